@@ -1,0 +1,260 @@
+"""Pins the CPU oracle before anything is compared against it (no GPU needed).
+
+Every check here is something the oracle's own formula does not restate: the reference's known-answer demo,
+exact integer arithmetic, closed forms, an exact-rational model of the fused chain, numpy's independent
+float16 / float64 routines.
+"""
+import numpy as np
+import pytest
+
+from backup_1_amd import workloads
+from exact_chain import fma_chain, gemm_exact_chain
+
+
+def bits(x):
+    return np.ascontiguousarray(x).view(np.uint32)
+
+
+# ---------------------------------------------------------------- GEMM chain -----------------------------------
+def test_reference_known_answer_pattern(oracle):
+    # test/test/CUDA_GEMM/CUDA_GEMM.cpp:24-42, main runs 2048^3 (:112-116)
+    M, K, N = 64, 2048, 48
+    A, B, printed, closed = workloads.known_answer_pattern(M, K, N)
+    assert abs(closed - 28612147.2) < 1e-3          # 0.01*(K-1)K(2K-1)/6 at K = 2048
+    D = oracle.sgemm_chain(A, B)
+    assert np.all(D == D[0, 0])                      # every element identical by construction
+    tol = 1e-5 * np.sqrt(K)
+    assert abs(float(D[0, 0]) - closed) / closed < tol
+    assert abs(float(D[0, 0]) - printed) / printed < tol
+    # and the chain itself, bit for bit, from exact rational arithmetic
+    assert bits(D[0, 0]) == bits(fma_chain(A[0, :], B[:, 0]))
+
+
+@pytest.mark.parametrize("shape", [(5, 7, 3), (17, 33, 9), (1, 1, 1), (2, 64, 2)])
+def test_chain_matches_exact_rational_model(oracle, shape):
+    M, K, N = shape
+    A = workloads.normal((M, K), 11)
+    B = workloads.uniform_pm1((K, N), 12)
+    C = workloads.normal((M, N), 13)
+    for fast in (False, True):
+        assert np.array_equal(bits(oracle.sgemm_chain(A, B, fast=fast)), bits(gemm_exact_chain(A, B)))
+        assert np.array_equal(bits(oracle.sgemm_chain(A, B, C, fast=fast)), bits(gemm_exact_chain(A, B, C)))
+
+
+def test_small_integer_products_are_exact(oracle):
+    M, K, N = 37, 1500, 53
+    A = workloads.small_ints((M, K), 1)
+    B = workloads.small_ints((K, N), 2)
+    want = (A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32)
+    assert np.array_equal(oracle.sgemm_chain(A, B, fast=False), want)
+    assert np.array_equal(oracle.sgemm_chain(A, B, fast=True), want)
+    assert np.array_equal(oracle.decx_cpu_sgemm(A, B), want)
+
+
+def test_permutation_identity_and_zero_A(oracle):
+    M, K = 29, 40
+    A = workloads.normal((M, K), 3)
+    perm = np.random.Generator(np.random.PCG64(4)).permutation(K)
+    P = np.zeros((K, K), dtype=np.float32)
+    P[perm, np.arange(K)] = 1.0                      # column j picks A[:, perm[j]]
+    assert np.array_equal(bits(oracle.sgemm_chain(A, P)), bits(A[:, perm]))
+    assert np.array_equal(bits(oracle.sgemm_chain(A, np.eye(K, dtype=np.float32))), bits(A))
+    C = workloads.normal((M, K), 5)
+    assert np.array_equal(bits(oracle.sgemm_chain(np.zeros_like(A), P, C)), bits(C))
+
+
+def test_transposed_operand_would_fail(oracle):
+    # a swapped/transposed operand must not slip through the checks above: A@B != (B.T@A.T) laid out the same
+    A = workloads.small_ints((8, 8), 6)
+    B = workloads.small_ints((8, 8), 7)
+    assert not np.array_equal(oracle.sgemm_chain(A, B), oracle.sgemm_chain(B, A))
+
+
+@pytest.mark.parametrize("shape", [(33, 70, 19), (128, 256, 130), (7, 1500, 45), (300, 9, 1031)])
+def test_fast_chain_bit_identical_to_scalar(oracle, shape):
+    M, K, N = shape
+    A = workloads.normal((M, K), 21)
+    B = workloads.normal((K, N), 22)
+    C = workloads.normal((M, N), 23)
+    assert np.array_equal(bits(oracle.sgemm_chain(A, B, fast=True)), bits(oracle.sgemm_chain(A, B, fast=False)))
+    assert np.array_equal(bits(oracle.sgemm_chain(A, B, C, fast=True)), bits(oracle.sgemm_chain(A, B, C, fast=False)))
+    rows = np.array([0, M - 1, M // 2], dtype=np.int32)
+    assert np.array_equal(bits(oracle.sgemm_chain_rows(A, B, rows)), bits(oracle.sgemm_chain(A, B, fast=False)[rows]))
+
+
+def test_pitched_operands(oracle):
+    # DECX containers are pitched (Matrix.h:24-27, :260): model with slices of wider arrays holding NaN padding
+    M, K, N = 10, 13, 11
+    Abuf = np.full((M, 16), np.nan, dtype=np.float32)
+    Bbuf = np.full((K, 16), np.nan, dtype=np.float32)
+    Abuf[:, :K] = workloads.normal((M, K), 31)
+    Bbuf[:, :N] = workloads.normal((K, N), 32)
+    A, B = Abuf[:, :K], Bbuf[:, :N]
+    want = gemm_exact_chain(A, B)
+    assert np.array_equal(bits(oracle.sgemm_chain(A, B, fast=False)), bits(want))
+    assert np.array_equal(bits(oracle.sgemm_chain(A, B, fast=True)), bits(want))
+
+
+# ---------------------------------------------------------------- DECX_cpu thread-pool SGEMM ------------------
+# variants of the reference dispatch: N%16 in {0,8}, M%32, K%64, panel count % 4 (sgemm_callers.h:1116-1248)
+_VARIANTS = []
+for n in (64, 72, 48, 56, 16, 8, 80, 104):          # panel counts 4,5(w8),3,4(w8),1,1(w8),5,7(w8)
+    for m in (96, 100):
+        for k in (128, 136):
+            _VARIANTS.append((m, k, n))
+_VARIANTS += [(1024, 1024, 1024), (31, 64, 16), (33, 8, 24), (200, 67, 50), (3, 5, 7)]
+
+
+@pytest.mark.parametrize("shape", _VARIANTS)
+def test_decx_cpu_sgemm_bit_identical_to_chain(oracle, shape):
+    M, K, N = shape
+    A = workloads.uniform_pm1((M, K), 41)
+    B = workloads.uniform_pm1((K, N), 42)
+    got = oracle.decx_cpu_sgemm(A, B)
+    want = oracle.sgemm_chain(A, B, fast=(M * N * K > 1 << 22))
+    assert np.array_equal(bits(got), bits(want))
+
+
+def test_decx_cpu_sgemm_thread_counts(oracle):
+    A = workloads.uniform_pm1((200, 300), 43)
+    B = workloads.uniform_pm1((300, 120), 44)
+    want = oracle.sgemm_chain(A, B)
+    for t in (1, 2, 5, 16, 64):
+        assert np.array_equal(bits(oracle.decx_cpu_sgemm(A, B, nthreads=t)), bits(want))
+    assert oracle.pool_size(64) == 16                # reference arrays are MAX_THREAD_NUM 16 (thread_pool.h:18)
+
+
+# ---------------------------------------------------------------- convolution ---------------------------------
+def _conv_bruteforce_f64(src, filt, flag):
+    H, W, C = src.shape
+    N, kh, kw, _ = filt.shape
+    oy, ox = (kh // 2, kw // 2) if flag == 1 else (0, 0)
+    Ho, Wo = (H, W) if flag == 1 else (H - 2 * (kh // 2), W - 2 * (kw // 2))
+    out = np.zeros((Ho, Wo, N), dtype=np.float64)
+    for y in range(Ho):
+        for x in range(Wo):
+            for n in range(N):
+                s = 0.0
+                for ki in range(kh):
+                    for kj in range(kw):
+                        sy, sx = y + ki - oy, x + kj - ox
+                        if 0 <= sy < H and 0 <= sx < W:
+                            for c in range(C):
+                                s += float(src[sy, sx, c]) * float(filt[n, ki, kj, c])
+                out[y, x, n] = s
+    return out
+
+
+def test_conv_all_ones_counts_in_image_taps(oracle):
+    # 3x3 same-size conv of ones with ones: C * (#taps inside the image) = 9C interior, 6C edge, 4C corner
+    H, W, C, N = 9, 12, 8, 4
+    src = np.ones((H, W, C), dtype=np.float32)
+    filt = np.ones((N, 3, 3, C), dtype=np.float32)
+    d = oracle.conv2_chain(src, filt, 1)
+    assert d.shape == (H, W, N)
+    assert np.all(d[1:-1, 1:-1] == 9 * C) and np.all(d[0, 1:-1] == 6 * C) and np.all(d[1:-1, 0] == 6 * C)
+    assert d[0, 0, 0] == 4 * C and d[-1, -1, -1] == 4 * C and d[0, -1, 1] == 4 * C
+    v = oracle.conv2_chain(src, filt, 0)
+    assert v.shape == (H - 2, W - 2, N) and np.all(v == 9 * C)
+    # config-4 numbers: C = 64 -> 576 / 384 / 256
+    assert 9 * 64 == 576 and 6 * 64 == 384 and 4 * 64 == 256
+
+
+def test_conv_impulse_gives_reversed_filter(oracle):
+    # cross-correlation (im2col.cuh:150-163): an impulse at (py,px,c0) makes dst(py-di, px-dj, n) = filt[n, kh/2+di, kw/2+dj, c0]
+    H, W, C, N, kh, kw = 11, 13, 4, 3, 5, 3
+    filt = workloads.normal((N, kh, kw, C), 51)
+    src = np.zeros((H, W, C), dtype=np.float32)
+    py, px, c0 = 5, 6, 2
+    src[py, px, c0] = 1.0
+    d = oracle.conv2_chain(src, filt, 1)
+    for di in range(-(kh // 2), kh // 2 + 1):
+        for dj in range(-(kw // 2), kw // 2 + 1):
+            assert np.array_equal(d[py - di, px - dj, :], filt[:, kh // 2 + di, kw // 2 + dj, c0])
+    d[py - kh // 2:py + kh // 2 + 1, px - kw // 2:px + kw // 2 + 1] = 0
+    assert not d.any()
+
+
+@pytest.mark.parametrize("case", [(6, 7, 4, 3, 3, 3, 1), (6, 7, 4, 3, 3, 3, 0), (5, 9, 8, 2, 5, 3, 1), (8, 8, 4, 5, 1, 1, 1),
+                                  (9, 6, 4, 2, 3, 5, 0)])
+def test_conv_vs_bruteforce(oracle, case):
+    H, W, C, N, kh, kw, flag = case
+    src = workloads.small_ints((H, W, C), 61)
+    filt = workloads.small_ints((N, kh, kw, C), 62)
+    want = _conv_bruteforce_f64(src, filt, flag)
+    assert np.array_equal(oracle.conv2_chain(src, filt, flag).astype(np.float64), want)     # integer-exact
+    srcr = workloads.uniform_01((H, W, C), 63)
+    filtr = workloads.normal((N, kh, kw, C), 64, sigma=0.05)
+    got = oracle.conv2_chain(srcr, filtr, flag)
+    np.testing.assert_allclose(got, _conv_bruteforce_f64(srcr, filtr, flag), rtol=0, atol=1e-5)
+
+
+def test_conv_chain_order_is_tap_major_channel_minor(oracle):
+    # bit-exact against the exact-rational chain run in k = (ki*kw+kj)*dpitch + c order (im2col.cuh:153);
+    # a channel-major or flipped order rounds differently on this data
+    H, W, C, N, kh, kw = 4, 5, 4, 2, 3, 3
+    src = workloads.normal((H, W, C), 71)
+    filt = workloads.normal((N, kh, kw, C), 72)
+    got = oracle.conv2_chain(src, filt, 1)
+    for (y, x, n) in [(0, 0, 0), (2, 3, 1), (3, 4, 0), (1, 2, 1)]:
+        a, b = [], []
+        for ki in range(kh):
+            for kj in range(kw):
+                sy, sx = y + ki - 1, x + kj - 1
+                for c in range(C):
+                    a.append(src[sy, sx, c] if (0 <= sy < H and 0 <= sx < W) else np.float32(0))
+                    b.append(filt[n, ki, kj, c])
+        assert bits(got[y, x, n]) == bits(fma_chain(a, b))
+
+
+def test_conv_strided_containers_and_bad_flag(oracle):
+    # Tensor rows are padded to wpitch = ceil4(W) pixels, filters to ceil4(kw) (Tensor.h:162-184, TensorArray.h:174-198)
+    H, W, C, N, kh, kw = 5, 6, 4, 2, 3, 3
+    sbuf = np.full((H, 8, C), np.nan, dtype=np.float32)
+    fbuf = np.full((N, kh, 4, C), np.nan, dtype=np.float32)
+    sbuf[:, :W] = workloads.small_ints((H, W, C), 81)
+    fbuf[:, :, :kw] = workloads.small_ints((N, kh, kw, C), 82)
+    got = oracle.conv2_chain(sbuf[:, :W], fbuf[:, :, :kw], 1)
+    want = _conv_bruteforce_f64(np.ascontiguousarray(sbuf[:, :W]), np.ascontiguousarray(fbuf[:, :, :kw]), 1)
+    assert np.array_equal(got.astype(np.float64), want)
+    with pytest.raises(ValueError):
+        oracle.conv2_chain(sbuf[:, :W], fbuf[:, :, :kw], 2)
+
+
+# ---------------------------------------------------------------- fp16 ----------------------------------------
+def test_half_conversion_matches_numpy_and_ieee(oracle):
+    known = {1.0: 0x3C00, -2.0: 0xC000, 65504.0: 0x7BFF, 65520.0: 0x7C00, 65519.99: 0x7BFF, 5.9604645e-8: 0x0001,
+             2.9802322e-8: 0x0000, 0.0: 0x0000, 1.0009765625: 0x3C01, 1.00048828125: 0x3C00, 1.00146484375: 0x3C02,
+             6.1035156e-5: 0x0400, 6.097555e-5: 0x03FF}
+    x = np.array(list(known.keys()), dtype=np.float32)
+    assert list(oracle.float_to_half(x)) == list(known.values())
+    r = np.random.Generator(np.random.PCG64(91))
+    v = np.concatenate([workloads.uniform_pm1((100000,), 92), workloads.normal((50000,), 93) * 1000,
+                        (r.random(50000, dtype=np.float32) * 1e-4).astype(np.float32),
+                        r.integers(0, 1 << 32, 200000, dtype=np.uint64).astype(np.uint32).view(np.float32)])
+    v = v[np.isfinite(v)]
+    with np.errstate(over="ignore"):
+        assert np.array_equal(oracle.float_to_half(v), v.astype(np.float16).view(np.uint16))
+    allh = np.arange(65536, dtype=np.uint16)
+    f = oracle.half_to_float(allh)
+    nf = allh.view(np.float16).astype(np.float32)
+    assert np.array_equal(f.view(np.uint32)[~np.isnan(nf)], nf.view(np.uint32)[~np.isnan(nf)])
+    assert np.all(np.isnan(f[np.isnan(nf)]))
+
+
+def test_f64_rows(oracle):
+    M, K, N = 20, 300, 70
+    A = workloads.small_ints((M, K), 101)
+    B = workloads.small_ints((K, N), 102)
+    rows = np.array([0, 7, 19], dtype=np.int32)
+    ref, ab = oracle.gemm_f64_rows_f16(oracle.float_to_half(A), oracle.float_to_half(B), rows)
+    assert np.array_equal(ref, (A.astype(np.int64) @ B.astype(np.int64))[rows].astype(np.float64))
+    assert np.array_equal(ab, (np.abs(A).astype(np.int64) @ np.abs(B).astype(np.int64))[rows].astype(np.float64))
+    Ar, Br = workloads.uniform_pm1((M, K), 103), workloads.uniform_pm1((K, N), 104)
+    ref32, ab32 = oracle.gemm_f64_rows_f32(Ar, Br, rows)
+    np.testing.assert_allclose(ref32, (Ar.astype(np.float64) @ Br.astype(np.float64))[rows], rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(ab32, (np.abs(Ar).astype(np.float64) @ np.abs(Br).astype(np.float64))[rows], rtol=1e-12)
+    Ah, Bh = oracle.float_to_half(Ar), oracle.float_to_half(Br)
+    refh, _ = oracle.gemm_f64_rows_f16(Ah, Bh, rows)
+    want = (Ah.view(np.float16).astype(np.float64) @ Bh.view(np.float16).astype(np.float64))[rows]
+    np.testing.assert_allclose(refh, want, rtol=1e-12, atol=1e-12)
