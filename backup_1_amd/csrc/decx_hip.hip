@@ -1,0 +1,387 @@
+// C ABI of libdecx_hip.so: device bring-up, memory, and the dispatch of the GEMM / convolution kernels.
+// Declarations and the reference interface each entry point stands in for: include/decx_hip.h.
+#include "../../include/decx_hip.h"
+
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "hgemm_tile.hpp"
+#include "sgemm_tile.hpp"
+
+using namespace decx_hip;
+
+namespace {
+
+struct Runtime {
+    bool is_init = false;
+    int device = -1;
+    int compute_units = 0;
+    int clock_khz = 0;
+    size_t hbm_bytes = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    int sgemm_variant = 0;
+    int hgemm_variant = 0;
+};
+Runtime g_rt;
+
+thread_local char g_err[512] = "No error\n";   // SUCCESS string of the reference, core/error.h:61
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    return fail(DECX_HIP_FAIL_HIP_BASE + (int)e, "%s: %s\n", what, hipGetErrorString(e));
+}
+
+#define HIP_TRY(expr)                                   \
+    do {                                                \
+        hipError_t e_ = (expr);                         \
+        if (e_ != hipSuccess) return hip_fail(e_, #expr); \
+    } while (0)
+
+int need_init() { return fail(DECX_HIP_FAIL_NOT_INIT, "CUDA should be initialized first\n"); }   // core/error.h:60
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int cdiv(int a, int b) { return (a + b - 1) / b; }
+
+// ---------------------------------------------------------------------------------------------------------------
+// fp32 launchers
+// ---------------------------------------------------------------------------------------------------------------
+template <class S, class ASrc, class BSrc, class Out>
+int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, float* D, const Out& out, int M, int N,
+                      int K) {
+    auto kern = sgemm_tile_kernel<S, ASrc, BSrc, Out>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)S::LDS_BYTES));
+        attr_done = true;
+    }
+    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    const long total = (long)tiles_m * tiles_n;
+    if (total > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
+    const int group_m = tiles_m < 8 ? tiles_m : 8;
+    hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream, a, b, Cin, ldc, D, out, M,
+                       N, K, tiles_m, tiles_n, group_m);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+// Tile shapes (variant numbers of decx_hip_set_sgemm_variant):
+//   1: 256x256x16, 2x2 waves of 128x128   -- large problems, highest reuse per LDS byte
+//   2: 128x128x16, 2x2 waves of  64x64    -- small problems, several workgroups per CU
+//   3: 256x128x16, 2x2 waves of 128x64    -- narrow N (the convolution's 128 filters)
+typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
+typedef SgemmShape<128, 128, 16, 2, 2> SShapeSmall;
+typedef SgemmShape<256, 128, 16, 2, 2> SShapeTall;
+
+int pick_sgemm_variant(int M, int N) {
+    if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 3) return g_rt.sgemm_variant;
+    const int cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+    const long big = (long)cdiv(M, 256) * cdiv(N, 256);
+    if (big * 10 >= (long)cus * 8) return 1;                 // at least ~0.8 tiles per CU
+    const long tall = (long)cdiv(M, 256) * cdiv(N, 128);
+    if (tall * 10 >= (long)cus * 7) return 3;
+    return 2;
+}
+
+template <class ASrc, class BSrc, class Out>
+int dispatch_sgemm(int variant, const ASrc& a, const BSrc& b, const float* Cin, int ldc, float* D, const Out& out, int M,
+                   int N, int K) {
+    switch (variant) {
+        case 1: return launch_sgemm_tile<SShapeBig>(a, b, Cin, ldc, D, out, M, N, K);
+        case 3: return launch_sgemm_tile<SShapeTall>(a, b, Cin, ldc, D, out, M, N, K);
+        default: return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K);
+    }
+}
+
+int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
+                  int N, int K) {
+    if (!g_rt.is_init) return need_init();
+    if (!A || !B || !D) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "null matrix pointer\n");
+    if (M <= 0 || N <= 0 || K <= 0) return fail(DECX_HIP_FAIL_DIMS, "Matrix Dims don't match each other");
+    if (lda < K || ldb < N || ldd < N || (Cin && ldc < N))
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "leading dimension smaller than the row length\n");
+    const int variant = pick_sgemm_variant(M, N);
+    const bool vec_a = aligned16(A) && lda % 4 == 0;
+    const bool vec_b = aligned16(B) && ldb % 4 == 0 && ldb >= 4;
+    DenseOut out{ldd};
+    if (vec_a && vec_b) {
+        DenseA<true> a{A, lda, M, K};
+        DenseB<true> b{B, ldb, N, K};
+        return dispatch_sgemm(variant, a, b, Cin, ldc, D, out, M, N, K);
+    }
+    // unaligned operands: element-wise loaders, one tile shape only
+    DenseA<false> a{A, lda, M, K};
+    DenseB<false> b{B, ldb, N, K};
+    return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K);
+}
+
+int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt, int N, int kh,
+                 int kw, size_t filt_stride, size_t filt_row_stride, float* dst, int dst_dpitch, size_t dst_row_stride,
+                 int flag) {
+    if (!g_rt.is_init) return need_init();
+    if (flag != DECX_HIP_CONV_NO_COMPENSATE && flag != DECX_HIP_CONV_ZERO_COMPENSATE)
+        return fail(DECX_HIP_FAIL_ERROR_FLAG, "This flag is meaningless in current context\n");   // core/error.h:67
+    if (!src || !filt || !dst) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "null tensor pointer\n");
+    if (H <= 0 || W <= 0 || N <= 0 || kh <= 0 || kw <= 0 || dpitch <= 0)
+        return fail(DECX_HIP_FAIL_DIMS, "Tensor Dims don't match each other");
+    if (dpitch % 4 != 0 || src_row_stride % 4 != 0 || filt_stride % 4 != 0 || filt_row_stride % 4 != 0 ||
+        !aligned16(src) || !aligned16(filt))
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "tensors must be 16-byte aligned with channel pitch a multiple of 4\n");
+    const int Hout = flag ? H : H - 2 * (kh / 2), Wout = flag ? W : W - 2 * (kw / 2);
+    if (Hout <= 0 || Wout <= 0) return fail(DECX_HIP_FAIL_DIMS, "kernel larger than the image\n");
+    if (src_row_stride < (size_t)W * dpitch || filt_row_stride < (size_t)kw * dpitch ||
+        filt_stride < (size_t)(kh - 1) * filt_row_stride + (size_t)kw * dpitch || dst_dpitch < N ||
+        dst_row_stride < (size_t)Wout * dst_dpitch)
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "stride smaller than the extent it spans\n");
+    const long Ml = (long)Hout * Wout, Kl = (long)kh * kw * dpitch;
+    if (Ml > 0x7fffffffL || Kl > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large\n");
+    const int M = (int)Ml, K = (int)Kl;
+    Im2colA a{src, H, W, dpitch, kh, kw, flag ? kh / 2 : 0, flag ? kw / 2 : 0, Wout, M, K, src_row_stride};
+    FilterB b{filt, N, K, dpitch, kw, filt_stride, filt_row_stride};
+    TensorOut out{Wout, dst_dpitch, dst_row_stride};
+    return dispatch_sgemm(pick_sgemm_variant(M, N), a, b, nullptr, 0, dst, out, M, N, K);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// fp16 launchers
+// ---------------------------------------------------------------------------------------------------------------
+// Tile shapes (variant numbers of decx_hip_set_hgemm_variant):
+//   1: 256x256x32, 2x2 waves of 128x128
+//   2: 128x128x32, 2x2 waves of  64x64
+typedef HgemmShape<256, 256, 32, 2, 2> HShapeBig;
+typedef HgemmShape<128, 128, 32, 2, 2> HShapeSmall;
+
+template <class S, bool VEC>
+int launch_hgemm_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
+                      int ldd, int M, int N, int K) {
+    auto kern = hgemm_tile_kernel<S, VEC>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)S::LDS_BYTES));
+        attr_done = true;
+    }
+    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    const long total = (long)tiles_m * tiles_n;
+    if (total > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
+    const int group_m = tiles_m < 8 ? tiles_m : 8;
+    hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream,
+                       reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
+                       reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N, K,
+                       tiles_m, tiles_n, group_m);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
+                  int ldd, int M, int N, int K) {
+    if (!g_rt.is_init) return need_init();
+    if (!A || !B || !D) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "null matrix pointer\n");
+    if (M <= 0 || N <= 0 || K <= 0) return fail(DECX_HIP_FAIL_DIMS, "Matrix Dims don't match each other");
+    if (lda < K || ldb < N || ldd < N || (Cin && ldc < N))
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "leading dimension smaller than the row length\n");
+    const bool vec = aligned16(A) && aligned16(B) && lda % 8 == 0 && ldb % 8 == 0 && ldb >= 8;
+    if (!vec) return launch_hgemm_tile<HShapeSmall, false>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
+    int variant = g_rt.hgemm_variant;
+    if (variant < 1 || variant > 2) {
+        const int cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+        variant = ((long)cdiv(M, 256) * cdiv(N, 256) * 10 >= (long)cus * 8) ? 1 : 2;
+    }
+    if (variant == 1) return launch_hgemm_tile<HShapeBig, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
+    return launch_hgemm_tile<HShapeSmall, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
+}
+
+int finish(int rc) {
+    if (rc != 0) return rc;
+    HIP_TRY(hipStreamSynchronize(g_rt.stream));
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int decx_hip_init(int* device) {
+    if (!g_rt.is_init) {
+        int count = 0;
+        HIP_TRY(hipGetDeviceCount(&count));
+        if (count <= 0) return fail(DECX_HIP_FAIL_NOT_INIT, "no HIP device visible\n");
+        int dev = 0;
+        HIP_TRY(hipGetDevice(&dev));
+        hipDeviceProp_t prop;
+        HIP_TRY(hipGetDeviceProperties(&prop, dev));
+        if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+            return fail(DECX_HIP_FAIL_NOT_INIT, "device %d is %s; this library carries gfx950 code only\n", dev,
+                        prop.gcnArchName);
+        g_rt.device = dev;
+        g_rt.compute_units = prop.multiProcessorCount;
+        g_rt.clock_khz = prop.clockRate;
+        g_rt.hbm_bytes = prop.totalGlobalMem;
+        HIP_TRY(hipStreamCreateWithFlags(&g_rt.stream, hipStreamNonBlocking));
+        HIP_TRY(hipEventCreate(&g_rt.ev_start));
+        HIP_TRY(hipEventCreate(&g_rt.ev_stop));
+        g_rt.is_init = true;
+    }
+    if (device) *device = g_rt.device;
+    return 0;
+}
+
+int decx_hip_is_init(void) { return g_rt.is_init ? 1 : 0; }
+
+int decx_hip_device_info(int* compute_units, int* clock_khz, size_t* hbm_bytes) {
+    if (!g_rt.is_init) return need_init();
+    if (compute_units) *compute_units = g_rt.compute_units;
+    if (clock_khz) *clock_khz = g_rt.clock_khz;
+    if (hbm_bytes) *hbm_bytes = g_rt.hbm_bytes;
+    return 0;
+}
+
+int decx_hip_malloc(void** dptr, size_t bytes) {
+    if (!g_rt.is_init) return need_init();
+    if (!dptr) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "null output pointer\n");
+    *dptr = nullptr;
+    if (hipMalloc(dptr, bytes ? bytes : 1) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(DECX_HIP_FAIL_ALLOCATION, "Fail to allocate memory\n");   // core/error.h:65
+    }
+    return 0;
+}
+
+int decx_hip_free(void* dptr) {
+    if (!dptr) return 0;
+    HIP_TRY(hipFree(dptr));
+    return 0;
+}
+
+int decx_hip_memset(void* dptr, int value, size_t bytes) {
+    if (!g_rt.is_init) return need_init();
+    HIP_TRY(hipMemsetAsync(dptr, value, bytes, g_rt.stream));
+    HIP_TRY(hipStreamSynchronize(g_rt.stream));
+    return 0;
+}
+
+int decx_hip_host_malloc(void** hptr, size_t bytes) {
+    if (!g_rt.is_init) return need_init();
+    if (!hptr) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "null output pointer\n");
+    *hptr = nullptr;
+    if (hipHostMalloc(hptr, bytes ? bytes : 1, hipHostMallocDefault) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(DECX_HIP_FAIL_ALLOCATION, "Fail to allocate memory\n");
+    }
+    return 0;
+}
+
+int decx_hip_host_free(void* hptr) {
+    if (!hptr) return 0;
+    HIP_TRY(hipHostFree(hptr));
+    return 0;
+}
+
+static hipMemcpyKind copy_kind(int direction) {
+    switch (direction) {
+        case DECX_HIP_H2D: return hipMemcpyHostToDevice;
+        case DECX_HIP_D2H: return hipMemcpyDeviceToHost;
+        default: return hipMemcpyDeviceToDevice;
+    }
+}
+
+int decx_hip_memcpy2d(void* dst, size_t dst_pitch_bytes, const void* src, size_t src_pitch_bytes, size_t width_bytes,
+                      size_t rows, int direction) {
+    if (!g_rt.is_init) return need_init();
+    if (direction < DECX_HIP_H2D || direction > DECX_HIP_D2D) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "bad copy direction\n");
+    if (width_bytes == 0 || rows == 0) return 0;
+    if (dst_pitch_bytes < width_bytes || src_pitch_bytes < width_bytes)
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "pitch smaller than the row width\n");
+    HIP_TRY(hipMemcpy2DAsync(dst, dst_pitch_bytes, src, src_pitch_bytes, width_bytes, rows, copy_kind(direction),
+                             g_rt.stream));
+    HIP_TRY(hipStreamSynchronize(g_rt.stream));
+    return 0;
+}
+
+int decx_hip_memcpy(void* dst, const void* src, size_t bytes, int direction) {
+    if (!g_rt.is_init) return need_init();
+    if (direction < DECX_HIP_H2D || direction > DECX_HIP_D2D) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "bad copy direction\n");
+    if (bytes == 0) return 0;
+    HIP_TRY(hipMemcpyAsync(dst, src, bytes, copy_kind(direction), g_rt.stream));
+    HIP_TRY(hipStreamSynchronize(g_rt.stream));
+    return 0;
+}
+
+int decx_hip_sync(void) {
+    if (!g_rt.is_init) return need_init();
+    HIP_TRY(hipDeviceSynchronize());
+    return 0;
+}
+
+int decx_hip_sgemm_async(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd,
+                         int M, int N, int K) {
+    return sgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
+}
+int decx_hip_sgemm(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
+                   int N, int K) {
+    return finish(sgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K));
+}
+
+int decx_hip_hgemm_f32acc_async(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
+                                uint16_t* D, int ldd, int M, int N, int K) {
+    return hgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
+}
+int decx_hip_hgemm_f32acc(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
+                          int ldd, int M, int N, int K) {
+    return finish(hgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K));
+}
+
+int decx_hip_conv2_im2col_f32_async(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt,
+                                    int N, int kh, int kw, size_t filt_stride, size_t filt_row_stride, float* dst,
+                                    int dst_dpitch, size_t dst_row_stride, int flag) {
+    return conv_enqueue(src, H, W, dpitch, src_row_stride, filt, N, kh, kw, filt_stride, filt_row_stride, dst, dst_dpitch,
+                        dst_row_stride, flag);
+}
+int decx_hip_conv2_im2col_f32(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt, int N,
+                              int kh, int kw, size_t filt_stride, size_t filt_row_stride, float* dst, int dst_dpitch,
+                              size_t dst_row_stride, int flag) {
+    return finish(conv_enqueue(src, H, W, dpitch, src_row_stride, filt, N, kh, kw, filt_stride, filt_row_stride, dst,
+                               dst_dpitch, dst_row_stride, flag));
+}
+
+int decx_hip_timer_start(void) {
+    if (!g_rt.is_init) return need_init();
+    HIP_TRY(hipEventRecord(g_rt.ev_start, g_rt.stream));
+    return 0;
+}
+
+int decx_hip_timer_stop(float* milliseconds) {
+    if (!g_rt.is_init) return need_init();
+    HIP_TRY(hipEventRecord(g_rt.ev_stop, g_rt.stream));
+    HIP_TRY(hipEventSynchronize(g_rt.ev_stop));
+    float ms = 0.f;
+    HIP_TRY(hipEventElapsedTime(&ms, g_rt.ev_start, g_rt.ev_stop));
+    if (milliseconds) *milliseconds = ms;
+    return 0;
+}
+
+const char* decx_hip_last_error(void) { return g_err; }
+
+int decx_hip_set_sgemm_variant(int variant) {
+    int prev = g_rt.sgemm_variant;
+    g_rt.sgemm_variant = variant;
+    return prev;
+}
+int decx_hip_set_hgemm_variant(int variant) {
+    int prev = g_rt.hgemm_variant;
+    g_rt.hgemm_variant = variant;
+    return prev;
+}
+
+}  // extern "C"

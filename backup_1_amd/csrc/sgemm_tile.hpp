@@ -1,0 +1,352 @@
+// fp32 MFMA contraction tile for gfx950, shared by the dense GEMM and the fused im2col convolution.
+//
+// One workgroup owns a BM x BN tile of the result and walks K in steps of BK.  Its waves are laid out WAVES_M x
+// WAVES_N, each owning a (BM/WAVES_M) x (BN/WAVES_N) sub-tile as a grid of 32x32 v_mfma_f32_32x32x2_f32 blocks
+// whose accumulators stay in registers for the whole K walk.
+//
+// Staging: global -> registers -> LDS, two LDS buffers, one barrier per K step; the loads for step t+1 are issued
+// before the MFMAs of step t.  Both operands are kept in LDS as float4 "k-quads":
+//   A quad (q, m) = A[m][4q .. 4q+3]          at  As[q][m]             (row of BM+4 quads: the +4 staggers the four
+//                                                                       q-planes over the banks for the staging stores)
+//   B quad (q, n) = B[4q .. 4q+3][n]          at  Bs[q][n + (n >> 4)]  (4x4 register transpose while staging; the
+//                                                                       n>>4 skew keeps the 64-byte-strided staging
+//                                                                       stores off each other's banks)
+// so that one ds_read_b128 per 32-row block feeds four MFMAs.  The MFMA's two k-slots (lanes 0-31 / 32-63) take
+// quads 2s and 2s+1: within a quad pair the products are summed in the order k = 8s+e (lanes 0-31) and 8s+4+e
+// (lanes 32-63), e = 0..3 -- a fixed permutation of k inside each group of 8, applied identically to A and B.
+//
+// Ragged edges: rows >= M and columns >= N are read from clamped (valid) addresses and never stored; only the last,
+// partial K step zero-fills (both operands, so that 0 * Inf cannot appear).  No padded copies exist anywhere.
+#pragma once
+#include <type_traits>
+#include "tile_common.hpp"
+
+namespace decx_hip {
+
+// ---------------------------------------------------------------------------------------------------------------
+// A-operand sources.  Interface:
+//   RowState row_state(int m)                       per-row values that do not change along K
+//   template<bool TAIL> f32x4 load(rs, k)           A[m][k..k+3]; TAIL zero-fills elements with k >= K
+//   size_t out_offset(int m)                        where row m of the result starts, in elements
+// ---------------------------------------------------------------------------------------------------------------
+template <bool VEC>
+struct DenseA {
+    const float* A;
+    int lda, M, K;
+    struct RowState {
+        const float* row;
+    };
+    __device__ __forceinline__ RowState row_state(int m) const {
+        RowState rs;
+        rs.row = A + (size_t)(m < M ? m : M - 1) * lda;
+        return rs;
+    }
+    template <bool TAIL>
+    __device__ __forceinline__ f32x4 load(const RowState& rs, int k) const {
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        if (VEC) {
+            if (!TAIL) {
+                v = *reinterpret_cast<const f32x4*>(rs.row + k);
+            } else if (k < K) {
+                v = *reinterpret_cast<const f32x4*>(rs.row + k);   // lda % 4 == 0 keeps the quad inside the pitch
+                if (k + 1 >= K) v[1] = 0.f;
+                if (k + 2 >= K) v[2] = 0.f;
+                if (k + 3 >= K) v[3] = 0.f;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (k + e < K) v[e] = rs.row[k + e];
+        }
+        return v;
+    }
+};
+
+// The im2col view of a channel-innermost tensor: row m = (y, x) of the output, column k = (ki*kw + kj)*dpitch + c.
+struct Im2colA {
+    const float* src;
+    int H, W, dpitch, kh, kw, oy, ox, Wout, Mtot, K;
+    size_t row_stride;
+    struct RowState {
+        int y, x;   // output pixel, already shifted by (-oy, -ox)
+    };
+    __device__ __forceinline__ RowState row_state(int m) const {
+        if (m >= Mtot) m = Mtot - 1;
+        RowState rs;
+        rs.y = m / Wout - oy;
+        rs.x = m % Wout - ox;
+        return rs;
+    }
+    template <bool TAIL>
+    __device__ __forceinline__ f32x4 load(const RowState& rs, int k) const {
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        if (TAIL && k >= K) return v;           // K = kh*kw*dpitch is a multiple of 4: quads never straddle it
+        const int tap = k / dpitch, c = k - tap * dpitch;
+        const int ki = tap / kw, kj = tap - ki * kw;
+        const int sy = rs.y + ki, sx = rs.x + kj;
+        if (sy >= 0 && sy < H && sx >= 0 && sx < W)
+            v = *reinterpret_cast<const f32x4*>(src + (size_t)sy * row_stride + (size_t)sx * dpitch + c);
+        return v;
+    }
+};
+
+// Result addressing: dense matrices (row m at m*ld) or the convolution's output tensor (pixel (y,x) at
+// y*row_stride + x*dpitch).
+struct DenseOut {
+    int ld;
+    __device__ __forceinline__ size_t offset(int m) const { return (size_t)m * ld; }
+};
+struct TensorOut {
+    int Wout, dpitch;
+    size_t row_stride;
+    __device__ __forceinline__ size_t offset(int m) const {
+        const int y = m / Wout, x = m - y * Wout;
+        return (size_t)y * row_stride + (size_t)x * dpitch;
+    }
+};
+
+// ---------------------------------------------------------------------------------------------------------------
+// B-operand sources.  Interface (S = SgemmShape):
+//   quads<S>()                                   staging registers (float4) per thread and K step
+//   load<S, TAIL>(stage, tid, k0, bn0)           fetch this thread's share of B[k0 .. k0+BK) x [bn0 .. bn0+BN)
+//   store<S>(plane, stage, tid)                  write it to the LDS planes as k-quads at [q][n + (n >> 4)]
+// ---------------------------------------------------------------------------------------------------------------
+// B as a row-major K x N matrix: a thread takes a 4(k) x 4(n) block with four 16-byte row loads (consecutive lanes
+// -> consecutive column groups, so a wave reads whole rows) and transposes it in registers into four k-quads.
+template <bool VEC>
+struct DenseB {
+    const float* B;
+    int ldb, N, K;
+    template <class S>
+    static constexpr int tasks() { return S::KQ * (S::BN / 4); }
+    template <class S>
+    static constexpr int passes() { return (tasks<S>() + S::NT - 1) / S::NT; }
+    template <class S>
+    static constexpr int quads() { return 4 * passes<S>(); }
+
+    template <class S, bool TAIL>
+    __device__ __forceinline__ void load(f32x4* st, int tid, int k0, int bn0) const {
+        constexpr int CG = S::BN / 4;
+#pragma unroll
+        for (int p = 0; p < passes<S>(); ++p) {
+            const int task = tid + p * S::NT;
+            if (tasks<S>() % S::NT != 0 && task >= tasks<S>()) break;
+            const int q = task / CG, cg = task % CG;
+            const int col = bn0 + 4 * cg;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int k = k0 + 4 * q + r;
+                f32x4 v = {0.f, 0.f, 0.f, 0.f};
+                if (!TAIL || k < K) {
+                    if (VEC) {
+                        const int cc = col <= ldb - 4 ? col : ldb - 4;   // stay inside the pitch; such columns are never stored
+                        v = *reinterpret_cast<const f32x4*>(B + (size_t)k * ldb + cc);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (col + e < N) v[e] = B[(size_t)k * ldb + col + e];
+                    }
+                }
+                st[4 * p + r] = v;
+            }
+        }
+    }
+    template <class S>
+    __device__ __forceinline__ void store(f32x4* plane, const f32x4* st, int tid) const {
+        constexpr int CG = S::BN / 4;
+#pragma unroll
+        for (int p = 0; p < passes<S>(); ++p) {
+            const int task = tid + p * S::NT;
+            if (tasks<S>() % S::NT != 0 && task >= tasks<S>()) break;
+            const int q = task / CG, cg = task % CG;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int n = 4 * cg + j;
+                f32x4 t = {st[4 * p + 0][j], st[4 * p + 1][j], st[4 * p + 2][j], st[4 * p + 3][j]};
+                plane[q * S::B_ROW + n + (n >> 4)] = t;
+            }
+        }
+    }
+};
+
+// B as a bank of N filters, filter n holding its taps channel-innermost: column n of the lowered GEMM is filter n and
+// four consecutive k (same tap, four channels) are already contiguous in memory, so a k-quad is one 16-byte load.
+struct FilterB {
+    const float* filt;
+    int N, K, dpitch, kw;
+    size_t filt_stride, filt_row_stride;
+    template <class S>
+    static constexpr int quads() { return S::KQ * S::BN / S::NT; }
+
+    template <class S, bool TAIL>
+    __device__ __forceinline__ void load(f32x4* st, int tid, int k0, int bn0) const {
+        static_assert((S::KQ * S::BN) % S::NT == 0, "filter staging must divide evenly");
+#pragma unroll
+        for (int j = 0; j < quads<S>(); ++j) {
+            const int id = tid + j * S::NT;
+            const int q = id % S::KQ;
+            int n = bn0 + id / S::KQ;
+            if (n >= N) n = N - 1;
+            const int k = k0 + 4 * q;
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            if (!TAIL || k < K) {
+                const int tap = k / dpitch, c = k - tap * dpitch;
+                const int ki = tap / kw, kj = tap - ki * kw;
+                v = *reinterpret_cast<const f32x4*>(filt + (size_t)n * filt_stride + (size_t)ki * filt_row_stride +
+                                                    (size_t)kj * dpitch + c);
+            }
+            st[j] = v;
+        }
+    }
+    template <class S>
+    __device__ __forceinline__ void store(f32x4* plane, const f32x4* st, int tid) const {
+#pragma unroll
+        for (int j = 0; j < quads<S>(); ++j) {
+            const int id = tid + j * S::NT;
+            const int q = id % S::KQ, n = id / S::KQ;
+            plane[q * S::B_ROW + n + (n >> 4)] = st[j];
+        }
+    }
+};
+
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_>
+struct SgemmShape {
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+    static constexpr int NT = WAVES_M * WAVES_N * kWave;
+    static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    static constexpr int MI = WM / 32, NI = WN / 32;
+    static constexpr int KQ = BK / 4;                         // k-quads per step
+    static constexpr int A_ROW = BM + 4;                      // quads per A plane
+    static constexpr int B_ROW = BN + BN / 16;                // quads per B plane
+    static constexpr int A_PASSES = (BM * KQ) / NT;           // float4 global loads of A per thread per step
+    static constexpr size_t LDS_BYTES = 2 * (size_t)KQ * (A_ROW + B_ROW) * sizeof(f32x4);
+    static_assert(BM % (WAVES_M * 32) == 0 && BN % (WAVES_N * 32) == 0, "wave tile must be whole 32x32 blocks");
+    static_assert(BK % 8 == 0, "a K step is whole quad pairs");
+    static_assert((BM * KQ) % NT == 0, "A staging must divide evenly");
+    static_assert(NT % KQ == 0, "A staging: KQ lanes per row");
+};
+
+template <class S, class ASrc, class BSrc, class Out>
+__global__ __launch_bounds__(S::NT) void sgemm_tile_kernel(ASrc a_src, BSrc b_src, const float* Cin, int ldc, float* D,
+                                                           Out out, int M, int N, int K, int tiles_m, int tiles_n,
+                                                           int group_m) {
+    constexpr int BM = S::BM, BN = S::BN, BK = S::BK, NT = S::NT, KQ = S::KQ, MI = S::MI, NI = S::NI;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    f32x4* As = reinterpret_cast<f32x4*>(lds_raw);                       // [2][KQ][A_ROW]
+    f32x4* Bs = As + 2 * KQ * S::A_ROW;                                  // [2][KQ][B_ROW]
+
+    const TileCoord tc = xcd_grouped_tile(blockIdx.x, tiles_m, tiles_n, group_m);
+    const int bm0 = tc.tm * BM, bn0 = tc.tn * BN;
+    const int tid = threadIdx.x;
+    const int wave = tid / kWave, lane = tid % kWave;
+    const int wm0 = (wave / S::WAVES_N) * S::WM, wn0 = (wave % S::WAVES_N) * S::WN;
+    const int li = lane & 31, lh = lane >> 5;
+
+    // ---- staging assignment -------------------------------------------------------------------------------
+    // A: KQ consecutive lanes cover one row's BK floats (one 16-byte quad each)
+    const int a_q = tid % KQ, a_r = tid / KQ;
+    constexpr int A_RSTEP = NT / KQ;
+    typename ASrc::RowState a_rs[S::A_PASSES];
+#pragma unroll
+    for (int p = 0; p < S::A_PASSES; ++p) a_rs[p] = a_src.row_state(bm0 + a_r + p * A_RSTEP);
+    f32x4 a_stage[S::A_PASSES];
+    f32x4 b_stage[BSrc::template quads<S>()];
+
+    auto load_stage = [&](int k0, auto tail_tag) {
+        constexpr bool TAIL = decltype(tail_tag)::value;
+#pragma unroll
+        for (int p = 0; p < S::A_PASSES; ++p) a_stage[p] = a_src.template load<TAIL>(a_rs[p], k0 + 4 * a_q);
+        b_src.template load<S, TAIL>(b_stage, tid, k0, bn0);
+    };
+
+    auto store_stage = [&](int buf) {
+        f32x4* Ab = As + buf * KQ * S::A_ROW;
+#pragma unroll
+        for (int p = 0; p < S::A_PASSES; ++p) Ab[a_q * S::A_ROW + a_r + p * A_RSTEP] = a_stage[p];
+        b_src.template store<S>(Bs + buf * KQ * S::B_ROW, b_stage, tid);
+    };
+
+    // ---- accumulators: start from C for dst = A*B + C (the reference pre-loads them too, GEMM.cuh:223) ---------
+    f32x16 acc[MI][NI];
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
+    if (Cin != nullptr) {
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                if (m < M) {
+                    const float* crow = Cin + (size_t)m * ldc;
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni) {
+                        const int n = bn0 + wn0 + ni * 32 + li;
+                        if (n < N) acc[mi][ni][r] = crow[n];
+                    }
+                }
+            }
+    }
+
+    const int full_steps = K / BK;
+    const int steps = (K + BK - 1) / BK;
+
+    if (full_steps > 0) load_stage(0, std::false_type{});
+    else load_stage(0, std::true_type{});
+    store_stage(0);
+    __syncthreads();
+
+    for (int t = 0; t < steps; ++t) {
+        const int buf = t & 1;
+        if (t + 1 < steps) {
+            if (t + 1 < full_steps) load_stage((t + 1) * BK, std::false_type{});
+            else load_stage((t + 1) * BK, std::true_type{});
+        }
+        const f32x4* Ab = As + buf * KQ * S::A_ROW;
+        const f32x4* Bb = Bs + buf * KQ * S::B_ROW;
+#pragma unroll
+        for (int s = 0; s < KQ / 2; ++s) {
+            f32x4 af[MI], bf[NI];
+            const int q = 2 * s + lh;
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi) af[mi] = Ab[q * S::A_ROW + wm0 + mi * 32 + li];
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni) {
+                const int n = wn0 + ni * 32 + li;
+                bf[ni] = Bb[q * S::B_ROW + n + (n >> 4)];
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni)
+                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[mi][e], bf[ni][e], acc[mi][ni], 0, 0, 0);
+        }
+        if (t + 1 < steps) {
+            store_stage(buf ^ 1);     // that buffer was last read before the previous barrier
+            __syncthreads();
+        }
+    }
+
+    // ---- epilogue: each lane holds column li of its 32-wide block; a half-wave writes 128 contiguous bytes ------
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+            if (m < M) {
+                float* drow = D + out.offset(m);
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni) {
+                    const int n = bn0 + wn0 + ni * 32 + li;
+                    if (n < N) drow[n] = acc[mi][ni][r];
+                }
+            }
+        }
+}
+
+}  // namespace decx_hip

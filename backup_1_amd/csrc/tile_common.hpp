@@ -1,0 +1,44 @@
+// Shared pieces of the gfx950 contraction kernels: vector types, the XCD-aware tile walk, status codes.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace decx_hip {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;      // CDNA wavefront width
+constexpr int kXcds = 8;       // MI355X: 8 accelerator complex dies, 32 CUs and one 4 MiB L2 each
+
+struct TileCoord {
+    int tm, tn;
+};
+
+// Workgroups are handed to the 8 XCDs round-robin by linear id.  Re-number them so that the ids living on one XCD
+// form one contiguous run of a "grouped" raster (group_m tile-rows tall, walked column by column): the tiles that
+// are resident on an XCD at the same time then share A row-panels and B column-panels in that XCD's private L2.
+__device__ __forceinline__ TileCoord xcd_grouped_tile(int pid, int tiles_m, int tiles_n, int group_m) {
+    const int total = tiles_m * tiles_n;
+    const int xcd = pid % kXcds;
+    const int local = pid / kXcds;
+    const int base = total / kXcds, rem = total % kXcds;
+    const int start = xcd * base + (xcd < rem ? xcd : rem);
+    const int id = start + local;
+    const int per_group = group_m * tiles_n;
+    const int group = id / per_group;
+    const int first_m = group * group_m;
+    const int rows = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
+    const int in_group = id - group * per_group;
+    TileCoord t;
+    t.tm = first_m + in_group % rows;
+    t.tn = in_group / rows;
+    return t;
+}
+
+}  // namespace decx_hip

@@ -1,0 +1,135 @@
+/*
+ * C ABI of the MI355X (gfx950) dense-contraction library, libdecx_hip.so.
+ *
+ * This is the boundary the DECX C++ API (de::cuda::GEMM, de::cuda::Conv2_MK_im2col and the Matrix / GPU_Matrix /
+ * Tensor / TensorArray containers) binds to.  DECX itself has no FFI layer: its API functions call CUDA directly.
+ * Each entry point below names the piece of the reference it stands in for (paths relative to the reference tree).
+ *
+ * Conventions
+ *   - plain pointers and sizes only; every matrix / tensor pointer is a DEVICE pointer unless the name says host;
+ *   - dimensions are the true (unpadded) ones, leading dimensions ("ld", "stride", "pitch") are in ELEMENTS;
+ *   - return value 0 = success, 1..0x10 = the matching decx::DECX_error_types value (handles/decx_handles.h:6-38),
+ *     >= 1000 = 1000 + hipError_t.  Nothing here calls exit(); the reference does on CUDA errors (core/error.h:32-45);
+ *   - calls without the _async suffix block until the result is complete, like the reference's API functions
+ *     (cudaDeviceSynchronize at GEMM.h:122, :450; conv2_mk_im2col.h:268);
+ *   - one process drives one GPU; the library is not thread-safe (neither is the reference: global pools, no locks).
+ */
+#ifndef DECX_HIP_H_
+#define DECX_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* decx::DECX_error_types values used on this path (handles/decx_handles.h:6-38) */
+#define DECX_HIP_SUCCESS              0x00
+#define DECX_HIP_FAIL_NOT_INIT        0x01
+#define DECX_HIP_FAIL_DIMS            0x03
+#define DECX_HIP_FAIL_ERROR_FLAG      0x0b
+#define DECX_HIP_FAIL_ERROR_PARAMS    0x0d
+#define DECX_HIP_FAIL_ALLOCATION      0x10
+#define DECX_HIP_FAIL_HIP_BASE        1000
+
+/* decx::conv_property (convolution/CUDA/conv_flags.h:16-20) */
+#define DECX_HIP_CONV_NO_COMPENSATE   0
+#define DECX_HIP_CONV_ZERO_COMPENSATE 1
+
+/* copy directions for decx_hip_memcpy / decx_hip_memcpy2d */
+#define DECX_HIP_H2D 1
+#define DECX_HIP_D2H 2
+#define DECX_HIP_D2D 3
+
+/* de::InitCuda() (core/configs/config.h:73-78): selects the current device, checks it is gfx950, creates the
+ * library's stream.  *device (nullable) receives the device ordinal.  Every compute entry point returns
+ * DECX_HIP_FAIL_NOT_INIT before this has succeeded (the decx::cuP.is_init gate, GEMM.h:63). */
+int decx_hip_init(int* device);
+int decx_hip_is_init(void);
+
+/* Number of compute units and the shader clock in kHz of the initialised device (decx::cuP.prop, config.h:75). */
+int decx_hip_device_info(int* compute_units, int* clock_khz, size_t* hbm_bytes);
+
+/* decx::alloc::_device_malloc / _device_dealloc (core/allocators.h:119-247), without the pool behind them. */
+int decx_hip_malloc(void** dptr, size_t bytes);
+int decx_hip_free(void* dptr);
+/* cudaMemset in _GPU_Matrix::alloc_data_space (classes/GPU_Matrix.h:142-168) */
+int decx_hip_memset(void* dptr, int value, size_t bytes);
+/* decx::alloc::_host_fixed_page_malloc (cudaHostAlloc, store type Page_Locked, classes/store_types.h:24-28) */
+int decx_hip_host_malloc(void** hptr, size_t bytes);
+int decx_hip_host_free(void* hptr);
+/* cudaMemcpy2D in _GPU_Matrix::Load_from_host / Load_to_host (classes/GPU_Matrix.h:334-354) and the
+ * cudaMemcpy2DAsync calls of the host-matrix GEMM (GEMM.h:109-120).  Pitches and width in BYTES. */
+int decx_hip_memcpy2d(void* dst, size_t dst_pitch_bytes, const void* src, size_t src_pitch_bytes, size_t width_bytes,
+                      size_t rows, int direction);
+int decx_hip_memcpy(void* dst, const void* src, size_t bytes, int direction);
+/* cudaDeviceSynchronize */
+int decx_hip_sync(void);
+
+/* de::cuda::GEMM(GPU_Matrix<float>& A, B, dst)            GEMM.h:398-454  (Cin == NULL)
+ * de::cuda::GEMM(GPU_Matrix<float>& A, B, C, dst)         GEMM.h:46       (Cin != NULL, dst = A*B + C)
+ * and, between the H2D / D2H copies, the kernel step of the host-matrix overloads (decx::sGEMM_part,
+ * GEMM3_macros.h:65-78).  Replaces cu_GEMM_fp32_spec / _ABC_spec (GEMM.cuh:31, :206) and the ragged variants
+ * (GEMM_nonuniform.cuh:32-693).
+ *   D[i*ldd + j] = Cin[i*ldc + j] + sum_k A[i*lda + k] * B[k*ldb + j],  0<=i<M, 0<=j<N, 0<=k<K, fp32 throughout.
+ * M, N, K are arbitrary positive sizes: ragged edges are handled inside the kernel, no padded copies are made.
+ * Cin may alias D.  Fast path needs A, B 16-byte aligned with lda, ldb multiples of 4 (always true for DECX
+ * containers, whose pitch is a multiple of 8 floats, Matrix.h:24-27); otherwise a slower element-wise loader runs. */
+int decx_hip_sgemm(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
+                   int N, int K);
+int decx_hip_sgemm_async(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd,
+                         int M, int N, int K);
+
+/* de::cuda::GEMM(GPU_Matrix<de::Half>& ...)               GEMM.h:457-519 (+ the A*B+C overload, GEMM.h:49)
+ * Replaces cu_GEMM_fp16_spec and its variants (GEMM.cuh:119, :297; GEMM_nonuniform.cuh:712-1334).
+ * Operands and result are IEEE binary16 bit patterns (de::Half{unsigned short val}, classes/classes_util.h:58-63).
+ * Products are accumulated in fp32 and rounded to binary16 (nearest even) once, on store; the reference accumulates
+ * in binary16 (GEMM_kernel_def.cuh:100-121), which this library deliberately does not reproduce.
+ * Fast path needs A, B 16-byte aligned with lda, ldb multiples of 8 (DECX pitch is a multiple of 16 halves). */
+int decx_hip_hgemm_f32acc(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
+                          int ldd, int M, int N, int K);
+int decx_hip_hgemm_f32acc_async(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
+                                uint16_t* D, int ldd, int M, int N, int K);
+
+/* de::cuda::Conv2_MK_im2col(Tensor<float>& src, TensorArray<float>& kernel, Tensor<float>& dst, int flag)
+ * (convolution/CUDA/im2col/conv2_mk_im2col.h:25, :278-306): the device part, i.e. what cu_sIm2Col_r8_within
+ * (im2col.cuh:86-178) followed by cu_conv_eq_mm (eq_GEMM.cuh:109-209) produce.  The patch matrix is never built:
+ * the GEMM's A-tile loader reads the tensor directly.
+ *   src  : H x W pixels, dpitch channels each (dpitch % 4 == 0), pixel (y,x) at src + y*src_row_stride + x*dpitch
+ *          (Tensor.h:389-394);
+ *   filt : N filters kh x kw x dpitch, tap (ki,kj) of filter n at filt + n*filt_stride + ki*filt_row_stride + kj*dpitch
+ *          (TensorArray.h:521-525);
+ *   dst  : dst(y,x,n) at dst + y*dst_row_stride + x*dst_dpitch + n;
+ *   flag : DECX_HIP_CONV_ZERO_COMPENSATE -> H x W outputs, input taken as 0 outside the image;
+ *          DECX_HIP_CONV_NO_COMPENSATE   -> (H-2*(kh/2)) x (W-2*(kw/2)) outputs;  anything else -> DECX_HIP_FAIL_ERROR_FLAG.
+ *   dst(y,x,n) = sum over k = (ki*kw + kj)*dpitch + c of src(y+ki-oy, x+kj-ox, c) * filt(n,ki,kj,c),
+ *   (oy,ox) = (kh/2, kw/2) for ZERO_COMPENSATE, (0,0) otherwise: cross-correlation, stride 1 (im2col.cuh:150-163).
+ * Channels c in [C, dpitch) are read like any other, so the containers' zero padding must be zero.
+ * Columns x >= W_out of a dst row (the wpitch padding) are not written. */
+int decx_hip_conv2_im2col_f32(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt, int N,
+                              int kh, int kw, size_t filt_stride, size_t filt_row_stride, float* dst, int dst_dpitch,
+                              size_t dst_row_stride, int flag);
+int decx_hip_conv2_im2col_f32_async(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt,
+                                    int N, int kh, int kw, size_t filt_stride, size_t filt_row_stride, float* dst,
+                                    int dst_dpitch, size_t dst_row_stride, int flag);
+
+/* Timing on the library's own stream (the reference's demos time with clock(), CUDA_GEMM.cpp:43-46, :93-96).
+ * start records an event, stop records another, waits for it and returns the elapsed milliseconds. */
+int decx_hip_timer_start(void);
+int decx_hip_timer_stop(float* milliseconds);
+
+/* Message of the most recent failure on this thread of control ("No error\n" if none), a static string the caller
+ * must not free -- the char* error_string of de::DH (handles/decx_handles.h:42-49). */
+const char* decx_hip_last_error(void);
+
+/* Tile-shape override for experiments: 0 = automatic choice by problem shape; other values select a fixed
+ * kernel variant (see the table in backup_1_amd/csrc/decx_hip.hip).  Returns the previous value.  Results never depend on it
+ * beyond fp32 summation order. */
+int decx_hip_set_sgemm_variant(int variant);
+int decx_hip_set_hgemm_variant(int variant);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DECX_HIP_H_ */

@@ -17,3 +17,11 @@ def oracle():
     import oracle as _oracle
     _oracle.lib()
     return _oracle
+
+
+@pytest.fixture(scope="session")
+def gpu():
+    """Initialise the device through the C ABI.  No fallback: a missing library or device is a failure."""
+    from backup_1_amd import capi
+    capi.init()
+    return capi

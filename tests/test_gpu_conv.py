@@ -1,0 +1,68 @@
+"""Fused im2col convolution parity on the GPU (decx_hip_conv2_im2col_f32) against the CPU oracle."""
+import numpy as np
+import pytest
+
+from backup_1_amd import workloads
+from gpu_helpers import gpu_conv
+
+pytestmark = pytest.mark.gpu
+
+CASES = [  # H, W, C, N, kh, kw, flag
+    (6, 7, 4, 3, 3, 3, 1), (6, 7, 4, 3, 3, 3, 0), (5, 9, 8, 2, 5, 3, 1), (8, 8, 4, 5, 1, 1, 1), (9, 6, 4, 2, 3, 5, 0),
+    (33, 31, 3, 7, 3, 3, 1), (40, 50, 16, 130, 3, 3, 1), (21, 23, 6, 5, 7, 7, 1), (21, 23, 6, 5, 7, 7, 0),
+    (30, 30, 64, 128, 3, 3, 1), (17, 19, 4, 1, 17, 17, 1), (64, 64, 32, 64, 5, 5, 0),
+]
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+@pytest.mark.parametrize("case", CASES)
+def test_integer_exact(gpu, oracle, case, variant):
+    H, W, C, N, kh, kw, flag = case
+    src = workloads.small_ints((H, W, C), 100 + H, -4, 4)
+    filt = workloads.small_ints((N, kh, kw, C), 200 + N, -4, 4)
+    assert np.array_equal(gpu_conv(src, filt, flag, variant=variant), oracle.conv2_chain(src, filt, flag))
+
+
+def test_all_ones_counts_taps(gpu):
+    H, W, C, N = 20, 24, 64, 8
+    d = gpu_conv(np.ones((H, W, C), np.float32), np.ones((N, 3, 3, C), np.float32), 1)
+    assert np.all(d[1:-1, 1:-1] == 576) and np.all(d[0, 1:-1] == 384) and np.all(d[1:-1, -1] == 384)
+    assert d[0, 0, 0] == 256 and d[-1, -1, -1] == 256
+
+
+def test_impulse_gives_reversed_filter(gpu):
+    H, W, C, N, kh, kw = 11, 13, 4, 3, 5, 3
+    filt = workloads.normal((N, kh, kw, C), 51)
+    src = np.zeros((H, W, C), dtype=np.float32)
+    src[5, 6, 2] = 1.0
+    d = gpu_conv(src, filt, 1)
+    for di in range(-2, 3):
+        for dj in range(-1, 2):
+            assert np.array_equal(d[5 - di, 6 - dj, :], filt[:, 2 + di, 1 + dj, 2])
+
+
+def test_config4_224x224x64_128_filters(gpu, oracle):
+    src, filt = workloads.conv_case()
+    ref = oracle.conv2_chain(src, filt, 1)
+    # scale = sum |a||b| per output: the same convolution on absolute values, in fp64 via the oracle's f32 chain is
+    # accurate enough for a scale
+    scale = oracle.conv2_chain(np.abs(src), np.abs(filt), 1).astype(np.float64)
+    K = 3 * 3 * 64
+    for variant in (0, 1, 2, 3):
+        got = gpu_conv(src, filt, 1, variant=variant)
+        err = float(np.max(np.abs(got.astype(np.float64) - ref) / scale))
+        print("conv 224x224x64 (*) 128x3x3x64 variant %d: max |x-r|/sum|a||b| = %.3e (bound %.3e)" %
+              (variant, err, 1e-5 * np.sqrt(K)))
+        assert err < 4e-7 * np.sqrt(K) + 2e-7 < 1e-5 * np.sqrt(K)
+    si, fi = workloads.small_ints((224, 224, 64), 71, -4, 4), workloads.small_ints((128, 3, 3, 64), 72, -4, 4)
+    assert np.array_equal(gpu_conv(si, fi, 1), oracle.conv2_chain(si, fi, 1))
+
+
+def test_bad_flag_and_bad_layout(gpu):
+    L = gpu.lib()
+    buf = gpu.DeviceBuffer(1 << 16)
+    args = lambda flag, dp=4: (buf.ptr, 8, 8, dp, 8 * dp, buf.ptr, 2, 3, 3, 3 * 4 * dp, 4 * dp, buf.ptr, 4, 32, flag)
+    assert L.decx_hip_conv2_im2col_f32(*args(2)) == 0x0b          # DECX_FAIL_ErrorFlag
+    assert "meaningless" in gpu.last_error()
+    assert L.decx_hip_conv2_im2col_f32(*args(1, dp=3)) == 0x0d    # channel pitch not a multiple of 4
+    assert L.decx_hip_conv2_im2col_f32(*args(1)) == 0

@@ -1,0 +1,106 @@
+"""fp16-in / fp32-accumulate GEMM parity on the GPU (decx_hip_hgemm_f32acc) against an fp64 host product.
+
+Tolerance of the path: |x - r| <= 2e-3 relative, taken as max |x - r| / sum_k|a||b| with r the fp64 product of the
+binary16 operands.  Integer data gives a stricter check: the fp32 accumulation is exact, so the result must equal the
+exact product rounded once to binary16.
+"""
+import numpy as np
+import pytest
+
+from backup_1_amd import workloads
+from gpu_helpers import gpu_hgemm, rel_err_vs_abs_scale
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-3
+
+
+def to_bits(x):
+    return x.astype(np.float16).view(np.uint16)
+
+
+def from_bits(b):
+    return b.view(np.float16).astype(np.float64)
+
+
+SHAPES = [(1, 1, 1), (3, 5, 7), (31, 17, 33), (32, 32, 32), (128, 32, 128), (129, 33, 130), (256, 256, 256),
+          (300, 70, 500), (257, 1500, 255), (64, 8, 1000), (1000, 3, 64), (513, 129, 259)]
+
+
+@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_integer_exact_all_tiles(gpu, shape, variant):
+    M, K, N = shape
+    A = workloads.small_ints((M, K), 3000 + M, -4, 4)
+    B = workloads.small_ints((K, N), 4000 + N, -4, 4)
+    got = gpu_hgemm(to_bits(A), to_bits(B), variant=variant)
+    with np.errstate(over="ignore"):
+        want = (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float16).view(np.uint16)   # one RNE rounding
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("shape", [(5, 7, 9), (130, 33, 77)])
+def test_unaligned_pitch(gpu, shape):
+    M, K, N = shape
+    A = workloads.small_ints((M, K), 13, -4, 4)
+    B = workloads.small_ints((K, N), 14, -4, 4)
+    got = gpu_hgemm(to_bits(A), to_bits(B), align=1)
+    assert np.array_equal(got, (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float16).view(np.uint16))
+
+
+def test_a_times_b_plus_c(gpu):
+    M, K, N = 200, 150, 300
+    A, B = workloads.small_ints((M, K), 21, -3, 3), workloads.small_ints((K, N), 22, -3, 3)
+    C = workloads.small_ints((M, N), 23, -50, 50)
+    want = (A.astype(np.float64) @ B.astype(np.float64) + C).astype(np.float16).view(np.uint16)
+    for variant in (1, 2):
+        assert np.array_equal(gpu_hgemm(to_bits(A), to_bits(B), to_bits(C), variant=variant), want)
+
+
+def test_rounding_to_half_is_nearest_even(gpu):
+    # single products that are exact in fp32 and lie exactly half-way between two binary16 numbers
+    A = np.array([[683.0], [293.0], [439.0]], dtype=np.float32)
+    B = np.array([[3.0, 7.0, 14.0]], dtype=np.float32)
+    got = gpu_hgemm(to_bits(A), to_bits(B)).view(np.float16).astype(np.float32)
+    assert got[0, 0] == 2048.0      # 2049: tie between 2048 (even mantissa) and 2050
+    assert got[1, 1] == 2052.0      # 2051: tie between 2050 and 2052 (even mantissa)
+    assert got[2, 2] == 6144.0      # 6146: tie between 6144 (even mantissa) and 6148
+
+
+@pytest.mark.parametrize("case", [(1024, 1024, 1024), (777, 1333, 901)])
+def test_random_vs_fp64(gpu, oracle, case):
+    M, K, N = case
+    A, B = workloads.uniform_pm1((M, K), 61), workloads.uniform_pm1((K, N), 62)
+    Ab, Bb = oracle.float_to_half(A), oracle.float_to_half(B)
+    rows = np.arange(0, M, max(1, M // 50), dtype=np.int32)
+    ref, scale = oracle.gemm_f64_rows_f16(Ab, Bb, rows)
+    for variant in (1, 2):
+        got = from_bits(gpu_hgemm(Ab, Bb, variant=variant))[rows]
+        err = rel_err_vs_abs_scale(got, ref, scale)
+        print("%s variant %d: max |x-r|/sum|a||b| = %.3e (bound %.1e)" % (case, variant, err, TOL))
+        assert err < TOL
+        # elementwise: within half a binary16 ulp of the fp64 value plus the fp32 accumulation error
+        assert np.all(np.abs(got - ref) <= np.abs(ref) * 2.0 ** -11 + scale * 1e-6 + 1e-7)
+
+
+def test_config5_8192_cube_sampled_rows(gpu, oracle):
+    n = 8192
+    A, B = workloads.gemm_square(n, seed=5)
+    Ab, Bb = oracle.float_to_half(A), oracle.float_to_half(B)
+    del A, B
+    got = gpu_hgemm(Ab, Bb)
+    rows = np.random.Generator(np.random.PCG64(63)).choice(n, size=64, replace=False).astype(np.int32)
+    ref, scale = oracle.gemm_f64_rows_f16(Ab, Bb, rows)
+    g = from_bits(got[rows])
+    err = rel_err_vs_abs_scale(g, ref, scale)
+    print("8192^3 fp16: max |x-r|/sum|a||b| on 64 rows = %.3e (bound %.1e); max |x-r|/max|r| = %.3e" %
+          (err, TOL, np.max(np.abs(g - ref)) / np.max(np.abs(ref))))
+    assert err < TOL
+    assert np.all(np.abs(g - ref) <= np.abs(ref) * 2.0 ** -11 + scale * 1e-6 + 1e-7)
+    # full-size integer property: C @ 1 == A @ (B @ 1) exactly while every C element is exact in binary16 (|c| <= 2048)
+    Ai = workloads.small_ints((n, n), 64, -1, 1) * (workloads.uniform_01((n, n), 65) < 0.02)
+    Bi = workloads.small_ints((n, n), 66, -1, 1)
+    goti = from_bits(gpu_hgemm(to_bits(Ai), to_bits(Bi)))
+    assert np.max(np.abs(goti)) <= 2048
+    assert np.array_equal(goti.sum(axis=1), Ai.astype(np.float64) @ Bi.astype(np.float64).sum(axis=1))
+    assert np.array_equal(goti.sum(axis=0), Ai.astype(np.float64).sum(axis=0) @ Bi.astype(np.float64))

@@ -1,0 +1,131 @@
+"""fp32 GEMM parity on the GPU, through the C ABI (decx_hip_sgemm), against the CPU oracle.
+
+Two kinds of check:
+  * bit-exact on small-integer data (every partial sum is exact in fp32, so MFMA order cannot matter): pins indexing,
+    ragged edges, the K tail, pitches and the A*B+C path exactly;
+  * tolerance on the seeded benchmark data: max |x - r| / sum_k|a||b| <= 1e-5 * sqrt(K) against the reference's
+    single-accumulator fused chain.  The observed error is far below that bound; it is asserted against a tighter
+    working bound as well so that a regression in accuracy shows up.
+"""
+import numpy as np
+import pytest
+
+from backup_1_amd import workloads
+from gpu_helpers import gpu_sgemm, rel_err_vs_abs_scale
+
+pytestmark = pytest.mark.gpu
+
+TOL = lambda K: 1e-5 * np.sqrt(K)            # stated tolerance of the path
+TIGHT = lambda K: 4e-7 * np.sqrt(K) + 2e-7   # working bound: a few ulp of random-walk rounding
+
+
+def exact_int_product(A, B):
+    return (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32)
+
+
+SHAPES = [(1, 1, 1), (3, 5, 7), (31, 17, 33), (32, 16, 32), (128, 16, 128), (129, 17, 130), (256, 256, 256),
+          (300, 70, 500), (257, 1500, 255), (64, 8, 1000), (1000, 3, 64), (513, 129, 259)]
+
+
+@pytest.mark.parametrize("variant", [1, 2, 3])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_integer_exact_all_tiles(gpu, shape, variant):
+    M, K, N = shape
+    A = workloads.small_ints((M, K), 1000 + M)
+    B = workloads.small_ints((K, N), 2000 + N)
+    got = gpu_sgemm(A, B, variant=variant)
+    assert np.array_equal(got, exact_int_product(A, B))
+
+
+@pytest.mark.parametrize("shape", [(5, 7, 9), (130, 33, 77), (256, 64, 250)])
+def test_unaligned_pitch_uses_elementwise_loader(gpu, shape):
+    M, K, N = shape
+    A = workloads.small_ints((M, K), 11)
+    B = workloads.small_ints((K, N), 12)
+    assert np.array_equal(gpu_sgemm(A, B, align=1), exact_int_product(A, B))
+
+
+@pytest.mark.parametrize("variant", [1, 2, 3])
+def test_a_times_b_plus_c(gpu, oracle, variant):
+    M, K, N = 200, 150, 300
+    A, B, C = workloads.small_ints((M, K), 21), workloads.small_ints((K, N), 22), workloads.small_ints((M, N), 23, -100, 100)
+    want = exact_int_product(A, B) + C
+    assert np.array_equal(gpu_sgemm(A, B, C, variant=variant), want)
+    assert np.array_equal(gpu_sgemm(A, B, C, variant=variant, inplace=True), want)       # GEMM.h:206 passes dst as C
+    assert np.array_equal(gpu_sgemm(np.zeros_like(A), B, C, variant=variant), C)          # A = 0  =>  dst = C
+    Ar, Br, Cr = workloads.normal((M, K), 24), workloads.normal((K, N), 25), workloads.normal((M, N), 26)
+    ref = oracle.sgemm_chain(Ar, Br, Cr)
+    scale = np.abs(Ar).astype(np.float64) @ np.abs(Br).astype(np.float64) + np.abs(Cr)
+    assert rel_err_vs_abs_scale(gpu_sgemm(Ar, Br, Cr, variant=variant), ref, scale) < TIGHT(K)
+
+
+def test_reference_known_answer_pattern(gpu):
+    # test/test/CUDA_GEMM/CUDA_GEMM.cpp:59-109 on GPU_Matrix, main runs <2048,2048,2048>; a 512-row slab keeps it quick
+    M, K, N = 512, 2048, 2048
+    A, B, printed, closed = workloads.known_answer_pattern(M, K, N)
+    got = gpu_sgemm(A, B)
+    assert np.all(got == got[0, 0])
+    assert abs(float(got[0, 0]) - closed) / closed < TOL(K)
+    assert abs(float(got[0, 0]) - printed) / printed < TOL(K)
+
+
+def test_permutation_matrix_moves_columns_exactly(gpu):
+    M, K = 300, 260
+    A = workloads.normal((M, K), 31)
+    perm = np.random.Generator(np.random.PCG64(32)).permutation(K)
+    P = np.zeros((K, K), dtype=np.float32)
+    P[perm, np.arange(K)] = 1.0
+    assert np.array_equal(gpu_sgemm(A, P).view(np.uint32), A[:, perm].view(np.uint32))
+
+
+def test_config1_1024_cube_vs_chain(gpu, oracle):
+    A, B = workloads.gemm_square(1024)
+    ref = oracle.sgemm_chain(A, B)
+    scale = np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)
+    for variant in (0, 1, 2, 3):
+        err = rel_err_vs_abs_scale(gpu_sgemm(A, B, variant=variant), ref, scale)
+        print("1024^3 variant %d: max |x-r|/sum|a||b| = %.3e (bound %.3e)" % (variant, err, TOL(1024)))
+        assert err < TIGHT(1024) < TOL(1024)
+
+
+def test_config3_ragged_vs_chain_and_integer_exact(gpu, oracle):
+    M, K, N = 3000, 1500, 4500
+    Ai, Bi = workloads.small_ints((M, K), 41), workloads.small_ints((K, N), 42)
+    assert np.array_equal(gpu_sgemm(Ai, Bi), exact_int_product(Ai, Bi))
+    A, B = workloads.gemm_ragged()
+    ref = oracle.sgemm_chain(A, B)
+    scale = np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)
+    err = rel_err_vs_abs_scale(gpu_sgemm(A, B), ref, scale)
+    print("ragged 3000x1500x4500: max |x-r|/sum|a||b| = %.3e (bound %.3e)" % (err, TOL(K)))
+    assert err < TIGHT(K) < TOL(K)
+
+
+@pytest.mark.parametrize("n", [4096, 8192])
+def test_config2_large_squares(gpu, oracle, n):
+    # full-size properties that do not need an O(n^3) host product:
+    #   integer data:  C @ 1 == A @ (B @ 1)  and  1^T @ C == (1^T @ A) @ B, exactly (all values are small integers)
+    #   plus sampled rows against the oracle chain, bit-exact for integers and within tolerance for the seeded data.
+    Ai, Bi = workloads.small_ints((n, n), 51, -4, 4), workloads.small_ints((n, n), 52, -4, 4)
+    got = gpu_sgemm(Ai, Bi).astype(np.float64)
+    A64, B64 = Ai.astype(np.float64), Bi.astype(np.float64)
+    assert np.array_equal(got.sum(axis=1), A64 @ B64.sum(axis=1))
+    assert np.array_equal(got.sum(axis=0), A64.sum(axis=0) @ B64)
+    rows = np.random.Generator(np.random.PCG64(53)).choice(n, size=24, replace=False).astype(np.int32)
+    assert np.array_equal(got[rows].astype(np.float32), oracle.sgemm_chain_rows(Ai, Bi, rows))
+    del got, A64, B64
+    A, B = workloads.gemm_square(n)
+    got = gpu_sgemm(A, B)
+    ref = oracle.sgemm_chain_rows(A, B, rows)
+    _, scale = oracle.gemm_f64_rows_f32(A, B, rows)
+    err = rel_err_vs_abs_scale(got[rows], ref, scale)
+    print("%d^3: max |x-r|/sum|a||b| on 24 rows = %.3e (bound %.3e)" % (n, err, TOL(n)))
+    assert err < TIGHT(n) < TOL(n)
+
+
+def test_bad_arguments_are_reported_not_executed(gpu):
+    L = gpu.lib()
+    buf = gpu.DeviceBuffer(4096)
+    assert L.decx_hip_sgemm(buf.ptr, 8, buf.ptr, 8, None, 0, buf.ptr, 8, 0, 8, 8) == 0x03       # empty matrix
+    assert L.decx_hip_sgemm(buf.ptr, 4, buf.ptr, 8, None, 0, buf.ptr, 8, 8, 8, 8) == 0x0d       # lda < K
+    assert L.decx_hip_sgemm(None, 8, buf.ptr, 8, None, 0, buf.ptr, 8, 8, 8, 8) == 0x0d
+    assert gpu.last_error().strip() != ""
