@@ -1,0 +1,183 @@
+#!/usr/bin/env python3
+"""Benchmark of the dense-contraction path on one MI355X.
+
+A "step" is one de::cuda::GEMM-on-GPU_Matrix equivalent: one call of decx_hip_sgemm on device-resident operands.
+Headline workload (the configuration the metric is quoted on): fp32 square GEMM, M = N = K = 8192, row-major,
+entries uniform[-1,1] from a fixed seed.  The same JSON line also carries, under "also", the other configurations the
+metric names (fp16 8192^3 with fp32 accumulation, fp32 4096^3, the ragged 3000x1500x4500 GEMM, the fused im2col
+convolution), each timed the same way, and a CPU baseline (the restated DECX_cpu thread-pool SGEMM from oracle/) timed
+on this box's host cores on a bounded slab of the headline workload.
+
+Prints ONE JSON line on stdout; progress goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MATRIX_TFLOPS = 157.3     # MI355X dense fp32 MFMA
+PEAK_FP16_MATRIX_TFLOPS = 2516.6    # MI355X dense fp16 MFMA (2.5 PFLOP/s)
+
+
+def log(msg):
+    print("[bench] " + msg, file=sys.stderr, flush=True)
+
+
+def time_launches(capi, launch, steps, warmup):
+    """Returns (wall ms per step, HIP-event ms per step) for `steps` back-to-back launches on the library's stream."""
+    for _ in range(warmup):
+        launch()
+    capi.sync()
+    t0 = time.perf_counter()
+    capi.timer_start()
+    for _ in range(steps):
+        launch()
+    ev_ms = capi.timer_stop()
+    capi.sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return wall_ms / steps, ev_ms / steps
+
+
+def bench_sgemm(capi, workloads, M, K, N, steps, warmup, seed, dist="uniform"):
+    if dist == "uniform":
+        A, B = workloads.uniform_pm1((M, K), seed), workloads.uniform_pm1((K, N), seed + 1)
+    else:
+        A, B = workloads.normal((M, K), seed), workloads.normal((K, N), seed + 1)
+    pad8 = lambda x: (x + 7) // 8 * 8
+    lda, ldb, ldd = pad8(K), pad8(N), pad8(N)
+    Ab = np.zeros((M, lda), np.float32); Ab[:, :K] = A
+    Bb = np.zeros((K, ldb), np.float32); Bb[:, :N] = B
+    dA, dB = capi.DeviceBuffer.from_numpy(Ab), capi.DeviceBuffer.from_numpy(Bb)
+    dD = capi.DeviceBuffer(M * ldd * 4)
+    launch = lambda: capi.sgemm(dA.ptr, lda, dB.ptr, ldb, dD.ptr, ldd, M, N, K, blocking=False)
+    wall, ev = time_launches(capi, launch, steps, warmup)
+    flops = 2.0 * M * N * K
+    return {"ms_wall": wall, "ms_kernel": ev, "tflops": flops / (wall * 1e-3) / 1e12, "tflops_kernel": flops / (ev * 1e-3) / 1e12,
+            "flops": flops, "A": A, "B": B}
+
+
+def bench_hgemm(capi, workloads, n, steps, warmup, seed):
+    A = workloads.uniform_pm1((n, n), seed).astype(np.float16).view(np.uint16)
+    B = workloads.uniform_pm1((n, n), seed + 1).astype(np.float16).view(np.uint16)
+    dA, dB = capi.DeviceBuffer.from_numpy(A), capi.DeviceBuffer.from_numpy(B)
+    dD = capi.DeviceBuffer(n * n * 2)
+    launch = lambda: capi.hgemm(dA.ptr, n, dB.ptr, n, dD.ptr, n, n, n, n, blocking=False)
+    wall, ev = time_launches(capi, launch, steps, warmup)
+    flops = 2.0 * n * n * n
+    return {"ms_wall": wall, "ms_kernel": ev, "tflops": flops / (wall * 1e-3) / 1e12, "tflops_kernel": flops / (ev * 1e-3) / 1e12}
+
+
+def bench_conv(capi, workloads, steps, warmup):
+    H = W = 224; C = 64; N = 128; kh = kw = 3
+    src, filt = workloads.conv_case()
+    fb = np.zeros((N, kh, 4, C), np.float32); fb[:, :, :kw, :] = filt       # TensorArray: wpitch = ceil4(kw)
+    dS, dF = capi.DeviceBuffer.from_numpy(src), capi.DeviceBuffer.from_numpy(fb)
+    dD = capi.DeviceBuffer(H * W * N * 4)
+    launch = lambda: capi.conv2_im2col(dS.ptr, H, W, C, W * C, dF.ptr, N, kh, kw, kh * 4 * C, 4 * C, dD.ptr, N, W * N, 1,
+                                       blocking=False)
+    wall, ev = time_launches(capi, launch, steps, warmup)
+    flops = 2.0 * H * W * N * kh * kw * C
+    return {"ms_wall": wall, "ms_kernel": ev, "tflops": flops / (wall * 1e-3) / 1e12, "tflops_kernel": flops / (ev * 1e-3) / 1e12}
+
+
+def cpu_baseline(A, B, rows):
+    """The restated DECX_cpu thread-pool SGEMM (oracle/, kind "port") on the first `rows` rows of the headline A times
+    the full B: B re-pack included, 12 tasks on a pool of min(hardware threads, 16) workers, as the reference sizes it."""
+    import oracle
+    N = B.shape[1]
+    out = np.zeros((rows, N), np.float32)
+    workers = oracle.pool_size(0)
+    best = None
+    for _ in range(2):
+        t0 = time.perf_counter()
+        oracle.decx_cpu_sgemm(A[:rows], B, out=out)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    flops = 2.0 * rows * N * A.shape[1]
+    return {"value": flops / best / 1e12, "unit": "TFLOP/s", "cores": min(workers, 12), "kind": "port",
+            "sample": "restated DECX_cpu thread-pool SGEMM (B re-pack + 32x16x64 AVX2 FMA blocks, 3x4 task grid, pool of %d "
+                      "workers, g++ -O2) on rows 0..%d of the 8192^3 fp32 workload x full B, best of 2, %.2f s" %
+                      (workers, rows - 1, best)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--size", type=int, default=8192, help="square size of the headline fp32 GEMM")
+    ap.add_argument("--only", default="", help="comma list of: headline,fp16,sq4096,ragged,conv,cpu (default all)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); --gpus %d is not supported. "
+              "value is one GPU's throughput." % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    only = set(filter(None, args.only.split(",")))
+    want = lambda k: not only or k in only
+
+    from backup_1_amd import capi, workloads
+    capi.init()
+    info = capi.device_info()
+    log("device: %d CUs, %.0f MHz" % (info["compute_units"], info["clock_khz"] / 1e3))
+
+    n = args.size
+    log("headline: fp32 GEMM %d^3" % n)
+    head = bench_sgemm(capi, workloads, n, n, n, args.steps, args.warmup, 1234)
+    log("  %.3f ms/step wall, %.3f ms/launch by HIP events -> %.1f TFLOP/s" % (head["ms_wall"], head["ms_kernel"], head["tflops"]))
+
+    also = {}
+    side_steps = max(5, min(args.steps, 20))
+    if want("fp16"):
+        r = bench_hgemm(capi, workloads, 8192, side_steps, args.warmup, 5)
+        also["fp16_8192_f32acc"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
+                                    "frac_of_fp16_dense_peak": round(r["tflops_kernel"] / PEAK_FP16_MATRIX_TFLOPS, 4)}
+        log("fp16 8192^3: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+    if want("sq4096"):
+        r = bench_sgemm(capi, workloads, 4096, 4096, 4096, side_steps, args.warmup, 1234)
+        also["fp32_4096"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
+                             "frac_of_fp32_matrix_peak": round(r["tflops_kernel"] / PEAK_FP32_MATRIX_TFLOPS, 4)}
+        log("fp32 4096^3: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+    if want("ragged"):
+        r = bench_sgemm(capi, workloads, 3000, 1500, 4500, side_steps, args.warmup, 4321, dist="normal")
+        also["fp32_ragged_3000x1500x4500"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
+                                              "frac_of_fp32_matrix_peak": round(r["tflops_kernel"] / PEAK_FP32_MATRIX_TFLOPS, 4)}
+        log("fp32 ragged: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+    if want("conv"):
+        r = bench_conv(capi, workloads, side_steps, args.warmup)
+        also["fp32_conv_224x224x64_128f3x3_fused_im2col"] = {
+            "tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
+            "frac_of_fp32_matrix_peak": round(r["tflops_kernel"] / PEAK_FP32_MATRIX_TFLOPS, 4)}
+        log("conv: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+
+    cpu = None
+    if want("cpu"):
+        log("cpu baseline (oracle port of the DECX_cpu thread-pool SGEMM) ...")
+        cpu = cpu_baseline(head["A"], head["B"], rows=min(n, 3072))
+        log("  %.4f TFLOP/s on %d cores" % (cpu["value"], cpu["cores"]))
+
+    achieved = head["tflops_kernel"]
+    line = {
+        "metric": "GEMM TFLOP/s at 8192^3 fp32 (fraction of MI355X fp32 matrix peak under roofline.frac; fp16 and conv under also)",
+        "value": round(head["tflops"], 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(head["ms_wall"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "fp32 square GEMM C=A*B, M=N=K=%d, row-major, uniform[-1,1] seed 1234, device-resident "
+                               "operands (GPU_Matrix path)" % n},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_MATRIX_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_FP32_MATRIX_TFLOPS, 4), "traffic": None,
+                     "kernel": "sgemm_tile_kernel", "flop_per_launch": head["flops"],
+                     "avg_launch_ms_hip_events": round(head["ms_kernel"], 4)},
+        "cpu_baseline": cpu,
+        "also": also,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()
