@@ -1,0 +1,239 @@
+// DECX-named API functions over the C ABI (include/decx_hip.h).  Reference call stacks mirrored here:
+//   host-matrix GEMM      GEMM/CUDA/large_squares/GEMM.h:56-131   (re_construct dst, H2D, kernel, D2H)
+//   GPU_Matrix GEMM       GEMM.h:398-454 (fp32), :457-519 (fp16)
+//   Conv2_MK_im2col       convolution/CUDA/im2col/conv2_mk_im2col.h:278-306 (+ :57-274 host drivers)
+// Differences on purpose: device copies keep the host pitch (no padding to 128/16 multiples, GEMM.h:80-104 pads);
+// errors of the GPU runtime come back in the DH instead of exiting the process; Conv2_MK_im2col fills its DH and
+// rejects unknown flags (the reference returns an unfilled DH, conv2_mk_im2col.h:301-305).
+#include <cmath>
+#include <cstring>
+
+#include "decx_classes.hpp"
+
+namespace {
+
+char kSuccess[] = "No error\n";                                              // core/error.h:61
+char kGemmDims[] = "The width of matrix A and the height of matrix B are required to be same";   // core/error.h GEMM_DimNMatch
+char kMDims[] = "Matrix Dims don't match each other";
+char kNotFactory[] = "Container was not created by this library's factories\n";
+
+de::DH ok() { return de::DH{decx::DECX_SUCCESS, kSuccess}; }
+de::DH from_status(int rc) {
+    if (rc == 0) return ok();
+    return de::DH{rc, const_cast<char*>(decx_hip_last_error())};
+}
+de::DH not_init() {
+    static char msg[] = "CUDA should be initialized first\n";               // core/error.h:60
+    return de::DH{decx::DECX_FAIL_not_init, msg};
+}
+de::DH alloc_fail() {
+    static char msg[] = "Fail to allocate memory\n";                          // core/error.h:65
+    return de::DH{decx::DECX_FAIL_ALLOCATION, msg};
+}
+
+struct DeviceTemp {   // a device buffer freed on scope exit
+    void* ptr = nullptr;
+    int alloc(size_t bytes) { return decx_hip_malloc(&ptr, bytes); }
+    ~DeviceTemp() { if (ptr) decx_hip_free(ptr); }
+};
+
+template <typename T> struct GemmCall;
+template <> struct GemmCall<float> {
+    static int run(const float* A, int lda, const float* B, int ldb, const float* C, int ldc, float* D, int ldd, int M,
+                   int N, int K) { return decx_hip_sgemm(A, lda, B, ldb, C, ldc, D, ldd, M, N, K); }
+};
+template <> struct GemmCall<de::Half> {
+    static int run(const de::Half* A, int lda, const de::Half* B, int ldb, const de::Half* C, int ldc, de::Half* D, int ldd,
+                   int M, int N, int K) {
+        return decx_hip_hgemm_f32acc(reinterpret_cast<const uint16_t*>(A), lda, reinterpret_cast<const uint16_t*>(B), ldb,
+                                     reinterpret_cast<const uint16_t*>(C), ldc, reinterpret_cast<uint16_t*>(D), ldd, M, N, K);
+    }
+};
+
+template <typename T>
+de::DH gemm_host(de::Matrix<T>& A_, de::Matrix<T>& B_, de::Matrix<T>* C_, de::Matrix<T>& dst_) {
+    auto* A = dynamic_cast<decx::_Matrix<T>*>(&A_);
+    auto* B = dynamic_cast<decx::_Matrix<T>*>(&B_);
+    auto* C = C_ ? dynamic_cast<decx::_Matrix<T>*>(C_) : nullptr;
+    auto* dst = dynamic_cast<decx::_Matrix<T>*>(&dst_);
+    if (!A || !B || !dst || (C_ && !C)) return de::DH{decx::DECX_FAIL_ErrorParams, kNotFactory};
+    if (!decx_hip_is_init()) return not_init();                                           // GEMM.h:63
+    if (A->width != B->height) return de::DH{decx::DECX_FAIL_DimsNotMatching, kGemmDims}; // GEMM.h:68
+    if (C && (C->width != B->width || C->height != A->height))                            // GEMM.h:154-157
+        return de::DH{decx::DECX_FAIL_DimsNotMatching, kMDims};
+    const int M = (int)A->height, K = (int)A->width, N = (int)B->width;
+    // C may be the same object as dst: read it before dst is re-constructed
+    DeviceTemp dA, dB, dD;
+    if (dA.alloc(A->total_bytes) || dB.alloc(B->total_bytes)) return alloc_fail();
+    int rc = decx_hip_memcpy2d(dA.ptr, (size_t)A->pitch * sizeof(T), A->Mat.ptr, (size_t)A->pitch * sizeof(T),
+                               (size_t)K * sizeof(T), M, DECX_HIP_H2D);
+    if (rc) return from_status(rc);
+    rc = decx_hip_memcpy2d(dB.ptr, (size_t)B->pitch * sizeof(T), B->Mat.ptr, (size_t)B->pitch * sizeof(T),
+                           (size_t)N * sizeof(T), K, DECX_HIP_H2D);
+    if (rc) return from_status(rc);
+    const uint pitch_d = decx::ceil_to((uint)N, decx::matrix_align<T>());
+    if (dD.alloc((size_t)pitch_d * M * sizeof(T))) return alloc_fail();
+    if (C) {   // the reference uploads C into the dst device buffer and accumulates in place (GEMM.h:196-206)
+        rc = decx_hip_memcpy2d(dD.ptr, (size_t)pitch_d * sizeof(T), C->Mat.ptr, (size_t)C->pitch * sizeof(T),
+                               (size_t)N * sizeof(T), M, DECX_HIP_H2D);
+        if (rc) return from_status(rc);
+    }
+    if (!dst->re_construct((uint)N, (uint)M, decx::Page_Locked)) return alloc_fail();     // GEMM.h:73
+    rc = GemmCall<T>::run(static_cast<const T*>(dA.ptr), (int)A->pitch, static_cast<const T*>(dB.ptr), (int)B->pitch,
+                          C ? static_cast<const T*>(dD.ptr) : nullptr, (int)pitch_d, static_cast<T*>(dD.ptr), (int)pitch_d,
+                          M, N, K);
+    if (rc) return from_status(rc);
+    rc = decx_hip_memcpy2d(dst->Mat.ptr, (size_t)dst->pitch * sizeof(T), dD.ptr, (size_t)pitch_d * sizeof(T),
+                           (size_t)N * sizeof(T), M, DECX_HIP_D2H);                        // only the valid columns, GEMM.h:119-120
+    return from_status(rc);
+}
+
+template <typename T>
+de::DH gemm_device(de::GPU_Matrix<T>& A_, de::GPU_Matrix<T>& B_, de::GPU_Matrix<T>* C_, de::GPU_Matrix<T>& dst_) {
+    auto* A = dynamic_cast<decx::_GPU_Matrix<T>*>(&A_);
+    auto* B = dynamic_cast<decx::_GPU_Matrix<T>*>(&B_);
+    auto* C = C_ ? dynamic_cast<decx::_GPU_Matrix<T>*>(C_) : nullptr;
+    auto* dst = dynamic_cast<decx::_GPU_Matrix<T>*>(&dst_);
+    if (!A || !B || !dst || (C_ && !C)) return de::DH{decx::DECX_FAIL_ErrorParams, kNotFactory};
+    if (!decx_hip_is_init()) return not_init();                                           // GEMM.h:403
+    if (A->width != B->height) return de::DH{decx::DECX_FAIL_DimsNotMatching, kGemmDims}; // GEMM.h:408
+    if (C && (C->width != B->width || C->height != A->height)) return de::DH{decx::DECX_FAIL_DimsNotMatching, kMDims};
+    if (C != dst && !dst->re_construct(B->width, A->height))                              // GEMM.h:414 (fp16 too: defect D7 not kept)
+        return dst->last_status == DECX_HIP_FAIL_ALLOCATION ? alloc_fail() : from_status(dst->last_status);
+    return from_status(GemmCall<T>::run(A->Mat.ptr, (int)A->pitch, B->Mat.ptr, (int)B->pitch, C ? C->Mat.ptr : nullptr,
+                                        C ? (int)C->pitch : 0, dst->Mat.ptr, (int)dst->pitch, (int)A->height,
+                                        (int)B->width, (int)A->width));
+}
+
+}  // namespace
+
+namespace de {
+
+void InitCuda() {
+    int dev = -1;
+    (void)decx_hip_init(&dev);   // failures surface as DECX_FAIL_not_init on the first compute call
+}
+void release_all_tmp() {}
+
+// IEEE binary32 -> binary16, round to nearest even
+Half Float2Half(const float& x) {
+    uint32_t u;
+    std::memcpy(&u, &x, 4);
+    const uint32_t sign = (u >> 16) & 0x8000u, mag = u & 0x7fffffffu;
+    Half h;
+    if (mag > 0x7f800000u) { h.val = (unsigned short)(sign | 0x7e00u); return h; }           // NaN
+    if (mag >= 0x477ff000u) { h.val = (unsigned short)(sign | 0x7c00u); return h; }          // overflow to inf
+    if (mag < 0x33000001u) { h.val = (unsigned short)sign; return h; }                       // underflow to zero
+    const int e = (int)(mag >> 23) - 127;
+    const uint32_t man = (mag & 0x7fffffu) | 0x800000u;
+    const int shift = e >= -14 ? 13 : 13 + (-14 - e);
+    uint32_t q = man >> shift;
+    const uint32_t rem = man & ((1u << shift) - 1u), halfway = 1u << (shift - 1);
+    if (rem > halfway || (rem == halfway && (q & 1u))) ++q;
+    h.val = (unsigned short)(sign | (e >= -14 ? ((uint32_t)(e + 14) << 10) + q : q));
+    return h;
+}
+float Half2Float(const Half& x) {
+    const uint32_t sign = (uint32_t)(x.val & 0x8000u) << 16, e = (x.val >> 10) & 0x1fu;
+    uint32_t m = x.val & 0x3ffu, u;
+    if (e == 0) {
+        if (m == 0) u = sign;
+        else {
+            int s = 0;
+            while (!(m & 0x400u)) { m <<= 1; ++s; }
+            u = sign | (uint32_t)(113 - s) << 23 | (m & 0x3ffu) << 13;
+        }
+    } else if (e == 31) u = sign | 0x7f800000u | m << 13;
+    else u = sign | (e + 112u) << 23 | m << 13;
+    float f;
+    std::memcpy(&f, &u, 4);
+    return f;
+}
+
+// ---- factories ----------------------------------------------------------------------------------------------
+template <typename T> Matrix<T>& CreateMatrixRef() { return *(new decx::_Matrix<T>()); }
+template <typename T> Matrix<T>* CreateMatrixPtr() { return new decx::_Matrix<T>(); }
+template <typename T> Matrix<T>& CreateMatrixRef(const uint w, const uint h, const int st) { return *(new decx::_Matrix<T>(w, h, st)); }
+template <typename T> Matrix<T>* CreateMatrixPtr(const uint w, const uint h, const int st) { return new decx::_Matrix<T>(w, h, st); }
+template <typename T> GPU_Matrix<T>& CreateGPUMatrixRef() { return *(new decx::_GPU_Matrix<T>()); }
+template <typename T> GPU_Matrix<T>* CreateGPUMatrixPtr() { return new decx::_GPU_Matrix<T>(); }
+template <typename T> GPU_Matrix<T>& CreateGPUMatrixRef(const uint w, const uint h) { return *(new decx::_GPU_Matrix<T>(w, h)); }
+template <typename T> GPU_Matrix<T>* CreateGPUMatrixPtr(const uint w, const uint h) { return new decx::_GPU_Matrix<T>(w, h); }
+template <typename T> Tensor<T>& CreateTensorRef() { return *(new decx::_Tensor<T>()); }
+template <typename T> Tensor<T>* CreateTensorPtr() { return new decx::_Tensor<T>(); }
+template <typename T> Tensor<T>& CreateTensorRef(const uint w, const uint h, const uint d, const int f) { return *(new decx::_Tensor<T>(w, h, d, f)); }
+template <typename T> Tensor<T>* CreateTensorPtr(const uint w, const uint h, const uint d, const int f) { return new decx::_Tensor<T>(w, h, d, f); }
+template <typename T> TensorArray<T>& CreateTensorArrayRef() { return *(new decx::_TensorArray<T>()); }
+template <typename T> TensorArray<T>* CreateTensorArrayPtr() { return new decx::_TensorArray<T>(); }
+template <typename T> TensorArray<T>& CreateTensorArrayRef(const uint w, const uint h, const uint d, const uint n, const int f) { return *(new decx::_TensorArray<T>(w, h, d, n, f)); }
+template <typename T> TensorArray<T>* CreateTensorArrayPtr(const uint w, const uint h, const uint d, const uint n, const int f) { return new decx::_TensorArray<T>(w, h, d, n, f); }
+
+#define DECX_INSTANTIATE_MATRIX(T)                                                     \
+    template Matrix<T>& CreateMatrixRef<T>();                                          \
+    template Matrix<T>* CreateMatrixPtr<T>();                                          \
+    template Matrix<T>& CreateMatrixRef<T>(const uint, const uint, const int);         \
+    template Matrix<T>* CreateMatrixPtr<T>(const uint, const uint, const int);         \
+    template GPU_Matrix<T>& CreateGPUMatrixRef<T>();                                   \
+    template GPU_Matrix<T>* CreateGPUMatrixPtr<T>();                                   \
+    template GPU_Matrix<T>& CreateGPUMatrixRef<T>(const uint, const uint);             \
+    template GPU_Matrix<T>* CreateGPUMatrixPtr<T>(const uint, const uint);
+DECX_INSTANTIATE_MATRIX(float)
+DECX_INSTANTIATE_MATRIX(Half)
+template Tensor<float>& CreateTensorRef<float>();
+template Tensor<float>* CreateTensorPtr<float>();
+template Tensor<float>& CreateTensorRef<float>(const uint, const uint, const uint, const int);
+template Tensor<float>* CreateTensorPtr<float>(const uint, const uint, const uint, const int);
+template TensorArray<float>& CreateTensorArrayRef<float>();
+template TensorArray<float>* CreateTensorArrayPtr<float>();
+template TensorArray<float>& CreateTensorArrayRef<float>(const uint, const uint, const uint, const uint, const int);
+template TensorArray<float>* CreateTensorArrayPtr<float>(const uint, const uint, const uint, const uint, const int);
+
+// ---- GEMM ---------------------------------------------------------------------------------------------------
+namespace cuda {
+DH GEMM(Matrix<float>& A, Matrix<float>& B, Matrix<float>& dst) { return gemm_host<float>(A, B, nullptr, dst); }
+DH GEMM(Matrix<float>& A, Matrix<float>& B, Matrix<float>& C, Matrix<float>& dst) { return gemm_host<float>(A, B, &C, dst); }
+DH GEMM(Matrix<Half>& A, Matrix<Half>& B, Matrix<Half>& dst) { return gemm_host<Half>(A, B, nullptr, dst); }
+DH GEMM(Matrix<Half>& A, Matrix<Half>& B, Matrix<Half>& C, Matrix<Half>& dst) { return gemm_host<Half>(A, B, &C, dst); }
+DH GEMM(GPU_Matrix<float>& A, GPU_Matrix<float>& B, GPU_Matrix<float>& dst) { return gemm_device<float>(A, B, nullptr, dst); }
+DH GEMM(GPU_Matrix<float>& A, GPU_Matrix<float>& B, GPU_Matrix<float>& C, GPU_Matrix<float>& dst) { return gemm_device<float>(A, B, &C, dst); }
+DH GEMM(GPU_Matrix<Half>& A, GPU_Matrix<Half>& B, GPU_Matrix<Half>& dst) { return gemm_device<Half>(A, B, nullptr, dst); }
+DH GEMM(GPU_Matrix<Half>& A, GPU_Matrix<Half>& B, GPU_Matrix<Half>& C, GPU_Matrix<Half>& dst) { return gemm_device<Half>(A, B, &C, dst); }
+
+// ---- convolution ----------------------------------------------------------------------------------------------
+DH Conv2_MK_im2col(Tensor<float>& src_, TensorArray<float>& kernel_, Tensor<float>& dst_, const int flag) {
+    auto* src = dynamic_cast<decx::_Tensor<float>*>(&src_);
+    auto* ker = dynamic_cast<decx::_TensorArray<float>*>(&kernel_);
+    auto* dst = dynamic_cast<decx::_Tensor<float>*>(&dst_);
+    if (!src || !ker || !dst) return DH{decx::DECX_FAIL_ErrorParams, kNotFactory};
+    if (!decx_hip_is_init()) return not_init();                                           // conv2_mk_im2col.h:285-289
+    if (flag != decx::de_conv_no_compensate && flag != decx::de_conv_zero_compensate) {
+        static char msg[] = "This flag is meaningless in current context\n";              // core/error.h:67
+        return DH{decx::DECX_FAIL_ErrorFlag, msg};
+    }
+    if (src->depth != ker->depth) {
+        static char msg[] = "Tensor Dims don't match each other";
+        return DH{decx::DECX_FAIL_DimsNotMatching, msg};
+    }
+    const int H = (int)src->height, W = (int)src->width, kh = (int)ker->height, kw = (int)ker->width;
+    const int Hout = flag ? H : H - 2 * (kh / 2), Wout = flag ? W : W - 2 * (kw / 2);     // conv2_mk_im2col.h:63-66, :173-176
+    if (Hout <= 0 || Wout <= 0) {
+        static char msg[] = "Tensor Dims don't match each other";
+        return DH{decx::DECX_FAIL_DimsNotMatching, msg};
+    }
+    if (!dst->re_construct((uint)Wout, (uint)Hout, ker->tensor_num, decx::Page_Locked)) return alloc_fail();   // :178
+    DeviceTemp dS, dK, dD;
+    if (dS.alloc(src->total_bytes) || dK.alloc(ker->total_bytes) || dD.alloc(dst->total_bytes)) return alloc_fail();
+    int rc = decx_hip_memcpy(dS.ptr, src->Tens.ptr, src->total_bytes, DECX_HIP_H2D);
+    if (rc) return from_status(rc);
+    rc = decx_hip_memcpy(dK.ptr, ker->TensArr.ptr, ker->total_bytes, DECX_HIP_H2D);
+    if (rc) return from_status(rc);
+    rc = decx_hip_memset(dD.ptr, 0, dst->total_bytes);   // the width / channel padding of dst stays zero
+    if (rc) return from_status(rc);
+    rc = decx_hip_conv2_im2col_f32(static_cast<const float*>(dS.ptr), H, W, (int)src->dpitch, src->dp_x_wp,
+                                   static_cast<const float*>(dK.ptr), (int)ker->tensor_num, kh, kw, ker->_gap, ker->dp_x_wp,
+                                   static_cast<float*>(dD.ptr), (int)dst->dpitch, dst->dp_x_wp, flag);
+    if (rc) return from_status(rc);
+    return from_status(decx_hip_memcpy(dst->Tens.ptr, dD.ptr, dst->total_bytes, DECX_HIP_D2H));   // :266
+}
+}  // namespace cuda
+}  // namespace de

@@ -1,0 +1,288 @@
+// Concrete containers behind the abstract classes of DECX.h, with the reference's layout rules:
+//   Matrix / GPU_Matrix : row pitch = width rounded up to 8 (4-byte), 16 (2-byte), 4 (8-byte), 32 (1-byte) elements
+//                         (classes/Matrix.h:24-27, :253-322; GPU_Matrix.h:211-271)
+//   Tensor              : channel-innermost, dpitch = ceil4(depth), wpitch = ceil4(width), row stride dp_x_wp,
+//                         zero-filled on allocation (classes/Tensor.h:162-184, :312, :389-394)
+//   TensorArray         : tensor_num tensors back to back, stride _gap = dp_x_wp * height
+//                         (classes/TensorArray.h:174-198, :349-352, :521-525)
+// Field names follow the reference so that code reading them ports directly.
+#pragma once
+#include <cstdlib>
+#include <cstring>
+
+#include "../../include/decx_hip.h"
+#include "DECX.h"
+
+namespace decx {
+
+inline uint ceil_to(uint v, uint a) { return (v + a - 1) / a * a; }
+
+template <typename T>
+constexpr uint matrix_align() {
+    return sizeof(T) == 4 ? 8 : sizeof(T) == 2 ? 16 : sizeof(T) == 8 ? 4 : 32;
+}
+
+// Host storage: pinned (Page_Locked) through the C ABI when a device is initialised, else 64-byte aligned pageable.
+struct HostBlock {
+    void* ptr = nullptr;
+    bool pinned = false;
+    bool alloc(size_t bytes, int store_type) {
+        free();
+        if (bytes == 0) bytes = 64;
+        if (store_type == Page_Locked && decx_hip_is_init()) {
+            if (decx_hip_host_malloc(&ptr, bytes) == 0) {
+                pinned = true;
+                return true;
+            }
+            ptr = nullptr;
+        }
+        pinned = false;
+        ptr = std::aligned_alloc(64, (bytes + 63) / 64 * 64);
+        return ptr != nullptr;
+    }
+    void free() {
+        if (!ptr) return;
+        if (pinned) decx_hip_host_free(ptr);
+        else std::free(ptr);
+        ptr = nullptr;
+    }
+};
+
+template <typename T>
+struct PtrInfo {   // the reference's decx::PtrInfo<T> exposes .ptr (core/memory_management/MemBlock.h:45-133)
+    T* ptr = nullptr;
+};
+
+template <typename T>
+class _Matrix : public de::Matrix<T> {
+    HostBlock block_;
+
+public:
+    uint width = 0, height = 0;
+    unsigned short Store_Type = Page_Default;
+    size_t element_num = 0, total_bytes = 0;     // padded (pitch * height)
+    uint pitch = 0;
+    PtrInfo<T> Mat;
+    size_t _element_num = 0, _total_bytes = 0;   // true (width * height)
+
+    _Matrix() {}
+    _Matrix(uint w, uint h, int store_type) { construct(w, h, store_type); }
+    void attribute_assign(uint w, uint h, int store_type) {
+        width = w;
+        height = h;
+        Store_Type = (unsigned short)store_type;
+        pitch = ceil_to(w, matrix_align<T>());
+        _element_num = (size_t)w * h;
+        _total_bytes = _element_num * sizeof(T);
+        element_num = (size_t)pitch * h;
+        total_bytes = element_num * sizeof(T);
+    }
+    bool construct(uint w, uint h, int store_type) {
+        attribute_assign(w, h, store_type);
+        bool ok = block_.alloc(total_bytes, store_type);
+        Mat.ptr = static_cast<T*>(block_.ptr);
+        return ok;
+    }
+    bool re_construct(uint w, uint h, int store_type) {
+        if (Mat.ptr && w == width && h == height && store_type == Store_Type) return true;
+        return construct(w, h, store_type);
+    }
+    uint Width() override { return width; }
+    uint Height() override { return height; }
+    size_t TotalBytes() override { return total_bytes; }
+    T& index(const int row, const int col) override { return Mat.ptr[(size_t)pitch * row + col]; }
+    void release() override {
+        block_.free();
+        Mat.ptr = nullptr;
+    }
+    de::Matrix<T>& operator=(de::Matrix<T>& src) override {   // shallow alias in the reference; deep copy is the safe reading
+        _Matrix<T>& s = dynamic_cast<_Matrix<T>&>(src);
+        if (&s != this) {
+            construct(s.width, s.height, s.Store_Type);
+            std::memcpy(Mat.ptr, s.Mat.ptr, total_bytes);
+        }
+        return *this;
+    }
+    ~_Matrix() override { release(); }
+};
+
+template <typename T>
+class _GPU_Matrix : public de::GPU_Matrix<T> {
+public:
+    uint width = 0, height = 0;
+    size_t element_num = 0, total_bytes = 0;     // padded
+    uint pitch = 0;
+    PtrInfo<T> Mat;                              // DEVICE pointer
+    size_t _element_num = 0, _total_bytes = 0;
+    int last_status = 0;                         // status of the most recent allocation / copy
+
+    _GPU_Matrix() {}
+    _GPU_Matrix(uint w, uint h) { construct(w, h); }
+    void attribute_assign(uint w, uint h) {
+        width = w;
+        height = h;
+        pitch = ceil_to(w, matrix_align<T>());
+        _element_num = (size_t)w * h;
+        _total_bytes = _element_num * sizeof(T);
+        element_num = (size_t)pitch * h;
+        total_bytes = element_num * sizeof(T);
+    }
+    bool construct(uint w, uint h) {
+        release();
+        attribute_assign(w, h);
+        void* p = nullptr;
+        last_status = decx_hip_malloc(&p, total_bytes);
+        if (last_status != 0) return false;
+        Mat.ptr = static_cast<T*>(p);
+        last_status = decx_hip_memset(p, 0, total_bytes);   // the whole pitched buffer (the reference clears only width*height bytes)
+        return last_status == 0;
+    }
+    bool re_construct(uint w, uint h) {
+        if (Mat.ptr && w == width && h == height) return true;
+        return construct(w, h);
+    }
+    uint Width() override { return width; }
+    uint Height() override { return height; }
+    size_t TotalBytes() override { return total_bytes; }
+    void Load_from_host(de::Matrix<T>& src) override {
+        _Matrix<T>& s = dynamic_cast<_Matrix<T>&>(src);
+        if (s.width != width || s.height != height) { last_status = DECX_HIP_FAIL_DIMS; return; }
+        last_status = decx_hip_memcpy2d(Mat.ptr, (size_t)pitch * sizeof(T), s.Mat.ptr, (size_t)s.pitch * sizeof(T),
+                                        (size_t)width * sizeof(T), height, DECX_HIP_H2D);
+    }
+    void Load_to_host(de::Matrix<T>& dst) override {
+        _Matrix<T>& d = dynamic_cast<_Matrix<T>&>(dst);
+        if (d.width != width || d.height != height) { last_status = DECX_HIP_FAIL_DIMS; return; }
+        last_status = decx_hip_memcpy2d(d.Mat.ptr, (size_t)d.pitch * sizeof(T), Mat.ptr, (size_t)pitch * sizeof(T),
+                                        (size_t)width * sizeof(T), height, DECX_HIP_D2H);
+    }
+    void release() override {
+        if (Mat.ptr) decx_hip_free(Mat.ptr);
+        Mat.ptr = nullptr;
+    }
+    de::GPU_Matrix<T>& operator=(de::GPU_Matrix<T>& src) override {
+        _GPU_Matrix<T>& s = dynamic_cast<_GPU_Matrix<T>&>(src);
+        if (&s != this && construct(s.width, s.height))
+            last_status = decx_hip_memcpy(Mat.ptr, s.Mat.ptr, total_bytes, DECX_HIP_D2D);
+        return *this;
+    }
+    ~_GPU_Matrix() override { release(); }
+};
+
+template <typename T>
+class _Tensor : public de::Tensor<T> {
+    HostBlock block_;
+
+public:
+    uint width = 0, height = 0, depth = 0;
+    int _store_type = Page_Default;
+    uint dpitch = 0, wpitch = 0;
+    size_t dp_x_wp = 0;
+    PtrInfo<T> Tens;
+    size_t element_num = 0, _element_num = 0, total_bytes = 0;
+
+    _Tensor() {}
+    _Tensor(uint w, uint h, uint d, int store_type) { construct(w, h, d, store_type); }
+    void attribute_assign(uint w, uint h, uint d, int store_type) {
+        width = w;
+        height = h;
+        depth = d;
+        _store_type = store_type;
+        wpitch = ceil_to(w, 4);
+        dpitch = ceil_to(d, 4);
+        dp_x_wp = (size_t)dpitch * wpitch;
+        element_num = (size_t)d * w * h;
+        _element_num = (size_t)h * dp_x_wp;
+        total_bytes = _element_num * sizeof(T);
+    }
+    bool construct(uint w, uint h, uint d, int store_type) {
+        attribute_assign(w, h, d, store_type);
+        bool ok = block_.alloc(total_bytes, store_type);
+        Tens.ptr = static_cast<T*>(block_.ptr);
+        if (ok) std::memset(Tens.ptr, 0, total_bytes);
+        return ok;
+    }
+    bool re_construct(uint w, uint h, uint d, int store_type) {
+        if (Tens.ptr && w == width && h == height && d == depth && store_type == _store_type) {
+            std::memset(Tens.ptr, 0, total_bytes);
+            return true;
+        }
+        return construct(w, h, d, store_type);
+    }
+    uint Width() override { return width; }
+    uint Height() override { return height; }
+    uint Depth() override { return depth; }
+    T& index(const int x, const int y, const int z) override { return Tens.ptr[(size_t)x * dp_x_wp + (size_t)y * dpitch + z]; }
+    de::Tensor<T>& operator=(de::Tensor<T>& src) override {
+        _Tensor<T>& s = dynamic_cast<_Tensor<T>&>(src);
+        if (&s != this) {
+            construct(s.width, s.height, s.depth, s._store_type);
+            std::memcpy(Tens.ptr, s.Tens.ptr, total_bytes);
+        }
+        return *this;
+    }
+    void release() override {
+        block_.free();
+        Tens.ptr = nullptr;
+    }
+    ~_Tensor() override { release(); }
+};
+
+template <typename T>
+class _TensorArray : public de::TensorArray<T> {
+    HostBlock block_;
+
+public:
+    uint width = 0, height = 0, depth = 0, tensor_num = 0;
+    int _store_type = Page_Default;
+    uint dpitch = 0, wpitch = 0;
+    size_t dp_x_wp = 0, _gap = 0;
+    PtrInfo<T> TensArr;
+    size_t element_num = 0, _element_num = 0, total_bytes = 0;
+
+    _TensorArray() {}
+    _TensorArray(uint w, uint h, uint d, uint n, int store_type) { construct(w, h, d, n, store_type); }
+    void attribute_assign(uint w, uint h, uint d, uint n, int store_type) {
+        width = w;
+        height = h;
+        depth = d;
+        tensor_num = n;
+        _store_type = store_type;
+        wpitch = ceil_to(w, 4);
+        dpitch = ceil_to(d, 4);
+        dp_x_wp = (size_t)dpitch * wpitch;
+        _gap = dp_x_wp * h;
+        element_num = (size_t)d * w * h * n;
+        _element_num = (size_t)n * _gap;
+        total_bytes = _element_num * sizeof(T);
+    }
+    bool construct(uint w, uint h, uint d, uint n, int store_type) {
+        attribute_assign(w, h, d, n, store_type);
+        bool ok = block_.alloc(total_bytes, store_type);
+        TensArr.ptr = static_cast<T*>(block_.ptr);
+        if (ok) std::memset(TensArr.ptr, 0, total_bytes);
+        return ok;
+    }
+    uint Width() override { return width; }
+    uint Height() override { return height; }
+    uint Depth() override { return depth; }
+    uint TensorNum() override { return tensor_num; }
+    T& index(const int x, const int y, const int z, const int tensor_id) override {
+        return TensArr.ptr[(size_t)tensor_id * _gap + (size_t)x * dp_x_wp + (size_t)y * dpitch + z];
+    }
+    de::TensorArray<T>& operator=(de::TensorArray<T>& src) override {
+        _TensorArray<T>& s = dynamic_cast<_TensorArray<T>&>(src);
+        if (&s != this) {
+            construct(s.width, s.height, s.depth, s.tensor_num, s._store_type);
+            std::memcpy(TensArr.ptr, s.TensArr.ptr, total_bytes);
+        }
+        return *this;
+    }
+    void release() override {
+        block_.free();
+        TensArr.ptr = nullptr;
+    }
+    ~_TensorArray() override { release(); }
+};
+
+}  // namespace decx

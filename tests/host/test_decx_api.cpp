@@ -1,0 +1,298 @@
+// Exercises the DECX-named C++ API (backup_1_amd/host/DECX.h) the way the reference's demo programs do
+// (test/test/CUDA_GEMM/CUDA_GEMM.cpp, test/test/"generating classes"/*.h), but with assertions, and checks results
+// against the CPU oracle (liboracle.so).  Usage: test_decx_api cpu | gpu
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "../../backup_1_amd/host/DECX.h"
+
+extern "C" {
+void oracle_sgemm_chain_fast(const float* A, long lda, const float* B, long ldb, const float* Cin, long ldc, float* D,
+                             long ldd, int M, int N, int K, int nthreads);
+int oracle_conv2_chain(const float* src, int H, int W, int dpitch, long src_row_stride, const float* filt, int N, int kh,
+                       int kw, long filt_stride, long filt_row_stride, float* dst, int dst_dpitch, long dst_row_stride,
+                       int flag, int nthreads);
+void oracle_gemm_f64_rows_f16(const uint16_t* A, long lda, const uint16_t* B, long ldb, const int* rows, int nrows,
+                              double* out, double* abs_out, int N, int K, int nthreads);
+}
+
+static int g_fail = 0;
+#define CHECK(cond)                                                                  \
+    do {                                                                             \
+        if (!(cond)) { std::printf("  CHECK FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond); ++g_fail; } \
+    } while (0)
+#define RUN(fn)                                   \
+    do {                                          \
+        int before = g_fail;                      \
+        std::printf("RUN  %s\n", #fn); std::fflush(stdout); \
+        fn();                                     \
+        std::printf("%s %s\n", g_fail == before ? "PASS" : "FAIL", #fn); std::fflush(stdout); \
+    } while (0)
+
+static std::mt19937 rng(12345);
+static float small_int() { return (float)((int)(rng() % 9) - 4); }
+static float unif() { return (float)((rng() >> 8) * (1.0 / 8388608.0) - 1.0); }
+
+template <class F>
+static void fill(de::Matrix<float>& m, F f) {
+    for (uint i = 0; i < m.Height(); ++i)
+        for (uint j = 0; j < m.Width(); ++j) m.index(i, j) = f();
+}
+static std::vector<float> dense(de::Matrix<float>& m) {
+    std::vector<float> v((size_t)m.Height() * m.Width());
+    for (uint i = 0; i < m.Height(); ++i)
+        for (uint j = 0; j < m.Width(); ++j) v[(size_t)i * m.Width() + j] = m.index(i, j);
+    return v;
+}
+static std::vector<float> chain(de::Matrix<float>& A, de::Matrix<float>& B, de::Matrix<float>* C = nullptr) {
+    int M = A.Height(), K = A.Width(), N = B.Width();
+    std::vector<float> a = dense(A), b = dense(B), c, d((size_t)M * N);
+    if (C) c = dense(*C);
+    oracle_sgemm_chain_fast(a.data(), K, b.data(), N, C ? c.data() : nullptr, N, d.data(), N, M, N, K, 0);
+    return d;
+}
+
+// ------------------------------------------------------------------ CPU-only checks ----------------------------
+static void containers_follow_reference_pitch_rules() {
+    de::Matrix<float>& m = de::CreateMatrixRef<float>(13, 7, decx::Page_Default);
+    CHECK(m.Width() == 13 && m.Height() == 7 && m.TotalBytes() == 16u * 7 * 4);     // pitch = ceil8(13) = 16
+    m.index(6, 12) = 3.5f;
+    CHECK((&m.index(6, 12)) - (&m.index(0, 0)) == 6 * 16 + 12);
+    de::Matrix<de::Half>& h = de::CreateMatrixRef<de::Half>(17, 3, decx::Page_Default);
+    CHECK(h.TotalBytes() == 32u * 3 * 2);                                             // pitch = ceil16(17) = 32
+    de::Tensor<float>& t = de::CreateTensorRef<float>(5, 6, 3, decx::Page_Default);  // width 5, height 6, depth 3
+    CHECK(t.Width() == 5 && t.Height() == 6 && t.Depth() == 3);
+    CHECK((&t.index(1, 0, 0)) - (&t.index(0, 0, 0)) == 8 * 4);                        // wpitch 8, dpitch 4
+    CHECK((&t.index(0, 1, 0)) - (&t.index(0, 0, 0)) == 4);
+    bool zero = true;
+    for (int i = 0; i < 6 * 8 * 4; ++i) zero = zero && (&t.index(0, 0, 0))[i] == 0.0f;
+    CHECK(zero);                                                                      // Tensor.h:312 zero-fills
+    de::TensorArray<float>& ta = de::CreateTensorArrayRef<float>(3, 3, 64, 5, decx::Page_Default);
+    CHECK(ta.TensorNum() == 5 && (&ta.index(0, 0, 0, 1)) - (&ta.index(0, 0, 0, 0)) == 3 * 4 * 64);   // _gap
+    CHECK((&ta.index(1, 2, 7, 0)) - (&ta.index(0, 0, 0, 0)) == 1 * 4 * 64 + 2 * 64 + 7);
+    m.release(); h.release(); t.release(); ta.release();
+}
+
+static void half_conversion() {
+    CHECK(de::Float2Half(1.0f).val == 0x3C00 && de::Float2Half(-2.0f).val == 0xC000);
+    CHECK(de::Float2Half(65504.0f).val == 0x7BFF && de::Float2Half(65520.0f).val == 0x7C00);
+    CHECK(de::Float2Half(1.00048828125f).val == 0x3C00 && de::Float2Half(1.00146484375f).val == 0x3C02);   // ties to even
+    CHECK(de::Float2Half(5.9604645e-8f).val == 0x0001 && de::Float2Half(2.9802322e-8f).val == 0x0000);
+    for (unsigned v = 0; v < 0x7C00; ++v) {
+        de::Half h; h.val = (unsigned short)v;
+        CHECK(de::Float2Half(de::Half2Float(h)).val == v);
+        if (g_fail) break;
+    }
+}
+
+static void gemm_refuses_before_init() {
+    de::Matrix<float>& A = de::CreateMatrixRef<float>(8, 8, decx::Page_Default);
+    de::Matrix<float>& B = de::CreateMatrixRef<float>(8, 8, decx::Page_Default);
+    de::Matrix<float>& C = de::CreateMatrixRef<float>();
+    de::DH h = de::cuda::GEMM(A, B, C);
+    CHECK(h.error_type == decx::DECX_FAIL_not_init && std::strstr(h.error_string, "initialized first"));
+    de::Tensor<float>& s = de::CreateTensorRef<float>(8, 8, 4, decx::Page_Default);
+    de::TensorArray<float>& k = de::CreateTensorArrayRef<float>(3, 3, 4, 2, decx::Page_Default);
+    de::Tensor<float>& d = de::CreateTensorRef<float>();
+    CHECK(de::cuda::Conv2_MK_im2col(s, k, d, 1).error_type == decx::DECX_FAIL_not_init);
+}
+
+static void cpu_sgemm_case(int M, int K, int N, bool ints) {
+    de::Matrix<float>& A = de::CreateMatrixRef<float>(K, M, decx::Page_Default);
+    de::Matrix<float>& B = de::CreateMatrixRef<float>(N, K, decx::Page_Default);
+    de::Matrix<float>& C = de::CreateMatrixRef<float>();
+    if (ints) { fill(A, small_int); fill(B, small_int); } else { fill(A, unif); fill(B, unif); }
+    de::DH h = de::cpu::sgemm(A, B, C);
+    CHECK(h.error_type == decx::DECX_SUCCESS && C.Width() == (uint)N && C.Height() == (uint)M);
+    std::vector<float> got = dense(C), want = chain(A, B);
+    CHECK(std::memcmp(got.data(), want.data(), got.size() * 4) == 0);                // bit-identical to the fused chain
+    A.release(); B.release(); C.release();
+}
+static void cpu_sgemm_matches_chain_bit_for_bit() {
+    cpu_sgemm_case(1024, 1024, 1024, false);      // config 1
+    cpu_sgemm_case(100, 136, 72, false);
+    cpu_sgemm_case(33, 7, 9, false);
+    cpu_sgemm_case(1, 1, 1, false);
+    cpu_sgemm_case(301, 150, 455, true);
+    de::Matrix<float>& A = de::CreateMatrixRef<float>(10, 4, decx::Page_Default);
+    de::Matrix<float>& B = de::CreateMatrixRef<float>(4, 11, decx::Page_Default);
+    de::Matrix<float>& C = de::CreateMatrixRef<float>();
+    CHECK(de::cpu::sgemm(A, B, C).error_type == decx::DECX_FAIL_DimsNotMatching);    // sgemm.h:35-38
+}
+
+// ------------------------------------------------------------------ GPU checks --------------------------------
+static double rel_err(const std::vector<float>& got, const std::vector<float>& ref, double scale) {
+    double e = 0;
+    for (size_t i = 0; i < got.size(); ++i) e = std::fmax(e, std::fabs((double)got[i] - ref[i]) / scale);
+    return e;
+}
+
+template <int M, int N, int K>
+static void cuda_gemm_mem_exch() {     // CUDA_GEMM.cpp:15-57
+    de::Matrix<float>& A = de::CreateMatrixRef<float>(K, M, 0);
+    de::Matrix<float>& B = de::CreateMatrixRef<float>(N, K, 0);
+    de::Matrix<float>& C = de::CreateMatrixRef<float>(N, M, 0);
+    for (uint i = 0; i < A.Height(); ++i) for (uint j = 0; j < A.Width(); ++j) A.index(i, j) = j * 0.1;
+    for (uint i = 0; i < B.Height(); ++i) for (uint j = 0; j < B.Width(); ++j) B.index(i, j) = i * 0.1;
+    float sum = 0;
+    for (int i = 0; i < K; ++i) sum += (0.1 * i * 0.1 * i);
+    de::DH h = de::cuda::GEMM(A, B, C);
+    CHECK(h.error_type == decx::DECX_SUCCESS);
+    bool all = true;
+    for (uint i = 0; i < C.Height(); ++i)
+        for (uint j = 0; j < C.Width(); ++j) all = all && std::fabs(C.index(i, j) - sum) / sum < 1e-5 * std::sqrt((double)K);
+    CHECK(all);
+    A.release(); B.release(); C.release();
+}
+template <int M, int N, int K>
+static void cuda_gemm_on_GPU() {       // CUDA_GEMM.cpp:59-109
+    de::Matrix<float>& A = de::CreateMatrixRef<float>(K, M, 0);
+    de::Matrix<float>& B = de::CreateMatrixRef<float>(N, K, 0);
+    de::Matrix<float>& C = de::CreateMatrixRef<float>(N, M, 0);
+    de::GPU_Matrix<float>& dA = de::CreateGPUMatrixRef<float>(K, M);
+    de::GPU_Matrix<float>& dB = de::CreateGPUMatrixRef<float>(N, K);
+    de::GPU_Matrix<float>& dC = de::CreateGPUMatrixRef<float>(N, M);
+    for (uint i = 0; i < A.Height(); ++i) for (uint j = 0; j < A.Width(); ++j) A.index(i, j) = j * 0.1;
+    for (uint i = 0; i < B.Height(); ++i) for (uint j = 0; j < B.Width(); ++j) B.index(i, j) = i * 0.1;
+    float sum = 0;
+    for (int i = 0; i < K; ++i) sum += (0.1 * i * 0.1 * i);
+    dA.Load_from_host(A); dB.Load_from_host(B);
+    de::DH h = de::cuda::GEMM(dA, dB, dC);
+    CHECK(h.error_type == decx::DECX_SUCCESS);
+    dC.Load_to_host(C);
+    bool all = true;
+    for (uint i = 0; i < C.Height(); ++i)
+        for (uint j = 0; j < C.Width(); ++j) all = all && std::fabs(C.index(i, j) - sum) / sum < 1e-5 * std::sqrt((double)K);
+    CHECK(all);
+    A.release(); B.release(); C.release(); dA.release(); dB.release(); dC.release();
+}
+static void reference_demo_known_answer() {
+    cuda_gemm_mem_exch<512, 1024, 2048>();
+    cuda_gemm_on_GPU<2048, 2048, 2048>();        // what the reference's main() runs (CUDA_GEMM.cpp:112-116)
+}
+
+static void gemm_fp32_all_flavours() {
+    const int M = 300, K = 150, N = 450;     // ragged everywhere
+    de::Matrix<float>& A = de::CreateMatrixRef<float>(K, M, 0);
+    de::Matrix<float>& B = de::CreateMatrixRef<float>(N, K, 0);
+    de::Matrix<float>& C = de::CreateMatrixRef<float>(N, M, 0);
+    de::Matrix<float>& D = de::CreateMatrixRef<float>();
+    fill(A, small_int); fill(B, small_int); fill(C, small_int);
+    CHECK(de::cuda::GEMM(A, B, D).error_type == 0 && D.Width() == (uint)N && D.Height() == (uint)M);
+    CHECK(dense(D) == chain(A, B));                                        // integer data: exact
+    CHECK(de::cuda::GEMM(A, B, C, D).error_type == 0);
+    CHECK(dense(D) == chain(A, B, &C));
+    std::vector<float> want = chain(A, B, &C);
+    CHECK(de::cuda::GEMM(A, B, C, C).error_type == 0);                     // dst aliasing C
+    CHECK(dense(C) == want);
+    // device-resident flavours
+    de::GPU_Matrix<float>& dA = de::CreateGPUMatrixRef<float>(K, M);
+    de::GPU_Matrix<float>& dB = de::CreateGPUMatrixRef<float>(N, K);
+    de::GPU_Matrix<float>& dC = de::CreateGPUMatrixRef<float>(N, M);
+    de::GPU_Matrix<float>& dD = de::CreateGPUMatrixRef<float>();          // empty: GEMM sizes it (GEMM.h:414)
+    fill(A, unif); fill(B, unif); fill(C, unif);
+    dA.Load_from_host(A); dB.Load_from_host(B); dC.Load_from_host(C);
+    CHECK(de::cuda::GEMM(dA, dB, dD).error_type == 0 && dD.Width() == (uint)N && dD.Height() == (uint)M);
+    de::Matrix<float>& R = de::CreateMatrixRef<float>(N, M, 0);
+    dD.Load_to_host(R);
+    CHECK(rel_err(dense(R), chain(A, B), K * 0.33) < 1e-5 * std::sqrt((double)K));
+    CHECK(de::cuda::GEMM(dA, dB, dC, dD).error_type == 0);
+    dD.Load_to_host(R);
+    CHECK(rel_err(dense(R), chain(A, B, &C), K * 0.33) < 1e-5 * std::sqrt((double)K));
+    // dims mismatch -> 0x03 (GEMM.h:68, :408)
+    de::Matrix<float>& Bad = de::CreateMatrixRef<float>(N, K + 1, 0);
+    de::DH h = de::cuda::GEMM(A, Bad, D);
+    CHECK(h.error_type == decx::DECX_FAIL_DimsNotMatching && std::strstr(h.error_string, "width of matrix A"));
+    de::GPU_Matrix<float>& dBad = de::CreateGPUMatrixRef<float>(N, K + 1);
+    CHECK(de::cuda::GEMM(dA, dBad, dD).error_type == decx::DECX_FAIL_DimsNotMatching);
+}
+
+static void gemm_fp16_flavours() {
+    const int M = 130, K = 200, N = 77;
+    de::Matrix<de::Half>& A = de::CreateMatrixRef<de::Half>(K, M, 0);
+    de::Matrix<de::Half>& B = de::CreateMatrixRef<de::Half>(N, K, 0);
+    de::Matrix<de::Half>& D = de::CreateMatrixRef<de::Half>();
+    std::vector<uint16_t> a((size_t)M * K), b((size_t)K * N);
+    for (int i = 0; i < M; ++i) for (int j = 0; j < K; ++j) { A.index(i, j) = de::Float2Half(unif()); a[(size_t)i * K + j] = A.index(i, j).val; }
+    for (int i = 0; i < K; ++i) for (int j = 0; j < N; ++j) { B.index(i, j) = de::Float2Half(unif()); b[(size_t)i * N + j] = B.index(i, j).val; }
+    std::vector<int> rows(M);
+    for (int i = 0; i < M; ++i) rows[i] = i;
+    std::vector<double> ref((size_t)M * N), scale((size_t)M * N);
+    oracle_gemm_f64_rows_f16(a.data(), K, b.data(), N, rows.data(), M, ref.data(), scale.data(), N, K, 0);
+    auto check = [&](de::Matrix<de::Half>& R) {
+        double e = 0;
+        for (int i = 0; i < M; ++i)
+            for (int j = 0; j < N; ++j)
+                e = std::fmax(e, std::fabs(de::Half2Float(R.index(i, j)) - ref[(size_t)i * N + j]) / scale[(size_t)i * N + j]);
+        return e;
+    };
+    CHECK(de::cuda::GEMM(A, B, D).error_type == 0 && D.Width() == (uint)N && D.Height() == (uint)M);
+    CHECK(check(D) < 2e-3);
+    de::GPU_Matrix<de::Half>& dA = de::CreateGPUMatrixRef<de::Half>(K, M);
+    de::GPU_Matrix<de::Half>& dB = de::CreateGPUMatrixRef<de::Half>(N, K);
+    de::GPU_Matrix<de::Half>& dD = de::CreateGPUMatrixRef<de::Half>();    // not pre-sized: the fp32 behaviour (GEMM.h:414)
+    dA.Load_from_host(A); dB.Load_from_host(B);
+    CHECK(de::cuda::GEMM(dA, dB, dD).error_type == 0);
+    de::Matrix<de::Half>& R = de::CreateMatrixRef<de::Half>(N, M, 0);
+    dD.Load_to_host(R);
+    CHECK(check(R) < 2e-3);
+}
+
+static void conv_case(int H, int W, int C, int N, int kh, int kw, int flag) {
+    de::Tensor<float>& src = de::CreateTensorRef<float>(W, H, C, 0);
+    de::TensorArray<float>& ker = de::CreateTensorArrayRef<float>(kw, kh, C, N, 0);
+    de::Tensor<float>& dst = de::CreateTensorRef<float>();
+    for (int y = 0; y < H; ++y) for (int x = 0; x < W; ++x) for (int c = 0; c < C; ++c) src.index(y, x, c) = small_int();
+    for (int n = 0; n < N; ++n) for (int i = 0; i < kh; ++i) for (int j = 0; j < kw; ++j) for (int c = 0; c < C; ++c) ker.index(i, j, c, n) = small_int();
+    de::DH h = de::cuda::Conv2_MK_im2col(src, ker, dst, flag);
+    CHECK(h.error_type == decx::DECX_SUCCESS);
+    const int Ho = flag ? H : H - 2 * (kh / 2), Wo = flag ? W : W - 2 * (kw / 2);
+    CHECK(dst.Width() == (uint)Wo && dst.Height() == (uint)Ho && dst.Depth() == (uint)N);
+    const long s_row = &src.index(1, 0, 0) - &src.index(0, 0, 0), dp = &src.index(0, 1, 0) - &src.index(0, 0, 0);
+    const long k_gap = N > 1 ? &ker.index(0, 0, 0, 1) - &ker.index(0, 0, 0, 0) : (long)kh * ((kw + 3) / 4 * 4) * dp;
+    const long k_row = kh > 1 ? &ker.index(1, 0, 0, 0) - &ker.index(0, 0, 0, 0) : (long)((kw + 3) / 4 * 4) * dp;
+    std::vector<float> want((size_t)Ho * Wo * N);
+    CHECK(oracle_conv2_chain(&src.index(0, 0, 0), H, W, (int)dp, s_row, &ker.index(0, 0, 0, 0), N, kh, kw, k_gap, k_row,
+                             want.data(), N, (long)Wo * N, flag, 0) == 0);
+    bool same = true;
+    for (int y = 0; y < Ho; ++y) for (int x = 0; x < Wo; ++x) for (int n = 0; n < N; ++n)
+        same = same && dst.index(y, x, n) == want[((size_t)y * Wo + x) * N + n];
+    CHECK(same);
+    src.release(); ker.release(); dst.release();
+}
+static void conv_flavours_and_flags() {
+    conv_case(20, 22, 8, 6, 3, 3, decx::de_conv_zero_compensate);
+    conv_case(20, 22, 8, 6, 3, 3, decx::de_conv_no_compensate);
+    conv_case(33, 31, 3, 7, 5, 3, decx::de_conv_zero_compensate);
+    conv_case(56, 56, 64, 128, 3, 3, decx::de_conv_zero_compensate);
+    de::Tensor<float>& s = de::CreateTensorRef<float>(8, 8, 4, 0);
+    de::TensorArray<float>& k = de::CreateTensorArrayRef<float>(3, 3, 4, 2, 0);
+    de::Tensor<float>& d = de::CreateTensorRef<float>();
+    de::DH h = de::cuda::Conv2_MK_im2col(s, k, d, 7);
+    CHECK(h.error_type == decx::DECX_FAIL_ErrorFlag);
+    de::TensorArray<float>& k2 = de::CreateTensorArrayRef<float>(3, 3, 8, 2, 0);
+    CHECK(de::cuda::Conv2_MK_im2col(s, k2, d, 1).error_type == decx::DECX_FAIL_DimsNotMatching);
+}
+
+int main(int argc, char** argv) {
+    std::string mode = argc > 1 ? argv[1] : "cpu";
+    if (mode == "cpu") {
+        RUN(containers_follow_reference_pitch_rules);
+        RUN(half_conversion);
+        RUN(gemm_refuses_before_init);
+        RUN(cpu_sgemm_matches_chain_bit_for_bit);
+    } else {
+        de::InitCuda();
+        RUN(reference_demo_known_answer);
+        RUN(gemm_fp32_all_flavours);
+        RUN(gemm_fp16_flavours);
+        RUN(conv_flavours_and_flags);
+    }
+    std::printf("%s: %d failure(s)\n", mode.c_str(), g_fail);
+    return g_fail ? 1 : 0;
+}
