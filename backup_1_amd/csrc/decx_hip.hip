@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <cstring>
 
+#include "hgemm_dma_tile.hpp"
 #include "hgemm_tile.hpp"
 #include "sgemm_tile.hpp"
 
@@ -161,11 +162,35 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
 //   2: 128x128x32, 2x2 waves of  64x64
 typedef HgemmShape<256, 256, 32, 2, 2> HShapeBig;
 typedef HgemmShape<128, 128, 32, 2, 2> HShapeSmall;
+//   3: 256x256x32, 2x2 waves of 128x128, 4-stage LDS-DMA pipeline
+typedef HgemmDmaShape<256, 256, 32, 2, 2, 4> HShapeDma;
 
 template <class S, bool VEC>
 int launch_hgemm_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                       int ldd, int M, int N, int K) {
     auto kern = hgemm_tile_kernel<S, VEC>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)S::LDS_BYTES));
+        attr_done = true;
+    }
+    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    const long total = (long)tiles_m * tiles_n;
+    if (total > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
+    const int group_m = tiles_m < 8 ? tiles_m : 8;
+    hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream,
+                       reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
+                       reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N, K,
+                       tiles_m, tiles_n, group_m);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+template <class S>
+int launch_hgemm_dma_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
+                          uint16_t* D, int ldd, int M, int N, int K) {
+    auto kern = hgemm_dma_kernel<S>;
     static bool attr_done = false;
     if (!attr_done) {
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -194,10 +219,11 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
     const bool vec = aligned16(A) && aligned16(B) && lda % 8 == 0 && ldb % 8 == 0 && ldb >= 8;
     if (!vec) return launch_hgemm_tile<HShapeSmall, false>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
     int variant = g_rt.hgemm_variant;
-    if (variant < 1 || variant > 2) {
+    if (variant < 1 || variant > 3) {
         const int cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
-        variant = ((long)cdiv(M, 256) * cdiv(N, 256) * 10 >= (long)cus * 8) ? 1 : 2;
+        variant = ((long)cdiv(M, 256) * cdiv(N, 256) * 10 >= (long)cus * 8) ? 3 : 2;
     }
+    if (variant == 3) return launch_hgemm_dma_tile<HShapeDma>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
     if (variant == 1) return launch_hgemm_tile<HShapeBig, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
     return launch_hgemm_tile<HShapeSmall, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
 }
