@@ -57,10 +57,10 @@ inline int cdiv(int a, int b) { return (a + b - 1) / b; }
 // ---------------------------------------------------------------------------------------------------------------
 // fp32 launchers
 // ---------------------------------------------------------------------------------------------------------------
-template <class S, class ASrc, class BSrc, class Out>
-int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, float* D, const Out& out, int M, int N,
-                      int K) {
-    auto kern = sgemm_tile_kernel<S, ASrc, BSrc, Out>;
+template <class S, class ASrc, class BSrc, class Out, bool HAS_C>
+int launch_sgemm_tile_c(const ASrc& a, const BSrc& b, const float* Cin, int ldc, float* D, const Out& out, int M, int N,
+                        int K) {
+    auto kern = sgemm_tile_kernel<S, ASrc, BSrc, Out, HAS_C>;
     static bool attr_done = false;
     if (!attr_done) {
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -75,6 +75,13 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
                        N, K, tiles_m, tiles_n, group_m);
     HIP_TRY(hipGetLastError());
     return 0;
+}
+
+template <class S, class ASrc, class BSrc, class Out>
+int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, float* D, const Out& out, int M, int N,
+                      int K) {
+    if (Cin != nullptr) return launch_sgemm_tile_c<S, ASrc, BSrc, Out, true>(a, b, Cin, ldc, D, out, M, N, K);
+    return launch_sgemm_tile_c<S, ASrc, BSrc, Out, false>(a, b, Cin, ldc, D, out, M, N, K);
 }
 
 // Tile shapes (variant numbers of decx_hip_set_sgemm_variant):

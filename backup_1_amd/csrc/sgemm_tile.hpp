@@ -226,7 +226,7 @@ struct SgemmShape {
     static_assert(NT % KQ == 0, "A staging: KQ lanes per row");
 };
 
-template <class S, class ASrc, class BSrc, class Out>
+template <class S, class ASrc, class BSrc, class Out, bool HAS_C>
 __global__ __launch_bounds__(S::NT) void sgemm_tile_kernel(ASrc a_src, BSrc b_src, const float* Cin, int ldc, float* D,
                                                            Out out, int M, int N, int K, int tiles_m, int tiles_n,
                                                            int group_m) {
@@ -266,7 +266,6 @@ __global__ __launch_bounds__(S::NT) void sgemm_tile_kernel(ASrc a_src, BSrc b_sr
         b_src.template store<S>(Bs + buf * KQ * S::B_ROW, b_stage, tid);
     };
 
-    // ---- accumulators: start from C for dst = A*B + C (the reference pre-loads them too, GEMM.cuh:223) ---------
     f32x16 acc[MI][NI];
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
@@ -274,37 +273,8 @@ __global__ __launch_bounds__(S::NT) void sgemm_tile_kernel(ASrc a_src, BSrc b_sr
         for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
-    if (Cin != nullptr) {
-#pragma unroll
-        for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-                if (m < M) {
-                    const float* crow = Cin + (size_t)m * ldc;
-#pragma unroll
-                    for (int ni = 0; ni < NI; ++ni) {
-                        const int n = bn0 + wn0 + ni * 32 + li;
-                        if (n < N) acc[mi][ni][r] = crow[n];
-                    }
-                }
-            }
-    }
 
-    const int full_steps = K / BK;
-    const int steps = (K + BK - 1) / BK;
-
-    if (full_steps > 0) load_stage(0, std::false_type{});
-    else load_stage(0, std::true_type{});
-    store_stage(0);
-    __syncthreads();
-
-    for (int t = 0; t < steps; ++t) {
-        const int buf = t & 1;
-        if (t + 1 < steps) {
-            if (t + 1 < full_steps) load_stage((t + 1) * BK, std::false_type{});
-            else load_stage((t + 1) * BK, std::true_type{});
-        }
+    auto compute_stage = [&](int buf) {
         const f32x4* Ab = As + buf * KQ * S::A_ROW;
         const f32x4* Bb = Bs + buf * KQ * S::B_ROW;
 #pragma unroll
@@ -326,13 +296,40 @@ __global__ __launch_bounds__(S::NT) void sgemm_tile_kernel(ASrc a_src, BSrc b_sr
                     for (int ni = 0; ni < NI; ++ni)
                         acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[mi][e], bf[ni][e], acc[mi][ni], 0, 0, 0);
         }
-        if (t + 1 < steps) {
-            store_stage(buf ^ 1);     // that buffer was last read before the previous barrier
+    };
+
+    // K walk.  The loop over full steps is straight-line (load next, compute current, stage next, one barrier); the
+    // partial last step, if any, is peeled out so that its masking code never sits on the main path.
+    const int full_steps = K / BK;
+    const bool has_tail = full_steps * BK < K;
+
+    if (full_steps > 0) load_stage(0, std::false_type{});
+    else load_stage(0, std::true_type{});
+    store_stage(0);
+    __syncthreads();
+
+    for (int t = 0; t + 1 < full_steps; ++t) {
+        load_stage((t + 1) * BK, std::false_type{});
+        __builtin_amdgcn_sched_barrier(0);   // keep the global loads ahead of the MFMAs: their latency hides behind them
+        compute_stage(t & 1);
+        __builtin_amdgcn_sched_barrier(0);
+        store_stage((t + 1) & 1);     // that buffer was last read before the previous barrier
+        __syncthreads();
+    }
+    if (full_steps > 0) {
+        if (has_tail) load_stage(full_steps * BK, std::true_type{});
+        compute_stage((full_steps - 1) & 1);
+        if (has_tail) {
+            store_stage(full_steps & 1);
             __syncthreads();
+            compute_stage(full_steps & 1);
         }
+    } else {
+        compute_stage(0);             // K < BK: the prologue staged the only, partial step
     }
 
-    // ---- epilogue: each lane holds column li of its 32-wide block; a half-wave writes 128 contiguous bytes ------
+    // ---- epilogue: each lane holds column li of its 32-wide block; a half-wave writes 128 contiguous bytes.
+    // dst = A*B + C adds C here (C may alias dst: every element is read and written by the same lane).
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
@@ -340,10 +337,11 @@ __global__ __launch_bounds__(S::NT) void sgemm_tile_kernel(ASrc a_src, BSrc b_sr
             const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
             if (m < M) {
                 float* drow = D + out.offset(m);
+                const float* crow = HAS_C ? Cin + (size_t)m * ldc : nullptr;
 #pragma unroll
                 for (int ni = 0; ni < NI; ++ni) {
                     const int n = bn0 + wn0 + ni * 32 + li;
-                    if (n < N) drow[n] = acc[mi][ni][r];
+                    if (n < N) drow[n] = HAS_C ? acc[mi][ni][r] + crow[n] : acc[mi][ni][r];
                 }
             }
         }
