@@ -89,8 +89,8 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //   2: 128x128x16, 2x2 waves of  64x64    -- small problems, several workgroups per CU
 //   3: 256x128x16, 2x2 waves of 128x64    -- narrow N (the convolution's 128 filters)
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
-typedef SgemmShape<128, 128, 16, 2, 2> SShapeSmall;
-typedef SgemmShape<256, 128, 16, 2, 2> SShapeTall;
+typedef SgemmShape<128, 128, 16, 2, 2, 2> SShapeSmall;
+typedef SgemmShape<256, 128, 16, 2, 2, 2> SShapeTall;
 
 int pick_sgemm_variant(int M, int N) {
     if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 3) return g_rt.sgemm_variant;

@@ -26,7 +26,10 @@ namespace decx_hip {
 // ---------------------------------------------------------------------------------------------------------------
 // A-operand sources.  Interface:
 //   RowState row_state(int m)                       per-row values that do not change along K
-//   template<bool TAIL> f32x4 load(rs, k)           A[m][k..k+3]; TAIL zero-fills elements with k >= K
+//   template<bool TAIL> f32x4 load(rs, k, keep)     A[m][k..k+3] read from an always-valid address; the caller replaces
+//                                                   the quad by zeros when keep comes back false (deferred, so that the
+//                                                   load itself stays branch-free and nothing waits on it early);
+//                                                   TAIL additionally zero-fills elements with k >= K
 //   size_t out_offset(int m)                        where row m of the result starts, in elements
 // ---------------------------------------------------------------------------------------------------------------
 template <bool VEC>
@@ -42,7 +45,8 @@ struct DenseA {
         return rs;
     }
     template <bool TAIL>
-    __device__ __forceinline__ f32x4 load(const RowState& rs, int k) const {
+    __device__ __forceinline__ f32x4 load(const RowState& rs, int k, bool& keep) const {
+        keep = true;
         f32x4 v = {0.f, 0.f, 0.f, 0.f};
         if (VEC) {
             if (!TAIL) {
@@ -78,15 +82,16 @@ struct Im2colA {
         return rs;
     }
     template <bool TAIL>
-    __device__ __forceinline__ f32x4 load(const RowState& rs, int k) const {
-        f32x4 v = {0.f, 0.f, 0.f, 0.f};
-        if (TAIL && k >= K) return v;           // K = kh*kw*dpitch is a multiple of 4: quads never straddle it
-        const int tap = k / dpitch, c = k - tap * dpitch;
+    __device__ __forceinline__ f32x4 load(const RowState& rs, int k, bool& keep) const {
+        // K = kh*kw*dpitch is a multiple of 4: quads never straddle it
+        const bool k_ok = !TAIL || k < K;
+        const int kk = k_ok ? k : 0;
+        const int tap = kk / dpitch, c = kk - tap * dpitch;
         const int ki = tap / kw, kj = tap - ki * kw;
         const int sy = rs.y + ki, sx = rs.x + kj;
-        if (sy >= 0 && sy < H && sx >= 0 && sx < W)
-            v = *reinterpret_cast<const f32x4*>(src + (size_t)sy * row_stride + (size_t)sx * dpitch + c);
-        return v;
+        keep = k_ok && sy >= 0 && sy < H && sx >= 0 && sx < W;
+        const int cy = sy < 0 ? 0 : (sy >= H ? H - 1 : sy), cx = sx < 0 ? 0 : (sx >= W ? W - 1 : sx);
+        return *reinterpret_cast<const f32x4*>(src + (size_t)cy * row_stride + (size_t)cx * dpitch + c);
     }
 };
 
@@ -209,9 +214,10 @@ struct FilterB {
     }
 };
 
-template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_>
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int WAVES_PER_SIMD_ = 1>
 struct SgemmShape {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+    static constexpr int WAVES_PER_SIMD = WAVES_PER_SIMD_;   // occupancy the register budget is held to
     static constexpr int NT = WAVES_M * WAVES_N * kWave;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     static constexpr int MI = WM / 32, NI = WN / 32;
@@ -227,7 +233,7 @@ struct SgemmShape {
 };
 
 template <class S, class ASrc, class BSrc, class Out, bool HAS_C>
-__global__ __launch_bounds__(S::NT) void sgemm_tile_kernel(ASrc a_src, BSrc b_src, const float* Cin, int ldc, float* D,
+__global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(ASrc a_src, BSrc b_src, const float* Cin, int ldc, float* D,
                                                            Out out, int M, int N, int K, int tiles_m, int tiles_n,
                                                            int group_m) {
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, NT = S::NT, KQ = S::KQ, MI = S::MI, NI = S::NI;
@@ -250,19 +256,23 @@ __global__ __launch_bounds__(S::NT) void sgemm_tile_kernel(ASrc a_src, BSrc b_sr
 #pragma unroll
     for (int p = 0; p < S::A_PASSES; ++p) a_rs[p] = a_src.row_state(bm0 + a_r + p * A_RSTEP);
     f32x4 a_stage[S::A_PASSES];
+    bool a_keep[S::A_PASSES];
     f32x4 b_stage[BSrc::template quads<S>()];
 
     auto load_stage = [&](int k0, auto tail_tag) {
         constexpr bool TAIL = decltype(tail_tag)::value;
 #pragma unroll
-        for (int p = 0; p < S::A_PASSES; ++p) a_stage[p] = a_src.template load<TAIL>(a_rs[p], k0 + 4 * a_q);
+        for (int p = 0; p < S::A_PASSES; ++p) a_stage[p] = a_src.template load<TAIL>(a_rs[p], k0 + 4 * a_q, a_keep[p]);
         b_src.template load<S, TAIL>(b_stage, tid, k0, bn0);
     };
 
     auto store_stage = [&](int buf) {
         f32x4* Ab = As + buf * KQ * S::A_ROW;
 #pragma unroll
-        for (int p = 0; p < S::A_PASSES; ++p) Ab[a_q * S::A_ROW + a_r + p * A_RSTEP] = a_stage[p];
+        for (int p = 0; p < S::A_PASSES; ++p) {
+            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+            Ab[a_q * S::A_ROW + a_r + p * A_RSTEP] = a_keep[p] ? a_stage[p] : zero;
+        }
         b_src.template store<S>(Bs + buf * KQ * S::B_ROW, b_stage, tid);
     };
 
@@ -274,32 +284,40 @@ __global__ __launch_bounds__(S::NT) void sgemm_tile_kernel(ASrc a_src, BSrc b_sr
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
 
-    auto compute_stage = [&](int buf) {
+    // Fragments of one quad pair s: per 32-row / 32-column block one float4 = four consecutive k of this lane's k-slot.
+    auto read_frags = [&](int buf, int s, f32x4* af, f32x4* bf) {
         const f32x4* Ab = As + buf * KQ * S::A_ROW;
         const f32x4* Bb = Bs + buf * KQ * S::B_ROW;
+        const int q = 2 * s + lh;
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi) af[mi] = Ab[q * S::A_ROW + wm0 + mi * 32 + li];
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) {
+            const int n = wn0 + ni * 32 + li;
+            bf[ni] = Bb[q * S::B_ROW + n + (n >> 4)];
+        }
+    };
+    // MFMAs number lo .. hi-1 of a quad pair, in the order (e, mi, ni); a full pair is 4*MI*NI of them.
+    constexpr int PAIR_MFMAS = 4 * MI * NI;
+    auto mfma_range = [&](const f32x4* af, const f32x4* bf, auto lo_tag, auto hi_tag) {
+        constexpr int LO = decltype(lo_tag)::value, HI = decltype(hi_tag)::value;
+#pragma unroll
+        for (int i = LO; i < HI; ++i) {
+            const int e = i / (MI * NI), mi = (i / NI) % MI, ni = i % NI;
+            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[mi][e], bf[ni][e], acc[mi][ni], 0, 0, 0);
+        }
+    };
+    auto compute_stage = [&](int buf) {      // unpipelined: used for the peeled steps only
 #pragma unroll
         for (int s = 0; s < KQ / 2; ++s) {
             f32x4 af[MI], bf[NI];
-            const int q = 2 * s + lh;
-#pragma unroll
-            for (int mi = 0; mi < MI; ++mi) af[mi] = Ab[q * S::A_ROW + wm0 + mi * 32 + li];
-#pragma unroll
-            for (int ni = 0; ni < NI; ++ni) {
-                const int n = wn0 + ni * 32 + li;
-                bf[ni] = Bb[q * S::B_ROW + n + (n >> 4)];
-            }
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-#pragma unroll
-                for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-                    for (int ni = 0; ni < NI; ++ni)
-                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[mi][e], bf[ni][e], acc[mi][ni], 0, 0, 0);
+            read_frags(buf, s, af, bf);
+            mfma_range(af, bf, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
         }
     };
 
-    // K walk.  The loop over full steps is straight-line (load next, compute current, stage next, one barrier); the
-    // partial last step, if any, is peeled out so that its masking code never sits on the main path.
+    // K walk.  Full steps run a software-pipelined loop; the partial last step, if any, is peeled out so that its
+    // masking code never sits on the main path.
     const int full_steps = K / BK;
     const bool has_tail = full_steps * BK < K;
 
@@ -308,21 +326,70 @@ __global__ __launch_bounds__(S::NT) void sgemm_tile_kernel(ASrc a_src, BSrc b_sr
     store_stage(0);
     __syncthreads();
 
-    for (int t = 0; t + 1 < full_steps; ++t) {
-        load_stage((t + 1) * BK, std::false_type{});
-        __builtin_amdgcn_sched_barrier(0);   // keep the global loads ahead of the MFMAs: their latency hides behind them
-        compute_stage(t & 1);
-        __builtin_amdgcn_sched_barrier(0);
-        store_stage((t + 1) & 1);     // that buffer was last read before the previous barrier
-        __syncthreads();
-    }
     if (full_steps > 0) {
+        static_assert(KQ == 4, "the pipelined loop is written for two quad pairs per K step");
+        constexpr int VMEM_OPS = S::A_PASSES + BSrc::template quads<S>();     // global loads per thread and step
+        constexpr int FRAG_OPS = MI + NI;                                     // ds_read_b128 per quad pair
+        constexpr int WRITE_OPS = S::A_PASSES + BSrc::template quads<S>();    // ds_write_b128 per thread and step
+        f32x4 af0[MI], bf0[NI], af1[MI], bf1[NI];
+        read_frags(0, 0, af0, bf0);
+        // Steady state of one K step t (LDS buffer t&1 holds it, fragments of its first quad pair are in af0/bf0):
+        //   pair 0 MFMAs   interleaved with: global loads of step t+1, LDS reads of pair 1
+        //   pair 1 MFMAs   interleaved with: LDS writes of step t+1 into the other buffer
+        //   barrier, then the LDS reads of step t+1's pair 0 hide behind the last few MFMAs of pair 1.
+        // Every memory instruction sits between MFMAs, so the matrix pipe is never starved by an in-order wait.
+        for (int t = 0; t + 1 < full_steps; ++t) {
+            const int buf = t & 1;
+            load_stage((t + 1) * BK, std::false_type{});
+            read_frags(buf, 1, af1, bf1);
+            mfma_range(af0, bf0, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
+            // scheduling-group masks: 0x002 VALU, 0x008 MFMA, 0x020 VMEM read, 0x100 DS read, 0x200 DS write
+            constexpr int G0 = PAIR_MFMAS / (VMEM_OPS + FRAG_OPS) > 0 ? PAIR_MFMAS / (VMEM_OPS + FRAG_OPS) : 1;
+#pragma unroll
+            for (int i = 0; i < VMEM_OPS; ++i) {          // global loads first: they need the longest lead
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, G0, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < FRAG_OPS; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, G0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+
+            constexpr int LATE = MI * NI < PAIR_MFMAS / 4 ? MI * NI : PAIR_MFMAS / 4;   // MFMAs kept for after the barrier
+            constexpr int EARLY = PAIR_MFMAS - LATE;
+            store_stage(buf ^ 1);             // that buffer was last read before the previous barrier
+            mfma_range(af1, bf1, std::integral_constant<int, 0>{}, std::integral_constant<int, EARLY>{});
+            // the staged registers are first touched (register transposes, then LDS writes) half-way through these
+            // MFMAs, which is what gives the global loads their lead
+            constexpr int G1 = (EARLY / 2) / WRITE_OPS > 0 ? (EARLY / 2) / WRITE_OPS : 1;
+            __builtin_amdgcn_sched_group_barrier(0x008, EARLY - G1 * WRITE_OPS, 1);
+#pragma unroll
+            for (int i = 0; i < WRITE_OPS; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x002, 4, 1);
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 1);
+                __builtin_amdgcn_sched_group_barrier(0x008, G1, 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            read_frags(buf ^ 1, 0, af0, bf0);
+            mfma_range(af1, bf1, std::integral_constant<int, EARLY>{}, std::integral_constant<int, PAIR_MFMAS>{});
+            __builtin_amdgcn_sched_group_barrier(0x100, FRAG_OPS, 2);
+            __builtin_amdgcn_sched_group_barrier(0x008, LATE, 2);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // last full step: its first fragments are already in af0/bf0
+        const int buf = (full_steps - 1) & 1;
         if (has_tail) load_stage(full_steps * BK, std::true_type{});
-        compute_stage((full_steps - 1) & 1);
+        read_frags(buf, 1, af1, bf1);
+        mfma_range(af0, bf0, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
+        mfma_range(af1, bf1, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
         if (has_tail) {
-            store_stage(full_steps & 1);
+            store_stage(buf ^ 1);
             __syncthreads();
-            compute_stage(full_steps & 1);
+            compute_stage(buf ^ 1);
         }
     } else {
         compute_stage(0);             // K < BK: the prologue staged the only, partial step

@@ -112,6 +112,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--size", type=int, default=8192, help="square size of the headline fp32 GEMM")
+    ap.add_argument("--sgemm-variant", type=int, default=0, help="force a fp32 tile shape (0 = automatic)")
+    ap.add_argument("--hgemm-variant", type=int, default=0, help="force a fp16 tile shape (0 = automatic)")
     ap.add_argument("--only", default="", help="comma list of: headline,fp16,sq4096,ragged,conv,cpu (default all)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -124,6 +126,8 @@ def main():
     from backup_1_amd import capi, workloads
     capi.init()
     info = capi.device_info()
+    capi.lib().decx_hip_set_sgemm_variant(args.sgemm_variant)
+    capi.lib().decx_hip_set_hgemm_variant(args.hgemm_variant)
     log("device: %d CUs, %.0f MHz" % (info["compute_units"], info["clock_khz"] / 1e3))
 
     n = args.size
