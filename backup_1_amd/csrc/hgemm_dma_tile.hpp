@@ -6,15 +6,17 @@
 // never passes through VGPRs and several K steps can be in flight at once.  The swizzle is applied on the GLOBAL
 // side: lane L of a 64-unit chunk fetches the unit whose swizzled slot is L.
 //
-// Pipeline with STAGES LDS buffers: at the top of step t the wave waits until its own loads of step t have landed
-// (vmcnt <= loads issued after them), all waves meet at one barrier (which also guarantees everybody finished reading
-// the buffer of step t-1), then the loads of step t+STAGES-1 are issued into that freed buffer and step t is computed.
+// Pipeline with STAGES LDS buffers, one barrier per K step, placed inside the step's last MFMA block: before it the
+// wave waits until its own loads of step t+1 have landed (vmcnt <= loads issued after them); once all waves are past
+// it nobody reads step t's buffer any more, so the loads of step t+STAGES go out at once and the first fragments of
+// step t+1 are fetched, all of it between the remaining MFMAs of step t.
 // The loads are issued through inline asm so that the compiler's wait-count insertion does not serialise them; the
 // waits are written out explicitly.  M0 (the LDS base of such a load) is written only by those asm statements.
 //
 // The last, partial K step (K % BK != 0) cannot zero-fill through the DMA path and is staged through registers.
 // Requires 16-byte aligned operands with lda, ldb multiples of 8.
 #pragma once
+#include <type_traits>
 #include "hgemm_tile.hpp"
 
 namespace decx_hip {
@@ -46,13 +48,17 @@ __device__ __forceinline__ void wait_dma_then_barrier() {
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" : : "n"(N) : "memory");
 }
 
-template <class S>
+template <class S, bool HAS_C>
 __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __restrict__ A, int lda,
                                                           const _Float16* __restrict__ B, int ldb, const _Float16* Cin,
                                                           int ldc, _Float16* D, int ldd, int M, int N, int K, int tiles_m,
                                                           int tiles_n, int group_m) {
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, NT = S::NT, UA = S::UA, UB = S::UB, MI = S::MI, NI = S::NI;
     constexpr int STAGES = S::STAGES;
+    constexpr int KS = BK / 16;                                // MFMA k-blocks per K step
+    constexpr int BLK = MI * NI;                               // MFMAs per k-block
+    static_assert(KS == 2, "the hand-placed schedule below is written for two k-blocks per K step");
+    static_assert(BLK >= S::LOADS && BLK % 2 == 0, "the post-barrier half block must have a slot per DMA load");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     u32x4* lds = reinterpret_cast<u32x4*>(lds_raw);            // [STAGES][A_UNITS | B_UNITS]
     const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds_raw;
@@ -64,7 +70,7 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
     const int wm0 = (wave / S::WAVES_N) * S::WM, wn0 = (wave % S::WAVES_N) * S::WN;
     const int li = lane & 31, lh = lane >> 5;
 
-    // ---- per-lane global sources of this wave's DMA loads (advance by one K step per stage) -----------------------
+    // ---- per-lane global sources of this wave's DMA loads; they advance by one K step after every issue ----------
     const _Float16* a_src[S::A_LOADS];
     const _Float16* b_src[S::B_LOADS];
 #pragma unroll
@@ -87,17 +93,23 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
     }
     const size_t b_step = (size_t)BK * ldb;
 
-    auto issue_stage = [&](int stage, int t) {
+    // load number j (A loads first, then B) of the next K step to be fetched, into LDS buffer `stage`
+    auto issue_one = [&](int stage, int j) {
         const uint32_t base = lds_base + (uint32_t)stage * (S::STAGE_UNITS * 16);
+        if (j < S::A_LOADS) {
+            dma_load16(a_src[j], base + (uint32_t)(wave * S::A_LOADS + j) * 1024u);
+            a_src[j] += BK;
+        } else {
+            const int jb = j - S::A_LOADS;
+            dma_load16(b_src[jb], base + (uint32_t)(S::A_UNITS * 16) + (uint32_t)(wave * S::B_LOADS + jb) * 1024u);
+            b_src[jb] += b_step;
+        }
+    };
+    auto issue_stage = [&](int stage) {
 #pragma unroll
-        for (int j = 0; j < S::A_LOADS; ++j)
-            dma_load16(a_src[j] + (size_t)t * BK, base + (uint32_t)(wave * S::A_LOADS + j) * 1024u);
-#pragma unroll
-        for (int j = 0; j < S::B_LOADS; ++j)
-            dma_load16(b_src[j] + (size_t)t * b_step, base + (uint32_t)(S::A_UNITS * 16) + (uint32_t)(wave * S::B_LOADS + j) * 1024u);
+        for (int j = 0; j < S::LOADS; ++j) issue_one(stage, j);
     };
 
-    // ---- accumulators ------------------------------------------------------------------------------------------------
     f32x16 acc[MI][NI];
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
@@ -108,77 +120,107 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
 
     const int full_steps = K / BK;
 
-    // prologue: fill STAGES-1 buffers (issue nothing for steps that do not exist)
+    // prologue: every LDS buffer gets a K step (issue nothing for steps that do not exist)
 #pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s)
-        if (s < full_steps) issue_stage(s, s);
+    for (int s = 0; s < STAGES; ++s)
+        if (s < full_steps) issue_stage(s);
 
-    if (Cin != nullptr) {
-#pragma unroll
-        for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-                if (m < M) {
-                    const _Float16* crow = Cin + (size_t)m * ldc;
-#pragma unroll
-                    for (int ni = 0; ni < NI; ++ni) {
-                        const int n = bn0 + wn0 + ni * 32 + li;
-                        if (n < N) acc[mi][ni][r] = (float)crow[n];
-                    }
-                }
-            }
-    }
-
-    // transposed-read geometry of this lane (see hgemm_tile.hpp)
+    // ---- fragment reads -------------------------------------------------------------------------------------------
+    // byte offsets inside one LDS buffer; the swizzles depend on the lane only through these loop-invariant terms
     const int tg = lane >> 4, ts = lane & 15;
-    const int t_row = 8 * (tg >> 1) + (ts >> 2);
-    const int t_col = 16 * (tg & 1) + 4 * (ts & 3);
-
-    auto compute_stage = [&](int stage) {
+    const int t_row = 8 * (tg >> 1) + (ts >> 2);               // transposed read: row inside a 16-row k-block (+4: high half)
+    const int t_col = 16 * (tg & 1) + 4 * (ts & 3);            // and column inside a 32-column block
+    typedef short i16x8 __attribute__((ext_vector_type(8)));
+    struct Frags {
+        f16x8 a[MI];
+        i16x4 b_lo[NI], b_hi[NI];
+    };
+    // The 3*... reads of one k-block, numbered in the order the MFMAs (mi-major) first need them:
+    //   0: a[0], then b_lo/b_hi of ni = 0..NI-1, then a[1..MI-1]
+    constexpr int FRAG_READS = MI + 2 * NI;
+    auto read_one = [&](Frags& f, int stage, int ks, int r) {
         const u32x4* Ab = lds + stage * S::STAGE_UNITS;
         const unsigned char* Bb = reinterpret_cast<const unsigned char*>(Ab + S::A_UNITS);
+        if (r == 0 || r > 2 * NI) {
+            const int mi = r == 0 ? 0 : r - 2 * NI;
+            u32x4 raw = Ab[a_unit_slot(wm0 + mi * 32 + li, 2 * ks + lh, UA)];
+            f.a[mi] = __builtin_bit_cast(f16x8, raw);
+        } else {
+            const int ni = (r - 1) / 2, hi = (r - 1) % 2;
+            const int col = wn0 + ni * 32 + t_col;
+            const int k = 16 * ks + t_row + 4 * hi;
+            const int off = b_unit_slot(k, col >> 3, UB) * 16 + (col & 7) * 2;
+            i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(Bb + off));
+            if (hi) f.b_hi[ni] = v;
+            else f.b_lo[ni] = v;
+        }
+    };
+    auto mfma_one = [&](const Frags& f, int i) {
+        const int mi = i / NI, ni = i % NI;
+        i16x8 both = {f.b_lo[ni][0], f.b_lo[ni][1], f.b_lo[ni][2], f.b_lo[ni][3],
+                      f.b_hi[ni][0], f.b_hi[ni][1], f.b_hi[ni][2], f.b_hi[ni][3]};
+        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.a[mi], __builtin_bit_cast(f16x8, both), acc[mi][ni], 0, 0, 0);
+    };
+#define DECX_PIN() __builtin_amdgcn_sched_barrier(0)
+
+    Frags f0, f1;
+
+    // One K step.  f0 holds the fragments of its first k-block on entry and those of the NEXT step's first k-block on
+    // exit.  Source order is the issue order (every slot is pinned): memory instructions ride between MFMAs.
+    //   block 0 (f0): MFMA i + LDS read i of block 1                          (reads finish ahead of block 1)
+    //   block 1 (f1): first half plain, then wait for the next step's data + barrier -- at this point every wave has
+    //                 finished reading this step's buffer, so it is refilled right away (DMA loads of step t+STAGES),
+    //                 and the next step's first fragments are read, all between the MFMAs of the second half.
+    auto k_step = [&](int stg, int next, auto wait_tag, bool refill, bool has_next) {
+        constexpr int WAITN = decltype(wait_tag)::value;
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            f16x8 af[MI], bf[NI];
+        for (int i = 0; i < BLK; ++i) {
+            if (i < FRAG_READS) read_one(f1, stg, 1, i);
+            mfma_one(f0, i);
+            DECX_PIN();
+        }
 #pragma unroll
-            for (int mi = 0; mi < MI; ++mi) {
-                u32x4 raw = Ab[a_unit_slot(wm0 + mi * 32 + li, 2 * ks + lh, UA)];
-                af[mi] = __builtin_bit_cast(f16x8, raw);
+        for (int i = 0; i < BLK / 2; ++i) {
+            mfma_one(f1, i);
+            DECX_PIN();
+        }
+        if (has_next) {
+            wait_dma_then_barrier<WAITN>();
+            DECX_PIN();
+        }
+        constexpr int SLOTS = BLK - BLK / 2;                   // MFMAs left; spread FRAG_READS reads and LOADS loads over them
+#pragma unroll
+        for (int i = 0; i < SLOTS; ++i) {
+            if (refill && i < S::LOADS) issue_one(stg, i);
+            if (has_next) {
+#pragma unroll
+                for (int r = (i * FRAG_READS) / SLOTS; r < ((i + 1) * FRAG_READS) / SLOTS; ++r) read_one(f0, next, 0, r);
             }
-#pragma unroll
-            for (int ni = 0; ni < NI; ++ni) {
-                const int col = wn0 + ni * 32 + t_col;
-                const int k_lo = 16 * ks + t_row, k_hi = k_lo + 4;
-                const int off_lo = b_unit_slot(k_lo, col >> 3, UB) * 16 + (col & 7) * 2;
-                const int off_hi = b_unit_slot(k_hi, col >> 3, UB) * 16 + (col & 7) * 2;
-                i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(Bb + off_lo));
-                i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(Bb + off_hi));
-                typedef short i16x8 __attribute__((ext_vector_type(8)));
-                i16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                bf[ni] = __builtin_bit_cast(f16x8, both);
-            }
-#pragma unroll
-            for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-                for (int ni = 0; ni < NI; ++ni)
-                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mi], bf[ni], acc[mi][ni], 0, 0, 0);
+            mfma_one(f1, BLK / 2 + i);
+            DECX_PIN();
         }
     };
 
-    // ---- main loop over full K steps -------------------------------------------------------------------------------
-    // unrolled by STAGES so that every LDS buffer index is a compile-time constant
-    for (int t0 = 0; t0 < full_steps; t0 += STAGES) {
+    if (full_steps > 0) {
+        wait_dma_then_barrier<0>();                            // step 0 (and whatever else the prologue fetched) has landed
 #pragma unroll
-        for (int s = 0; s < STAGES; ++s) {
-            const int t = t0 + s;
-            if (t < full_steps) {
-                // groups issued after step t's: min(STAGES-2, full_steps-1-t); the steady-state count is a constant
-                if (t + STAGES - 2 < full_steps) wait_dma_then_barrier<S::LOADS*(STAGES - 2)>();
-                else wait_dma_then_barrier<0>();
-                if (t + STAGES - 1 < full_steps) issue_stage((s + STAGES - 1) % STAGES, t + STAGES - 1);
-                compute_stage(s);
-            }
+        for (int r = 0; r < FRAG_READS; ++r) read_one(f0, 0, 0, r);
+        DECX_PIN();
+
+        // steady state: every step refills its buffer (t + STAGES < full_steps).  Before the barrier of step t the data of
+        // step t+1 must have landed; the loads of steps t+2 .. t+STAGES-1, issued later, may still be in flight.
+        const int steady = full_steps > STAGES ? full_steps - STAGES : 0;
+        int stg = 0;
+        for (int t = 0; t < steady; ++t) {
+            const int next = stg + 1 == STAGES ? 0 : stg + 1;
+            k_step(stg, next, std::integral_constant<int, S::LOADS*(STAGES - 2)>{}, true, true);
+            stg = next;
+        }
+        // the last (<= STAGES) steps: nothing left to fetch, conservative waits
+        for (int t = steady; t < full_steps; ++t) {
+            const int next = stg + 1 == STAGES ? 0 : stg + 1;
+            k_step(stg, next, std::integral_constant<int, 0>{}, false, t + 1 < full_steps);
+            stg = next;
         }
     }
 
@@ -230,9 +272,17 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
             Bb[b_unit_slot(id / UB, id % UB, UB)] = b_stage[p];
         }
         __syncthreads();
-        compute_stage(0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+            for (int r = 0; r < FRAG_READS; ++r) read_one(f0, 0, ks, r);
+#pragma unroll
+            for (int i = 0; i < BLK; ++i) mfma_one(f0, i);
+        }
     }
+#undef DECX_PIN
 
+    // ---- epilogue: round once to binary16; dst = A*B + C adds C (as fp32) first ---------------------------------------
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
@@ -240,10 +290,11 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
             const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
             if (m < M) {
                 _Float16* drow = D + (size_t)m * ldd;
+                const _Float16* crow = HAS_C ? Cin + (size_t)m * ldc : nullptr;
 #pragma unroll
                 for (int ni = 0; ni < NI; ++ni) {
                     const int n = bn0 + wn0 + ni * 32 + li;
-                    if (n < N) drow[n] = (_Float16)acc[mi][ni][r];
+                    if (n < N) drow[n] = (_Float16)(HAS_C ? acc[mi][ni][r] + (float)crow[n] : acc[mi][ni][r]);
                 }
             }
         }
