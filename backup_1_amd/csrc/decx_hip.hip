@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "hgemm_dma_tile.hpp"
@@ -25,6 +26,7 @@ struct Runtime {
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     int sgemm_variant = 0;
     int hgemm_variant = 0;
+    int group_m = 8;   // tile-rows per raster group of the XCD-aware tile walk (env DECX_HIP_GROUP_M overrides, for tuning)
 };
 Runtime g_rt;
 
@@ -70,7 +72,7 @@ int launch_sgemm_tile_c(const ASrc& a, const BSrc& b, const float* Cin, int ldc,
     const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
     const long total = (long)tiles_m * tiles_n;
     if (total > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
-    const int group_m = tiles_m < 8 ? tiles_m : 8;
+    const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
     hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream, a, b, Cin, ldc, D, out, M,
                        N, K, tiles_m, tiles_n, group_m);
     HIP_TRY(hipGetLastError());
@@ -171,6 +173,10 @@ typedef HgemmShape<256, 256, 32, 2, 2> HShapeBig;
 typedef HgemmShape<128, 128, 32, 2, 2> HShapeSmall;
 //   3: 256x256x32, 2x2 waves of 128x128, 4-stage LDS-DMA pipeline
 typedef HgemmDmaShape<256, 256, 32, 2, 2, 4> HShapeDma;
+//   4: 256x256x64, 2x2 waves of 128x128, 2-stage LDS-DMA pipeline (whole 128-byte lines of A per row and step)
+typedef HgemmDmaShape<256, 256, 64, 2, 2, 2> HShapeDma64;
+//   5: 256x256x32, 5-stage
+typedef HgemmDmaShape<256, 256, 32, 2, 2, 5> HShapeDma5;
 
 template <class S, bool VEC>
 int launch_hgemm_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
@@ -185,7 +191,7 @@ int launch_hgemm_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb, co
     const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
     const long total = (long)tiles_m * tiles_n;
     if (total > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
-    const int group_m = tiles_m < 8 ? tiles_m : 8;
+    const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
     hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream,
                        reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
                        reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N, K,
@@ -209,7 +215,7 @@ int launch_hgemm_dma_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb
     const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
     const long total = (long)tiles_m * tiles_n;
     if (total > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
-    const int group_m = tiles_m < 8 ? tiles_m : 8;
+    const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
     hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream,
                        reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
                        reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N, K,
@@ -228,11 +234,13 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
     const bool vec = aligned16(A) && aligned16(B) && lda % 8 == 0 && ldb % 8 == 0 && ldb >= 8;
     if (!vec) return launch_hgemm_tile<HShapeSmall, false>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
     int variant = g_rt.hgemm_variant;
-    if (variant < 1 || variant > 3) {
+    if (variant < 1 || variant > 5) {
         const int cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
-        variant = ((long)cdiv(M, 256) * cdiv(N, 256) * 10 >= (long)cus * 8) ? 3 : 2;
+        variant = ((long)cdiv(M, 256) * cdiv(N, 256) * 10 >= (long)cus * 8) ? 4 : 2;
     }
     if (variant == 3) return launch_hgemm_dma_tile<HShapeDma>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
+    if (variant == 4) return launch_hgemm_dma_tile<HShapeDma64>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
+    if (variant == 5) return launch_hgemm_dma_tile<HShapeDma5>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
     if (variant == 1) return launch_hgemm_tile<HShapeBig, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
     return launch_hgemm_tile<HShapeSmall, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
 }
@@ -266,6 +274,7 @@ int decx_hip_init(int* device) {
         HIP_TRY(hipStreamCreateWithFlags(&g_rt.stream, hipStreamNonBlocking));
         HIP_TRY(hipEventCreate(&g_rt.ev_start));
         HIP_TRY(hipEventCreate(&g_rt.ev_stop));
+        if (const char* gm = getenv("DECX_HIP_GROUP_M")) { int v = atoi(gm); if (v > 0) g_rt.group_m = v; }
         g_rt.is_init = true;
     }
     if (device) *device = g_rt.device;

@@ -57,8 +57,7 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
     constexpr int STAGES = S::STAGES;
     constexpr int KS = BK / 16;                                // MFMA k-blocks per K step
     constexpr int BLK = MI * NI;                               // MFMAs per k-block
-    static_assert(KS == 2, "the hand-placed schedule below is written for two k-blocks per K step");
-    static_assert(BLK >= S::LOADS && BLK % 2 == 0, "the post-barrier half block must have a slot per DMA load");
+    static_assert(KS >= 2, "the schedule below needs at least two k-blocks per K step");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     u32x4* lds = reinterpret_cast<u32x4*>(lds_raw);            // [STAGES][A_UNITS | B_UNITS]
     const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds_raw;
@@ -173,33 +172,45 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
     //                 and the next step's first fragments are read, all between the MFMAs of the second half.
     auto k_step = [&](int stg, int next, auto wait_tag, bool refill, bool has_next) {
         constexpr int WAITN = decltype(wait_tag)::value;
+        // k-blocks 0 .. KS-2: MFMA i of block b rides with LDS read i of block b+1 (fragment sets alternate f0, f1)
 #pragma unroll
-        for (int i = 0; i < BLK; ++i) {
-            if (i < FRAG_READS) read_one(f1, stg, 1, i);
-            mfma_one(f0, i);
-            DECX_PIN();
+        for (int b = 0; b + 1 < KS; ++b) {
+#pragma unroll
+            for (int i = 0; i < BLK; ++i) {
+                if (i < FRAG_READS) read_one((b & 1) ? f0 : f1, stg, b + 1, i);
+                mfma_one((b & 1) ? f1 : f0, i);
+                DECX_PIN();
+            }
         }
+        // last k-block: a few MFMAs, the barrier, then refill + next step's first fragments between the rest
+        Frags& fl = ((KS - 1) & 1) ? f1 : f0;
+        Frags& fn = ((KS - 1) & 1) ? f0 : f1;      // receives the next step's block 0 (KS even: this is f0 again)
+        constexpr int PRE = BLK / 4;
 #pragma unroll
-        for (int i = 0; i < BLK / 2; ++i) {
-            mfma_one(f1, i);
+        for (int i = 0; i < PRE; ++i) {
+            mfma_one(fl, i);
             DECX_PIN();
         }
         if (has_next) {
             wait_dma_then_barrier<WAITN>();
             DECX_PIN();
         }
-        constexpr int SLOTS = BLK - BLK / 2;                   // MFMAs left; spread FRAG_READS reads and LOADS loads over them
+        constexpr int SLOTS = BLK - PRE;
 #pragma unroll
         for (int i = 0; i < SLOTS; ++i) {
-            if (refill && i < S::LOADS) issue_one(stg, i);
+            if (refill) {
+#pragma unroll
+                for (int j = (i * S::LOADS) / SLOTS; j < ((i + 1) * S::LOADS) / SLOTS; ++j) issue_one(stg, j);
+            }
             if (has_next) {
 #pragma unroll
-                for (int r = (i * FRAG_READS) / SLOTS; r < ((i + 1) * FRAG_READS) / SLOTS; ++r) read_one(f0, next, 0, r);
+                for (int r = (i * FRAG_READS) / SLOTS; r < ((i + 1) * FRAG_READS) / SLOTS; ++r) read_one(fn, next, 0, r);
             }
-            mfma_one(f1, BLK / 2 + i);
+            mfma_one(fl, PRE + i);
             DECX_PIN();
         }
     };
+    static_assert(KS % 2 == 0, "fragment sets must line up across K steps (block 0 always in f0)");
 
     if (full_steps > 0) {
         wait_dma_then_barrier<0>();                            // step 0 (and whatever else the prologue fetched) has landed
