@@ -93,15 +93,24 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
 typedef SgemmShape<128, 128, 16, 2, 2, 2> SShapeSmall;
 typedef SgemmShape<256, 128, 16, 2, 2, 2> SShapeTall;
+//   4: 224x128x16, 1x4 waves of 224x32    -- 7/8 of shape 3 per tile: fills more CUs when M/256 tiles leave many idle
+typedef SgemmShape<224, 128, 16, 1, 4, 2> SShape224;
 
+// Tile shape by a small cost model: a CU works through ceil(tiles / CUs) tiles one after another, a tile costs its area
+// divided by how well that shape keeps the matrix pipe busy (measured on 8192^3, relative to shape 1).
 int pick_sgemm_variant(int M, int N) {
-    if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 3) return g_rt.sgemm_variant;
-    const int cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
-    const long big = (long)cdiv(M, 256) * cdiv(N, 256);
-    if (big * 10 >= (long)cus * 8) return 1;                 // at least ~0.8 tiles per CU
-    const long tall = (long)cdiv(M, 256) * cdiv(N, 128);
-    if (tall * 10 >= (long)cus * 7) return 3;
-    return 2;
+    if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 4) return g_rt.sgemm_variant;
+    const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+    struct Cand { int variant, bm, bn; double eff; };
+    const Cand cands[] = {{1, 256, 256, 1.00}, {3, 256, 128, 0.95}, {4, 224, 128, 0.85}, {2, 128, 128, 0.90}};
+    int best = 1;
+    double best_cost = 0.0;
+    for (const Cand& c : cands) {
+        const long tiles = (long)cdiv(M, c.bm) * cdiv(N, c.bn);
+        const double cost = (double)((tiles + cus - 1) / cus) * c.bm * c.bn / c.eff;
+        if (best_cost == 0.0 || cost < best_cost) { best_cost = cost; best = c.variant; }
+    }
+    return best;
 }
 
 template <class ASrc, class BSrc, class Out>
@@ -110,6 +119,7 @@ int dispatch_sgemm(int variant, const ASrc& a, const BSrc& b, const float* Cin, 
     switch (variant) {
         case 1: return launch_sgemm_tile<SShapeBig>(a, b, Cin, ldc, D, out, M, N, K);
         case 3: return launch_sgemm_tile<SShapeTall>(a, b, Cin, ldc, D, out, M, N, K);
+        case 4: return launch_sgemm_tile<SShape224>(a, b, Cin, ldc, D, out, M, N, K);
         default: return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K);
     }
 }
@@ -159,7 +169,7 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
     const int M = (int)Ml, K = (int)Kl;
     Im2colA a{src, H, W, dpitch, kh, kw, flag ? kh / 2 : 0, flag ? kw / 2 : 0, Wout, M, K, src_row_stride};
     FilterB b{filt, N, K, dpitch, kw, filt_stride, filt_row_stride};
-    TensorOut out{Wout, dst_dpitch, dst_row_stride};
+    TensorOut out{Wout, dst_dpitch, dst_row_stride, dst_row_stride == (size_t)Wout * dst_dpitch};
     return dispatch_sgemm(pick_sgemm_variant(M, N), a, b, nullptr, 0, dst, out, M, N, K);
 }
 

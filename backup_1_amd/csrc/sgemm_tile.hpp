@@ -26,12 +26,37 @@ namespace decx_hip {
 // ---------------------------------------------------------------------------------------------------------------
 // A-operand sources.  Interface:
 //   RowState row_state(int m)                       per-row values that do not change along K
-//   template<bool TAIL> f32x4 load(rs, k, keep)     A[m][k..k+3] read from an always-valid address; the caller replaces
+//   KState k_state(k) / advance(ks, dk)             position of a k-quad, moved on by whole K steps
+//   template<bool TAIL> f32x4 load(rs, ks, keep)    A[m][k..k+3] read from an always-valid address; the caller replaces
 //                                                   the quad by zeros when keep comes back false (deferred, so that the
 //                                                   load itself stays branch-free and nothing waits on it early);
 //                                                   TAIL additionally zero-fills elements with k >= K
 //   size_t out_offset(int m)                        where row m of the result starts, in elements
 // ---------------------------------------------------------------------------------------------------------------
+// Position of one k index inside the im2col ordering k = (ki*kw + kj)*dpitch + c.  Decoded once (two integer
+// divisions), then advanced by whole K steps with additions only.
+struct TapWalk {
+    int k, c, ki, kj;
+    __device__ __forceinline__ void init(int k_, int dpitch, int kw) {
+        k = k_;
+        const int tap = k_ / dpitch;
+        c = k_ - tap * dpitch;
+        ki = tap / kw;
+        kj = tap - ki * kw;
+    }
+    __device__ __forceinline__ void advance(int dk, int dpitch, int kw) {
+        k += dk;
+        c += dk;
+        while (c >= dpitch) {
+            c -= dpitch;
+            if (++kj == kw) {
+                kj = 0;
+                ++ki;
+            }
+        }
+    }
+};
+
 template <bool VEC>
 struct DenseA {
     const float* A;
@@ -39,13 +64,19 @@ struct DenseA {
     struct RowState {
         const float* row;
     };
+    struct KState {
+        int k;
+    };
+    __device__ __forceinline__ KState k_state(int k) const { return KState{k}; }
+    __device__ __forceinline__ void advance(KState& ks, int dk) const { ks.k += dk; }
     __device__ __forceinline__ RowState row_state(int m) const {
         RowState rs;
         rs.row = A + (size_t)(m < M ? m : M - 1) * lda;
         return rs;
     }
     template <bool TAIL>
-    __device__ __forceinline__ f32x4 load(const RowState& rs, int k, bool& keep) const {
+    __device__ __forceinline__ f32x4 load(const RowState& rs, const KState& ks, bool& keep) const {
+        const int k = ks.k;
         keep = true;
         f32x4 v = {0.f, 0.f, 0.f, 0.f};
         if (VEC) {
@@ -67,31 +98,38 @@ struct DenseA {
 };
 
 // The im2col view of a channel-innermost tensor: row m = (y, x) of the output, column k = (ki*kw + kj)*dpitch + c.
+// Per row the element offset of its top-left tap is kept; per K step one tap offset is added to it, so a load costs
+// two coordinate adds, two unsigned range checks and one 64-bit add.
 struct Im2colA {
     const float* src;
     int H, W, dpitch, kh, kw, oy, ox, Wout, Mtot, K;
     size_t row_stride;
     struct RowState {
-        int y, x;   // output pixel, already shifted by (-oy, -ox)
+        int y, x;          // output pixel shifted by (-oy, -ox): the image position of tap (0, 0)
+        long base;         // y*row_stride + x*dpitch (may be negative: it is only used together with an in-image tap)
     };
     __device__ __forceinline__ RowState row_state(int m) const {
         if (m >= Mtot) m = Mtot - 1;
         RowState rs;
         rs.y = m / Wout - oy;
         rs.x = m % Wout - ox;
+        rs.base = (long)rs.y * (long)row_stride + (long)rs.x * dpitch;
         return rs;
     }
+    typedef TapWalk KState;
+    __device__ __forceinline__ KState k_state(int k) const {
+        KState ks;
+        ks.init(k, dpitch, kw);
+        return ks;
+    }
+    __device__ __forceinline__ void advance(KState& ks, int dk) const { ks.advance(dk, dpitch, kw); }
     template <bool TAIL>
-    __device__ __forceinline__ f32x4 load(const RowState& rs, int k, bool& keep) const {
-        // K = kh*kw*dpitch is a multiple of 4: quads never straddle it
-        const bool k_ok = !TAIL || k < K;
-        const int kk = k_ok ? k : 0;
-        const int tap = kk / dpitch, c = kk - tap * dpitch;
-        const int ki = tap / kw, kj = tap - ki * kw;
-        const int sy = rs.y + ki, sx = rs.x + kj;
-        keep = k_ok && sy >= 0 && sy < H && sx >= 0 && sx < W;
-        const int cy = sy < 0 ? 0 : (sy >= H ? H - 1 : sy), cx = sx < 0 ? 0 : (sx >= W ? W - 1 : sx);
-        return *reinterpret_cast<const f32x4*>(src + (size_t)cy * row_stride + (size_t)cx * dpitch + c);
+    __device__ __forceinline__ f32x4 load(const RowState& rs, const KState& ks, bool& keep) const {
+        // K = kh*kw*dpitch is a multiple of 4: quads never straddle it.  A tap outside the image (or k >= K, TAIL only)
+        // reads the tensor's first quad instead and is zeroed by the caller.
+        const long tap_off = (long)ks.ki * (long)row_stride + (long)(ks.kj * dpitch + ks.c);
+        keep = (unsigned)(rs.y + ks.ki) < (unsigned)H && (unsigned)(rs.x + ks.kj) < (unsigned)W && (!TAIL || ks.k < K);
+        return *reinterpret_cast<const f32x4*>(src + (keep ? rs.base + tap_off : 0L));
     }
 };
 
@@ -104,7 +142,9 @@ struct DenseOut {
 struct TensorOut {
     int Wout, dpitch;
     size_t row_stride;
+    bool dense;      // row_stride == Wout*dpitch: pixel m simply starts at m*dpitch, no division needed
     __device__ __forceinline__ size_t offset(int m) const {
+        if (dense) return (size_t)m * dpitch;
         const int y = m / Wout, x = m - y * Wout;
         return (size_t)y * row_stride + (size_t)x * dpitch;
     }
@@ -113,7 +153,8 @@ struct TensorOut {
 // ---------------------------------------------------------------------------------------------------------------
 // B-operand sources.  Interface (S = SgemmShape):
 //   quads<S>()                                   staging registers (float4) per thread and K step
-//   load<S, TAIL>(stage, tid, k0, bn0)           fetch this thread's share of B[k0 .. k0+BK) x [bn0 .. bn0+BN)
+//   KState k_state<S>(tid) / advance<S>(ks)      position of the K step to fetch next
+//   load<S, TAIL>(stage, tid, ks, bn0)           fetch this thread's share of B[k0 .. k0+BK) x [bn0 .. bn0+BN)
 //   store<S>(plane, stage, tid)                  write it to the LDS planes as k-quads at [q][n + (n >> 4)]
 // ---------------------------------------------------------------------------------------------------------------
 // B as a row-major K x N matrix: a thread takes a 4(k) x 4(n) block with four 16-byte row loads (consecutive lanes
@@ -128,9 +169,17 @@ struct DenseB {
     static constexpr int passes() { return (tasks<S>() + S::NT - 1) / S::NT; }
     template <class S>
     static constexpr int quads() { return 4 * passes<S>(); }
+    struct KState {
+        int k0;
+    };
+    template <class S>
+    __device__ __forceinline__ KState k_state(int tid) const { return KState{0}; }
+    template <class S>
+    __device__ __forceinline__ void advance(KState& ks) const { ks.k0 += S::BK; }
 
     template <class S, bool TAIL>
-    __device__ __forceinline__ void load(f32x4* st, int tid, int k0, int bn0) const {
+    __device__ __forceinline__ void load(f32x4* st, int tid, const KState& ks, int bn0) const {
+        const int k0 = ks.k0;
         constexpr int CG = S::BN / 4;
 #pragma unroll
         for (int p = 0; p < passes<S>(); ++p) {
@@ -182,24 +231,28 @@ struct FilterB {
     size_t filt_stride, filt_row_stride;
     template <class S>
     static constexpr int quads() { return S::KQ * S::BN / S::NT; }
+    typedef TapWalk KState;       // every quad of a thread has the same k-quad index q = tid % KQ (NT is a multiple of KQ)
+    template <class S>
+    __device__ __forceinline__ KState k_state(int tid) const {
+        KState ks;
+        ks.init(4 * (tid % S::KQ), dpitch, kw);
+        return ks;
+    }
+    template <class S>
+    __device__ __forceinline__ void advance(KState& ks) const { ks.advance(S::BK, dpitch, kw); }
 
     template <class S, bool TAIL>
-    __device__ __forceinline__ void load(f32x4* st, int tid, int k0, int bn0) const {
-        static_assert((S::KQ * S::BN) % S::NT == 0, "filter staging must divide evenly");
+    __device__ __forceinline__ void load(f32x4* st, int tid, const KState& ks, int bn0) const {
+        static_assert((S::KQ * S::BN) % S::NT == 0 && S::NT % S::KQ == 0, "filter staging must divide evenly");
+        const bool k_ok = !TAIL || ks.k < K;
+        const size_t tap_off = k_ok ? (size_t)ks.ki * filt_row_stride + (size_t)ks.kj * dpitch + ks.c : 0;
 #pragma unroll
         for (int j = 0; j < quads<S>(); ++j) {
             const int id = tid + j * S::NT;
-            const int q = id % S::KQ;
             int n = bn0 + id / S::KQ;
             if (n >= N) n = N - 1;
-            const int k = k0 + 4 * q;
-            f32x4 v = {0.f, 0.f, 0.f, 0.f};
-            if (!TAIL || k < K) {
-                const int tap = k / dpitch, c = k - tap * dpitch;
-                const int ki = tap / kw, kj = tap - ki * kw;
-                v = *reinterpret_cast<const f32x4*>(filt + (size_t)n * filt_stride + (size_t)ki * filt_row_stride +
-                                                    (size_t)kj * dpitch + c);
-            }
+            f32x4 v = *reinterpret_cast<const f32x4*>(filt + (size_t)n * filt_stride + tap_off);
+            if (TAIL && !k_ok) v = f32x4{0.f, 0.f, 0.f, 0.f};
             st[j] = v;
         }
     }
@@ -224,11 +277,11 @@ struct SgemmShape {
     static constexpr int KQ = BK / 4;                         // k-quads per step
     static constexpr int A_ROW = BM + 4;                      // quads per A plane
     static constexpr int B_ROW = BN + BN / 16;                // quads per B plane
-    static constexpr int A_PASSES = (BM * KQ) / NT;           // float4 global loads of A per thread per step
+    static constexpr int A_PASSES = (BM * KQ + NT - 1) / NT;  // float4 global loads of A per thread per step (last may be partial)
+    static constexpr bool A_PARTIAL = (BM * KQ) % NT != 0;
     static constexpr size_t LDS_BYTES = 2 * (size_t)KQ * (A_ROW + B_ROW) * sizeof(f32x4);
     static_assert(BM % (WAVES_M * 32) == 0 && BN % (WAVES_N * 32) == 0, "wave tile must be whole 32x32 blocks");
     static_assert(BK % 8 == 0, "a K step is whole quad pairs");
-    static_assert((BM * KQ) % NT == 0, "A staging must divide evenly");
     static_assert(NT % KQ == 0, "A staging: KQ lanes per row");
 };
 
@@ -254,22 +307,34 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
     constexpr int A_RSTEP = NT / KQ;
     typename ASrc::RowState a_rs[S::A_PASSES];
 #pragma unroll
-    for (int p = 0; p < S::A_PASSES; ++p) a_rs[p] = a_src.row_state(bm0 + a_r + p * A_RSTEP);
+    for (int p = 0; p < S::A_PASSES; ++p) {
+        const int r = a_r + p * A_RSTEP;
+        a_rs[p] = a_src.row_state(bm0 + (S::A_PARTIAL && r >= BM ? 0 : r));
+    }
     f32x4 a_stage[S::A_PASSES];
     bool a_keep[S::A_PASSES];
     f32x4 b_stage[BSrc::template quads<S>()];
+    typename ASrc::KState a_ks = a_src.k_state(4 * a_q);       // this thread's k-quad of the next K step to fetch
+    typename BSrc::KState b_ks = b_src.template k_state<S>(tid);
 
-    auto load_stage = [&](int k0, auto tail_tag) {
+    // fetches the next K step (steps are always taken in order) and moves the k positions on
+    auto load_stage = [&](auto tail_tag) {
         constexpr bool TAIL = decltype(tail_tag)::value;
 #pragma unroll
-        for (int p = 0; p < S::A_PASSES; ++p) a_stage[p] = a_src.template load<TAIL>(a_rs[p], k0 + 4 * a_q, a_keep[p]);
-        b_src.template load<S, TAIL>(b_stage, tid, k0, bn0);
+        for (int p = 0; p < S::A_PASSES; ++p) {
+            if (S::A_PARTIAL && a_r + p * A_RSTEP >= BM) continue;
+            a_stage[p] = a_src.template load<TAIL>(a_rs[p], a_ks, a_keep[p]);
+        }
+        b_src.template load<S, TAIL>(b_stage, tid, b_ks, bn0);
+        a_src.advance(a_ks, BK);
+        b_src.template advance<S>(b_ks);
     };
 
     auto store_stage = [&](int buf) {
         f32x4* Ab = As + buf * KQ * S::A_ROW;
 #pragma unroll
         for (int p = 0; p < S::A_PASSES; ++p) {
+            if (S::A_PARTIAL && a_r + p * A_RSTEP >= BM) continue;
             const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
             Ab[a_q * S::A_ROW + a_r + p * A_RSTEP] = a_keep[p] ? a_stage[p] : zero;
         }
@@ -321,8 +386,8 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
     const int full_steps = K / BK;
     const bool has_tail = full_steps * BK < K;
 
-    if (full_steps > 0) load_stage(0, std::false_type{});
-    else load_stage(0, std::true_type{});
+    if (full_steps > 0) load_stage(std::false_type{});
+    else load_stage(std::true_type{});
     store_stage(0);
     __syncthreads();
 
@@ -340,7 +405,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         // Every memory instruction sits between MFMAs, so the matrix pipe is never starved by an in-order wait.
         for (int t = 0; t + 1 < full_steps; ++t) {
             const int buf = t & 1;
-            load_stage((t + 1) * BK, std::false_type{});
+            load_stage(std::false_type{});
             read_frags(buf, 1, af1, bf1);
             mfma_range(af0, bf0, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
             // scheduling-group masks: 0x002 VALU, 0x008 MFMA, 0x020 VMEM read, 0x100 DS read, 0x200 DS write
@@ -382,7 +447,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         }
         // last full step: its first fragments are already in af0/bf0
         const int buf = (full_steps - 1) & 1;
-        if (has_tail) load_stage(full_steps * BK, std::true_type{});
+        if (has_tail) load_stage(std::true_type{});
         read_frags(buf, 1, af1, bf1);
         mfma_range(af0, bf0, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
         mfma_range(af1, bf1, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
