@@ -20,7 +20,7 @@ SYMBOLS = [
     "decx_hip_host_malloc", "decx_hip_host_free", "decx_hip_memcpy2d", "decx_hip_memcpy", "decx_hip_sync",
     "decx_hip_sgemm", "decx_hip_sgemm_async", "decx_hip_hgemm_f32acc", "decx_hip_hgemm_f32acc_async",
     "decx_hip_conv2_im2col_f32", "decx_hip_conv2_im2col_f32_async", "decx_hip_timer_start", "decx_hip_timer_stop",
-    "decx_hip_last_error", "decx_hip_set_sgemm_variant", "decx_hip_set_hgemm_variant",
+    "decx_hip_last_error", "decx_hip_set_sgemm_variant", "decx_hip_set_hgemm_variant", "decx_hip_copy_kernel",
 ]
 
 
@@ -55,6 +55,7 @@ def lib():
             "decx_hip_hgemm_f32acc_async": ([P, I, P, I, P, I, P, I, I, I, I], I),
             "decx_hip_conv2_im2col_f32": ([P, I, I, I, Z, P, I, I, I, Z, Z, P, I, Z, I], I),
             "decx_hip_conv2_im2col_f32_async": ([P, I, I, I, Z, P, I, I, I, Z, Z, P, I, Z, I], I),
+            "decx_hip_copy_kernel": ([P, P, Z], I),
             "decx_hip_timer_start": ([], I), "decx_hip_timer_stop": ([PF], I),
             "decx_hip_last_error": ([], ctypes.c_char_p),
             "decx_hip_set_sgemm_variant": ([I], I), "decx_hip_set_hgemm_variant": ([I], I),

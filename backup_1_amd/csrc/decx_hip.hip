@@ -255,6 +255,13 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
     return launch_hgemm_tile<HShapeSmall, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
 }
 
+// Plain streaming copy, 16 bytes per lane and iteration: the known-size kernel that hardware traffic counters
+// (FETCH_SIZE / WRITE_SIZE) are calibrated against.
+__global__ __launch_bounds__(256) void copy_kernel(f32x4* __restrict__ dst, const f32x4* __restrict__ src, size_t quads) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < quads; i += stride) dst[i] = src[i];
+}
+
 int finish(int rc) {
     if (rc != 0) return rc;
     HIP_TRY(hipStreamSynchronize(g_rt.stream));
@@ -407,6 +414,18 @@ int decx_hip_conv2_im2col_f32(const float* src, int H, int W, int dpitch, size_t
                               size_t dst_row_stride, int flag) {
     return finish(conv_enqueue(src, H, W, dpitch, src_row_stride, filt, N, kh, kw, filt_stride, filt_row_stride, dst,
                                dst_dpitch, dst_row_stride, flag));
+}
+
+int decx_hip_copy_kernel(void* dst, const void* src, size_t bytes) {
+    if (!g_rt.is_init) return need_init();
+    if (!dst || !src || bytes % 16 != 0 || !aligned16(dst) || !aligned16(src))
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "copy needs 16-byte aligned pointers and a multiple of 16 bytes\n");
+    if (bytes == 0) return 0;
+    const int blocks = g_rt.compute_units > 0 ? g_rt.compute_units * 8 : 2048;
+    hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(256), 0, g_rt.stream, static_cast<f32x4*>(dst),
+                       static_cast<const f32x4*>(src), bytes / 16);
+    HIP_TRY(hipGetLastError());
+    return finish(0);
 }
 
 int decx_hip_timer_start(void) {

@@ -23,6 +23,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_MATRIX_TFLOPS = 157.3     # MI355X dense fp32 MFMA
 PEAK_FP16_MATRIX_TFLOPS = 2516.6    # MI355X dense fp16 MFMA (2.5 PFLOP/s)
+# HBM-side bytes per launch of the headline kernel (fp32 8192^3), from the FETCH_SIZE / WRITE_SIZE counter runs
+# summarised in profiles/hbm_traffic_fetch_write_size.txt (read factor 2.0, write factor 1.0 against a copy kernel).
+# Counters cannot be read from inside this script; the figure is only reported for the workload it was measured on.
+MEASURED_TRAFFIC_BYTES_FP32_8192 = 3.755e9
 
 
 def log(msg):
@@ -159,6 +163,15 @@ def main():
             "frac_of_fp32_matrix_peak": round(r["tflops_kernel"] / PEAK_FP32_MATRIX_TFLOPS, 4)}
         log("conv: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
 
+    if "copy" in only:
+        # calibration launch for the traffic counters: 1 GiB read + 1 GiB written by a plain copy kernel
+        nbytes = 1 << 30
+        src, dst = capi.DeviceBuffer(nbytes), capi.DeviceBuffer(nbytes)
+        src.fill(1)
+        for _ in range(3):
+            capi.check(capi.lib().decx_hip_copy_kernel(dst.ptr, src.ptr, nbytes))
+        also["copy_1GiB"] = {"bytes_read": nbytes, "bytes_written": nbytes}
+
     cpu = None
     if want("cpu"):
         log("cpu baseline (oracle port of the DECX_cpu thread-pool SGEMM) ...")
@@ -174,7 +187,8 @@ def main():
         "config": {"workload": "fp32 square GEMM C=A*B, M=N=K=%d, row-major, uniform[-1,1] seed 1234, device-resident "
                                "operands (GPU_Matrix path)" % n},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_MATRIX_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_FP32_MATRIX_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved / PEAK_FP32_MATRIX_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES_FP32_8192 if (n == 8192 and args.sgemm_variant in (0, 1)) else None,
                      "kernel": "sgemm_tile_kernel", "flop_per_launch": head["flops"],
                      "avg_launch_ms_hip_events": round(head["ms_kernel"], 4)},
         "cpu_baseline": cpu,

@@ -114,6 +114,11 @@ int decx_hip_conv2_im2col_f32_async(const float* src, int H, int W, int dpitch, 
                                     int N, int kh, int kw, size_t filt_stride, size_t filt_row_stride, float* dst,
                                     int dst_dpitch, size_t dst_row_stride, int flag);
 
+/* A plain device-to-device streaming copy kernel of `bytes` bytes (16-byte aligned, multiple of 16).  It has no
+ * counterpart in the reference: it exists so that hardware traffic counters read for the kernels above can be scaled
+ * by what the same counters read for a kernel whose traffic is known exactly.  Blocks until complete. */
+int decx_hip_copy_kernel(void* dst, const void* src, size_t bytes);
+
 /* Timing on the library's own stream (the reference's demos time with clock(), CUDA_GEMM.cpp:43-46, :93-96).
  * start records an event, stop records another, waits for it and returns the elapsed milliseconds. */
 int decx_hip_timer_start(void);
