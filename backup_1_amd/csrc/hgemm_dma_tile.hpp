@@ -37,9 +37,11 @@ struct HgemmDmaShape : HgemmShape<BM_, BN_, BK_, WAVES_M_, WAVES_N_> {
     static_assert(STAGES >= 2, "need at least double buffering");
 };
 
-// One 16-byte-per-lane load from global memory straight into LDS at lds_base + 16*lane (lds_base wave-uniform).
-__device__ __forceinline__ void dma_load16(const void* gptr, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_base) : "memory", "m0");
+// One 16-byte-per-lane load from global memory (wave-uniform base + per-lane byte offset) straight into LDS at
+// lds_base + 16*lane (lds_base wave-uniform).
+__device__ __forceinline__ void dma_load16(const void* sbase, uint32_t lane_off, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 : : "v"(lane_off), "s"(sbase), "s"(lds_base) : "memory", "m0");
 }
 
 template <int N>
@@ -69,9 +71,12 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
     const int wm0 = (wave / S::WAVES_N) * S::WM, wn0 = (wave % S::WAVES_N) * S::WN;
     const int li = lane & 31, lh = lane >> 5;
 
-    // ---- per-lane global sources of this wave's DMA loads; they advance by one K step after every issue ----------
-    const _Float16* a_src[S::A_LOADS];
-    const _Float16* b_src[S::B_LOADS];
+    // ---- global sources of this wave's DMA loads: a wave-uniform base per operand that advances by one K step per
+    // fetched step, plus loop-invariant per-lane byte offsets (rows of this tile only, so 32 bits are plenty)
+    int m_first = bm0 < M ? bm0 : M - 1;
+    const _Float16* a_base = A + (size_t)m_first * lda;        // + BK halves per step
+    const _Float16* b_base = B;                                // + BK rows per step
+    uint32_t a_off[S::A_LOADS], b_off[S::B_LOADS];
 #pragma unroll
     for (int j = 0; j < S::A_LOADS; ++j) {
         const int chunk = wave * S::A_LOADS + j;               // 64 units = 64/UA rows
@@ -79,7 +84,7 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
         const int q = (lane % UA) ^ ((r / (16 / UA)) % UA);    // the unit whose swizzled slot is this lane
         int m = bm0 + r;
         if (m >= M) m = M - 1;
-        a_src[j] = A + (size_t)m * lda + 8 * q;
+        a_off[j] = (uint32_t)(((size_t)(m - m_first) * lda + 8 * q) * sizeof(_Float16));
     }
 #pragma unroll
     for (int j = 0; j < S::B_LOADS; ++j) {
@@ -88,20 +93,23 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
         const int u = (lane % UB) ^ ((kr & 3) << 2);
         int col = bn0 + 8 * u;
         if (col > ldb - 8) col = ldb - 8;                      // stay inside the pitch; such columns are never stored
-        b_src[j] = B + (size_t)kr * ldb + col;
+        b_off[j] = (uint32_t)(((size_t)kr * ldb + col) * sizeof(_Float16));
     }
     const size_t b_step = (size_t)BK * ldb;
 
-    // load number j (A loads first, then B) of the next K step to be fetched, into LDS buffer `stage`
+    // load number j (A loads first, then B) of the next K step to be fetched, into LDS buffer `stage`; the bases move
+    // on after the last load of a step
     auto issue_one = [&](int stage, int j) {
         const uint32_t base = lds_base + (uint32_t)stage * (S::STAGE_UNITS * 16);
         if (j < S::A_LOADS) {
-            dma_load16(a_src[j], base + (uint32_t)(wave * S::A_LOADS + j) * 1024u);
-            a_src[j] += BK;
+            dma_load16(a_base, a_off[j], base + (uint32_t)(wave * S::A_LOADS + j) * 1024u);
         } else {
             const int jb = j - S::A_LOADS;
-            dma_load16(b_src[jb], base + (uint32_t)(S::A_UNITS * 16) + (uint32_t)(wave * S::B_LOADS + jb) * 1024u);
-            b_src[jb] += b_step;
+            dma_load16(b_base, b_off[jb], base + (uint32_t)(S::A_UNITS * 16) + (uint32_t)(wave * S::B_LOADS + jb) * 1024u);
+        }
+        if (j == S::LOADS - 1) {
+            a_base += BK;
+            b_base += b_step;
         }
     };
     auto issue_stage = [&](int stage) {
@@ -125,7 +133,9 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
         if (s < full_steps) issue_stage(s);
 
     // ---- fragment reads -------------------------------------------------------------------------------------------
-    // byte offsets inside one LDS buffer; the swizzles depend on the lane only through these loop-invariant terms
+    // Loop-invariant per-lane byte offsets inside one LDS buffer; everything else about a read (row block, k-block,
+    // low/high half) is a compile-time constant that folds into the instruction's offset field, because the swizzle
+    // terms only depend on address bits those constants do not touch.
     const int tg = lane >> 4, ts = lane & 15;
     const int t_row = 8 * (tg >> 1) + (ts >> 2);               // transposed read: row inside a 16-row k-block (+4: high half)
     const int t_col = 16 * (tg & 1) + 4 * (ts & 3);            // and column inside a 32-column block
@@ -134,22 +144,28 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
         f16x8 a[MI];
         i16x4 b_lo[NI], b_hi[NI];
     };
-    // The 3*... reads of one k-block, numbered in the order the MFMAs (mi-major) first need them:
+    uint32_t a_frag_off[KS], b_frag_off[NI];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) a_frag_off[ks] = (uint32_t)a_unit_slot(wm0 + li, 2 * ks + lh, UA) * 16u;   // + mi*32 rows
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) {
+        const int col = wn0 + ni * 32 + t_col;
+        b_frag_off[ni] = (uint32_t)(S::A_UNITS * 16) + (uint32_t)b_unit_slot(t_row, col >> 3, UB) * 16u + (uint32_t)(col & 7) * 2u;
+    }
+    static_assert(32 % (16 / UA) == 0 && (32 / (16 / UA)) % UA == 0, "row blocks of 32 must not change the A swizzle");
+    // The reads of one k-block, numbered in the order the MFMAs (mi-major) first need them:
     //   0: a[0], then b_lo/b_hi of ni = 0..NI-1, then a[1..MI-1]
     constexpr int FRAG_READS = MI + 2 * NI;
     auto read_one = [&](Frags& f, int stage, int ks, int r) {
-        const u32x4* Ab = lds + stage * S::STAGE_UNITS;
-        const unsigned char* Bb = reinterpret_cast<const unsigned char*>(Ab + S::A_UNITS);
+        const unsigned char* buf = lds_raw + (size_t)stage * (S::STAGE_UNITS * 16);
         if (r == 0 || r > 2 * NI) {
             const int mi = r == 0 ? 0 : r - 2 * NI;
-            u32x4 raw = Ab[a_unit_slot(wm0 + mi * 32 + li, 2 * ks + lh, UA)];
+            u32x4 raw = *reinterpret_cast<const u32x4*>(buf + a_frag_off[ks] + mi * (32 * UA * 16));
             f.a[mi] = __builtin_bit_cast(f16x8, raw);
         } else {
             const int ni = (r - 1) / 2, hi = (r - 1) % 2;
-            const int col = wn0 + ni * 32 + t_col;
-            const int k = 16 * ks + t_row + 4 * hi;
-            const int off = b_unit_slot(k, col >> 3, UB) * 16 + (col & 7) * 2;
-            i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(Bb + off));
+            const unsigned char* p = buf + b_frag_off[ni] + (16 * ks + 4 * hi) * (UB * 16);   // rows k and k+4 share k & 3
+            i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)p);
             if (hi) f.b_hi[ni] = v;
             else f.b_lo[ni] = v;
         }
