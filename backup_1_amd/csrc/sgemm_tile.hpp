@@ -8,7 +8,7 @@
 // before the MFMAs of step t.  Both operands are kept in LDS as float4 "k-quads":
 //   A quad (q, m) = A[m][4q .. 4q+3]          at  As[q][m]             (row of BM+4 quads: the +4 staggers the four
 //                                                                       q-planes over the banks for the staging stores)
-//   B quad (q, n) = B[4q .. 4q+3][n]          at  Bs[q][n + (n >> 4)]  (4x4 register transpose while staging; the
+//   B quad (q, n) = B[4q .. 4q+3][n]          at  Bs[q][b_slot(n)]  (4x4 register transpose while staging; the
 //                                                                       n>>4 skew keeps the 64-byte-strided staging
 //                                                                       stores off each other's banks)
 // so that one ds_read_b128 per 32-row block feeds four MFMAs.  The MFMA's two k-slots (lanes 0-31 / 32-63) take
@@ -33,6 +33,15 @@ namespace decx_hip {
 //                                                   TAIL additionally zero-fills elements with k >= K
 //   size_t out_offset(int m)                        where row m of the result starts, in elements
 // ---------------------------------------------------------------------------------------------------------------
+// Slot of column n inside a B plane: bits 3-4 of n are folded onto bits 0-1.
+// Measured on gfx950 (two active lanes hitting the same banks, SQ_LDS_BANK_CONFLICT): ds_read_b128 services a wave in
+// four phases -- lanes {0-3, 12-15, 20-23, 24-27} and {4-11, 16-19, 28-31} of each half-wave -- and a phase is
+// conflict-free when its 16-byte accesses fall into distinct slots mod 16; ds_write_b128 goes in eight phases of 8
+// consecutive lanes, conflict-free when the slots are distinct mod 8.  With this fold the fragment reads (32
+// consecutive columns per half-wave) and the staging stores (every 4th column per instruction) both qualify.  Rows of A
+// need no fold: consecutive slots are read, and the planes are 2 slots out of step for the staging stores.
+__device__ __forceinline__ int b_slot(int n) { return n ^ ((n >> 3) & 3); }
+
 // Position of one k index inside the im2col ordering k = (ki*kw + kj)*dpitch + c.  Decoded once (two integer
 // divisions), then advanced by whole K steps with additions only.
 struct TapWalk {
@@ -155,7 +164,7 @@ struct TensorOut {
 //   quads<S>()                                   staging registers (float4) per thread and K step
 //   KState k_state<S>(tid) / advance<S>(ks)      position of the K step to fetch next
 //   load<S, TAIL>(stage, tid, ks, bn0)           fetch this thread's share of B[k0 .. k0+BK) x [bn0 .. bn0+BN)
-//   store<S>(plane, stage, tid)                  write it to the LDS planes as k-quads at [q][n + (n >> 4)]
+//   store<S>(plane, stage, tid)                  write it to the LDS planes as k-quads at [q][b_slot(n)]
 // ---------------------------------------------------------------------------------------------------------------
 // B as a row-major K x N matrix: a thread takes a 4(k) x 4(n) block with four 16-byte row loads (consecutive lanes
 // -> consecutive column groups, so a wave reads whole rows) and transposes it in registers into four k-quads.
@@ -217,7 +226,7 @@ struct DenseB {
             for (int j = 0; j < 4; ++j) {
                 const int n = 4 * cg + j;
                 f32x4 t = {st[4 * p + 0][j], st[4 * p + 1][j], st[4 * p + 2][j], st[4 * p + 3][j]};
-                plane[q * S::B_ROW + n + (n >> 4)] = t;
+                plane[q * S::B_ROW + b_slot(n)] = t;
             }
         }
     }
@@ -262,7 +271,7 @@ struct FilterB {
         for (int j = 0; j < quads<S>(); ++j) {
             const int id = tid + j * S::NT;
             const int q = id % S::KQ, n = id / S::KQ;
-            plane[q * S::B_ROW + n + (n >> 4)] = st[j];
+            plane[q * S::B_ROW + b_slot(n)] = st[j];
         }
     }
 };
@@ -275,8 +284,8 @@ struct SgemmShape {
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     static constexpr int MI = WM / 32, NI = WN / 32;
     static constexpr int KQ = BK / 4;                         // k-quads per step
-    static constexpr int A_ROW = BM + 4;                      // quads per A plane
-    static constexpr int B_ROW = BN + BN / 16;                // quads per B plane
+    static constexpr int A_ROW = BM + 2;                      // quads per A plane (planes 2 slots out of step mod 8)
+    static constexpr int B_ROW = BN + 2;                      // quads per B plane
     static constexpr int A_PASSES = (BM * KQ + NT - 1) / NT;  // float4 global loads of A per thread per step (last may be partial)
     static constexpr bool A_PARTIAL = (BM * KQ) % NT != 0;
     static constexpr size_t LDS_BYTES = 2 * (size_t)KQ * (A_ROW + B_ROW) * sizeof(f32x4);
@@ -359,7 +368,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
 #pragma unroll
         for (int ni = 0; ni < NI; ++ni) {
             const int n = wn0 + ni * 32 + li;
-            bf[ni] = Bb[q * S::B_ROW + n + (n >> 4)];
+            bf[ni] = Bb[q * S::B_ROW + b_slot(n)];
         }
     };
     // MFMAs number lo .. hi-1 of a quad pair, in the order (e, mi, ni); a full pair is 4*MI*NI of them.
