@@ -119,6 +119,38 @@ public:
     virtual ~TensorArray() {}
 };
 
+// classes/GPU_Tensor.h:19-47.  Device-resident tensor with the host Tensor's layout (dpitch = ceil4(depth),
+// wpitch = ceil4(width)).
+template <typename T>
+class GPU_Tensor {
+public:
+    GPU_Tensor() {}
+    virtual uint Width() = 0;
+    virtual uint Height() = 0;
+    virtual uint Depth() = 0;
+    virtual GPU_Tensor<T>& operator=(GPU_Tensor<T>& src) = 0;
+    virtual void Load_from_host(Tensor<T>& src) = 0;
+    virtual void Load_to_host(Tensor<T>& dst) = 0;
+    virtual void release() = 0;
+    virtual ~GPU_Tensor() {}
+};
+
+// classes/GPU_TensorArray.h:24-52
+template <typename T>
+class GPU_TensorArray {
+public:
+    GPU_TensorArray() {}
+    virtual uint Width() = 0;
+    virtual uint Height() = 0;
+    virtual uint Depth() = 0;
+    virtual uint TensorNum() = 0;
+    virtual void Load_from_host(TensorArray<T>& src) = 0;
+    virtual void Load_to_host(TensorArray<T>& dst) = 0;
+    virtual GPU_TensorArray<T>& operator=(GPU_TensorArray<T>& src) = 0;
+    virtual void release() = 0;
+    virtual ~GPU_TensorArray() {}
+};
+
 // factories: classes/Matrix.h:430-476, GPU_Matrix.h:361-435, Tensor.h:401-463, TensorArray.h:440-474.
 // Instantiated for float and de::Half (Matrix, GPU_Matrix) and float (Tensor, TensorArray).
 template <typename T> Matrix<T>& CreateMatrixRef();
@@ -138,6 +170,16 @@ template <typename T> TensorArray<T>* CreateTensorArrayPtr();
 template <typename T> TensorArray<T>& CreateTensorArrayRef(const uint width, const uint height, const uint depth, const uint tensor_num, const int flag);
 template <typename T> TensorArray<T>* CreateTensorArrayPtr(const uint width, const uint height, const uint depth, const uint tensor_num, const int flag);
 
+// classes/GPU_Tensor.h:385-397, GPU_TensorArray.h (same pattern); instantiated for float
+template <typename T> GPU_Tensor<T>& CreateGPUTensorRef();
+template <typename T> GPU_Tensor<T>* CreateGPUTensorPtr();
+template <typename T> GPU_Tensor<T>& CreateGPUTensorRef(const uint width, const uint height, const uint depth);
+template <typename T> GPU_Tensor<T>* CreateGPUTensorPtr(const uint width, const uint height, const uint depth);
+template <typename T> GPU_TensorArray<T>& CreateGPUTensorArrayRef();
+template <typename T> GPU_TensorArray<T>* CreateGPUTensorArrayPtr();
+template <typename T> GPU_TensorArray<T>& CreateGPUTensorArrayRef(const uint width, const uint height, const uint depth, const uint tensor_num);
+template <typename T> GPU_TensorArray<T>* CreateGPUTensorArrayPtr(const uint width, const uint height, const uint depth, const uint tensor_num);
+
 // core/configs/config.h:62, :73-78.  The name is kept for drop-in use; it initialises the HIP device.
 void InitCuda();
 // core/memory_management/Memory_pool.h:23-37.  There are no pools here; kept as a no-op.
@@ -155,6 +197,10 @@ DH GEMM(GPU_Matrix<Half>& A, GPU_Matrix<Half>& B, GPU_Matrix<Half>& dst);
 DH GEMM(GPU_Matrix<Half>& A, GPU_Matrix<Half>& B, GPU_Matrix<Half>& C, GPU_Matrix<Half>& dst);
 // convolution/CUDA/im2col/conv2_mk_im2col.h:25.  flag: decx::conv_property.
 DH Conv2_MK_im2col(Tensor<float>& src, TensorArray<float>& kernel, Tensor<float>& dst, const int flag);
+// Device-resident flavour of the same convolution (the reference only has the host one; its GPU_Tensor /
+// GPU_TensorArray containers, classes/GPU_Tensor.h and GPU_TensorArray.h, are what it would take).  dst is
+// (re)constructed to the output size; no host copies are made.
+DH Conv2_MK_im2col(GPU_Tensor<float>& src, GPU_TensorArray<float>& kernel, GPU_Tensor<float>& dst, const int flag);
 }  // namespace cuda
 
 namespace cpu {

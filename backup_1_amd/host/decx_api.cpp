@@ -168,6 +168,23 @@ template <typename T> TensorArray<T>* CreateTensorArrayPtr() { return new decx::
 template <typename T> TensorArray<T>& CreateTensorArrayRef(const uint w, const uint h, const uint d, const uint n, const int f) { return *(new decx::_TensorArray<T>(w, h, d, n, f)); }
 template <typename T> TensorArray<T>* CreateTensorArrayPtr(const uint w, const uint h, const uint d, const uint n, const int f) { return new decx::_TensorArray<T>(w, h, d, n, f); }
 
+template <typename T> GPU_Tensor<T>& CreateGPUTensorRef() { return *(new decx::_GPU_Tensor<T>()); }
+template <typename T> GPU_Tensor<T>* CreateGPUTensorPtr() { return new decx::_GPU_Tensor<T>(); }
+template <typename T> GPU_Tensor<T>& CreateGPUTensorRef(const uint w, const uint h, const uint d) { return *(new decx::_GPU_Tensor<T>(w, h, d)); }
+template <typename T> GPU_Tensor<T>* CreateGPUTensorPtr(const uint w, const uint h, const uint d) { return new decx::_GPU_Tensor<T>(w, h, d); }
+template <typename T> GPU_TensorArray<T>& CreateGPUTensorArrayRef() { return *(new decx::_GPU_TensorArray<T>()); }
+template <typename T> GPU_TensorArray<T>* CreateGPUTensorArrayPtr() { return new decx::_GPU_TensorArray<T>(); }
+template <typename T> GPU_TensorArray<T>& CreateGPUTensorArrayRef(const uint w, const uint h, const uint d, const uint n) { return *(new decx::_GPU_TensorArray<T>(w, h, d, n)); }
+template <typename T> GPU_TensorArray<T>* CreateGPUTensorArrayPtr(const uint w, const uint h, const uint d, const uint n) { return new decx::_GPU_TensorArray<T>(w, h, d, n); }
+template GPU_Tensor<float>& CreateGPUTensorRef<float>();
+template GPU_Tensor<float>* CreateGPUTensorPtr<float>();
+template GPU_Tensor<float>& CreateGPUTensorRef<float>(const uint, const uint, const uint);
+template GPU_Tensor<float>* CreateGPUTensorPtr<float>(const uint, const uint, const uint);
+template GPU_TensorArray<float>& CreateGPUTensorArrayRef<float>();
+template GPU_TensorArray<float>* CreateGPUTensorArrayPtr<float>();
+template GPU_TensorArray<float>& CreateGPUTensorArrayRef<float>(const uint, const uint, const uint, const uint);
+template GPU_TensorArray<float>* CreateGPUTensorArrayPtr<float>(const uint, const uint, const uint, const uint);
+
 #define DECX_INSTANTIATE_MATRIX(T)                                                     \
     template Matrix<T>& CreateMatrixRef<T>();                                          \
     template Matrix<T>* CreateMatrixPtr<T>();                                          \
@@ -234,6 +251,28 @@ DH Conv2_MK_im2col(Tensor<float>& src_, TensorArray<float>& kernel_, Tensor<floa
                                    static_cast<float*>(dD.ptr), (int)dst->dpitch, dst->dp_x_wp, flag);
     if (rc) return from_status(rc);
     return from_status(decx_hip_memcpy(dst->Tens.ptr, dD.ptr, dst->total_bytes, DECX_HIP_D2H));   // :266
+}
+
+DH Conv2_MK_im2col(GPU_Tensor<float>& src_, GPU_TensorArray<float>& kernel_, GPU_Tensor<float>& dst_, const int flag) {
+    auto* src = dynamic_cast<decx::_GPU_Tensor<float>*>(&src_);
+    auto* ker = dynamic_cast<decx::_GPU_TensorArray<float>*>(&kernel_);
+    auto* dst = dynamic_cast<decx::_GPU_Tensor<float>*>(&dst_);
+    if (!src || !ker || !dst) return DH{decx::DECX_FAIL_ErrorParams, kNotFactory};
+    if (!decx_hip_is_init()) return not_init();
+    if (flag != decx::de_conv_no_compensate && flag != decx::de_conv_zero_compensate) {
+        static char msg[] = "This flag is meaningless in current context\n";
+        return DH{decx::DECX_FAIL_ErrorFlag, msg};
+    }
+    static char dims_msg[] = "Tensor Dims don't match each other";
+    if (src->depth != ker->depth) return DH{decx::DECX_FAIL_DimsNotMatching, dims_msg};
+    const int H = (int)src->height, W = (int)src->width, kh = (int)ker->height, kw = (int)ker->width;
+    const int Hout = flag ? H : H - 2 * (kh / 2), Wout = flag ? W : W - 2 * (kw / 2);
+    if (Hout <= 0 || Wout <= 0) return DH{decx::DECX_FAIL_DimsNotMatching, dims_msg};
+    if (!dst->re_construct((uint)Wout, (uint)Hout, ker->tensor_num))
+        return dst->last_status == DECX_HIP_FAIL_ALLOCATION ? alloc_fail() : from_status(dst->last_status);
+    return from_status(decx_hip_conv2_im2col_f32(src->Tens.ptr, H, W, (int)src->dpitch, src->dp_x_wp, ker->TensArr.ptr,
+                                                 (int)ker->tensor_num, kh, kw, ker->_gap, ker->dp_x_wp, dst->Tens.ptr,
+                                                 (int)dst->dpitch, dst->dp_x_wp, flag));
 }
 }  // namespace cuda
 }  // namespace de

@@ -285,4 +285,129 @@ public:
     ~_TensorArray() override { release(); }
 };
 
+template <typename T>
+class _GPU_Tensor : public de::GPU_Tensor<T> {
+public:
+    uint width = 0, height = 0, depth = 0;
+    uint dpitch = 0, wpitch = 0;
+    size_t dp_x_wp = 0;
+    PtrInfo<T> Tens;                             // DEVICE pointer
+    size_t element_num = 0, _element_num = 0, total_bytes = 0;
+    int last_status = 0;
+
+    _GPU_Tensor() {}
+    _GPU_Tensor(uint w, uint h, uint d) { construct(w, h, d); }
+    void attribute_assign(uint w, uint h, uint d) {
+        width = w;
+        height = h;
+        depth = d;
+        wpitch = ceil_to(w, 4);
+        dpitch = ceil_to(d, 4);
+        dp_x_wp = (size_t)dpitch * wpitch;
+        element_num = (size_t)d * w * h;
+        _element_num = (size_t)h * dp_x_wp;
+        total_bytes = _element_num * sizeof(T);
+    }
+    bool construct(uint w, uint h, uint d) {
+        release();
+        attribute_assign(w, h, d);
+        void* p = nullptr;
+        last_status = decx_hip_malloc(&p, total_bytes);
+        if (last_status != 0) return false;
+        Tens.ptr = static_cast<T*>(p);
+        last_status = decx_hip_memset(p, 0, total_bytes);
+        return last_status == 0;
+    }
+    bool re_construct(uint w, uint h, uint d) {
+        if (Tens.ptr && w == width && h == height && d == depth) return true;
+        return construct(w, h, d);
+    }
+    uint Width() override { return width; }
+    uint Height() override { return height; }
+    uint Depth() override { return depth; }
+    de::GPU_Tensor<T>& operator=(de::GPU_Tensor<T>& src) override {
+        _GPU_Tensor<T>& s = dynamic_cast<_GPU_Tensor<T>&>(src);
+        if (&s != this && construct(s.width, s.height, s.depth))
+            last_status = decx_hip_memcpy(Tens.ptr, s.Tens.ptr, total_bytes, DECX_HIP_D2D);
+        return *this;
+    }
+    void Load_from_host(de::Tensor<T>& src) override {
+        _Tensor<T>& s = dynamic_cast<_Tensor<T>&>(src);
+        if (s.width != width || s.height != height || s.depth != depth) { last_status = DECX_HIP_FAIL_DIMS; return; }
+        last_status = decx_hip_memcpy(Tens.ptr, s.Tens.ptr, total_bytes, DECX_HIP_H2D);     // identical layouts
+    }
+    void Load_to_host(de::Tensor<T>& dst) override {
+        _Tensor<T>& d = dynamic_cast<_Tensor<T>&>(dst);
+        if (d.width != width || d.height != height || d.depth != depth) { last_status = DECX_HIP_FAIL_DIMS; return; }
+        last_status = decx_hip_memcpy(d.Tens.ptr, Tens.ptr, total_bytes, DECX_HIP_D2H);
+    }
+    void release() override {
+        if (Tens.ptr) decx_hip_free(Tens.ptr);
+        Tens.ptr = nullptr;
+    }
+    ~_GPU_Tensor() override { release(); }
+};
+
+template <typename T>
+class _GPU_TensorArray : public de::GPU_TensorArray<T> {
+public:
+    uint width = 0, height = 0, depth = 0, tensor_num = 0;
+    uint dpitch = 0, wpitch = 0;
+    size_t dp_x_wp = 0, _gap = 0;
+    PtrInfo<T> TensArr;                          // DEVICE pointer
+    size_t element_num = 0, _element_num = 0, total_bytes = 0;
+    int last_status = 0;
+
+    _GPU_TensorArray() {}
+    _GPU_TensorArray(uint w, uint h, uint d, uint n) { construct(w, h, d, n); }
+    void attribute_assign(uint w, uint h, uint d, uint n) {
+        width = w;
+        height = h;
+        depth = d;
+        tensor_num = n;
+        wpitch = ceil_to(w, 4);
+        dpitch = ceil_to(d, 4);
+        dp_x_wp = (size_t)dpitch * wpitch;
+        _gap = dp_x_wp * h;
+        element_num = (size_t)d * w * h * n;
+        _element_num = (size_t)n * _gap;
+        total_bytes = _element_num * sizeof(T);
+    }
+    bool construct(uint w, uint h, uint d, uint n) {
+        release();
+        attribute_assign(w, h, d, n);
+        void* p = nullptr;
+        last_status = decx_hip_malloc(&p, total_bytes);
+        if (last_status != 0) return false;
+        TensArr.ptr = static_cast<T*>(p);
+        last_status = decx_hip_memset(p, 0, total_bytes);
+        return last_status == 0;
+    }
+    uint Width() override { return width; }
+    uint Height() override { return height; }
+    uint Depth() override { return depth; }
+    uint TensorNum() override { return tensor_num; }
+    void Load_from_host(de::TensorArray<T>& src) override {
+        _TensorArray<T>& s = dynamic_cast<_TensorArray<T>&>(src);
+        if (s.width != width || s.height != height || s.depth != depth || s.tensor_num != tensor_num) { last_status = DECX_HIP_FAIL_DIMS; return; }
+        last_status = decx_hip_memcpy(TensArr.ptr, s.TensArr.ptr, total_bytes, DECX_HIP_H2D);
+    }
+    void Load_to_host(de::TensorArray<T>& dst) override {
+        _TensorArray<T>& d = dynamic_cast<_TensorArray<T>&>(dst);
+        if (d.width != width || d.height != height || d.depth != depth || d.tensor_num != tensor_num) { last_status = DECX_HIP_FAIL_DIMS; return; }
+        last_status = decx_hip_memcpy(d.TensArr.ptr, TensArr.ptr, total_bytes, DECX_HIP_D2H);
+    }
+    de::GPU_TensorArray<T>& operator=(de::GPU_TensorArray<T>& src) override {
+        _GPU_TensorArray<T>& s = dynamic_cast<_GPU_TensorArray<T>&>(src);
+        if (&s != this && construct(s.width, s.height, s.depth, s.tensor_num))
+            last_status = decx_hip_memcpy(TensArr.ptr, s.TensArr.ptr, total_bytes, DECX_HIP_D2D);
+        return *this;
+    }
+    void release() override {
+        if (TensArr.ptr) decx_hip_free(TensArr.ptr);
+        TensArr.ptr = nullptr;
+    }
+    ~_GPU_TensorArray() override { release(); }
+};
+
 }  // namespace decx

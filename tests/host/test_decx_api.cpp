@@ -265,6 +265,33 @@ static void conv_case(int H, int W, int C, int N, int kh, int kw, int flag) {
     CHECK(same);
     src.release(); ker.release(); dst.release();
 }
+static void conv_device_resident() {
+    const int H = 30, W = 26, C = 12, N = 10, kh = 3, kw = 3;        // width not a multiple of 4: padded rows in dst
+    de::Tensor<float>& src = de::CreateTensorRef<float>(W, H, C, 0);
+    de::TensorArray<float>& ker = de::CreateTensorArrayRef<float>(kw, kh, C, N, 0);
+    for (int y = 0; y < H; ++y) for (int x = 0; x < W; ++x) for (int c = 0; c < C; ++c) src.index(y, x, c) = small_int();
+    for (int n = 0; n < N; ++n) for (int i = 0; i < kh; ++i) for (int j = 0; j < kw; ++j) for (int c = 0; c < C; ++c) ker.index(i, j, c, n) = small_int();
+    de::GPU_Tensor<float>& dsrc = de::CreateGPUTensorRef<float>(W, H, C);
+    de::GPU_TensorArray<float>& dker = de::CreateGPUTensorArrayRef<float>(kw, kh, C, N);
+    de::GPU_Tensor<float>& ddst = de::CreateGPUTensorRef<float>();
+    dsrc.Load_from_host(src); dker.Load_from_host(ker);
+    for (int flag = 0; flag < 2; ++flag) {
+        de::Tensor<float>& want = de::CreateTensorRef<float>();
+        CHECK(de::cuda::Conv2_MK_im2col(src, ker, want, flag).error_type == decx::DECX_SUCCESS);
+        CHECK(de::cuda::Conv2_MK_im2col(dsrc, dker, ddst, flag).error_type == decx::DECX_SUCCESS);
+        CHECK(ddst.Width() == want.Width() && ddst.Height() == want.Height() && ddst.Depth() == (uint)N);
+        de::Tensor<float>& got = de::CreateTensorRef<float>(want.Width(), want.Height(), N, 0);
+        ddst.Load_to_host(got);
+        bool same = true;
+        for (uint y = 0; y < want.Height(); ++y) for (uint x = 0; x < want.Width(); ++x) for (int n = 0; n < N; ++n)
+            same = same && got.index(y, x, n) == want.index(y, x, n);
+        CHECK(same);
+        want.release(); got.release();
+    }
+    CHECK(de::cuda::Conv2_MK_im2col(dsrc, dker, ddst, 5).error_type == decx::DECX_FAIL_ErrorFlag);
+    dsrc.release(); dker.release(); ddst.release(); src.release(); ker.release();
+}
+
 static void conv_flavours_and_flags() {
     conv_case(20, 22, 8, 6, 3, 3, decx::de_conv_zero_compensate);
     conv_case(20, 22, 8, 6, 3, 3, decx::de_conv_no_compensate);
@@ -292,6 +319,7 @@ int main(int argc, char** argv) {
         RUN(gemm_fp32_all_flavours);
         RUN(gemm_fp16_flavours);
         RUN(conv_flavours_and_flags);
+        RUN(conv_device_resident);
     }
     std::printf("%s: %d failure(s)\n", mode.c_str(), g_fail);
     return g_fail ? 1 : 0;
