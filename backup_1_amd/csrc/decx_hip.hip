@@ -56,12 +56,20 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 inline int cdiv(int a, int b) { return (a + b - 1) / b; }
 
+// A batch of `count` independent, equally shaped problems; the strides are in elements between consecutive problems.
+// Every launcher enqueues on `stream`.
+struct Batch {
+    int count = 1;
+    size_t stride_a = 0, stride_b = 0, stride_c = 0, stride_d = 0;
+    hipStream_t stream = nullptr;
+};
+
 // ---------------------------------------------------------------------------------------------------------------
 // fp32 launchers
 // ---------------------------------------------------------------------------------------------------------------
 template <class S, class ASrc, class BSrc, class Out, bool HAS_C>
 int launch_sgemm_tile_c(const ASrc& a, const BSrc& b, const float* Cin, int ldc, float* D, const Out& out, int M, int N,
-                        int K) {
+                        int K, const Batch& batch) {
     auto kern = sgemm_tile_kernel<S, ASrc, BSrc, Out, HAS_C>;
     static bool attr_done = false;
     if (!attr_done) {
@@ -71,34 +79,34 @@ int launch_sgemm_tile_c(const ASrc& a, const BSrc& b, const float* Cin, int ldc,
     }
     const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
     const long total = (long)tiles_m * tiles_n;
-    if (total > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
+    if (total > 0x7fffffffL || batch.count > 65535) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
     const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
-    hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream, a, b, Cin, ldc, D, out, M,
-                       N, K, tiles_m, tiles_n, group_m);
+    hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::LDS_BYTES, batch.stream, a, b, Cin,
+                       ldc, D, out, M, N, K, tiles_m, tiles_n, group_m, batch.stride_c, batch.stride_d);
     HIP_TRY(hipGetLastError());
     return 0;
 }
 
 template <class S, class ASrc, class BSrc, class Out>
 int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, float* D, const Out& out, int M, int N,
-                      int K) {
-    if (Cin != nullptr) return launch_sgemm_tile_c<S, ASrc, BSrc, Out, true>(a, b, Cin, ldc, D, out, M, N, K);
-    return launch_sgemm_tile_c<S, ASrc, BSrc, Out, false>(a, b, Cin, ldc, D, out, M, N, K);
+                      int K, const Batch& batch) {
+    if (Cin != nullptr) return launch_sgemm_tile_c<S, ASrc, BSrc, Out, true>(a, b, Cin, ldc, D, out, M, N, K, batch);
+    return launch_sgemm_tile_c<S, ASrc, BSrc, Out, false>(a, b, Cin, ldc, D, out, M, N, K, batch);
 }
 
 // Tile shapes (variant numbers of decx_hip_set_sgemm_variant):
 //   1: 256x256x16, 2x2 waves of 128x128   -- large problems, highest reuse per LDS byte
 //   2: 128x128x16, 2x2 waves of  64x64    -- small problems, several workgroups per CU
-//   3: 256x128x16, 2x2 waves of 128x64    -- narrow N (the convolution's 128 filters)
+//   3: 256x128x16, 2x2 waves of 128x64    -- narrow N
+//   4: 224x128x16, 1x4 waves of 224x32    -- 7/8 of shape 3 per tile: fills more CUs when M/256 tiles leave many idle
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
 typedef SgemmShape<128, 128, 16, 2, 2, 2> SShapeSmall;
 typedef SgemmShape<256, 128, 16, 2, 2, 2> SShapeTall;
-//   4: 224x128x16, 1x4 waves of 224x32    -- 7/8 of shape 3 per tile: fills more CUs when M/256 tiles leave many idle
 typedef SgemmShape<224, 128, 16, 1, 4, 2> SShape224;
 
 // Tile shape by a small cost model: a CU works through ceil(tiles / CUs) tiles one after another, a tile costs its area
 // divided by how well that shape keeps the matrix pipe busy (measured on 8192^3, relative to shape 1).
-int pick_sgemm_variant(int M, int N) {
+int pick_sgemm_variant(int M, int N, int batch) {
     if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 4) return g_rt.sgemm_variant;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     struct Cand { int variant, bm, bn; double eff; };
@@ -106,7 +114,7 @@ int pick_sgemm_variant(int M, int N) {
     int best = 1;
     double best_cost = 0.0;
     for (const Cand& c : cands) {
-        const long tiles = (long)cdiv(M, c.bm) * cdiv(N, c.bn);
+        const long tiles = (long)cdiv(M, c.bm) * cdiv(N, c.bn) * batch;
         const double cost = (double)((tiles + cus - 1) / cus) * c.bm * c.bn / c.eff;
         if (best_cost == 0.0 || cost < best_cost) { best_cost = cost; best = c.variant; }
     }
@@ -115,35 +123,44 @@ int pick_sgemm_variant(int M, int N) {
 
 template <class ASrc, class BSrc, class Out>
 int dispatch_sgemm(int variant, const ASrc& a, const BSrc& b, const float* Cin, int ldc, float* D, const Out& out, int M,
-                   int N, int K) {
+                   int N, int K, const Batch& batch) {
     switch (variant) {
-        case 1: return launch_sgemm_tile<SShapeBig>(a, b, Cin, ldc, D, out, M, N, K);
-        case 3: return launch_sgemm_tile<SShapeTall>(a, b, Cin, ldc, D, out, M, N, K);
-        case 4: return launch_sgemm_tile<SShape224>(a, b, Cin, ldc, D, out, M, N, K);
-        default: return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K);
+        case 1: return launch_sgemm_tile<SShapeBig>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 3: return launch_sgemm_tile<SShapeTall>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 4: return launch_sgemm_tile<SShape224>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        default: return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K, batch);
     }
 }
 
-int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
-                  int N, int K) {
+int check_gemm_args(const void* A, int lda, const void* B, int ldb, const void* Cin, int ldc, const void* D, int ldd, int M,
+                    int N, int K, const Batch& batch) {
     if (!g_rt.is_init) return need_init();
     if (!A || !B || !D) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "null matrix pointer\n");
-    if (M <= 0 || N <= 0 || K <= 0) return fail(DECX_HIP_FAIL_DIMS, "Matrix Dims don't match each other");
+    if (M <= 0 || N <= 0 || K <= 0 || batch.count <= 0) return fail(DECX_HIP_FAIL_DIMS, "Matrix Dims don't match each other");
     if (lda < K || ldb < N || ldd < N || (Cin && ldc < N))
         return fail(DECX_HIP_FAIL_ERROR_PARAMS, "leading dimension smaller than the row length\n");
-    const int variant = pick_sgemm_variant(M, N);
-    const bool vec_a = aligned16(A) && lda % 4 == 0;
-    const bool vec_b = aligned16(B) && ldb % 4 == 0 && ldb >= 4;
+    if (batch.count > 1 && (batch.stride_a < (size_t)(M - 1) * lda + K || batch.stride_b < (size_t)(K - 1) * ldb + N ||
+                            batch.stride_d < (size_t)(M - 1) * ldd + N || (Cin && batch.stride_c < (size_t)(M - 1) * ldc + N)))
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "batch stride smaller than one matrix\n");
+    return 0;
+}
+
+int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
+                  int N, int K, const Batch& batch) {
+    if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
+    const int variant = pick_sgemm_variant(M, N, batch.count);
+    const bool vec_a = aligned16(A) && lda % 4 == 0 && batch.stride_a % 4 == 0;
+    const bool vec_b = aligned16(B) && ldb % 4 == 0 && ldb >= 4 && batch.stride_b % 4 == 0;
     DenseOut out{ldd};
     if (vec_a && vec_b) {
-        DenseA<true> a{A, lda, M, K};
-        DenseB<true> b{B, ldb, N, K};
-        return dispatch_sgemm(variant, a, b, Cin, ldc, D, out, M, N, K);
+        DenseA<true> a{A, lda, M, K, batch.stride_a};
+        DenseB<true> b{B, ldb, N, K, batch.stride_b};
+        return dispatch_sgemm(variant, a, b, Cin, ldc, D, out, M, N, K, batch);
     }
     // unaligned operands: element-wise loaders, one tile shape only
-    DenseA<false> a{A, lda, M, K};
-    DenseB<false> b{B, ldb, N, K};
-    return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K);
+    DenseA<false> a{A, lda, M, K, batch.stride_a};
+    DenseB<false> b{B, ldb, N, K, batch.stride_b};
+    return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K, batch);
 }
 
 int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt, int N, int kh,
@@ -170,27 +187,29 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
     Im2colA a{src, H, W, dpitch, kh, kw, flag ? kh / 2 : 0, flag ? kw / 2 : 0, Wout, M, K, src_row_stride};
     FilterB b{filt, N, K, dpitch, kw, filt_stride, filt_row_stride};
     TensorOut out{Wout, dst_dpitch, dst_row_stride, dst_row_stride == (size_t)Wout * dst_dpitch};
-    return dispatch_sgemm(pick_sgemm_variant(M, N), a, b, nullptr, 0, dst, out, M, N, K);
+    Batch one;
+    one.stream = g_rt.stream;
+    return dispatch_sgemm(pick_sgemm_variant(M, N, 1), a, b, nullptr, 0, dst, out, M, N, K, one);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
 // fp16 launchers
 // ---------------------------------------------------------------------------------------------------------------
 // Tile shapes (variant numbers of decx_hip_set_hgemm_variant):
-//   1: 256x256x32, 2x2 waves of 128x128
-//   2: 128x128x32, 2x2 waves of  64x64
+//   1: 256x256x32, 2x2 waves of 128x128, register-staged
+//   2: 128x128x32, 2x2 waves of  64x64, register-staged (also the element-wise loader for unaligned operands)
+//   3: 256x256x32, 2x2 waves of 128x128, 4-stage LDS-DMA pipeline
+//   4: 256x256x64, 2x2 waves of 128x128, 2-stage LDS-DMA pipeline (whole 128-byte lines of A per row and step)
+//   5: 256x256x32, 2x2 waves of 128x128, 5-stage LDS-DMA pipeline
 typedef HgemmShape<256, 256, 32, 2, 2> HShapeBig;
 typedef HgemmShape<128, 128, 32, 2, 2> HShapeSmall;
-//   3: 256x256x32, 2x2 waves of 128x128, 4-stage LDS-DMA pipeline
 typedef HgemmDmaShape<256, 256, 32, 2, 2, 4> HShapeDma;
-//   4: 256x256x64, 2x2 waves of 128x128, 2-stage LDS-DMA pipeline (whole 128-byte lines of A per row and step)
 typedef HgemmDmaShape<256, 256, 64, 2, 2, 2> HShapeDma64;
-//   5: 256x256x32, 5-stage
 typedef HgemmDmaShape<256, 256, 32, 2, 2, 5> HShapeDma5;
 
 template <class S, bool VEC>
 int launch_hgemm_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
-                      int ldd, int M, int N, int K) {
+                      int ldd, int M, int N, int K, const Batch& batch) {
     auto kern = hgemm_tile_kernel<S, VEC>;
     static bool attr_done = false;
     if (!attr_done) {
@@ -200,19 +219,19 @@ int launch_hgemm_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb, co
     }
     const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
     const long total = (long)tiles_m * tiles_n;
-    if (total > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
+    if (total > 0x7fffffffL || batch.count > 65535) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
     const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
-    hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream,
+    hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::LDS_BYTES, batch.stream,
                        reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
                        reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N, K,
-                       tiles_m, tiles_n, group_m);
+                       tiles_m, tiles_n, group_m, batch.stride_a, batch.stride_b, batch.stride_c, batch.stride_d);
     HIP_TRY(hipGetLastError());
     return 0;
 }
 
 template <class S>
 int launch_hgemm_dma_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
-                          uint16_t* D, int ldd, int M, int N, int K) {
+                          uint16_t* D, int ldd, int M, int N, int K, const Batch& batch) {
     auto kern = Cin ? hgemm_dma_kernel<S, true> : hgemm_dma_kernel<S, false>;
     static bool attr_done = false;
     if (!attr_done) {
@@ -224,35 +243,129 @@ int launch_hgemm_dma_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb
     }
     const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
     const long total = (long)tiles_m * tiles_n;
-    if (total > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
+    if (total > 0x7fffffffL || batch.count > 65535) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
     const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
-    hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream,
+    hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::LDS_BYTES, batch.stream,
                        reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
                        reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N, K,
-                       tiles_m, tiles_n, group_m);
+                       tiles_m, tiles_n, group_m, batch.stride_a, batch.stride_b, batch.stride_c, batch.stride_d);
     HIP_TRY(hipGetLastError());
     return 0;
 }
 
 int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
-                  int ldd, int M, int N, int K) {
-    if (!g_rt.is_init) return need_init();
-    if (!A || !B || !D) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "null matrix pointer\n");
-    if (M <= 0 || N <= 0 || K <= 0) return fail(DECX_HIP_FAIL_DIMS, "Matrix Dims don't match each other");
-    if (lda < K || ldb < N || ldd < N || (Cin && ldc < N))
-        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "leading dimension smaller than the row length\n");
-    const bool vec = aligned16(A) && aligned16(B) && lda % 8 == 0 && ldb % 8 == 0 && ldb >= 8;
-    if (!vec) return launch_hgemm_tile<HShapeSmall, false>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
+                  int ldd, int M, int N, int K, const Batch& batch) {
+    if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
+    const bool vec = aligned16(A) && aligned16(B) && lda % 8 == 0 && ldb % 8 == 0 && ldb >= 8 && batch.stride_a % 8 == 0 &&
+                     batch.stride_b % 8 == 0;
+    if (!vec) return launch_hgemm_tile<HShapeSmall, false>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     int variant = g_rt.hgemm_variant;
     if (variant < 1 || variant > 5) {
         const int cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
-        variant = ((long)cdiv(M, 256) * cdiv(N, 256) * 10 >= (long)cus * 8) ? 4 : 2;
+        variant = ((long)cdiv(M, 256) * cdiv(N, 256) * batch.count * 10 >= (long)cus * 8) ? 4 : 2;
     }
-    if (variant == 3) return launch_hgemm_dma_tile<HShapeDma>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
-    if (variant == 4) return launch_hgemm_dma_tile<HShapeDma64>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
-    if (variant == 5) return launch_hgemm_dma_tile<HShapeDma5>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
-    if (variant == 1) return launch_hgemm_tile<HShapeBig, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
-    return launch_hgemm_tile<HShapeSmall, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
+    if (variant == 3) return launch_hgemm_dma_tile<HShapeDma>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 4) return launch_hgemm_dma_tile<HShapeDma64>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 5) return launch_hgemm_dma_tile<HShapeDma5>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 1) return launch_hgemm_tile<HShapeBig, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    return launch_hgemm_tile<HShapeSmall, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+}
+
+Batch single_on_library_stream() {
+    Batch b;
+    b.stream = g_rt.stream;
+    return b;
+}
+Batch batch_on_library_stream(int count, size_t sa, size_t sb, size_t sc, size_t sd) {
+    Batch b;
+    b.count = count;
+    b.stride_a = sa;
+    b.stride_b = sb;
+    b.stride_c = sc;
+    b.stride_d = sd;
+    b.stream = g_rt.stream;
+    return b;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Host-resident batches (the MatrixArray GEMM3 of the reference): one matrix triple per pipeline step, two device
+// buffer sets, uploads / kernel / downloads on three streams chained by events, so that the copies of steps i+1 and
+// i-1 run under the kernel of step i.
+// ---------------------------------------------------------------------------------------------------------------
+template <typename T, class Enqueue>
+int gemm3_host_pipeline(const T* hA, int lda, size_t plane_a, const T* hB, int ldb, size_t plane_b, const T* hC, int ldc,
+                        size_t plane_c, T* hD, int ldd, size_t plane_d, int M, int N, int K, int count, Enqueue enqueue) {
+    if (!g_rt.is_init) return need_init();
+    if (!hA || !hB || !hD) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "null matrix pointer\n");
+    if (M <= 0 || N <= 0 || K <= 0 || count <= 0) return fail(DECX_HIP_FAIL_DIMS, "Matrix Dims don't match each other");
+    if (lda < K || ldb < N || ldd < N || (hC && ldc < N))
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "leading dimension smaller than the row length\n");
+    const size_t bytes_a = (size_t)M * lda * sizeof(T), bytes_b = (size_t)K * ldb * sizeof(T), bytes_d = (size_t)M * ldd * sizeof(T);
+    struct Set { T *a = nullptr, *b = nullptr, *d = nullptr; hipEvent_t up = nullptr, done = nullptr, down = nullptr; } set[2];
+    hipStream_t s_up = nullptr, s_down = nullptr;
+    int rc = 0;
+    auto cleanup = [&] {
+        (void)hipDeviceSynchronize();
+        for (Set& s : set) {
+            if (s.a) (void)hipFree(s.a);
+            if (s.b) (void)hipFree(s.b);
+            if (s.d) (void)hipFree(s.d);
+            if (s.up) (void)hipEventDestroy(s.up);
+            if (s.done) (void)hipEventDestroy(s.done);
+            if (s.down) (void)hipEventDestroy(s.down);
+        }
+        if (s_up) (void)hipStreamDestroy(s_up);
+        if (s_down) (void)hipStreamDestroy(s_down);
+    };
+#define PIPE_TRY(expr)                                   \
+    do {                                                 \
+        hipError_t e_ = (expr);                          \
+        if (e_ != hipSuccess) { rc = hip_fail(e_, #expr); cleanup(); return rc; } \
+    } while (0)
+    for (Set& s : set) {
+        if (hipMalloc(&s.a, bytes_a) != hipSuccess || hipMalloc(&s.b, bytes_b) != hipSuccess || hipMalloc(&s.d, bytes_d) != hipSuccess) {
+            (void)hipGetLastError();
+            cleanup();
+            return fail(DECX_HIP_FAIL_ALLOCATION, "Fail to allocate memory\n");
+        }
+        PIPE_TRY(hipEventCreateWithFlags(&s.up, hipEventDisableTiming));
+        PIPE_TRY(hipEventCreateWithFlags(&s.done, hipEventDisableTiming));
+        PIPE_TRY(hipEventCreateWithFlags(&s.down, hipEventDisableTiming));
+    }
+    PIPE_TRY(hipStreamCreateWithFlags(&s_up, hipStreamNonBlocking));
+    PIPE_TRY(hipStreamCreateWithFlags(&s_down, hipStreamNonBlocking));
+    auto upload = [&](int i) -> hipError_t {
+        Set& s = set[i & 1];
+        hipError_t e;
+        if (i >= 2 && (e = hipStreamWaitEvent(s_up, s.done, 0)) != hipSuccess) return e;    // kernel i-2 has read a, b
+        if (hC && i >= 2 && (e = hipStreamWaitEvent(s_up, s.down, 0)) != hipSuccess) return e;   // and d was drained
+        if ((e = hipMemcpyAsync(s.a, hA + (size_t)i * plane_a, bytes_a, hipMemcpyHostToDevice, s_up)) != hipSuccess) return e;
+        if ((e = hipMemcpyAsync(s.b, hB + (size_t)i * plane_b, bytes_b, hipMemcpyHostToDevice, s_up)) != hipSuccess) return e;
+        if (hC && (e = hipMemcpy2DAsync(s.d, (size_t)ldd * sizeof(T), hC + (size_t)i * plane_c, (size_t)ldc * sizeof(T),
+                                        (size_t)N * sizeof(T), M, hipMemcpyHostToDevice, s_up)) != hipSuccess) return e;
+        return hipEventRecord(s.up, s_up);
+    };
+    PIPE_TRY(upload(0));
+    for (int i = 0; i < count; ++i) {
+        Set& s = set[i & 1];
+        if (i + 1 < count) PIPE_TRY(upload(i + 1));
+        PIPE_TRY(hipStreamWaitEvent(g_rt.stream, s.up, 0));
+        if (i >= 2) PIPE_TRY(hipStreamWaitEvent(g_rt.stream, s.down, 0));                   // result i-2 has left d
+        Batch one;
+        one.stream = g_rt.stream;
+        rc = enqueue(s.a, s.b, hC ? s.d : nullptr, s.d, one);
+        if (rc) { cleanup(); return rc; }
+        PIPE_TRY(hipEventRecord(s.done, g_rt.stream));
+        PIPE_TRY(hipStreamWaitEvent(s_down, s.done, 0));
+        PIPE_TRY(hipMemcpy2DAsync(hD + (size_t)i * plane_d, (size_t)ldd * sizeof(T), s.d, (size_t)ldd * sizeof(T),
+                                  (size_t)N * sizeof(T), M, hipMemcpyDeviceToHost, s_down));
+        PIPE_TRY(hipEventRecord(s.down, s_down));
+    }
+    PIPE_TRY(hipStreamSynchronize(s_down));
+    PIPE_TRY(hipStreamSynchronize(g_rt.stream));
+#undef PIPE_TRY
+    cleanup();
+    return 0;
 }
 
 // Plain streaming copy, 16 bytes per lane and iteration: the known-size kernel that hardware traffic counters
@@ -387,20 +500,49 @@ int decx_hip_sync(void) {
 
 int decx_hip_sgemm_async(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd,
                          int M, int N, int K) {
-    return sgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
+    return sgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, single_on_library_stream());
 }
 int decx_hip_sgemm(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
                    int N, int K) {
-    return finish(sgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K));
+    return finish(sgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, single_on_library_stream()));
+}
+int decx_hip_sgemm_batched(const float* A, int lda, size_t stride_a, const float* B, int ldb, size_t stride_b,
+                           const float* Cin, int ldc, size_t stride_c, float* D, int ldd, size_t stride_d, int M, int N, int K,
+                           int batch) {
+    return finish(sgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K,
+                                batch_on_library_stream(batch, stride_a, stride_b, stride_c, stride_d)));
 }
 
 int decx_hip_hgemm_f32acc_async(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
                                 uint16_t* D, int ldd, int M, int N, int K) {
-    return hgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K);
+    return hgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, single_on_library_stream());
 }
 int decx_hip_hgemm_f32acc(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                           int ldd, int M, int N, int K) {
-    return finish(hgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K));
+    return finish(hgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, single_on_library_stream()));
+}
+int decx_hip_hgemm_f32acc_batched(const uint16_t* A, int lda, size_t stride_a, const uint16_t* B, int ldb, size_t stride_b,
+                                  const uint16_t* Cin, int ldc, size_t stride_c, uint16_t* D, int ldd, size_t stride_d, int M,
+                                  int N, int K, int batch) {
+    return finish(hgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K,
+                                batch_on_library_stream(batch, stride_a, stride_b, stride_c, stride_d)));
+}
+
+int decx_hip_gemm3_host_f32(const float* hA, int lda, size_t plane_a, const float* hB, int ldb, size_t plane_b,
+                            const float* hC, int ldc, size_t plane_c, float* hD, int ldd, size_t plane_d, int M, int N, int K,
+                            int count) {
+    return gemm3_host_pipeline<float>(hA, lda, plane_a, hB, ldb, plane_b, hC, ldc, plane_c, hD, ldd, plane_d, M, N, K, count,
+                                      [&](const float* a, const float* b, const float* c, float* d, const Batch& one) {
+                                          return sgemm_enqueue(a, lda, b, ldb, c, ldd, d, ldd, M, N, K, one);
+                                      });
+}
+int decx_hip_gemm3_host_f16(const uint16_t* hA, int lda, size_t plane_a, const uint16_t* hB, int ldb, size_t plane_b,
+                            const uint16_t* hC, int ldc, size_t plane_c, uint16_t* hD, int ldd, size_t plane_d, int M, int N,
+                            int K, int count) {
+    return gemm3_host_pipeline<uint16_t>(hA, lda, plane_a, hB, ldb, plane_b, hC, ldc, plane_c, hD, ldd, plane_d, M, N, K, count,
+                                         [&](const uint16_t* a, const uint16_t* b, const uint16_t* c, uint16_t* d, const Batch& one) {
+                                             return hgemm_enqueue(a, lda, b, ldb, c, ldd, d, ldd, M, N, K, one);
+                                         });
 }
 
 int decx_hip_conv2_im2col_f32_async(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt,

@@ -54,9 +54,15 @@ template <class S, bool HAS_C>
 __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __restrict__ A, int lda,
                                                           const _Float16* __restrict__ B, int ldb, const _Float16* Cin,
                                                           int ldc, _Float16* D, int ldd, int M, int N, int K, int tiles_m,
-                                                          int tiles_n, int group_m) {
+                                                          int tiles_n, int group_m, size_t a_batch_stride,
+                                                          size_t b_batch_stride, size_t c_batch_stride, size_t d_batch_stride) {
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, NT = S::NT, UA = S::UA, UB = S::UB, MI = S::MI, NI = S::NI;
     constexpr int STAGES = S::STAGES;
+    // blockIdx.y walks a batch of independent problems of the same shape
+    A += (size_t)blockIdx.y * a_batch_stride;
+    B += (size_t)blockIdx.y * b_batch_stride;
+    if (HAS_C) Cin += (size_t)blockIdx.y * c_batch_stride;
+    D += (size_t)blockIdx.y * d_batch_stride;
     constexpr int KS = BK / 16;                                // MFMA k-blocks per K step
     constexpr int BLK = MI * NI;                               // MFMAs per k-block
     static_assert(KS >= 2, "the schedule below needs at least two k-blocks per K step");

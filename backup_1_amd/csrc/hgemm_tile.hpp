@@ -42,7 +42,13 @@ template <class S, bool VEC>
 __global__ __launch_bounds__(S::NT) void hgemm_tile_kernel(const _Float16* __restrict__ A, int lda,
                                                            const _Float16* __restrict__ B, int ldb, const _Float16* Cin,
                                                            int ldc, _Float16* D, int ldd, int M, int N, int K,
-                                                           int tiles_m, int tiles_n, int group_m) {
+                                                           int tiles_m, int tiles_n, int group_m, size_t a_batch_stride,
+                                                           size_t b_batch_stride, size_t c_batch_stride, size_t d_batch_stride) {
+    // blockIdx.y walks a batch of independent problems of the same shape
+    A += (size_t)blockIdx.y * a_batch_stride;
+    B += (size_t)blockIdx.y * b_batch_stride;
+    if (Cin != nullptr) Cin += (size_t)blockIdx.y * c_batch_stride;
+    D += (size_t)blockIdx.y * d_batch_stride;
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, NT = S::NT, UA = S::UA, UB = S::UB, MI = S::MI, NI = S::NI;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     u32x4* As = reinterpret_cast<u32x4*>(lds_raw);            // [2][A_UNITS]

@@ -70,6 +70,8 @@ template <bool VEC>
 struct DenseA {
     const float* A;
     int lda, M, K;
+    size_t batch_stride;      // elements between consecutive matrices of a batch (blockIdx.y walks the batch)
+    __device__ __forceinline__ void select_batch(int b) { A += (size_t)b * batch_stride; }
     struct RowState {
         const float* row;
     };
@@ -113,6 +115,7 @@ struct Im2colA {
     const float* src;
     int H, W, dpitch, kh, kw, oy, ox, Wout, Mtot, K;
     size_t row_stride;
+    __device__ __forceinline__ void select_batch(int) {}
     struct RowState {
         int y, x;          // output pixel shifted by (-oy, -ox): the image position of tap (0, 0)
         long base;         // y*row_stride + x*dpitch (may be negative: it is only used together with an in-image tap)
@@ -172,6 +175,8 @@ template <bool VEC>
 struct DenseB {
     const float* B;
     int ldb, N, K;
+    size_t batch_stride;
+    __device__ __forceinline__ void select_batch(int b) { B += (size_t)b * batch_stride; }
     template <class S>
     static constexpr int tasks() { return S::KQ * (S::BN / 4); }
     template <class S>
@@ -238,6 +243,7 @@ struct FilterB {
     const float* filt;
     int N, K, dpitch, kw;
     size_t filt_stride, filt_row_stride;
+    __device__ __forceinline__ void select_batch(int) {}
     template <class S>
     static constexpr int quads() { return S::KQ * S::BN / S::NT; }
     typedef TapWalk KState;       // every quad of a thread has the same k-quad index q = tid % KQ (NT is a multiple of KQ)
@@ -297,7 +303,12 @@ struct SgemmShape {
 template <class S, class ASrc, class BSrc, class Out, bool HAS_C>
 __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(ASrc a_src, BSrc b_src, const float* Cin, int ldc, float* D,
                                                            Out out, int M, int N, int K, int tiles_m, int tiles_n,
-                                                           int group_m) {
+                                                           int group_m, size_t c_batch_stride, size_t d_batch_stride) {
+    // blockIdx.y walks a batch of independent problems of the same shape
+    a_src.select_batch(blockIdx.y);
+    b_src.select_batch(blockIdx.y);
+    if (HAS_C) Cin += (size_t)blockIdx.y * c_batch_stride;
+    D += (size_t)blockIdx.y * d_batch_stride;
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, NT = S::NT, KQ = S::KQ, MI = S::MI, NI = S::NI;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     f32x4* As = reinterpret_cast<f32x4*>(lds_raw);                       // [2][KQ][A_ROW]

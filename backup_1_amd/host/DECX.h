@@ -119,6 +119,20 @@ public:
     virtual ~TensorArray() {}
 };
 
+// classes/MatrixArray.h:28-52.  MatrixNum equally sized host matrices back to back (pitch*height elements apart).
+template <typename T>
+class MatrixArray {
+public:
+    MatrixArray() {}
+    virtual uint Width() = 0;
+    virtual uint Height() = 0;
+    virtual uint MatrixNumber() = 0;
+    virtual T& index(uint row, uint col, size_t seq) = 0;
+    virtual MatrixArray<T>& operator=(MatrixArray<T>& src) = 0;
+    virtual void release() = 0;
+    virtual ~MatrixArray() {}
+};
+
 // classes/GPU_Tensor.h:19-47.  Device-resident tensor with the host Tensor's layout (dpitch = ceil4(depth),
 // wpitch = ceil4(width)).
 template <typename T>
@@ -170,6 +184,12 @@ template <typename T> TensorArray<T>* CreateTensorArrayPtr();
 template <typename T> TensorArray<T>& CreateTensorArrayRef(const uint width, const uint height, const uint depth, const uint tensor_num, const int flag);
 template <typename T> TensorArray<T>* CreateTensorArrayPtr(const uint width, const uint height, const uint depth, const uint tensor_num, const int flag);
 
+// classes/MatrixArray.h:377-389; instantiated for float and de::Half
+template <typename T> MatrixArray<T>& CreateMatrixArrayRef();
+template <typename T> MatrixArray<T>* CreateMatrixArrayPtr();
+template <typename T> MatrixArray<T>& CreateMatrixArrayRef(uint width, uint height, uint MatrixNum, const int flag);
+template <typename T> MatrixArray<T>* CreateMatrixArrayPtr(uint width, uint height, uint MatrixNum, const int flag);
+
 // classes/GPU_Tensor.h:385-397, GPU_TensorArray.h (same pattern); instantiated for float
 template <typename T> GPU_Tensor<T>& CreateGPUTensorRef();
 template <typename T> GPU_Tensor<T>* CreateGPUTensorPtr();
@@ -195,6 +215,12 @@ DH GEMM(GPU_Matrix<float>& A, GPU_Matrix<float>& B, GPU_Matrix<float>& dst);
 DH GEMM(GPU_Matrix<float>& A, GPU_Matrix<float>& B, GPU_Matrix<float>& C, GPU_Matrix<float>& dst);
 DH GEMM(GPU_Matrix<Half>& A, GPU_Matrix<Half>& B, GPU_Matrix<Half>& dst);
 DH GEMM(GPU_Matrix<Half>& A, GPU_Matrix<Half>& B, GPU_Matrix<Half>& C, GPU_Matrix<Half>& dst);
+// GEMM/CUDA/large_squares/GEMM3.h:27-36.  dst[i] = A[i] * B[i] (+ C[i]) for every matrix of the arrays, uploads and
+// downloads overlapped with the kernels.
+DH GEMM3(MatrixArray<float>& A, MatrixArray<float>& B, MatrixArray<float>& dst);
+DH GEMM3(MatrixArray<Half>& A, MatrixArray<Half>& B, MatrixArray<Half>& dst);
+DH GEMM3(MatrixArray<float>& A, MatrixArray<float>& B, MatrixArray<float>& C, MatrixArray<float>& dst);
+DH GEMM3(MatrixArray<Half>& A, MatrixArray<Half>& B, MatrixArray<Half>& C, MatrixArray<Half>& dst);
 // convolution/CUDA/im2col/conv2_mk_im2col.h:25.  flag: decx::conv_property.
 DH Conv2_MK_im2col(Tensor<float>& src, TensorArray<float>& kernel, Tensor<float>& dst, const int flag);
 // Device-resident flavour of the same convolution (the reference only has the host one; its GPU_Tensor /

@@ -105,6 +105,42 @@ de::DH gemm_device(de::GPU_Matrix<T>& A_, de::GPU_Matrix<T>& B_, de::GPU_Matrix<
                                         (int)B->width, (int)A->width));
 }
 
+template <typename T> struct Gemm3Call;
+template <> struct Gemm3Call<float> {
+    static int run(const float* A, int lda, size_t pa, const float* B, int ldb, size_t pb, const float* C, int ldc, size_t pc,
+                   float* D, int ldd, size_t pd, int M, int N, int K, int n) {
+        return decx_hip_gemm3_host_f32(A, lda, pa, B, ldb, pb, C, ldc, pc, D, ldd, pd, M, N, K, n);
+    }
+};
+template <> struct Gemm3Call<de::Half> {
+    static int run(const de::Half* A, int lda, size_t pa, const de::Half* B, int ldb, size_t pb, const de::Half* C, int ldc,
+                   size_t pc, de::Half* D, int ldd, size_t pd, int M, int N, int K, int n) {
+        return decx_hip_gemm3_host_f16(reinterpret_cast<const uint16_t*>(A), lda, pa, reinterpret_cast<const uint16_t*>(B), ldb, pb,
+                                       reinterpret_cast<const uint16_t*>(C), ldc, pc, reinterpret_cast<uint16_t*>(D), ldd, pd, M,
+                                       N, K, n);
+    }
+};
+
+template <typename T>
+de::DH gemm3_host(de::MatrixArray<T>& A_, de::MatrixArray<T>& B_, de::MatrixArray<T>* C_, de::MatrixArray<T>& dst_) {
+    auto* A = dynamic_cast<decx::_MatrixArray<T>*>(&A_);
+    auto* B = dynamic_cast<decx::_MatrixArray<T>*>(&B_);
+    auto* C = C_ ? dynamic_cast<decx::_MatrixArray<T>*>(C_) : nullptr;
+    auto* dst = dynamic_cast<decx::_MatrixArray<T>*>(&dst_);
+    if (!A || !B || !dst || (C_ && !C)) return de::DH{decx::DECX_FAIL_ErrorParams, kNotFactory};
+    if (!decx_hip_is_init()) return not_init();                                           // GEMM3.h:42-46
+    if (A->width != B->height) return de::DH{decx::DECX_FAIL_DimsNotMatching, kGemmDims};
+    static char num_msg[] = "The number of matrices don't match each other";             // core/error.h Matrix_number_not_matching
+    if (A->ArrayNumber != B->ArrayNumber || (C && C->ArrayNumber != A->ArrayNumber))
+        return de::DH{decx::DECX_FAIL_MNumNotMatching, num_msg};
+    if (C && (C->width != B->width || C->height != A->height)) return de::DH{decx::DECX_FAIL_DimsNotMatching, kMDims};
+    if (C != dst && !dst->re_construct(B->width, A->height, (uint)A->ArrayNumber, decx::Page_Locked)) return alloc_fail();
+    return from_status(Gemm3Call<T>::run(A->MatArr.ptr, (int)A->pitch, A->_plane, B->MatArr.ptr, (int)B->pitch, B->_plane,
+                                         C ? C->MatArr.ptr : nullptr, C ? (int)C->pitch : 0, C ? C->_plane : 0, dst->MatArr.ptr,
+                                         (int)dst->pitch, dst->_plane, (int)A->height, (int)B->width, (int)A->width,
+                                         (int)A->ArrayNumber));
+}
+
 }  // namespace
 
 namespace de {
@@ -176,6 +212,18 @@ template <typename T> GPU_TensorArray<T>& CreateGPUTensorArrayRef() { return *(n
 template <typename T> GPU_TensorArray<T>* CreateGPUTensorArrayPtr() { return new decx::_GPU_TensorArray<T>(); }
 template <typename T> GPU_TensorArray<T>& CreateGPUTensorArrayRef(const uint w, const uint h, const uint d, const uint n) { return *(new decx::_GPU_TensorArray<T>(w, h, d, n)); }
 template <typename T> GPU_TensorArray<T>* CreateGPUTensorArrayPtr(const uint w, const uint h, const uint d, const uint n) { return new decx::_GPU_TensorArray<T>(w, h, d, n); }
+template <typename T> MatrixArray<T>& CreateMatrixArrayRef() { return *(new decx::_MatrixArray<T>()); }
+template <typename T> MatrixArray<T>* CreateMatrixArrayPtr() { return new decx::_MatrixArray<T>(); }
+template <typename T> MatrixArray<T>& CreateMatrixArrayRef(uint w, uint h, uint n, const int f) { return *(new decx::_MatrixArray<T>(w, h, n, f)); }
+template <typename T> MatrixArray<T>* CreateMatrixArrayPtr(uint w, uint h, uint n, const int f) { return new decx::_MatrixArray<T>(w, h, n, f); }
+template MatrixArray<float>& CreateMatrixArrayRef<float>();
+template MatrixArray<float>* CreateMatrixArrayPtr<float>();
+template MatrixArray<float>& CreateMatrixArrayRef<float>(uint, uint, uint, const int);
+template MatrixArray<float>* CreateMatrixArrayPtr<float>(uint, uint, uint, const int);
+template MatrixArray<Half>& CreateMatrixArrayRef<Half>();
+template MatrixArray<Half>* CreateMatrixArrayPtr<Half>();
+template MatrixArray<Half>& CreateMatrixArrayRef<Half>(uint, uint, uint, const int);
+template MatrixArray<Half>* CreateMatrixArrayPtr<Half>(uint, uint, uint, const int);
 template GPU_Tensor<float>& CreateGPUTensorRef<float>();
 template GPU_Tensor<float>* CreateGPUTensorPtr<float>();
 template GPU_Tensor<float>& CreateGPUTensorRef<float>(const uint, const uint, const uint);
@@ -215,6 +263,11 @@ DH GEMM(GPU_Matrix<float>& A, GPU_Matrix<float>& B, GPU_Matrix<float>& dst) { re
 DH GEMM(GPU_Matrix<float>& A, GPU_Matrix<float>& B, GPU_Matrix<float>& C, GPU_Matrix<float>& dst) { return gemm_device<float>(A, B, &C, dst); }
 DH GEMM(GPU_Matrix<Half>& A, GPU_Matrix<Half>& B, GPU_Matrix<Half>& dst) { return gemm_device<Half>(A, B, nullptr, dst); }
 DH GEMM(GPU_Matrix<Half>& A, GPU_Matrix<Half>& B, GPU_Matrix<Half>& C, GPU_Matrix<Half>& dst) { return gemm_device<Half>(A, B, &C, dst); }
+
+DH GEMM3(MatrixArray<float>& A, MatrixArray<float>& B, MatrixArray<float>& dst) { return gemm3_host<float>(A, B, nullptr, dst); }
+DH GEMM3(MatrixArray<Half>& A, MatrixArray<Half>& B, MatrixArray<Half>& dst) { return gemm3_host<Half>(A, B, nullptr, dst); }
+DH GEMM3(MatrixArray<float>& A, MatrixArray<float>& B, MatrixArray<float>& C, MatrixArray<float>& dst) { return gemm3_host<float>(A, B, &C, dst); }
+DH GEMM3(MatrixArray<Half>& A, MatrixArray<Half>& B, MatrixArray<Half>& C, MatrixArray<Half>& dst) { return gemm3_host<Half>(A, B, &C, dst); }
 
 // ---- convolution ----------------------------------------------------------------------------------------------
 DH Conv2_MK_im2col(Tensor<float>& src_, TensorArray<float>& kernel_, Tensor<float>& dst_, const int flag) {

@@ -285,6 +285,61 @@ public:
     ~_TensorArray() override { release(); }
 };
 
+// classes/MatrixArray.h:222-239 (attributes), :367-370 (index)
+template <typename T>
+class _MatrixArray : public de::MatrixArray<T> {
+    HostBlock block_;
+
+public:
+    int _store_type = Page_Default;
+    PtrInfo<T> MatArr;
+    uint width = 0, height = 0, pitch = 0;
+    size_t element_num = 0, _element_num = 0, total_bytes = 0, ArrayNumber = 0;
+    size_t plane = 0, _plane = 0;                // true / padded elements per matrix
+
+    _MatrixArray() {}
+    _MatrixArray(uint w, uint h, uint n, int flag) { construct(w, h, n, flag); }
+    void attribute_assign(uint w, uint h, uint n, int flag) {
+        width = w;
+        height = h;
+        ArrayNumber = n;
+        _store_type = flag;
+        pitch = ceil_to(w, matrix_align<T>());
+        plane = (size_t)w * h;
+        _plane = (size_t)pitch * h;
+        element_num = plane * n;
+        _element_num = _plane * n;
+        total_bytes = _element_num * sizeof(T);
+    }
+    bool construct(uint w, uint h, uint n, int flag) {
+        attribute_assign(w, h, n, flag);
+        bool ok = block_.alloc(total_bytes, flag);
+        MatArr.ptr = static_cast<T*>(block_.ptr);
+        return ok;
+    }
+    bool re_construct(uint w, uint h, uint n, int flag) {
+        if (MatArr.ptr && w == width && h == height && n == ArrayNumber && flag == _store_type) return true;
+        return construct(w, h, n, flag);
+    }
+    uint Width() override { return width; }
+    uint Height() override { return height; }
+    uint MatrixNumber() override { return (uint)ArrayNumber; }
+    T& index(uint row, uint col, size_t seq) override { return MatArr.ptr[seq * _plane + (size_t)row * pitch + col]; }
+    de::MatrixArray<T>& operator=(de::MatrixArray<T>& src) override {
+        _MatrixArray<T>& s = dynamic_cast<_MatrixArray<T>&>(src);
+        if (&s != this) {
+            construct(s.width, s.height, (uint)s.ArrayNumber, s._store_type);
+            std::memcpy(MatArr.ptr, s.MatArr.ptr, total_bytes);
+        }
+        return *this;
+    }
+    void release() override {
+        block_.free();
+        MatArr.ptr = nullptr;
+    }
+    ~_MatrixArray() override { release(); }
+};
+
 template <typename T>
 class _GPU_Tensor : public de::GPU_Tensor<T> {
 public:

@@ -92,6 +92,29 @@ int decx_hip_hgemm_f32acc(const uint16_t* A, int lda, const uint16_t* B, int ldb
 int decx_hip_hgemm_f32acc_async(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
                                 uint16_t* D, int ldd, int M, int N, int K);
 
+/* Batched GEMM on device-resident data: `batch` independent problems of one shape in ONE launch; problem b uses
+ * A + b*stride_a, B + b*stride_b, Cin + b*stride_c (Cin nullable), D + b*stride_d (strides in elements).  This is the
+ * kernel step of de::cuda::GEMM3 over a MatrixArray (GEMM/CUDA/large_squares/GEMM3.h:27-36), whose matrices lie
+ * `_plane` = pitch*height elements apart (classes/MatrixArray.h:222-239), without its one-launch-per-matrix loop. */
+int decx_hip_sgemm_batched(const float* A, int lda, size_t stride_a, const float* B, int ldb, size_t stride_b,
+                           const float* Cin, int ldc, size_t stride_c, float* D, int ldd, size_t stride_d, int M, int N, int K,
+                           int batch);
+int decx_hip_hgemm_f32acc_batched(const uint16_t* A, int lda, size_t stride_a, const uint16_t* B, int ldb, size_t stride_b,
+                                  const uint16_t* Cin, int ldc, size_t stride_c, uint16_t* D, int ldd, size_t stride_d, int M,
+                                  int N, int K, int batch);
+
+/* de::cuda::GEMM3(MatrixArray<T>& A, B, [C,] dst) on HOST-resident arrays (GEMM3.h:40-300): the reference's pipeline of
+ * GEMM3_macros.h:140-374 -- upload of matrix i+1, kernel on matrix i and download of result i-1 overlap on three
+ * streams with two device buffer sets.  hA, hB, hC (nullable), hD are HOST pointers (pinned memory overlaps best);
+ * matrix i of an array starts plane_x elements after matrix i-1.  Device copies keep the host pitches (the reference
+ * pads them to 128/16 multiples, GEMM3.h:58-60). */
+int decx_hip_gemm3_host_f32(const float* hA, int lda, size_t plane_a, const float* hB, int ldb, size_t plane_b,
+                            const float* hC, int ldc, size_t plane_c, float* hD, int ldd, size_t plane_d, int M, int N, int K,
+                            int count);
+int decx_hip_gemm3_host_f16(const uint16_t* hA, int lda, size_t plane_a, const uint16_t* hB, int ldb, size_t plane_b,
+                            const uint16_t* hC, int ldc, size_t plane_c, uint16_t* hD, int ldd, size_t plane_d, int M, int N,
+                            int K, int count);
+
 /* de::cuda::Conv2_MK_im2col(Tensor<float>& src, TensorArray<float>& kernel, Tensor<float>& dst, int flag)
  * (convolution/CUDA/im2col/conv2_mk_im2col.h:25, :278-306): the device part, i.e. what cu_sIm2Col_r8_within
  * (im2col.cuh:86-178) followed by cu_conv_eq_mm (eq_GEMM.cuh:109-209) produce.  The patch matrix is never built:

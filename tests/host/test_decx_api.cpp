@@ -265,6 +265,55 @@ static void conv_case(int H, int W, int C, int N, int kh, int kw, int flag) {
     CHECK(same);
     src.release(); ker.release(); dst.release();
 }
+static void gemm3_matrix_arrays() {
+    const int M = 150, K = 90, N = 210, NUM = 5;
+    de::MatrixArray<float>& A = de::CreateMatrixArrayRef<float>(K, M, NUM, 0);
+    de::MatrixArray<float>& B = de::CreateMatrixArrayRef<float>(N, K, NUM, 0);
+    de::MatrixArray<float>& C = de::CreateMatrixArrayRef<float>(N, M, NUM, 0);
+    de::MatrixArray<float>& D = de::CreateMatrixArrayRef<float>();
+    CHECK(A.MatrixNumber() == (uint)NUM && (&A.index(0, 0, 1)) - (&A.index(0, 0, 0)) == 96 * M);   // pitch = ceil8(90) = 96
+    for (int s = 0; s < NUM; ++s) {
+        for (int i = 0; i < M; ++i) for (int j = 0; j < K; ++j) A.index(i, j, s) = small_int();
+        for (int i = 0; i < K; ++i) for (int j = 0; j < N; ++j) B.index(i, j, s) = small_int();
+        for (int i = 0; i < M; ++i) for (int j = 0; j < N; ++j) C.index(i, j, s) = small_int();
+    }
+    auto check = [&](de::MatrixArray<float>& R, bool with_c) {
+        bool same = R.Width() == (uint)N && R.Height() == (uint)M && R.MatrixNumber() == (uint)NUM;
+        for (int s = 0; s < NUM && same; ++s) {
+            std::vector<float> a((size_t)M * K), b((size_t)K * N), c((size_t)M * N), d((size_t)M * N);
+            for (int i = 0; i < M; ++i) for (int j = 0; j < K; ++j) a[(size_t)i * K + j] = A.index(i, j, s);
+            for (int i = 0; i < K; ++i) for (int j = 0; j < N; ++j) b[(size_t)i * N + j] = B.index(i, j, s);
+            for (int i = 0; i < M; ++i) for (int j = 0; j < N; ++j) c[(size_t)i * N + j] = C.index(i, j, s);
+            oracle_sgemm_chain_fast(a.data(), K, b.data(), N, with_c ? c.data() : nullptr, N, d.data(), N, M, N, K, 0);
+            for (int i = 0; i < M; ++i) for (int j = 0; j < N; ++j) same = same && R.index(i, j, s) == d[(size_t)i * N + j];
+        }
+        return same;
+    };
+    CHECK(de::cuda::GEMM3(A, B, D).error_type == decx::DECX_SUCCESS);
+    CHECK(check(D, false));                                          // integer data: exact, every matrix of the array
+    CHECK(de::cuda::GEMM3(A, B, C, D).error_type == decx::DECX_SUCCESS);
+    CHECK(check(D, true));
+    de::MatrixArray<float>& B4 = de::CreateMatrixArrayRef<float>(N, K, NUM - 1, 0);
+    CHECK(de::cuda::GEMM3(A, B4, D).error_type == decx::DECX_FAIL_MNumNotMatching);
+    // fp16 arrays against the fp64 product
+    de::MatrixArray<de::Half>& Ah = de::CreateMatrixArrayRef<de::Half>(K, M, 3, 0);
+    de::MatrixArray<de::Half>& Bh = de::CreateMatrixArrayRef<de::Half>(N, K, 3, 0);
+    de::MatrixArray<de::Half>& Dh = de::CreateMatrixArrayRef<de::Half>();
+    for (int s = 0; s < 3; ++s) {
+        for (int i = 0; i < M; ++i) for (int j = 0; j < K; ++j) Ah.index(i, j, s) = de::Float2Half(unif());
+        for (int i = 0; i < K; ++i) for (int j = 0; j < N; ++j) Bh.index(i, j, s) = de::Float2Half(unif());
+    }
+    CHECK(de::cuda::GEMM3(Ah, Bh, Dh).error_type == decx::DECX_SUCCESS);
+    double worst = 0;
+    for (int s = 0; s < 3; ++s)
+        for (int i = 0; i < M; i += 7) for (int j = 0; j < N; ++j) {
+            double r = 0, sc = 0;
+            for (int k = 0; k < K; ++k) { double x = de::Half2Float(Ah.index(i, k, s)), y = de::Half2Float(Bh.index(k, j, s)); r += x * y; sc += std::fabs(x * y); }
+            worst = std::fmax(worst, std::fabs(de::Half2Float(Dh.index(i, j, s)) - r) / sc);
+        }
+    CHECK(worst < 2e-3);
+}
+
 static void conv_device_resident() {
     const int H = 30, W = 26, C = 12, N = 10, kh = 3, kw = 3;        // width not a multiple of 4: padded rows in dst
     de::Tensor<float>& src = de::CreateTensorRef<float>(W, H, C, 0);
@@ -320,6 +369,7 @@ int main(int argc, char** argv) {
         RUN(gemm_fp16_flavours);
         RUN(conv_flavours_and_flags);
         RUN(conv_device_resident);
+        RUN(gemm3_matrix_arrays);
     }
     std::printf("%s: %d failure(s)\n", mode.c_str(), g_fail);
     return g_fail ? 1 : 0;

@@ -104,3 +104,21 @@ def test_config5_8192_cube_sampled_rows(gpu, oracle):
     assert np.max(np.abs(goti)) <= 2048
     assert np.array_equal(goti.sum(axis=1), Ai.astype(np.float64) @ Bi.astype(np.float64).sum(axis=1))
     assert np.array_equal(goti.sum(axis=0), Ai.astype(np.float64).sum(axis=0) @ Bi.astype(np.float64))
+
+
+@pytest.mark.parametrize("variant", [0, 2, 4])
+def test_batched_hgemm_one_launch(gpu, variant):
+    batch, M, K, N = 3, 256, 128, 512
+    A = workloads.small_ints((batch, M, K), 91, -3, 3)
+    B = workloads.small_ints((batch, K, N), 92, -3, 3)
+    dA, dB = gpu.DeviceBuffer.from_numpy(to_bits(A)), gpu.DeviceBuffer.from_numpy(to_bits(B))
+    dD = gpu.DeviceBuffer(batch * M * N * 2)
+    L = gpu.lib()
+    prev = L.decx_hip_set_hgemm_variant(variant)
+    try:
+        gpu.check(L.decx_hip_hgemm_f32acc_batched(dA.ptr, K, M * K, dB.ptr, N, K * N, None, 0, 0, dD.ptr, N, M * N, M, N, K, batch))
+    finally:
+        L.decx_hip_set_hgemm_variant(prev)
+    got = dD.download((batch, M, N), np.uint16)
+    want = np.einsum("bik,bkj->bij", A.astype(np.float64), B.astype(np.float64)).astype(np.float16).view(np.uint16)
+    assert np.array_equal(got, want)

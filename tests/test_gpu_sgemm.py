@@ -129,3 +129,48 @@ def test_bad_arguments_are_reported_not_executed(gpu):
     assert L.decx_hip_sgemm(buf.ptr, 4, buf.ptr, 8, None, 0, buf.ptr, 8, 8, 8, 8) == 0x0d       # lda < K
     assert L.decx_hip_sgemm(None, 8, buf.ptr, 8, None, 0, buf.ptr, 8, 8, 8, 8) == 0x0d
     assert gpu.last_error().strip() != ""
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2])
+def test_batched_gemm_one_launch(gpu, variant):
+    # decx_hip_sgemm_batched: every problem of the batch against the exact integer product, with and without C
+    batch, M, K, N = 5, 130, 70, 200
+    A = workloads.small_ints((batch, M, K), 71)
+    B = workloads.small_ints((batch, K, N), 72)
+    C = workloads.small_ints((batch, M, N), 73, -50, 50)
+    pad = lambda x: (x + 7) // 8 * 8
+    lda, ldb, ldd = pad(K), pad(N), pad(N)
+    Ab = np.full((batch, M, lda), np.nan, np.float32); Ab[:, :, :K] = A
+    Bb = np.full((batch, K, ldb), np.nan, np.float32); Bb[:, :, :N] = B
+    Cb = np.full((batch, M, ldd), np.nan, np.float32); Cb[:, :, :N] = C
+    dA, dB, dC = (gpu.DeviceBuffer.from_numpy(x) for x in (Ab, Bb, Cb))
+    dD = gpu.DeviceBuffer.from_numpy(np.full((batch, M, ldd), -5.0, np.float32))
+    L = gpu.lib()
+    prev = L.decx_hip_set_sgemm_variant(variant)
+    try:
+        gpu.check(L.decx_hip_sgemm_batched(dA.ptr, lda, M * lda, dB.ptr, ldb, K * ldb, None, 0, 0, dD.ptr, ldd, M * ldd, M, N, K, batch))
+        got = dD.download((batch, M, ldd), np.float32)
+        want = np.einsum("bik,bkj->bij", A.astype(np.float64), B.astype(np.float64))
+        assert np.array_equal(got[:, :, :N], want.astype(np.float32)) and np.all(got[:, :, N:] == -5.0)
+        gpu.check(L.decx_hip_sgemm_batched(dA.ptr, lda, M * lda, dB.ptr, ldb, K * ldb, dC.ptr, ldd, M * ldd, dD.ptr, ldd, M * ldd, M, N, K, batch))
+        got = dD.download((batch, M, ldd), np.float32)
+        assert np.array_equal(got[:, :, :N], (want + C).astype(np.float32))
+    finally:
+        L.decx_hip_set_sgemm_variant(prev)
+    assert L.decx_hip_sgemm_batched(dA.ptr, lda, 10, dB.ptr, ldb, K * ldb, None, 0, 0, dD.ptr, ldd, M * ldd, M, N, K, batch) == 0x0d
+
+
+def test_gemm3_host_pipeline(gpu):
+    # decx_hip_gemm3_host_f32: host arrays in, host arrays out, through the three-stream pipeline
+    count, M, K, N = 7, 96, 40, 120
+    A = workloads.small_ints((count, M, K), 81)
+    B = workloads.small_ints((count, K, N), 82)
+    C = workloads.small_ints((count, M, N), 83, -50, 50)
+    D = np.zeros((count, M, N), np.float32)
+    L = gpu.lib()
+    p = lambda a: a.ctypes.data
+    gpu.check(L.decx_hip_gemm3_host_f32(p(A), K, M * K, p(B), N, K * N, None, 0, 0, p(D), N, M * N, M, N, K, count))
+    want = np.einsum("bik,bkj->bij", A.astype(np.float64), B.astype(np.float64))
+    assert np.array_equal(D, want.astype(np.float32))
+    gpu.check(L.decx_hip_gemm3_host_f32(p(A), K, M * K, p(B), N, K * N, p(C), N, M * N, p(D), N, M * N, M, N, K, count))
+    assert np.array_equal(D, (want + C).astype(np.float32))
