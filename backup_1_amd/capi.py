@@ -21,7 +21,7 @@ SYMBOLS = [
     "decx_hip_sgemm", "decx_hip_sgemm_async", "decx_hip_hgemm_f32acc", "decx_hip_hgemm_f32acc_async",
     "decx_hip_conv2_im2col_f32", "decx_hip_conv2_im2col_f32_async", "decx_hip_timer_start", "decx_hip_timer_stop",
     "decx_hip_last_error", "decx_hip_set_sgemm_variant", "decx_hip_set_hgemm_variant", "decx_hip_copy_kernel",
-    "decx_hip_sgemm_batched", "decx_hip_hgemm_f32acc_batched", "decx_hip_gemm3_host_f32", "decx_hip_gemm3_host_f16",
+    "decx_hip_sgemm_splitk", "decx_hip_sgemm_batched", "decx_hip_hgemm_f32acc_batched", "decx_hip_gemm3_host_f32", "decx_hip_gemm3_host_f16",
 ]
 
 
@@ -57,6 +57,7 @@ def lib():
             "decx_hip_conv2_im2col_f32": ([P, I, I, I, Z, P, I, I, I, Z, Z, P, I, Z, I], I),
             "decx_hip_conv2_im2col_f32_async": ([P, I, I, I, Z, P, I, I, I, Z, Z, P, I, Z, I], I),
             "decx_hip_copy_kernel": ([P, P, Z], I),
+            "decx_hip_sgemm_splitk": ([P, I, P, I, P, I, P, I, I, I, I, I], I),
             "decx_hip_sgemm_batched": ([P, I, Z, P, I, Z, P, I, Z, P, I, Z, I, I, I, I], I),
             "decx_hip_hgemm_f32acc_batched": ([P, I, Z, P, I, Z, P, I, Z, P, I, Z, I, I, I, I], I),
             "decx_hip_gemm3_host_f32": ([P, I, Z, P, I, Z, P, I, Z, P, I, Z, I, I, I, I], I),

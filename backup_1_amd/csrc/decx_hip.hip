@@ -82,7 +82,47 @@ int launch_sgemm_tile_c(const ASrc& a, const BSrc& b, const float* Cin, int ldc,
     if (total > 0x7fffffffL || batch.count > 65535) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
     const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
     hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::LDS_BYTES, batch.stream, a, b, Cin,
-                       ldc, D, out, M, N, K, tiles_m, tiles_n, group_m, batch.stride_c, batch.stride_d);
+                       ldc, D, out, M, N, K, tiles_m, tiles_n, group_m, batch.stride_c, batch.stride_d, 0);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+// zero-fills the M x N region of a pitched matrix (the split-K kernel accumulates into it)
+__global__ __launch_bounds__(256) void zero_region_kernel(float* D, int ldd, int M, int N) {
+    const size_t total = (size_t)M * N;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x)
+        D[(i / N) * ldd + i % N] = 0.f;
+}
+
+// Split-K launch of one tile shape: `splits` K ranges of k_split_len each accumulate into D with atomics.
+template <class S>
+int launch_sgemm_splitk(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
+                        int N, int K, int splits, int k_split_len) {
+    typedef DenseA<true> ASrc;
+    typedef DenseB<true> BSrc;
+    const bool in_place = Cin == D;               // D already holds C: accumulate straight onto it
+    const bool add_c = Cin != nullptr && !in_place;
+    auto kern = add_c ? sgemm_tile_kernel<S, ASrc, BSrc, DenseOut, true, true> : sgemm_tile_kernel<S, ASrc, BSrc, DenseOut, false, true>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(sgemm_tile_kernel<S, ASrc, BSrc, DenseOut, true, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(sgemm_tile_kernel<S, ASrc, BSrc, DenseOut, false, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+        attr_done = true;
+    }
+    if (!in_place) {
+        const size_t total = (size_t)M * N;
+        const unsigned blocks = (unsigned)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+        hipLaunchKernelGGL(zero_region_kernel, dim3(blocks), dim3(256), 0, g_rt.stream, D, ldd, M, N);
+    }
+    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
+    ASrc a{A, lda, M, K, 0};
+    BSrc b{B, ldb, N, K, 0};
+    DenseOut out{ldd};
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)splits), dim3(S::NT), S::LDS_BYTES, g_rt.stream, a,
+                       b, Cin, ldc, D, out, M, N, K, tiles_m, tiles_n, group_m, (size_t)0, (size_t)0, k_split_len);
     HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -161,6 +201,29 @@ int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float*
     DenseA<false> a{A, lda, M, K, batch.stride_a};
     DenseB<false> b{B, ldb, N, K, batch.stride_b};
     return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K, batch);
+}
+
+// Split-K GEMM for problems whose M x N tile count leaves most CUs idle while K is long (the short-M / long-K shapes of
+// GEMM_Long_Lr, or a 1024^3 square).  splits <= 0 picks a count that fills the CUs about twice over.
+int sgemm_splitk_enqueue(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
+                         int N, int K, int splits) {
+    Batch one;
+    one.stream = g_rt.stream;
+    if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, one)) return rc;
+    if (!(aligned16(A) && aligned16(B) && lda % 4 == 0 && ldb % 4 == 0 && ldb >= 4))
+        return sgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, one);            // unaligned: plain path
+    const bool big_tiles = (long)cdiv(M, 256) * cdiv(N, 128) >= 16 && M > 128;
+    const int bm = big_tiles ? 256 : 128, bk = 16;
+    const long tiles = (long)cdiv(M, bm) * cdiv(N, 128);
+    const int cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+    const int max_splits = cdiv(K, 8 * bk) < 1024 ? cdiv(K, 8 * bk) : 1024;              // at least 8 K steps per range
+    if (splits <= 0) splits = (int)((2L * cus + tiles - 1) / tiles);
+    if (splits > max_splits) splits = max_splits;
+    if (splits <= 1) return sgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, one);
+    const int k_split_len = cdiv(cdiv(K, splits), bk) * bk;
+    splits = cdiv(K, k_split_len);                                                        // no empty range
+    if (big_tiles) return launch_sgemm_splitk<SShapeTall>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, splits, k_split_len);
+    return launch_sgemm_splitk<SShapeSmall>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, splits, k_split_len);
 }
 
 int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt, int N, int kh,
@@ -505,6 +568,10 @@ int decx_hip_sgemm_async(const float* A, int lda, const float* B, int ldb, const
 int decx_hip_sgemm(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
                    int N, int K) {
     return finish(sgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, single_on_library_stream()));
+}
+int decx_hip_sgemm_splitk(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
+                          int N, int K, int splits) {
+    return finish(sgemm_splitk_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, splits));
 }
 int decx_hip_sgemm_batched(const float* A, int lda, size_t stride_a, const float* B, int ldb, size_t stride_b,
                            const float* Cin, int ldc, size_t stride_c, float* D, int ldd, size_t stride_d, int M, int N, int K,

@@ -72,6 +72,7 @@ struct DenseA {
     int lda, M, K;
     size_t batch_stride;      // elements between consecutive matrices of a batch (blockIdx.y walks the batch)
     __device__ __forceinline__ void select_batch(int b) { A += (size_t)b * batch_stride; }
+    __device__ __forceinline__ void set_k_end(int k_end) { K = k_end; }      // split-K: this workgroup's K range ends here
     struct RowState {
         const float* row;
     };
@@ -116,6 +117,7 @@ struct Im2colA {
     int H, W, dpitch, kh, kw, oy, ox, Wout, Mtot, K;
     size_t row_stride;
     __device__ __forceinline__ void select_batch(int) {}
+    __device__ __forceinline__ void set_k_end(int k_end) { K = k_end; }
     struct RowState {
         int y, x;          // output pixel shifted by (-oy, -ox): the image position of tap (0, 0)
         long base;         // y*row_stride + x*dpitch (may be negative: it is only used together with an in-image tap)
@@ -165,7 +167,7 @@ struct TensorOut {
 // ---------------------------------------------------------------------------------------------------------------
 // B-operand sources.  Interface (S = SgemmShape):
 //   quads<S>()                                   staging registers (float4) per thread and K step
-//   KState k_state<S>(tid) / advance<S>(ks)      position of the K step to fetch next
+//   KState k_state<S>(tid, k_begin) / advance<S>(ks)   position of the K step to fetch next
 //   load<S, TAIL>(stage, tid, ks, bn0)           fetch this thread's share of B[k0 .. k0+BK) x [bn0 .. bn0+BN)
 //   store<S>(plane, stage, tid)                  write it to the LDS planes as k-quads at [q][b_slot(n)]
 // ---------------------------------------------------------------------------------------------------------------
@@ -177,6 +179,7 @@ struct DenseB {
     int ldb, N, K;
     size_t batch_stride;
     __device__ __forceinline__ void select_batch(int b) { B += (size_t)b * batch_stride; }
+    __device__ __forceinline__ void set_k_end(int k_end) { K = k_end; }
     template <class S>
     static constexpr int tasks() { return S::KQ * (S::BN / 4); }
     template <class S>
@@ -187,7 +190,7 @@ struct DenseB {
         int k0;
     };
     template <class S>
-    __device__ __forceinline__ KState k_state(int tid) const { return KState{0}; }
+    __device__ __forceinline__ KState k_state(int tid, int k_begin) const { return KState{k_begin}; }
     template <class S>
     __device__ __forceinline__ void advance(KState& ks) const { ks.k0 += S::BK; }
 
@@ -244,13 +247,14 @@ struct FilterB {
     int N, K, dpitch, kw;
     size_t filt_stride, filt_row_stride;
     __device__ __forceinline__ void select_batch(int) {}
+    __device__ __forceinline__ void set_k_end(int k_end) { K = k_end; }
     template <class S>
     static constexpr int quads() { return S::KQ * S::BN / S::NT; }
     typedef TapWalk KState;       // every quad of a thread has the same k-quad index q = tid % KQ (NT is a multiple of KQ)
     template <class S>
-    __device__ __forceinline__ KState k_state(int tid) const {
+    __device__ __forceinline__ KState k_state(int tid, int k_begin) const {
         KState ks;
-        ks.init(4 * (tid % S::KQ), dpitch, kw);
+        ks.init(k_begin + 4 * (tid % S::KQ), dpitch, kw);
         return ks;
     }
     template <class S>
@@ -300,10 +304,21 @@ struct SgemmShape {
     static_assert(NT % KQ == 0, "A staging: KQ lanes per row");
 };
 
-template <class S, class ASrc, class BSrc, class Out, bool HAS_C>
+// SPLIT_K: blockIdx.z selects a K range of k_split_len (a multiple of BK); every range adds its partial products to dst
+// with fp32 atomics, so dst must hold zeros beforehand and the summation order over ranges is not fixed.  C, if any, is
+// added by range 0.
+template <class S, class ASrc, class BSrc, class Out, bool HAS_C, bool SPLIT_K = false>
 __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(ASrc a_src, BSrc b_src, const float* Cin, int ldc, float* D,
                                                            Out out, int M, int N, int K, int tiles_m, int tiles_n,
-                                                           int group_m, size_t c_batch_stride, size_t d_batch_stride) {
+                                                           int group_m, size_t c_batch_stride, size_t d_batch_stride,
+                                                           int k_split_len) {
+    const int k_begin = SPLIT_K ? (int)blockIdx.z * k_split_len : 0;
+    if (SPLIT_K) {
+        const int k_end = k_begin + k_split_len < K ? k_begin + k_split_len : K;
+        a_src.set_k_end(k_end);
+        b_src.set_k_end(k_end);
+        K = k_end - k_begin;          // from here on K is the length of this workgroup's range
+    }
     // blockIdx.y walks a batch of independent problems of the same shape
     a_src.select_batch(blockIdx.y);
     b_src.select_batch(blockIdx.y);
@@ -334,8 +349,8 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
     f32x4 a_stage[S::A_PASSES];
     bool a_keep[S::A_PASSES];
     f32x4 b_stage[BSrc::template quads<S>()];
-    typename ASrc::KState a_ks = a_src.k_state(4 * a_q);       // this thread's k-quad of the next K step to fetch
-    typename BSrc::KState b_ks = b_src.template k_state<S>(tid);
+    typename ASrc::KState a_ks = a_src.k_state(k_begin + 4 * a_q);   // this thread's k-quad of the next K step to fetch
+    typename BSrc::KState b_ks = b_src.template k_state<S>(tid, k_begin);
 
     // fetches the next K step (steps are always taken in order) and moves the k positions on
     auto load_stage = [&](auto tail_tag) {
@@ -493,7 +508,11 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
 #pragma unroll
                 for (int ni = 0; ni < NI; ++ni) {
                     const int n = bn0 + wn0 + ni * 32 + li;
-                    if (n < N) drow[n] = HAS_C ? acc[mi][ni][r] + crow[n] : acc[mi][ni][r];
+                    if (n < N) {
+                        const float v = (HAS_C && (!SPLIT_K || blockIdx.z == 0)) ? acc[mi][ni][r] + crow[n] : acc[mi][ni][r];
+                        if (SPLIT_K) unsafeAtomicAdd(drow + n, v);      // hardware fp32 add in L2
+                        else drow[n] = v;
+                    }
                 }
             }
         }

@@ -215,6 +215,9 @@ DH GEMM(GPU_Matrix<float>& A, GPU_Matrix<float>& B, GPU_Matrix<float>& dst);
 DH GEMM(GPU_Matrix<float>& A, GPU_Matrix<float>& B, GPU_Matrix<float>& C, GPU_Matrix<float>& dst);
 DH GEMM(GPU_Matrix<Half>& A, GPU_Matrix<Half>& B, GPU_Matrix<Half>& dst);
 DH GEMM(GPU_Matrix<Half>& A, GPU_Matrix<Half>& B, GPU_Matrix<Half>& C, GPU_Matrix<Half>& dst);
+// GEMM/CUDA/extreme_shapes/GEMM_long_Lr.h:22.  dst = A * B for short-M / long-K shapes (split-K underneath).  Unlike
+// the reference it checks initialisation and dimensions, sizes dst, handles any shape and reports its status.
+DH GEMM_Long_Lr(GPU_Matrix<float>& A, GPU_Matrix<float>& B, GPU_Matrix<float>& dst);
 // GEMM/CUDA/large_squares/GEMM3.h:27-36.  dst[i] = A[i] * B[i] (+ C[i]) for every matrix of the arrays, uploads and
 // downloads overlapped with the kernels.
 DH GEMM3(MatrixArray<float>& A, MatrixArray<float>& B, MatrixArray<float>& dst);

@@ -264,6 +264,19 @@ DH GEMM(GPU_Matrix<float>& A, GPU_Matrix<float>& B, GPU_Matrix<float>& C, GPU_Ma
 DH GEMM(GPU_Matrix<Half>& A, GPU_Matrix<Half>& B, GPU_Matrix<Half>& dst) { return gemm_device<Half>(A, B, nullptr, dst); }
 DH GEMM(GPU_Matrix<Half>& A, GPU_Matrix<Half>& B, GPU_Matrix<Half>& C, GPU_Matrix<Half>& dst) { return gemm_device<Half>(A, B, &C, dst); }
 
+DH GEMM_Long_Lr(GPU_Matrix<float>& A_, GPU_Matrix<float>& B_, GPU_Matrix<float>& dst_) {
+    auto* A = dynamic_cast<decx::_GPU_Matrix<float>*>(&A_);
+    auto* B = dynamic_cast<decx::_GPU_Matrix<float>*>(&B_);
+    auto* dst = dynamic_cast<decx::_GPU_Matrix<float>*>(&dst_);
+    if (!A || !B || !dst) return DH{decx::DECX_FAIL_ErrorParams, kNotFactory};
+    if (!decx_hip_is_init()) return not_init();
+    if (A->width != B->height) return DH{decx::DECX_FAIL_DimsNotMatching, kGemmDims};
+    if (!dst->re_construct(B->width, A->height))
+        return dst->last_status == DECX_HIP_FAIL_ALLOCATION ? alloc_fail() : from_status(dst->last_status);
+    return from_status(decx_hip_sgemm_splitk(A->Mat.ptr, (int)A->pitch, B->Mat.ptr, (int)B->pitch, nullptr, 0, dst->Mat.ptr,
+                                             (int)dst->pitch, (int)A->height, (int)B->width, (int)A->width, 0));
+}
+
 DH GEMM3(MatrixArray<float>& A, MatrixArray<float>& B, MatrixArray<float>& dst) { return gemm3_host<float>(A, B, nullptr, dst); }
 DH GEMM3(MatrixArray<Half>& A, MatrixArray<Half>& B, MatrixArray<Half>& dst) { return gemm3_host<Half>(A, B, nullptr, dst); }
 DH GEMM3(MatrixArray<float>& A, MatrixArray<float>& B, MatrixArray<float>& C, MatrixArray<float>& dst) { return gemm3_host<float>(A, B, &C, dst); }

@@ -92,6 +92,15 @@ int decx_hip_hgemm_f32acc(const uint16_t* A, int lda, const uint16_t* B, int ldb
 int decx_hip_hgemm_f32acc_async(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
                                 uint16_t* D, int ldd, int M, int N, int K);
 
+/* de::cuda::GEMM_Long_Lr(GPU_Matrix<float>& A, B, dst) (GEMM/CUDA/extreme_shapes/GEMM_long_Lr.h:22-50; kernel
+ * GEMM_long_linear_region.cuh:73-131): fp32 GEMM for short-M / long-K shapes, whose M x N tiles alone leave most of the
+ * chip idle.  K is cut into `splits` ranges (<= 0: chosen from the CU count) that run as separate workgroups and add
+ * their partial products to D with fp32 atomics; the order in which ranges are added is not fixed, so results can
+ * differ in the last bits between runs (integer-valued data stays exact).  Same arguments and any-shape handling as
+ * decx_hip_sgemm (the reference kernel requires M % 16 == 0 and N, K % 64 == 0).  Cin may be NULL or alias D. */
+int decx_hip_sgemm_splitk(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
+                          int N, int K, int splits);
+
 /* Batched GEMM on device-resident data: `batch` independent problems of one shape in ONE launch; problem b uses
  * A + b*stride_a, B + b*stride_b, Cin + b*stride_c (Cin nullable), D + b*stride_d (strides in elements).  This is the
  * kernel step of de::cuda::GEMM3 over a MatrixArray (GEMM/CUDA/large_squares/GEMM3.h:27-36), whose matrices lie

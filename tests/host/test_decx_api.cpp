@@ -265,6 +265,23 @@ static void conv_case(int H, int W, int C, int N, int kh, int kw, int flag) {
     CHECK(same);
     src.release(); ker.release(); dst.release();
 }
+static void gemm_long_lr() {
+    const int M = 48, K = 16384, N = 200;        // short M, long K (GEMM_long_Lr.h's shape class), ragged N
+    de::Matrix<float>& A = de::CreateMatrixRef<float>(K, M, 0);
+    de::Matrix<float>& B = de::CreateMatrixRef<float>(N, K, 0);
+    de::Matrix<float>& R = de::CreateMatrixRef<float>(N, M, 0);
+    fill(A, small_int); fill(B, small_int);
+    de::GPU_Matrix<float>& dA = de::CreateGPUMatrixRef<float>(K, M);
+    de::GPU_Matrix<float>& dB = de::CreateGPUMatrixRef<float>(N, K);
+    de::GPU_Matrix<float>& dD = de::CreateGPUMatrixRef<float>();
+    dA.Load_from_host(A); dB.Load_from_host(B);
+    CHECK(de::cuda::GEMM_Long_Lr(dA, dB, dD).error_type == decx::DECX_SUCCESS && dD.Width() == (uint)N && dD.Height() == (uint)M);
+    dD.Load_to_host(R);
+    CHECK(dense(R) == chain(A, B));               // integer data: exact whatever the order of the K ranges
+    de::GPU_Matrix<float>& dBad = de::CreateGPUMatrixRef<float>(N, K + 8);
+    CHECK(de::cuda::GEMM_Long_Lr(dA, dBad, dD).error_type == decx::DECX_FAIL_DimsNotMatching);
+}
+
 static void gemm3_matrix_arrays() {
     const int M = 150, K = 90, N = 210, NUM = 5;
     de::MatrixArray<float>& A = de::CreateMatrixArrayRef<float>(K, M, NUM, 0);
@@ -370,6 +387,7 @@ int main(int argc, char** argv) {
         RUN(conv_flavours_and_flags);
         RUN(conv_device_resident);
         RUN(gemm3_matrix_arrays);
+        RUN(gemm_long_lr);
     }
     std::printf("%s: %d failure(s)\n", mode.c_str(), g_fail);
     return g_fail ? 1 : 0;

@@ -174,3 +174,48 @@ def test_gemm3_host_pipeline(gpu):
     assert np.array_equal(D, want.astype(np.float32))
     gpu.check(L.decx_hip_gemm3_host_f32(p(A), K, M * K, p(B), N, K * N, p(C), N, M * N, p(D), N, M * N, M, N, K, count))
     assert np.array_equal(D, (want + C).astype(np.float32))
+
+
+def _splitk(gpu, A, B, C=None, splits=0, inplace=False):
+    M, K = A.shape
+    _, N = B.shape
+    pad = lambda x: (x + 7) // 8 * 8
+    lda, ldb, ldd = pad(K), pad(N), pad(N)
+    Ab = np.full((M, lda), np.nan, np.float32); Ab[:, :K] = A
+    Bb = np.full((K, ldb), np.nan, np.float32); Bb[:, :N] = B
+    dA, dB = gpu.DeviceBuffer.from_numpy(Ab), gpu.DeviceBuffer.from_numpy(Bb)
+    Db = np.full((M, ldd), -9.0, np.float32)
+    dC = None
+    if C is not None:
+        Cb = np.full((M, ldd), np.nan, np.float32); Cb[:, :N] = C
+        if inplace:
+            Db[:, :N] = C
+        else:
+            dC = gpu.DeviceBuffer.from_numpy(Cb)
+    dD = gpu.DeviceBuffer.from_numpy(Db)
+    cptr = dD.ptr if (C is not None and inplace) else (dC.ptr if dC else None)
+    gpu.check(gpu.lib().decx_hip_sgemm_splitk(dA.ptr, lda, dB.ptr, ldb, cptr, ldd, dD.ptr, ldd, M, N, K, splits))
+    out = dD.download((M, ldd), np.float32)
+    assert np.all(out[:, N:] == -9.0), "split-K wrote into the pitch padding"
+    return out[:, :N].copy()
+
+
+@pytest.mark.parametrize("shape", [(16, 65536, 64), (48, 16384, 200), (300, 5000, 130), (1024, 1024, 1024), (7, 100, 5),
+                                   (512, 8200, 256)])
+def test_splitk_integer_exact_and_tolerance(gpu, oracle, shape):
+    # decx_hip_sgemm_splitk (GEMM_Long_Lr): atomics make the order of the K ranges free, integers stay exact
+    M, K, N = shape
+    A = workloads.small_ints((M, K), 301, -3, 3)
+    B = workloads.small_ints((K, N), 302, -3, 3)
+    C = workloads.small_ints((M, N), 303, -40, 40)
+    want = exact_int_product(A, B)
+    for splits in (0, 3, 64):
+        assert np.array_equal(_splitk(gpu, A, B, splits=splits), want)
+    assert np.array_equal(_splitk(gpu, A, B, C), want + C)
+    assert np.array_equal(_splitk(gpu, A, B, C, inplace=True), want + C)
+    Ar, Br = workloads.uniform_pm1((M, K), 304), workloads.uniform_pm1((K, N), 305)
+    rows = np.arange(0, M, max(1, M // 16), dtype=np.int32)
+    ref = oracle.sgemm_chain_rows(Ar, Br, rows)
+    _, scale = oracle.gemm_f64_rows_f32(Ar, Br, rows)
+    err = rel_err_vs_abs_scale(_splitk(gpu, Ar, Br)[rows], ref, scale)
+    assert err < TIGHT(K) < TOL(K)
