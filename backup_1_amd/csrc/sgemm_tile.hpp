@@ -286,10 +286,16 @@ struct FilterB {
     }
 };
 
-template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int WAVES_PER_SIMD_ = 1>
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int WAVES_PER_SIMD_ = 1,
+          int STAGE_SETS_ = (WAVES_PER_SIMD_ == 1 ? 2 : 1)>
 struct SgemmShape {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
     static constexpr int WAVES_PER_SIMD = WAVES_PER_SIMD_;   // occupancy the register budget is held to
+    // Staging register sets = how many K steps ahead of the MFMAs the global loads run.  Two sets hide more latency but
+    // cost A_PASSES + B quads more float4 registers per lane, which only the 512-register budget of one wave per SIMD
+    // holds without spilling.
+    static constexpr int STAGE_SETS = STAGE_SETS_;
+    static_assert(STAGE_SETS == 1 || STAGE_SETS == 2, "one or two K steps of prefetch");
     static constexpr int NT = WAVES_M * WAVES_N * kWave;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     static constexpr int MI = WM / 32, NI = WN / 32;
@@ -346,34 +352,40 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         const int r = a_r + p * A_RSTEP;
         a_rs[p] = a_src.row_state(bm0 + (S::A_PARTIAL && r >= BM ? 0 : r));
     }
-    f32x4 a_stage[S::A_PASSES];
-    bool a_keep[S::A_PASSES];
-    f32x4 b_stage[BSrc::template quads<S>()];
+    // With two staging register sets the K step fetched during step t is the one after next (t+2), so a global load
+    // has almost two steps of MFMAs to land before its data is moved into LDS; with one set it is step t+1.
+    constexpr int B_QUADS = BSrc::template quads<S>();
+    constexpr int SETS = S::STAGE_SETS;
+    f32x4 a_stage[SETS][S::A_PASSES];
+    bool a_keep[SETS][S::A_PASSES];
+    f32x4 b_stage[SETS][B_QUADS];
     typename ASrc::KState a_ks = a_src.k_state(k_begin + 4 * a_q);   // this thread's k-quad of the next K step to fetch
     typename BSrc::KState b_ks = b_src.template k_state<S>(tid, k_begin);
 
-    // fetches the next K step (steps are always taken in order) and moves the k positions on
-    auto load_stage = [&](auto tail_tag) {
+    // fetches the next K step (steps are always taken in order) into register set SET and moves the k positions on
+    auto load_stage = [&](auto set_tag, auto tail_tag) {
+        constexpr int SET = decltype(set_tag)::value;
         constexpr bool TAIL = decltype(tail_tag)::value;
 #pragma unroll
         for (int p = 0; p < S::A_PASSES; ++p) {
             if (S::A_PARTIAL && a_r + p * A_RSTEP >= BM) continue;
-            a_stage[p] = a_src.template load<TAIL>(a_rs[p], a_ks, a_keep[p]);
+            a_stage[SET][p] = a_src.template load<TAIL>(a_rs[p], a_ks, a_keep[SET][p]);
         }
-        b_src.template load<S, TAIL>(b_stage, tid, b_ks, bn0);
+        b_src.template load<S, TAIL>(b_stage[SET], tid, b_ks, bn0);
         a_src.advance(a_ks, BK);
         b_src.template advance<S>(b_ks);
     };
 
-    auto store_stage = [&](int buf) {
+    auto store_stage = [&](auto set_tag, int buf) {
+        constexpr int SET = decltype(set_tag)::value;
         f32x4* Ab = As + buf * KQ * S::A_ROW;
 #pragma unroll
         for (int p = 0; p < S::A_PASSES; ++p) {
             if (S::A_PARTIAL && a_r + p * A_RSTEP >= BM) continue;
             const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-            Ab[a_q * S::A_ROW + a_r + p * A_RSTEP] = a_keep[p] ? a_stage[p] : zero;
+            Ab[a_q * S::A_ROW + a_r + p * A_RSTEP] = a_keep[SET][p] ? a_stage[SET][p] : zero;
         }
-        b_src.template store<S>(Bs + buf * KQ * S::B_ROW, b_stage, tid);
+        b_src.template store<S>(Bs + buf * KQ * S::B_ROW, b_stage[SET], tid);
     };
 
     f32x16 acc[MI][NI];
@@ -416,83 +428,122 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         }
     };
 
-    // K walk.  Full steps run a software-pipelined loop; the partial last step, if any, is peeled out so that its
-    // masking code never sits on the main path.
+    // K walk over T steps (the last one partial when K % BK != 0; its loader zero-fills, so computing it is no
+    // different).  Step t lives in LDS buffer t&1.  Two sets: step t came through register set t&1; while it is
+    // computed, step t+2 is fetched into set t&1 (free since step t went to LDS during step t-1) and step t+1 moves from
+    // set (t+1)&1 into the other LDS buffer.  One set: step t+1 is fetched at the start of step t and moved to LDS in its
+    // second half.  The bulk of the steps (all whose fetch is a full step) run the software-pipelined body; the last
+    // few, with the masking loader, run a plain one.
     const int full_steps = K / BK;
-    const bool has_tail = full_steps * BK < K;
+    const int T = full_steps + (full_steps * BK < K ? 1 : 0);
+    typedef std::integral_constant<int, 0> Set0;
+    typedef std::integral_constant<int, 1> Set1;
 
-    if (full_steps > 0) load_stage(std::false_type{});
-    else load_stage(std::true_type{});
-    store_stage(0);
+    if (full_steps > 0) load_stage(Set0{}, std::false_type{});
+    else load_stage(Set0{}, std::true_type{});
+    store_stage(Set0{}, 0);
     __syncthreads();
-
-    if (full_steps > 0) {
-        static_assert(KQ == 4, "the pipelined loop is written for two quad pairs per K step");
-        constexpr int VMEM_OPS = S::A_PASSES + BSrc::template quads<S>();     // global loads per thread and step
-        constexpr int FRAG_OPS = MI + NI;                                     // ds_read_b128 per quad pair
-        constexpr int WRITE_OPS = S::A_PASSES + BSrc::template quads<S>();    // ds_write_b128 per thread and step
-        f32x4 af0[MI], bf0[NI], af1[MI], bf1[NI];
-        read_frags(0, 0, af0, bf0);
-        // Steady state of one K step t (LDS buffer t&1 holds it, fragments of its first quad pair are in af0/bf0):
-        //   pair 0 MFMAs   interleaved with: global loads of step t+1, LDS reads of pair 1
-        //   pair 1 MFMAs   interleaved with: LDS writes of step t+1 into the other buffer
-        //   barrier, then the LDS reads of step t+1's pair 0 hide behind the last few MFMAs of pair 1.
-        // Every memory instruction sits between MFMAs, so the matrix pipe is never starved by an in-order wait.
-        for (int t = 0; t + 1 < full_steps; ++t) {
-            const int buf = t & 1;
-            load_stage(std::false_type{});
-            read_frags(buf, 1, af1, bf1);
-            mfma_range(af0, bf0, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
-            // scheduling-group masks: 0x002 VALU, 0x008 MFMA, 0x020 VMEM read, 0x100 DS read, 0x200 DS write
-            constexpr int G0 = PAIR_MFMAS / (VMEM_OPS + FRAG_OPS) > 0 ? PAIR_MFMAS / (VMEM_OPS + FRAG_OPS) : 1;
-#pragma unroll
-            for (int i = 0; i < VMEM_OPS; ++i) {          // global loads first: they need the longest lead
-                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, G0, 0);
-            }
-#pragma unroll
-            for (int i = 0; i < FRAG_OPS; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x008, G0, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-
-            constexpr int LATE = MI * NI < PAIR_MFMAS / 4 ? MI * NI : PAIR_MFMAS / 4;   // MFMAs kept for after the barrier
-            constexpr int EARLY = PAIR_MFMAS - LATE;
-            store_stage(buf ^ 1);             // that buffer was last read before the previous barrier
-            mfma_range(af1, bf1, std::integral_constant<int, 0>{}, std::integral_constant<int, EARLY>{});
-            // the staged registers are first touched (register transposes, then LDS writes) half-way through these
-            // MFMAs, which is what gives the global loads their lead
-            constexpr int G1 = (EARLY / 2) / WRITE_OPS > 0 ? (EARLY / 2) / WRITE_OPS : 1;
-            __builtin_amdgcn_sched_group_barrier(0x008, EARLY - G1 * WRITE_OPS, 1);
-#pragma unroll
-            for (int i = 0; i < WRITE_OPS; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x002, 4, 1);
-                __builtin_amdgcn_sched_group_barrier(0x200, 1, 1);
-                __builtin_amdgcn_sched_group_barrier(0x008, G1, 1);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            __builtin_amdgcn_sched_barrier(0);
-            read_frags(buf ^ 1, 0, af0, bf0);
-            mfma_range(af1, bf1, std::integral_constant<int, EARLY>{}, std::integral_constant<int, PAIR_MFMAS>{});
-            __builtin_amdgcn_sched_group_barrier(0x100, FRAG_OPS, 2);
-            __builtin_amdgcn_sched_group_barrier(0x008, LATE, 2);
-            __builtin_amdgcn_sched_barrier(0);
+    if constexpr (SETS == 2) {
+        if (T > 1) {
+            if (full_steps > 1) load_stage(Set1{}, std::false_type{});
+            else load_stage(Set1{}, std::true_type{});
         }
-        // last full step: its first fragments are already in af0/bf0
-        const int buf = (full_steps - 1) & 1;
-        if (has_tail) load_stage(std::true_type{});
+    }
+
+    static_assert(KQ == 4, "the pipelined loop is written for two quad pairs per K step");
+    constexpr int VMEM_OPS = S::A_PASSES + B_QUADS;     // global loads per thread and step
+    constexpr int FRAG_OPS = MI + NI;                   // ds_read_b128 per quad pair
+    constexpr int WRITE_OPS = S::A_PASSES + B_QUADS;    // ds_write_b128 per thread and step
+    f32x4 af0[MI], bf0[NI], af1[MI], bf1[NI];
+
+    // Steady state of one K step t (fragments of its first quad pair are in af0/bf0):
+    //   pair 0 MFMAs   interleaved with: global loads of step t+SETS, LDS reads of pair 1
+    //   pair 1 MFMAs   interleaved with: LDS writes of step t+1 into the other buffer
+    //   barrier, then the LDS reads of step t+1's pair 0 hide behind the last few MFMAs of pair 1.
+    // Every memory instruction sits between MFMAs, so the matrix pipe is never starved by an in-order wait.
+    auto pipelined_step = [&](auto set_tag, int buf) {
+        constexpr int SET = decltype(set_tag)::value;
+        load_stage(set_tag, std::false_type{});
         read_frags(buf, 1, af1, bf1);
         mfma_range(af0, bf0, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
-        mfma_range(af1, bf1, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
-        if (has_tail) {
-            store_stage(buf ^ 1);
-            __syncthreads();
-            compute_stage(buf ^ 1);
+        // scheduling-group masks: 0x002 VALU, 0x008 MFMA, 0x020 VMEM read, 0x100 DS read, 0x200 DS write
+        constexpr int G0 = PAIR_MFMAS / (VMEM_OPS + FRAG_OPS) > 0 ? PAIR_MFMAS / (VMEM_OPS + FRAG_OPS) : 1;
+#pragma unroll
+        for (int i = 0; i < VMEM_OPS; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, G0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < FRAG_OPS; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, G0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        constexpr int LATE = MI * NI < PAIR_MFMAS / 4 ? MI * NI : PAIR_MFMAS / 4;   // MFMAs kept for after the barrier
+        constexpr int EARLY = PAIR_MFMAS - LATE;
+        // step t+1 sits in the other set when there are two; buffer buf^1 was last read before the previous barrier
+        store_stage(std::integral_constant<int, SETS == 2 ? 1 - SET : 0>{}, buf ^ 1);
+        mfma_range(af1, bf1, std::integral_constant<int, 0>{}, std::integral_constant<int, EARLY>{});
+        constexpr int G1 = (EARLY / 2) / WRITE_OPS > 0 ? (EARLY / 2) / WRITE_OPS : 1;
+        __builtin_amdgcn_sched_group_barrier(0x008, EARLY - G1 * WRITE_OPS, 1);
+#pragma unroll
+        for (int i = 0; i < WRITE_OPS; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x002, 4, 1);
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 1);
+            __builtin_amdgcn_sched_group_barrier(0x008, G1, 1);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(buf ^ 1, 0, af0, bf0);
+        mfma_range(af1, bf1, std::integral_constant<int, EARLY>{}, std::integral_constant<int, PAIR_MFMAS>{});
+        __builtin_amdgcn_sched_group_barrier(0x100, FRAG_OPS, 2);
+        __builtin_amdgcn_sched_group_barrier(0x008, LATE, 2);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    int t = 0;
+    if constexpr (SETS == 2) {
+        if (full_steps > 2) {
+            read_frags(0, 0, af0, bf0);
+            for (; t + 3 < full_steps; t += 2) {      // steps t and t+1 both fetch a full step (t+2, t+3 < full_steps)
+                pipelined_step(Set0{}, 0);
+                pipelined_step(Set1{}, 1);
+            }
+            if (t + 2 < full_steps) {
+                pipelined_step(Set0{}, 0);
+                ++t;
+            }
+        }
+        // the remaining steps: at most one more fetch, and that one is the partial step
+        for (; t < T; ++t) {
+            const int buf = t & 1;
+            if (t + 2 < T) {
+                if (buf == 0) load_stage(Set0{}, std::true_type{});
+                else load_stage(Set1{}, std::true_type{});
+            }
+            compute_stage(buf);
+            if (t + 1 < T) {
+                if (buf == 0) store_stage(Set1{}, 1);
+                else store_stage(Set0{}, 0);
+                __syncthreads();
+            }
         }
     } else {
-        compute_stage(0);             // K < BK: the prologue staged the only, partial step
+        if (full_steps > 1) {
+            read_frags(0, 0, af0, bf0);
+            for (; t + 1 < full_steps; ++t) pipelined_step(Set0{}, t & 1);   // fetches step t+1, a full one
+        }
+        for (; t < T; ++t) {
+            const int buf = t & 1;
+            if (t + 1 < T) load_stage(Set0{}, std::true_type{});
+            compute_stage(buf);
+            if (t + 1 < T) {
+                store_stage(Set0{}, buf ^ 1);
+                __syncthreads();
+            }
+        }
     }
 
     // ---- epilogue: each lane holds column li of its 32-wide block; a half-wave writes 128 contiguous bytes.
