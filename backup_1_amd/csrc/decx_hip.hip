@@ -139,15 +139,19 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //   2: 128x128x16, 2x2 waves of  64x64    -- small problems, several workgroups per CU
 //   3: 256x128x16, 2x2 waves of 128x64    -- narrow N
 //   4: 224x128x16, 1x4 waves of 224x32    -- 7/8 of shape 3 per tile: fills more CUs when M/256 tiles leave many idle
+//   5, 6: shapes 3 and 4 compiled for one wave per SIMD (512 registers, two staging sets) -- for launches that put at
+//         most one workgroup on a CU anyway, where a second resident workgroup cannot be what hides the load latency
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
 typedef SgemmShape<128, 128, 16, 2, 2, 2> SShapeSmall;
 typedef SgemmShape<256, 128, 16, 2, 2, 2> SShapeTall;
 typedef SgemmShape<224, 128, 16, 1, 4, 2> SShape224;
+typedef SgemmShape<256, 128, 16, 2, 2, 1> SShapeTallSolo;
+typedef SgemmShape<224, 128, 16, 1, 4, 1> SShape224Solo;
 
 // Tile shape by a small cost model: a CU works through ceil(tiles / CUs) tiles one after another, a tile costs its area
 // divided by how well that shape keeps the matrix pipe busy (measured on 8192^3, relative to shape 1).
 int pick_sgemm_variant(int M, int N, int batch) {
-    if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 4) return g_rt.sgemm_variant;
+    if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 6) return g_rt.sgemm_variant;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     struct Cand { int variant, bm, bn; double eff; };
     const Cand cands[] = {{1, 256, 256, 1.00}, {3, 256, 128, 0.95}, {4, 224, 128, 0.85}, {2, 128, 128, 0.90}};
@@ -156,7 +160,10 @@ int pick_sgemm_variant(int M, int N, int batch) {
     for (const Cand& c : cands) {
         const long tiles = (long)cdiv(M, c.bm) * cdiv(N, c.bn) * batch;
         const double cost = (double)((tiles + cus - 1) / cus) * c.bm * c.bn / c.eff;
-        if (best_cost == 0.0 || cost < best_cost) { best_cost = cost; best = c.variant; }
+        if (best_cost == 0.0 || cost < best_cost) {
+            best_cost = cost;
+            best = (tiles <= cus && c.variant >= 3) ? c.variant + 2 : c.variant;
+        }
     }
     return best;
 }
@@ -168,6 +175,8 @@ int dispatch_sgemm(int variant, const ASrc& a, const BSrc& b, const float* Cin, 
         case 1: return launch_sgemm_tile<SShapeBig>(a, b, Cin, ldc, D, out, M, N, K, batch);
         case 3: return launch_sgemm_tile<SShapeTall>(a, b, Cin, ldc, D, out, M, N, K, batch);
         case 4: return launch_sgemm_tile<SShape224>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 5: return launch_sgemm_tile<SShapeTallSolo>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 6: return launch_sgemm_tile<SShape224Solo>(a, b, Cin, ldc, D, out, M, N, K, batch);
         default: return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K, batch);
     }
 }
@@ -186,12 +195,12 @@ int check_gemm_args(const void* A, int lda, const void* B, int ldb, const void* 
 }
 
 int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
-                  int N, int K, const Batch& batch) {
+                  int N, int K, const Batch& batch, bool relu = false) {
     if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
     const int variant = pick_sgemm_variant(M, N, batch.count);
     const bool vec_a = aligned16(A) && lda % 4 == 0 && batch.stride_a % 4 == 0;
     const bool vec_b = aligned16(B) && ldb % 4 == 0 && ldb >= 4 && batch.stride_b % 4 == 0;
-    DenseOut out{ldd};
+    DenseOut out{ldd, relu};
     if (vec_a && vec_b) {
         DenseA<true> a{A, lda, M, K, batch.stride_a};
         DenseB<true> b{B, ldb, N, K, batch.stride_b};
@@ -228,7 +237,7 @@ int sgemm_splitk_enqueue(const float* A, int lda, const float* B, int ldb, const
 
 int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt, int N, int kh,
                  int kw, size_t filt_stride, size_t filt_row_stride, float* dst, int dst_dpitch, size_t dst_row_stride,
-                 int flag) {
+                 int flag, const float* bias = nullptr, bool relu = false) {
     if (!g_rt.is_init) return need_init();
     if (flag != DECX_HIP_CONV_NO_COMPENSATE && flag != DECX_HIP_CONV_ZERO_COMPENSATE)
         return fail(DECX_HIP_FAIL_ERROR_FLAG, "This flag is meaningless in current context\n");   // core/error.h:67
@@ -249,10 +258,11 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
     const int M = (int)Ml, K = (int)Kl;
     Im2colA a{src, H, W, dpitch, kh, kw, flag ? kh / 2 : 0, flag ? kw / 2 : 0, Wout, M, K, src_row_stride};
     FilterB b{filt, N, K, dpitch, kw, filt_stride, filt_row_stride};
-    TensorOut out{Wout, dst_dpitch, dst_row_stride, dst_row_stride == (size_t)Wout * dst_dpitch};
+    TensorOut out{Wout, dst_dpitch, dst_row_stride, dst_row_stride == (size_t)Wout * dst_dpitch, relu};
     Batch one;
     one.stream = g_rt.stream;
-    return dispatch_sgemm(pick_sgemm_variant(M, N, 1), a, b, nullptr, 0, dst, out, M, N, K, one);
+    // a bias is the "+ C" operand with row stride 0: every output pixel adds the same N values
+    return dispatch_sgemm(pick_sgemm_variant(M, N, 1), a, b, bias, 0, dst, out, M, N, K, one);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -438,6 +448,69 @@ __global__ __launch_bounds__(256) void copy_kernel(f32x4* __restrict__ dst, cons
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < quads; i += stride) dst[i] = src[i];
 }
 
+// Element-wise ReLU family of nn/operators/ReLU.h.  MODE 0: forward; 1: forward + record; 2: backward (dst = src where
+// the recorded bit is set, else 0 * src; ReLU.h:131-165).  The bit map has one byte per 8 consecutive floats: bits 4..7
+// = the first 16-byte quad's x,y,z,w, bits 0..3 = the second quad's (ReLU.h:86-123).
+// One quad per lane, no loop, streaming (non-temporal) accesses: every byte is touched once, consecutive lanes take
+// consecutive 16 bytes, and short-lived workgroups keep more loads in flight across the chip than a few long-lived ones
+// (measured: 6.7 TB/s against 5.2-5.8 TB/s for grid-stride loops of any unroll depth).  A map byte is assembled from
+// the two lanes of a quad pair with one lane exchange; the even lane stores it.
+template <int MODE>
+__global__ __launch_bounds__(256) void relu_kernel(const f32x4* __restrict__ src, f32x4* __restrict__ dst,
+                                                   unsigned char* __restrict__ rec_map, size_t quads) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const bool live = i < quads;              // quads is even in modes 1 and 2, so both lanes of a pair are live together
+    f32x4 q = {0.f, 0.f, 0.f, 0.f};
+    if (live) q = __builtin_nontemporal_load(src + i);
+    unsigned nibble = 0;
+    if (MODE == 2 && live) {
+        const unsigned byte = rec_map[i >> 1];
+        nibble = (i & 1) ? (byte & 15u) : (byte >> 4);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        if (MODE == 2) {
+            q[e] = (float)((nibble >> e) & 1u) * q[e];
+        } else {
+            const unsigned s = (~__float_as_uint(q[e])) >> 31;
+            q[e] = (float)s * q[e];
+            nibble |= s << e;
+        }
+    }
+    if (MODE == 1) {
+        const unsigned other = (unsigned)__shfl_xor((int)nibble, 1);
+        if (live && (i & 1) == 0) rec_map[i >> 1] = (unsigned char)((nibble << 4) | other);
+    }
+    if (live) __builtin_nontemporal_store(q, dst + i);
+}
+// the last n % 4 floats of the plain forward form
+__global__ void relu_tail_kernel(const float* __restrict__ src, float* __restrict__ dst, int n) {
+    const int i = threadIdx.x;
+    if (i < n) dst[i] = relu_by_sign(src[i]);
+}
+
+template <int MODE>
+int relu_enqueue(const float* src, float* dst, unsigned char* rec_map, size_t n) {
+    if (!g_rt.is_init) return need_init();
+    if (!src || !dst || (MODE != 0 && !rec_map)) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "null pointer\n");
+    if (!aligned16(src) || !aligned16(dst)) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "ReLU needs 16-byte aligned buffers\n");
+    if (MODE != 0 && n % 8 != 0)
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "the recorded forms work on whole groups of 8 floats (one map byte each)\n");
+    const size_t quads = MODE == 0 ? n / 4 : n / 8 * 2;
+    if (quads > 0) {
+        const size_t blocks = (quads + 255) / 256;
+        if (blocks > 0x7fffffffull) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "buffer too large for one launch\n");
+        hipLaunchKernelGGL(relu_kernel<MODE>, dim3((unsigned)blocks), dim3(256), 0, g_rt.stream,
+                           reinterpret_cast<const f32x4*>(src), reinterpret_cast<f32x4*>(dst), rec_map, quads);
+        HIP_TRY(hipGetLastError());
+    }
+    if (MODE == 0 && n % 4 != 0) {
+        hipLaunchKernelGGL(relu_tail_kernel, dim3(1), dim3(64), 0, g_rt.stream, src + quads * 4, dst + quads * 4, (int)(n % 4));
+        HIP_TRY(hipGetLastError());
+    }
+    return 0;
+}
+
 int finish(int rc) {
     if (rc != 0) return rc;
     HIP_TRY(hipStreamSynchronize(g_rt.stream));
@@ -569,6 +642,10 @@ int decx_hip_sgemm(const float* A, int lda, const float* B, int ldb, const float
                    int N, int K) {
     return finish(sgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, single_on_library_stream()));
 }
+int decx_hip_sgemm_relu(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
+                        int N, int K) {
+    return finish(sgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, single_on_library_stream(), true));
+}
 int decx_hip_sgemm_splitk(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
                           int N, int K, int splits) {
     return finish(sgemm_splitk_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, splits));
@@ -623,6 +700,22 @@ int decx_hip_conv2_im2col_f32(const float* src, int H, int W, int dpitch, size_t
                               size_t dst_row_stride, int flag) {
     return finish(conv_enqueue(src, H, W, dpitch, src_row_stride, filt, N, kh, kw, filt_stride, filt_row_stride, dst,
                                dst_dpitch, dst_row_stride, flag));
+}
+
+int decx_hip_conv2_im2col_f32_fused(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt,
+                                    int N, int kh, int kw, size_t filt_stride, size_t filt_row_stride, float* dst,
+                                    int dst_dpitch, size_t dst_row_stride, int flag, const float* bias, int relu) {
+    return finish(conv_enqueue(src, H, W, dpitch, src_row_stride, filt, N, kh, kw, filt_stride, filt_row_stride, dst,
+                               dst_dpitch, dst_row_stride, flag, bias, relu != 0));
+}
+
+int decx_hip_relu_f32(const float* src, float* dst, size_t n) { return finish(relu_enqueue<0>(src, dst, nullptr, n)); }
+int decx_hip_relu_f32_async(const float* src, float* dst, size_t n) { return relu_enqueue<0>(src, dst, nullptr, n); }
+int decx_hip_relu_f32_rec(const float* src, float* dst, unsigned char* rec_map, size_t n) {
+    return finish(relu_enqueue<1>(src, dst, rec_map, n));
+}
+int decx_hip_relu_f32_backward(const float* src, float* dst, const unsigned char* rec_map, size_t n) {
+    return finish(relu_enqueue<2>(src, dst, const_cast<unsigned char*>(rec_map), n));
 }
 
 int decx_hip_copy_kernel(void* dst, const void* src, size_t bytes) {

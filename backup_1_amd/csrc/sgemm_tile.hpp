@@ -147,16 +147,26 @@ struct Im2colA {
     }
 };
 
+// ReLU exactly as the reference's element-wise kernel computes it (nn/operators/ReLU.h:57-82): the value times
+// float(sign bit clear).  Hence a negative input gives -0.0f, -inf gives NaN, NaN stays NaN.
+__device__ __forceinline__ float relu_by_sign(float v) {
+    return (float)((~__float_as_uint(v)) >> 31) * v;
+}
+
 // Result addressing: dense matrices (row m at m*ld) or the convolution's output tensor (pixel (y,x) at
-// y*row_stride + x*dpitch).
+// y*row_stride + x*dpitch).  relu: apply relu_by_sign to every result element before it is stored.
 struct DenseOut {
     int ld;
+    bool relu = false;
     __device__ __forceinline__ size_t offset(int m) const { return (size_t)m * ld; }
+    __device__ __forceinline__ float finish(float v) const { return relu ? relu_by_sign(v) : v; }
 };
 struct TensorOut {
     int Wout, dpitch;
     size_t row_stride;
     bool dense;      // row_stride == Wout*dpitch: pixel m simply starts at m*dpitch, no division needed
+    bool relu = false;
+    __device__ __forceinline__ float finish(float v) const { return relu ? relu_by_sign(v) : v; }
     __device__ __forceinline__ size_t offset(int m) const {
         if (dense) return (size_t)m * dpitch;
         const int y = m / Wout, x = m - y * Wout;
@@ -562,7 +572,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
                     if (n < N) {
                         const float v = (HAS_C && (!SPLIT_K || blockIdx.z == 0)) ? acc[mi][ni][r] + crow[n] : acc[mi][ni][r];
                         if (SPLIT_K) unsafeAtomicAdd(drow + n, v);      // hardware fp32 add in L2
-                        else drow[n] = v;
+                        else drow[n] = out.finish(v);
                     }
                 }
             }

@@ -232,6 +232,16 @@ DH Conv2_MK_im2col(Tensor<float>& src, TensorArray<float>& kernel, Tensor<float>
 DH Conv2_MK_im2col(GPU_Tensor<float>& src, GPU_TensorArray<float>& kernel, GPU_Tensor<float>& dst, const int flag);
 }  // namespace cuda
 
+namespace nn {
+// nn/operators/ReLU.h:28-34.  Element-wise over the whole pitched buffer of src (padding included), with the
+// reference's arithmetic: value * float(sign bit clear).  dst must have src's dimensions (the reference prints a
+// message and still reports success; here the DH carries DECX_FAIL_DimsNotMatching).  rec_map takes one byte per 8
+// floats, filled linearly; ReLU_f_Rec sizes it to (pitch/8, height) if it is too small.
+DH ReLU_f(GPU_Matrix<float>& src, GPU_Matrix<float>& dst);
+DH ReLU_f_Rec(GPU_Matrix<float>& src, GPU_Matrix<float>& dst, GPU_Matrix<uchar>& rec_map);
+DH ReLU_f_Backward(GPU_Matrix<float>& src, GPU_Matrix<float>& dst, GPU_Matrix<uchar>& rec_map);
+}  // namespace nn
+
 namespace cpu {
 // GEMM/CPU/sgemm.h:22.  Host thread-pool SGEMM.
 DH sgemm(Matrix<float>& A, Matrix<float>& B, Matrix<float>& dst);

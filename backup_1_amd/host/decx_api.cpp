@@ -244,6 +244,7 @@ template GPU_TensorArray<float>* CreateGPUTensorArrayPtr<float>(const uint, cons
     template GPU_Matrix<T>* CreateGPUMatrixPtr<T>(const uint, const uint);
 DECX_INSTANTIATE_MATRIX(float)
 DECX_INSTANTIATE_MATRIX(Half)
+DECX_INSTANTIATE_MATRIX(uchar)
 template Tensor<float>& CreateTensorRef<float>();
 template Tensor<float>* CreateTensorPtr<float>();
 template Tensor<float>& CreateTensorRef<float>(const uint, const uint, const uint, const int);
@@ -341,4 +342,56 @@ DH Conv2_MK_im2col(GPU_Tensor<float>& src_, GPU_TensorArray<float>& kernel_, GPU
                                                  (int)dst->dpitch, dst->dp_x_wp, flag));
 }
 }  // namespace cuda
+
+// ---- nn::ReLU (nn/operators/ReLU.h:169-210) ----------------------------------------------------------------------
+namespace nn {
+namespace {
+struct ReluArgs {
+    decx::_GPU_Matrix<float>* src;
+    decx::_GPU_Matrix<float>* dst;
+    size_t len;         // floats the kernels run over: pitch * height (ReLU.h:175)
+    DH status;
+    bool ok;
+};
+ReluArgs relu_args(GPU_Matrix<float>& src_, GPU_Matrix<float>& dst_) {
+    ReluArgs r{dynamic_cast<decx::_GPU_Matrix<float>*>(&src_), dynamic_cast<decx::_GPU_Matrix<float>*>(&dst_), 0, DH{}, false};
+    static char dims_msg[] = "Matrix Dims don't match each other";
+    if (!r.src || !r.dst) r.status = DH{decx::DECX_FAIL_ErrorParams, kNotFactory};
+    else if (!decx_hip_is_init()) r.status = not_init();
+    else if (r.src->width != r.dst->width || r.src->height != r.dst->height || !r.src->Mat.ptr || !r.dst->Mat.ptr)
+        r.status = DH{decx::DECX_FAIL_DimsNotMatching, dims_msg};
+    else {
+        r.len = (size_t)r.src->pitch * r.src->height;
+        r.ok = true;
+    }
+    return r;
+}
+}  // namespace
+
+DH ReLU_f(GPU_Matrix<float>& src, GPU_Matrix<float>& dst) {
+    ReluArgs a = relu_args(src, dst);
+    if (!a.ok) return a.status;
+    return from_status(decx_hip_relu_f32(a.src->Mat.ptr, a.dst->Mat.ptr, a.len));
+}
+
+DH ReLU_f_Rec(GPU_Matrix<float>& src, GPU_Matrix<float>& dst, GPU_Matrix<uchar>& rec_map) {
+    ReluArgs a = relu_args(src, dst);
+    if (!a.ok) return a.status;
+    auto* map = dynamic_cast<decx::_GPU_Matrix<uchar>*>(&rec_map);
+    if (!map) return DH{decx::DECX_FAIL_ErrorParams, kNotFactory};
+    if ((!map->Mat.ptr || map->total_bytes < a.len / 8) && !map->re_construct(a.src->pitch / 8, a.src->height))
+        return map->last_status == DECX_HIP_FAIL_ALLOCATION ? alloc_fail() : from_status(map->last_status);
+    return from_status(decx_hip_relu_f32_rec(a.src->Mat.ptr, a.dst->Mat.ptr, map->Mat.ptr, a.len));
+}
+
+DH ReLU_f_Backward(GPU_Matrix<float>& src, GPU_Matrix<float>& dst, GPU_Matrix<uchar>& rec_map) {
+    ReluArgs a = relu_args(src, dst);
+    if (!a.ok) return a.status;
+    auto* map = dynamic_cast<decx::_GPU_Matrix<uchar>*>(&rec_map);
+    if (!map) return DH{decx::DECX_FAIL_ErrorParams, kNotFactory};
+    static char dims_msg[] = "Matrix Dims don't match each other";
+    if (!map->Mat.ptr || map->total_bytes < a.len / 8) return DH{decx::DECX_FAIL_DimsNotMatching, dims_msg};
+    return from_status(decx_hip_relu_f32_backward(a.src->Mat.ptr, a.dst->Mat.ptr, map->Mat.ptr, a.len));
+}
+}  // namespace nn
 }  // namespace de

@@ -23,6 +23,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_MATRIX_TFLOPS = 157.3     # MI355X dense fp32 MFMA
 PEAK_FP16_MATRIX_TFLOPS = 2516.6    # MI355X dense fp16 MFMA (2.5 PFLOP/s)
+PEAK_HBM_GBPS = 8000.0              # MI355X HBM3E
 # HBM-side bytes per launch of the headline kernel (fp32 8192^3), from the FETCH_SIZE / WRITE_SIZE counter runs
 # summarised in profiles/hbm_traffic_fetch_write_size.txt (read factor 2.0, write factor 1.0 against a copy kernel).
 # Counters cannot be read from inside this script; the figure is only reported for the workload it was measured on.
@@ -90,6 +91,36 @@ def bench_conv(capi, workloads, steps, warmup):
     return {"ms_wall": wall, "ms_kernel": ev, "tflops": flops / (wall * 1e-3) / 1e12, "tflops_kernel": flops / (ev * 1e-3) / 1e12}
 
 
+def bench_relu(capi, workloads, steps, warmup):
+    """de::nn::ReLU_f over a 8192 x 8192 fp32 matrix (256 MiB in, 256 MiB out): HBM-bound, 8 bytes per element."""
+    n = 8192 * 8192
+    x = workloads.normal((n,), 77)
+    dX, dY = capi.DeviceBuffer.from_numpy(x), capi.DeviceBuffer(n * 4)
+    launch = lambda: capi.check(capi.lib().decx_hip_relu_f32_async(dX.ptr, dY.ptr, n))
+    wall, ev = time_launches(capi, launch, steps, warmup)
+    return {"ms_wall": wall, "ms_kernel": ev, "gbps": 8.0 * n / (ev * 1e-3) / 1e9}
+
+
+def bench_conv_fused(capi, workloads, steps, warmup):
+    """config 4 with the bias + ReLU epilogue (decx_hip_conv2_im2col_f32_fused); same flop count as bench_conv."""
+    H = W = 224; C = 64; N = 128; kh = kw = 3
+    src, filt = workloads.conv_case()
+    fb = np.zeros((N, kh, 4, C), np.float32); fb[:, :, :kw, :] = filt
+    dS, dF = capi.DeviceBuffer.from_numpy(src), capi.DeviceBuffer.from_numpy(fb)
+    dB = capi.DeviceBuffer.from_numpy(workloads.normal((N,), 78))
+    dD = capi.DeviceBuffer(H * W * N * 4)
+    launch = lambda: capi.check(capi.lib().decx_hip_conv2_im2col_f32_fused(
+        dS.ptr, H, W, C, W * C, dF.ptr, N, kh, kw, kh * 4 * C, 4 * C, dD.ptr, N, W * N, 1, dB.ptr, 1))
+    ms = []
+    for i in range(warmup + steps):          # the fused entry point is synchronous: time whole calls
+        t0 = time.perf_counter()
+        launch()
+        if i >= warmup: ms.append((time.perf_counter() - t0) * 1e3)
+    flops = 2.0 * H * W * N * kh * kw * C
+    best = min(ms)
+    return {"ms_wall": best, "tflops": flops / (best * 1e-3) / 1e12}
+
+
 def cpu_baseline(A, B, rows):
     """The restated DECX_cpu thread-pool SGEMM (oracle/, kind "port") on the first `rows` rows of the headline A times
     the full B: B re-pack included, 12 tasks on a pool of min(hardware threads, 16) workers, as the reference sizes it."""
@@ -118,7 +149,7 @@ def main():
     ap.add_argument("--size", type=int, default=8192, help="square size of the headline fp32 GEMM")
     ap.add_argument("--sgemm-variant", type=int, default=0, help="force a fp32 tile shape (0 = automatic)")
     ap.add_argument("--hgemm-variant", type=int, default=0, help="force a fp16 tile shape (0 = automatic)")
-    ap.add_argument("--only", default="", help="comma list of: headline,fp16,sq4096,ragged,conv,cpu (default all)")
+    ap.add_argument("--only", default="", help="comma list of: headline,fp16,sq4096,ragged,conv,relu,cpu (default all)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); --gpus %d is not supported. "
@@ -162,6 +193,15 @@ def main():
             "tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
             "frac_of_fp32_matrix_peak": round(r["tflops_kernel"] / PEAK_FP32_MATRIX_TFLOPS, 4)}
         log("conv: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+
+    if want("relu"):
+        r = bench_relu(capi, workloads, side_steps, args.warmup)
+        also["relu_f32_8192x8192"] = {"GBps": round(r["gbps"], 1), "ms_per_step": round(r["ms_wall"], 4),
+                                      "frac_of_hbm_peak": round(r["gbps"] / PEAK_HBM_GBPS, 4)}
+        log("relu 8192x8192: %.4f ms -> %.0f GB/s" % (r["ms_wall"], r["gbps"]))
+        r = bench_conv_fused(capi, workloads, side_steps, args.warmup)
+        also["fp32_conv_bias_relu_fused_blocking_call"] = {"tflops": round(r["tflops"], 2), "ms_per_call": round(r["ms_wall"], 4)}
+        log("conv + bias + relu (one kernel, blocking call): %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
 
     if "copy" in only:
         # calibration launch for the traffic counters: 1 GiB read + 1 GiB written by a plain copy kernel

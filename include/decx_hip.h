@@ -146,6 +146,31 @@ int decx_hip_conv2_im2col_f32_async(const float* src, int H, int W, int dpitch, 
                                     int N, int kh, int kw, size_t filt_stride, size_t filt_row_stride, float* dst,
                                     int dst_dpitch, size_t dst_row_stride, int flag);
 
+/* The convolution above with the layer's element-wise tail applied to each result before it is stored, instead of in
+ * passes of their own over dst: an optional per-filter bias (N floats on the device, NULL for none) and, if relu != 0,
+ * the activation of de::nn::ReLU_f (nn/operators/ReLU.h:57-82) with its exact arithmetic (see decx_hip_relu_f32).
+ *   dst(y,x,n) = relu( conv(y,x,n) + bias[n] ). */
+int decx_hip_conv2_im2col_f32_fused(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt,
+                                    int N, int kh, int kw, size_t filt_stride, size_t filt_row_stride, float* dst,
+                                    int dst_dpitch, size_t dst_row_stride, int flag, const float* bias, int relu);
+/* decx_hip_sgemm followed by de::nn::ReLU_f on the result, in one kernel: D = relu(A*B + Cin). */
+int decx_hip_sgemm_relu(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
+                        int N, int K);
+
+/* de::nn::ReLU_f(GPU_Matrix<float>& src, dst)                    nn/operators/ReLU.h:28, :57-82, :169-180
+ * de::nn::ReLU_f_Rec(src, dst, GPU_Matrix<uchar>& rec_map)       ReLU.h:31, :98-127, :184-195
+ * de::nn::ReLU_f_Backward(src, dst, rec_map)                     ReLU.h:34, :131-165, :199-210
+ * over n consecutive floats (the reference passes pitch*height, padding included).  Arithmetic as in the reference:
+ *   forward : dst[i] = float(sign bit of src[i] clear) * src[i]  -- so negative inputs give -0.0f, -inf gives NaN;
+ *   rec     : forward, and byte j of rec_map records floats 8j..8j+7: bit 4+e = float 8j+e kept, bit e = float 8j+4+e
+ *             kept (e = 0..3);
+ *   backward: dst[i] = float(recorded bit of i) * src[i].
+ * src and dst 16-byte aligned (may be the same buffer); rec and backward need n % 8 == 0, rec_map holds n/8 bytes. */
+int decx_hip_relu_f32(const float* src, float* dst, size_t n);
+int decx_hip_relu_f32_async(const float* src, float* dst, size_t n);
+int decx_hip_relu_f32_rec(const float* src, float* dst, unsigned char* rec_map, size_t n);
+int decx_hip_relu_f32_backward(const float* src, float* dst, const unsigned char* rec_map, size_t n);
+
 /* A plain device-to-device streaming copy kernel of `bytes` bytes (16-byte aligned, multiple of 16).  It has no
  * counterpart in the reference: it exists so that hardware traffic counters read for the kernels above can be scaled
  * by what the same counters read for a kernel whose traffic is known exactly.  Blocks until complete. */

@@ -51,6 +51,12 @@ def lib():
         L.oracle_gemm_f64_rows_f16.restype = None
         L.oracle_gemm_f64_rows_f32.argtypes = [P, L_, P, L_, P, I, P, P, I, I, I]
         L.oracle_gemm_f64_rows_f32.restype = None
+        L.oracle_relu_f32.argtypes = [P, P, L_]
+        L.oracle_relu_f32.restype = None
+        L.oracle_relu_f32_rec.argtypes = [P, P, P, L_]
+        L.oracle_relu_f32_rec.restype = None
+        L.oracle_relu_f32_backward.argtypes = [P, P, P, L_]
+        L.oracle_relu_f32_backward.restype = None
         L.oracle_pool_size.argtypes = [I]
         L.oracle_pool_size.restype = I
         _lib = L
@@ -174,3 +180,31 @@ def gemm_f64_rows_f32(A, B, rows, nthreads=0):
     ab = np.empty((len(rows), N), dtype=np.float64)
     lib().oracle_gemm_f64_rows_f32(_p(A), _ld(A), _p(B), _ld(B), _p(rows), len(rows), _p(out), _p(ab), N, K, nthreads)
     return out, ab
+
+
+def relu(x):
+    """de::nn::ReLU_f arithmetic (nn/operators/ReLU.h:57-82) on a float32 array of any shape."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    lib().oracle_relu_f32(_p(x), _p(out), x.size)
+    return out
+
+
+def relu_rec(x):
+    """ReLU_f_Rec (ReLU.h:98-127): (dst, rec_map) with one map byte per 8 floats; x.size must be a multiple of 8."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    assert x.size % 8 == 0
+    out = np.empty_like(x)
+    rec = np.empty(x.size // 8, dtype=np.uint8)
+    lib().oracle_relu_f32_rec(_p(x), _p(out), _p(rec), x.size)
+    return out, rec
+
+
+def relu_backward(x, rec):
+    """ReLU_f_Backward (ReLU.h:131-165)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    rec = np.ascontiguousarray(rec, dtype=np.uint8)
+    assert x.size % 8 == 0 and rec.size == x.size // 8
+    out = np.empty_like(x)
+    lib().oracle_relu_f32_backward(_p(x), _p(out), _p(rec), x.size)
+    return out

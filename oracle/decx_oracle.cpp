@@ -27,6 +27,11 @@
 //                               fp64 7-loop brute force on tiny shapes, integer-exact vs int64.
 //   oracle_gemm_f64_rows_f16  : integer-exact vs int64, numpy float64 matmul on random data.
 //   oracle_float_to_half/back : numpy float16 casts (independent RNE implementation), IEEE known values.
+//   oracle_relu_f32[_rec|_backward] : restate srcs/nn/operators/ReLU.h:57-165 (value times float(sign bit clear); one
+//                               map byte per 8 floats).  The reference holds no test vectors for them; pinned by
+//                               numpy max(x,0) on finite data, the IEEE special cases the multiplication implies
+//                               (-x -> -0.0, -inf -> NaN, +inf kept), map bits against numpy's signbit/packbits, and
+//                               backward(rec(x)) identities.
 //
 // Build: make -C oracle   (g++ -O2 -mavx2 -mfma, see oracle/Makefile)
 
@@ -464,6 +469,39 @@ void oracle_gemm_f64_rows_f32(const float* A, long lda, const float* B, long ldb
             }
         }
     });
+}
+
+// nn/operators/ReLU.h:57-82: _sign = ~(bits & 0x80000000) >> 31 (unsigned), dst = float(_sign) * src.
+static inline float relu_by_sign(float v, unsigned* kept) {
+    uint32_t bits;
+    std::memcpy(&bits, &v, 4);
+    const unsigned s = (~(bits & 0x80000000u)) >> 31;
+    if (kept) *kept = s;
+    volatile float f = (float)s;       // keep the multiplication (0 * -inf must give NaN, 0 * -x must give -0)
+    return f * v;
+}
+void oracle_relu_f32(const float* src, float* dst, long n) {
+    for (long i = 0; i < n; ++i) dst[i] = relu_by_sign(src[i], nullptr);
+}
+// ReLU.h:86-127: thread t handles floats 8t..8t+7 as two float4; first quad -> bits 4..7, second quad -> bits 0..3.
+void oracle_relu_f32_rec(const float* src, float* dst, unsigned char* rec_map, long n) {
+    for (long t = 0; t < n / 8; ++t) {
+        unsigned mask = 0;
+        for (int e = 0; e < 8; ++e) {
+            unsigned s;
+            dst[8 * t + e] = relu_by_sign(src[8 * t + e], &s);
+            mask |= s << (e < 4 ? 4 + e : e - 4);
+        }
+        rec_map[t] = (unsigned char)mask;
+    }
+}
+// ReLU.h:131-165
+void oracle_relu_f32_backward(const float* src, float* dst, const unsigned char* rec_map, long n) {
+    for (long t = 0; t < n / 8; ++t)
+        for (int e = 0; e < 8; ++e) {
+            volatile float f = (float)((rec_map[t] >> (e < 4 ? 4 + e : e - 4)) & 1u);
+            dst[8 * t + e] = f * src[8 * t + e];
+        }
 }
 
 int oracle_pool_size(int nthreads) { return (int)global_pool(nthreads).size(); }

@@ -21,7 +21,7 @@ def pitched(arr, align, fill=np.nan):
     return buf, pitch
 
 
-def gpu_sgemm(A, B, C=None, align=8, variant=0, inplace=False):
+def gpu_sgemm(A, B, C=None, align=8, variant=0, inplace=False, relu=False):
     M, K = A.shape
     _, N = B.shape
     Ab, lda = pitched(A, align)
@@ -40,7 +40,11 @@ def gpu_sgemm(A, B, C=None, align=8, variant=0, inplace=False):
             dC = capi.DeviceBuffer.from_numpy(Cb)
     prev = capi.lib().decx_hip_set_sgemm_variant(variant)
     try:
-        capi.sgemm(dA.ptr, lda, dB.ptr, ldb, dD.ptr, ldd, M, N, K, dC.ptr if dC else None, ldc)
+        if relu:
+            capi.check(capi.lib().decx_hip_sgemm_relu(dA.ptr, lda, dB.ptr, ldb, dC.ptr if dC else None, ldc, dD.ptr, ldd,
+                                                      M, N, K))
+        else:
+            capi.sgemm(dA.ptr, lda, dB.ptr, ldb, dD.ptr, ldd, M, N, K, dC.ptr if dC else None, ldc)
     finally:
         capi.lib().decx_hip_set_sgemm_variant(prev)
     out = dD.download((M, ldd), np.float32)
@@ -83,8 +87,9 @@ def tensor_storage(t, wpitch_align=4, dpitch_align=4, pad_value=np.nan):
     return buf, wp, dp
 
 
-def gpu_conv(src, filt, flag, variant=0):
-    """src (H, W, C), filt (N, kh, kw, C) dense numpy -> dst (H_out, W_out, N), via DECX-style pitched storage."""
+def gpu_conv(src, filt, flag, variant=0, bias=None, relu=False):
+    """src (H, W, C), filt (N, kh, kw, C) dense numpy -> dst (H_out, W_out, N), via DECX-style pitched storage.
+    bias (N,) and/or relu select the fused entry point."""
     H, W, C = src.shape
     N, kh, kw, _ = filt.shape
     sbuf, swp, dp = tensor_storage(src)
@@ -100,8 +105,14 @@ def gpu_conv(src, filt, flag, variant=0):
                   capi.DeviceBuffer.from_numpy(sentinel))
     prev = capi.lib().decx_hip_set_sgemm_variant(variant)
     try:
-        capi.conv2_im2col(dS.ptr, H, W, dp, swp * dp, dF.ptr, N, kh, kw, kh * fwp * dp, fwp * dp, dD.ptr, ddp, dwp * ddp,
-                          flag)
+        if bias is None and not relu:
+            capi.conv2_im2col(dS.ptr, H, W, dp, swp * dp, dF.ptr, N, kh, kw, kh * fwp * dp, fwp * dp, dD.ptr, ddp,
+                              dwp * ddp, flag)
+        else:
+            dB = capi.DeviceBuffer.from_numpy(np.asarray(bias, dtype=np.float32)) if bias is not None else None
+            capi.check(capi.lib().decx_hip_conv2_im2col_f32_fused(
+                dS.ptr, H, W, dp, swp * dp, dF.ptr, N, kh, kw, kh * fwp * dp, fwp * dp, dD.ptr, ddp, dwp * ddp, flag,
+                dB.ptr if dB else None, 1 if relu else 0))
     finally:
         capi.lib().decx_hip_set_sgemm_variant(prev)
     out = dD.download((Ho, dwp, ddp), np.float32)

@@ -282,6 +282,54 @@ static void gemm_long_lr() {
     CHECK(de::cuda::GEMM_Long_Lr(dA, dBad, dD).error_type == decx::DECX_FAIL_DimsNotMatching);
 }
 
+static uint32_t bits_of(float v) { uint32_t b; std::memcpy(&b, &v, 4); return b; }
+static void nn_relu_family() {               // nn/operators/ReLU.h:28-34
+    const int W = 37, H = 13;                // pitch 40: the kernels run over the padding too
+    de::Matrix<float>& X = de::CreateMatrixRef<float>(W, H, 0);
+    de::Matrix<float>& G = de::CreateMatrixRef<float>(W, H, 0);
+    de::Matrix<float>& R = de::CreateMatrixRef<float>(W, H, 0);
+    fill(X, unif); fill(G, unif);
+    X.index(0, 0) = 0.f; X.index(0, 1) = -0.f; X.index(0, 2) = -INFINITY; X.index(0, 3) = INFINITY;
+    de::GPU_Matrix<float>& dX = de::CreateGPUMatrixRef<float>(W, H);
+    de::GPU_Matrix<float>& dY = de::CreateGPUMatrixRef<float>(W, H);
+    de::GPU_Matrix<float>& dG = de::CreateGPUMatrixRef<float>(W, H);
+    de::GPU_Matrix<uchar>& dMap = de::CreateGPUMatrixRef<uchar>();
+    dX.Load_from_host(X); dG.Load_from_host(G);
+    auto expect_forward = [&](de::Matrix<float>& got) {
+        int bad = 0;
+        for (int i = 0; i < H; ++i)
+            for (int j = 0; j < W; ++j) {
+                const float x = X.index(i, j), y = got.index(i, j);
+                if (std::isinf(x) && x < 0) bad += !std::isnan(y);                       // 0 * -inf
+                else if (std::signbit(x)) bad += bits_of(y) != 0x80000000u;             // 0 * negative = -0.0
+                else bad += bits_of(y) != bits_of(x);
+            }
+        return bad;
+    };
+    CHECK(de::nn::ReLU_f(dX, dY).error_type == decx::DECX_SUCCESS);
+    dY.Load_to_host(R);
+    CHECK(expect_forward(R) == 0);
+    de::GPU_Matrix<float>& dY2 = de::CreateGPUMatrixRef<float>(W, H);
+    CHECK(de::nn::ReLU_f_Rec(dX, dY2, dMap).error_type == decx::DECX_SUCCESS);
+    CHECK(dMap.TotalBytes() >= (size_t)40 * H / 8);
+    dY2.Load_to_host(R);
+    CHECK(expect_forward(R) == 0);
+    CHECK(de::nn::ReLU_f_Backward(dG, dY, dMap).error_type == decx::DECX_SUCCESS);
+    dY.Load_to_host(R);
+    int bad = 0;
+    for (int i = 0; i < H; ++i)
+        for (int j = 0; j < W; ++j) {
+            const float g = G.index(i, j);
+            const uint32_t want = std::signbit(X.index(i, j)) ? (bits_of(g) & 0x80000000u) : bits_of(g);   // 0 * g keeps g's sign
+            bad += bits_of(R.index(i, j)) != want;
+        }
+    CHECK(bad == 0);
+    de::GPU_Matrix<float>& dBad = de::CreateGPUMatrixRef<float>(W + 1, H);
+    CHECK(de::nn::ReLU_f(dX, dBad).error_type == decx::DECX_FAIL_DimsNotMatching);
+    de::GPU_Matrix<uchar>& dEmpty = de::CreateGPUMatrixRef<uchar>();
+    CHECK(de::nn::ReLU_f_Backward(dG, dY, dEmpty).error_type == decx::DECX_FAIL_DimsNotMatching);
+}
+
 static void gemm3_matrix_arrays() {
     const int M = 150, K = 90, N = 210, NUM = 5;
     de::MatrixArray<float>& A = de::CreateMatrixArrayRef<float>(K, M, NUM, 0);
@@ -388,6 +436,7 @@ int main(int argc, char** argv) {
         RUN(conv_device_resident);
         RUN(gemm3_matrix_arrays);
         RUN(gemm_long_lr);
+        RUN(nn_relu_family);
     }
     std::printf("%s: %d failure(s)\n", mode.c_str(), g_fail);
     return g_fail ? 1 : 0;

@@ -1,0 +1,108 @@
+"""ReLU family (decx_hip_relu_f32 / _rec / _backward) and the fused conv / GEMM epilogues on the GPU, against the
+CPU oracle's restatement of nn/operators/ReLU.h.  Everything here is bit-exact: the arithmetic is one multiplication
+by 0.0f or 1.0f per element."""
+import numpy as np
+import pytest
+
+from backup_1_amd import capi, workloads
+from gpu_helpers import gpu_conv, gpu_sgemm
+
+pytestmark = pytest.mark.gpu
+
+SPECIALS = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, 1e-45, -1e-45, 3.4e38, -3.4e38, 1.17549435e-38, -1.17549435e-38],
+                    dtype=np.float32)
+
+
+def bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+def same_bits_or_both_nan(got, ref):
+    nan = np.isnan(ref)
+    return np.array_equal(np.isnan(got), nan) and np.array_equal(bits(got)[~nan], bits(ref)[~nan])
+
+
+def data_with_specials(n, seed):
+    x = workloads.normal((n,), seed)
+    k = min(n, SPECIALS.size)
+    x[:k] = SPECIALS[:k]
+    return x
+
+
+def run_forward(x, inplace=False):
+    d_src = capi.DeviceBuffer.from_numpy(x)
+    d_dst = d_src if inplace else capi.DeviceBuffer.from_numpy(np.full(x.size + 8, -777.0, np.float32))
+    capi.check(capi.lib().decx_hip_relu_f32(d_src.ptr, d_dst.ptr, x.size))
+    if inplace:
+        return d_dst.download((x.size,), np.float32)
+    out = d_dst.download((x.size + 8,), np.float32)
+    assert np.all(out[x.size:] == -777.0), "wrote past n"
+    return out[:x.size]
+
+
+@pytest.mark.parametrize("n", [1, 7, 8, 9, 64, 1000, 4096, 65543, 1 << 20, (1 << 22) + 5])
+def test_forward_bit_exact(gpu, oracle, n):
+    x = data_with_specials(n, 900 + n % 97)
+    assert same_bits_or_both_nan(run_forward(x), oracle.relu(x))
+
+
+def test_forward_in_place_and_pitched_matrix(gpu, oracle):
+    # de::nn::ReLU_f runs over pitch*height floats of a GPU_Matrix, padding included (ReLU.h:169-180)
+    x = data_with_specials(37 * 104, 17)
+    assert same_bits_or_both_nan(run_forward(x, inplace=True), oracle.relu(x))
+
+
+@pytest.mark.parametrize("n", [8, 16, 8 * 777, 1 << 20, 8 * 500001])
+def test_rec_and_backward_bit_exact(gpu, oracle, n):
+    x = data_with_specials(n, 40 + n % 89)
+    g = workloads.normal((n,), 41 + n % 89)
+    d_x, d_y = capi.DeviceBuffer.from_numpy(x), capi.DeviceBuffer(n * 4)
+    d_map = capi.DeviceBuffer.from_numpy(np.full(n // 8 + 16, 0xAA, np.uint8))
+    capi.check(capi.lib().decx_hip_relu_f32_rec(d_x.ptr, d_y.ptr, d_map.ptr, n))
+    y, m = d_y.download((n,), np.float32), d_map.download((n // 8 + 16,), np.uint8)
+    ref_y, ref_m = oracle.relu_rec(x)
+    assert same_bits_or_both_nan(y, ref_y)
+    assert np.array_equal(m[:n // 8], ref_m) and np.all(m[n // 8:] == 0xAA)
+    d_g, d_gx = capi.DeviceBuffer.from_numpy(g), capi.DeviceBuffer(n * 4)
+    capi.check(capi.lib().decx_hip_relu_f32_backward(d_g.ptr, d_gx.ptr, d_map.ptr, n))
+    assert same_bits_or_both_nan(d_gx.download((n,), np.float32), oracle.relu_backward(g, ref_m))
+
+
+def test_argument_errors(gpu):
+    d = capi.DeviceBuffer(64)
+    L = capi.lib()
+    assert L.decx_hip_relu_f32(None, d.ptr, 8) == 0x0d
+    assert L.decx_hip_relu_f32_rec(d.ptr, d.ptr, d.ptr, 12) == 0x0d          # not whole map bytes
+    assert L.decx_hip_relu_f32_rec(d.ptr, d.ptr, None, 8) == 0x0d
+    assert L.decx_hip_relu_f32(d.ptr + 4, d.ptr, 4) == 0x0d                  # misaligned
+    assert L.decx_hip_relu_f32(d.ptr, d.ptr, 0) == 0
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6])
+def test_fused_conv_bias_relu_equals_separate_passes(gpu, oracle, variant):
+    H, W, C, N = 29, 31, 12, 70
+    src, filt = workloads.normal((H, W, C), 5), workloads.normal((N, 3, 3, C), 6)
+    bias = workloads.normal((N,), 7)
+    plain = gpu_conv(src, filt, 1, variant=variant)
+    # the fused kernel adds bias[n] to the finished fp32 sum and applies the activation: one fp32 add, one multiply
+    assert np.array_equal(bits(gpu_conv(src, filt, 1, variant=variant, bias=bias)), bits(plain + bias[None, None, :]))
+    assert np.array_equal(bits(gpu_conv(src, filt, 1, variant=variant, relu=True)), bits(oracle.relu(plain)))
+    both = gpu_conv(src, filt, 0, variant=variant, bias=bias, relu=True)
+    assert np.array_equal(bits(both), bits(oracle.relu(gpu_conv(src, filt, 0, variant=variant) + bias[None, None, :])))
+    assert np.signbit(both).any() and (both > 0).any()      # negative sums came out as -0.0, positive ones survived
+
+
+def test_fused_conv_integer_exact_against_oracle(gpu, oracle):
+    src = workloads.small_ints((40, 50, 16), 11, -4, 4)
+    filt = workloads.small_ints((130, 3, 3, 16), 12, -4, 4)
+    bias = workloads.small_ints((130,), 13, -50, 50)
+    ref = oracle.relu(oracle.conv2_chain(src, filt, 1) + bias[None, None, :])
+    assert np.array_equal(bits(gpu_conv(src, filt, 1, bias=bias, relu=True)), bits(ref))
+
+
+@pytest.mark.parametrize("shape", [(64, 64, 64), (300, 150, 450), (257, 1000, 129)])
+def test_sgemm_relu_epilogue(gpu, oracle, shape):
+    M, K, N = shape
+    A, B, C = workloads.normal((M, K), 1), workloads.normal((K, N), 2), workloads.normal((M, N), 3)
+    assert np.array_equal(bits(gpu_sgemm(A, B, relu=True)), bits(oracle.relu(gpu_sgemm(A, B))))
+    assert np.array_equal(bits(gpu_sgemm(A, B, C=C, relu=True)), bits(oracle.relu(gpu_sgemm(A, B, C=C))))

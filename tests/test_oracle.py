@@ -258,3 +258,46 @@ def test_f64_rows(oracle):
     refh, _ = oracle.gemm_f64_rows_f16(Ah, Bh, rows)
     want = (Ah.view(np.float16).astype(np.float64) @ Bh.view(np.float16).astype(np.float64))[rows]
     np.testing.assert_allclose(refh, want, rtol=1e-12, atol=1e-12)
+
+
+# ---- ReLU family (nn/operators/ReLU.h:57-165).  The reference holds no vectors for it; the restatement is pinned by
+# ---- an independent library routine on finite data, the IEEE special cases its multiplication implies, and identities.
+def test_relu_matches_numpy_maximum_on_finite_data(oracle):
+    x = workloads.normal((10007,), 3)
+    y = oracle.relu(x)
+    assert np.array_equal(y, np.maximum(x, np.float32(0)))            # value equality (-0.0 == 0.0)
+    assert np.array_equal(np.signbit(y), x < 0)                       # a zeroed negative keeps its sign: 0 * x = -0.0
+
+
+def test_relu_ieee_special_cases(oracle):
+    x = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 2.5], dtype=np.float32)
+    y = oracle.relu(x)
+    assert y[0] == 0 and not np.signbit(y[0])
+    assert y[1] == 0 and np.signbit(y[1])             # sign bit set -> multiplied by 0
+    assert y[2] == np.inf
+    assert np.isnan(y[3])                             # 0 * -inf
+    assert np.isnan(y[4])
+    assert y[5] == np.float32(1e-45) and y[6] == 0 and np.signbit(y[6]) and y[7] == 2.5
+
+
+def test_relu_rec_map_bits_match_packbits(oracle):
+    x = workloads.normal((8 * 1000,), 4)
+    y, rec = oracle.relu_rec(x)
+    assert np.array_equal(y.view(np.uint32), oracle.relu(x).view(np.uint32))
+    kept = (~np.signbit(x)).reshape(-1, 2, 4)          # [byte][quad][lane]
+    # byte = first quad in bits 4..7 (x -> bit 4 ... w -> bit 7), second quad in bits 0..3 (ReLU.h:105-113)
+    order = np.concatenate([kept[:, 1, :], kept[:, 0, :]], axis=1)       # bit 0 .. bit 7
+    assert np.array_equal(rec, np.packbits(order, axis=1, bitorder="little").ravel())
+
+
+def test_relu_backward_identities(oracle):
+    x, g = workloads.normal((8 * 513,), 5), workloads.normal((8 * 513,), 6)
+    _, rec = oracle.relu_rec(x)
+    gx = oracle.relu_backward(g, rec)
+    assert np.array_equal(gx, np.where(x >= 0, g, np.float32(0)))      # values
+    assert np.array_equal(np.signbit(gx), np.signbit(g))               # 0 * g and 1 * g both keep g's sign
+    ones = np.full(x.size // 8, 0xFF, np.uint8)
+    assert np.array_equal(oracle.relu_backward(g, ones).view(np.uint32), g.view(np.uint32))   # all kept: identity
+    assert np.all(oracle.relu_backward(g, np.zeros_like(ones)) == 0)
+    # backward with the map of x applied to x itself reproduces forward
+    assert np.array_equal(oracle.relu_backward(x, rec).view(np.uint32), oracle.relu(x).view(np.uint32))
