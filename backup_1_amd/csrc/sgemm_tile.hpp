@@ -42,8 +42,19 @@ namespace decx_hip {
 // need no fold: consecutive slots are read, and the planes are 2 slots out of step for the staging stores.
 __device__ __forceinline__ int b_slot(int n) { return n ^ ((n >> 3) & 3); }
 
+// A K step of dk as an increment of the im2col position (c, kj, ki): dk = (dki*kw + dkj)*dpitch + dc.  Worked out once
+// per kernel so that advancing is a handful of adds and selects.
+struct TapStep {
+    int dk, dc, dkj, dki;
+    __device__ __forceinline__ static TapStep make(int dk, int dpitch, int kw) {
+        const int taps = dk / dpitch, rows = taps / kw;
+        return TapStep{dk, dk - taps * dpitch, taps - rows * kw, rows};
+    }
+};
+
 // Position of one k index inside the im2col ordering k = (ki*kw + kj)*dpitch + c.  Decoded once (two integer
-// divisions), then advanced by whole K steps with additions only.
+// divisions), then advanced by whole K steps without divisions, loops or branches (control flow inside the K loop
+// would split its body into basic blocks and undo the instruction schedule).
 struct TapWalk {
     int k, c, ki, kj;
     __device__ __forceinline__ void init(int k_, int dpitch, int kw) {
@@ -53,16 +64,15 @@ struct TapWalk {
         ki = tap / kw;
         kj = tap - ki * kw;
     }
-    __device__ __forceinline__ void advance(int dk, int dpitch, int kw) {
-        k += dk;
-        c += dk;
-        while (c >= dpitch) {
-            c -= dpitch;
-            if (++kj == kw) {
-                kj = 0;
-                ++ki;
-            }
-        }
+    __device__ __forceinline__ void advance(const TapStep& st, int dpitch, int kw) {
+        k += st.dk;
+        c += st.dc;
+        const int carry_c = c >= dpitch ? 1 : 0;          // c < 2*dpitch: one carry at most
+        c -= carry_c ? dpitch : 0;
+        kj += st.dkj + carry_c;
+        const int carry_kj = kj >= kw ? 1 : 0;            // kj <= 2*kw - 1: one carry at most
+        kj -= carry_kj ? kw : 0;
+        ki += st.dki + carry_kj;
     }
 };
 
@@ -79,8 +89,12 @@ struct DenseA {
     struct KState {
         int k;
     };
+    struct KStep {
+        int dk;
+    };
     __device__ __forceinline__ KState k_state(int k) const { return KState{k}; }
-    __device__ __forceinline__ void advance(KState& ks, int dk) const { ks.k += dk; }
+    __device__ __forceinline__ KStep k_step(int dk) const { return KStep{dk}; }
+    __device__ __forceinline__ void advance(KState& ks, const KStep& st) const { ks.k += st.dk; }
     __device__ __forceinline__ RowState row_state(int m) const {
         RowState rs;
         rs.row = A + (size_t)(m < M ? m : M - 1) * lda;
@@ -136,7 +150,9 @@ struct Im2colA {
         ks.init(k, dpitch, kw);
         return ks;
     }
-    __device__ __forceinline__ void advance(KState& ks, int dk) const { ks.advance(dk, dpitch, kw); }
+    typedef TapStep KStep;
+    __device__ __forceinline__ KStep k_step(int dk) const { return TapStep::make(dk, dpitch, kw); }
+    __device__ __forceinline__ void advance(KState& ks, const KStep& st) const { ks.advance(st, dpitch, kw); }
     template <bool TAIL>
     __device__ __forceinline__ f32x4 load(const RowState& rs, const KState& ks, bool& keep) const {
         // K = kh*kw*dpitch is a multiple of 4: quads never straddle it.  A tap outside the image (or k >= K, TAIL only)
@@ -199,10 +215,14 @@ struct DenseB {
     struct KState {
         int k0;
     };
+    struct KStep {
+        int dk;
+    };
     template <class S>
     __device__ __forceinline__ KState k_state(int tid, int k_begin) const { return KState{k_begin}; }
     template <class S>
-    __device__ __forceinline__ void advance(KState& ks) const { ks.k0 += S::BK; }
+    __device__ __forceinline__ KStep k_step() const { return KStep{S::BK}; }
+    __device__ __forceinline__ void advance(KState& ks, const KStep& st) const { ks.k0 += st.dk; }
 
     template <class S, bool TAIL>
     __device__ __forceinline__ void load(f32x4* st, int tid, const KState& ks, int bn0) const {
@@ -267,8 +287,10 @@ struct FilterB {
         ks.init(k_begin + 4 * (tid % S::KQ), dpitch, kw);
         return ks;
     }
+    typedef TapStep KStep;
     template <class S>
-    __device__ __forceinline__ void advance(KState& ks) const { ks.advance(S::BK, dpitch, kw); }
+    __device__ __forceinline__ KStep k_step() const { return TapStep::make(S::BK, dpitch, kw); }
+    __device__ __forceinline__ void advance(KState& ks, const KStep& st) const { ks.advance(st, dpitch, kw); }
 
     template <class S, bool TAIL>
     __device__ __forceinline__ void load(f32x4* st, int tid, const KState& ks, int bn0) const {
@@ -310,9 +332,13 @@ struct SgemmShape {
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     static constexpr int MI = WM / 32, NI = WN / 32;
     static constexpr int KQ = BK / 4;                         // k-quads per step
-    static constexpr int A_ROW = BM + 2;                      // quads per A plane (planes 2 slots out of step mod 8)
+    static constexpr int A_PASSES = (BM * KQ + NT - 1) / NT;  // float4 global loads of A per thread per step
+    // When BM*KQ is not a multiple of NT the last pass covers rows past BM: they are staged like any other (loaded from
+    // the tile's first row, stored to plane rows BM .. A_STAGED_ROWS-1 that no wave reads), which keeps the K loop free of
+    // branches -- a divergent skip would split the loop body into basic blocks and undo its instruction schedule.
+    static constexpr int A_STAGED_ROWS = A_PASSES * (NT / KQ);
+    static constexpr int A_ROW = A_STAGED_ROWS + 2;           // quads per A plane (planes 2 slots out of step mod 8)
     static constexpr int B_ROW = BN + 2;                      // quads per B plane
-    static constexpr int A_PASSES = (BM * KQ + NT - 1) / NT;  // float4 global loads of A per thread per step (last may be partial)
     static constexpr bool A_PARTIAL = (BM * KQ) % NT != 0;
     static constexpr size_t LDS_BYTES = 2 * (size_t)KQ * (A_ROW + B_ROW) * sizeof(f32x4);
     static_assert(BM % (WAVES_M * 32) == 0 && BN % (WAVES_N * 32) == 0, "wave tile must be whole 32x32 blocks");
@@ -371,19 +397,18 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
     f32x4 b_stage[SETS][B_QUADS];
     typename ASrc::KState a_ks = a_src.k_state(k_begin + 4 * a_q);   // this thread's k-quad of the next K step to fetch
     typename BSrc::KState b_ks = b_src.template k_state<S>(tid, k_begin);
+    const typename ASrc::KStep a_step = a_src.k_step(BK);
+    const typename BSrc::KStep b_step = b_src.template k_step<S>();
 
     // fetches the next K step (steps are always taken in order) into register set SET and moves the k positions on
     auto load_stage = [&](auto set_tag, auto tail_tag) {
         constexpr int SET = decltype(set_tag)::value;
         constexpr bool TAIL = decltype(tail_tag)::value;
 #pragma unroll
-        for (int p = 0; p < S::A_PASSES; ++p) {
-            if (S::A_PARTIAL && a_r + p * A_RSTEP >= BM) continue;
-            a_stage[SET][p] = a_src.template load<TAIL>(a_rs[p], a_ks, a_keep[SET][p]);
-        }
+        for (int p = 0; p < S::A_PASSES; ++p) a_stage[SET][p] = a_src.template load<TAIL>(a_rs[p], a_ks, a_keep[SET][p]);
         b_src.template load<S, TAIL>(b_stage[SET], tid, b_ks, bn0);
-        a_src.advance(a_ks, BK);
-        b_src.template advance<S>(b_ks);
+        a_src.advance(a_ks, a_step);
+        b_src.advance(b_ks, b_step);
     };
 
     auto store_stage = [&](auto set_tag, int buf) {
@@ -391,7 +416,6 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         f32x4* Ab = As + buf * KQ * S::A_ROW;
 #pragma unroll
         for (int p = 0; p < S::A_PASSES; ++p) {
-            if (S::A_PARTIAL && a_r + p * A_RSTEP >= BM) continue;
             const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
             Ab[a_q * S::A_ROW + a_r + p * A_RSTEP] = a_keep[SET][p] ? a_stage[SET][p] : zero;
         }
