@@ -74,14 +74,14 @@ int launch_sgemm_tile_c(const ASrc& a, const BSrc& b, const float* Cin, int ldc,
     static bool attr_done = false;
     if (!attr_done) {
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)S::LDS_BYTES));
+                                    (int)S::template lds_bytes<BSrc>()));
         attr_done = true;
     }
     const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
     const long total = (long)tiles_m * tiles_n;
     if (total > 0x7fffffffL || batch.count > 65535) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
     const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
-    hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::LDS_BYTES, batch.stream, a, b, Cin,
+    hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::template lds_bytes<BSrc>(), batch.stream, a, b, Cin,
                        ldc, D, out, M, N, K, tiles_m, tiles_n, group_m, batch.stride_c, batch.stride_d, 0);
     HIP_TRY(hipGetLastError());
     return 0;
@@ -106,9 +106,9 @@ int launch_sgemm_splitk(const float* A, int lda, const float* B, int ldb, const 
     static bool attr_done = false;
     if (!attr_done) {
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(sgemm_tile_kernel<S, ASrc, BSrc, DenseOut, true, true>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::template lds_bytes<BSrc>()));
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(sgemm_tile_kernel<S, ASrc, BSrc, DenseOut, false, true>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::template lds_bytes<BSrc>()));
         attr_done = true;
     }
     if (!in_place) {
@@ -121,7 +121,7 @@ int launch_sgemm_splitk(const float* A, int lda, const float* B, int ldb, const 
     ASrc a{A, lda, M, K, 0};
     BSrc b{B, ldb, N, K, 0};
     DenseOut out{ldd};
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)splits), dim3(S::NT), S::LDS_BYTES, g_rt.stream, a,
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)splits), dim3(S::NT), S::template lds_bytes<BSrc>(), g_rt.stream, a,
                        b, Cin, ldc, D, out, M, N, K, tiles_m, tiles_n, group_m, (size_t)0, (size_t)0, k_split_len);
     HIP_TRY(hipGetLastError());
     return 0;
@@ -139,6 +139,9 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //   2: 128x128x16, 2x2 waves of  64x64    -- small problems, several workgroups per CU
 //   3: 256x128x16, 2x2 waves of 128x64    -- narrow N
 //   4: 224x128x16, 1x4 waves of 224x32    -- 7/8 of shape 3 per tile: fills more CUs when M/256 tiles leave many idle
+//   7: 256x256x16, 4x2 waves of  64x128   -- two waves per SIMD: the matrix pipe takes the next MFMA from the other wave
+//         while one wave issues its loads and LDS traffic (a lone wave leaves ~3.5 idle cycles between 64-cycle MFMAs);
+//         the default for large problems, 1-2 % ahead of shape 1
 //   5, 6: shapes 3 and 4 compiled for one wave per SIMD (512 registers, two staging sets) -- for launches that put at
 //         most one workgroup on a CU anyway, where a second resident workgroup cannot be what hides the load latency
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
@@ -147,22 +150,23 @@ typedef SgemmShape<256, 128, 16, 2, 2, 2> SShapeTall;
 typedef SgemmShape<224, 128, 16, 1, 4, 2> SShape224;
 typedef SgemmShape<256, 128, 16, 2, 2, 1> SShapeTallSolo;
 typedef SgemmShape<224, 128, 16, 1, 4, 1> SShape224Solo;
+typedef SgemmShape<256, 256, 16, 4, 2, 2, 2> SShapeBig8;
 
 // Tile shape by a small cost model: a CU works through ceil(tiles / CUs) tiles one after another, a tile costs its area
 // divided by how well that shape keeps the matrix pipe busy (measured on 8192^3, relative to shape 1).
 int pick_sgemm_variant(int M, int N, int batch) {
-    if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 6) return g_rt.sgemm_variant;
+    if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 7) return g_rt.sgemm_variant;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     struct Cand { int variant, bm, bn; double eff; };
-    const Cand cands[] = {{1, 256, 256, 1.00}, {3, 256, 128, 0.95}, {4, 224, 128, 0.85}, {2, 128, 128, 0.90}};
-    int best = 1;
+    const Cand cands[] = {{7, 256, 256, 1.00}, {3, 256, 128, 0.93}, {4, 224, 128, 0.83}, {2, 128, 128, 0.89}};
+    int best = 7;
     double best_cost = 0.0;
     for (const Cand& c : cands) {
         const long tiles = (long)cdiv(M, c.bm) * cdiv(N, c.bn) * batch;
         const double cost = (double)((tiles + cus - 1) / cus) * c.bm * c.bn / c.eff;
         if (best_cost == 0.0 || cost < best_cost) {
             best_cost = cost;
-            best = (tiles <= cus && c.variant >= 3) ? c.variant + 2 : c.variant;
+            best = (tiles <= cus && (c.variant == 3 || c.variant == 4)) ? c.variant + 2 : c.variant;
         }
     }
     return best;
@@ -177,6 +181,7 @@ int dispatch_sgemm(int variant, const ASrc& a, const BSrc& b, const float* Cin, 
         case 4: return launch_sgemm_tile<SShape224>(a, b, Cin, ldc, D, out, M, N, K, batch);
         case 5: return launch_sgemm_tile<SShapeTallSolo>(a, b, Cin, ldc, D, out, M, N, K, batch);
         case 6: return launch_sgemm_tile<SShape224Solo>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 7: return launch_sgemm_tile<SShapeBig8>(a, b, Cin, ldc, D, out, M, N, K, batch);
         default: return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K, batch);
     }
 }
@@ -200,7 +205,7 @@ int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float*
     const int variant = pick_sgemm_variant(M, N, batch.count);
     const bool vec_a = aligned16(A) && lda % 4 == 0 && batch.stride_a % 4 == 0;
     const bool vec_b = aligned16(B) && ldb % 4 == 0 && ldb >= 4 && batch.stride_b % 4 == 0;
-    DenseOut out{ldd, relu};
+    DenseOut out{ldd, relu, aligned16(D) && ldd % 4 == 0 && batch.stride_d % 4 == 0};
     if (vec_a && vec_b) {
         DenseA<true> a{A, lda, M, K, batch.stride_a};
         DenseB<true> b{B, ldb, N, K, batch.stride_b};

@@ -4,16 +4,22 @@
 // WAVES_N, each owning a (BM/WAVES_M) x (BN/WAVES_N) sub-tile as a grid of 32x32 v_mfma_f32_32x32x2_f32 blocks
 // whose accumulators stay in registers for the whole K walk.
 //
-// Staging: global -> registers -> LDS, two LDS buffers, one barrier per K step; the loads for step t+1 are issued
-// before the MFMAs of step t.  Both operands are kept in LDS as float4 "k-quads":
-//   A quad (q, m) = A[m][4q .. 4q+3]          at  As[q][m]             (row of BM+4 quads: the +4 staggers the four
-//                                                                       q-planes over the banks for the staging stores)
-//   B quad (q, n) = B[4q .. 4q+3][n]          at  Bs[q][b_slot(n)]  (4x4 register transpose while staging; the
-//                                                                       n>>4 skew keeps the 64-byte-strided staging
-//                                                                       stores off each other's banks)
+// Staging: global -> registers -> LDS, two LDS buffers, one barrier per K step; the loads run one or two K steps ahead
+// of the MFMAs.  A is kept in LDS as float4 "k-quads":
+//   A quad (q, m) = A[m][4q .. 4q+3]          at  As[q][m]             (plane rows 2 slots out of step mod 8, which
+//                                                                       keeps the staging stores off each other's banks)
 // so that one ds_read_b128 per 32-row block feeds four MFMAs.  The MFMA's two k-slots (lanes 0-31 / 32-63) take
 // quads 2s and 2s+1: within a quad pair the products are summed in the order k = 8s+e (lanes 0-31) and 8s+4+e
 // (lanes 32-63), e = 0..3 -- a fixed permutation of k inside each group of 8, applied identically to A and B.
+// B has two LDS layouts, chosen by its source:
+//   * a row-major K x N matrix (DenseB) stays row-major, Bs[k][n], exactly as loaded -- no transpose, no VALU work.
+//     The wave's 32x32 blocks then take INTERLEAVED columns: lane li of block ni owns column NI*li + ni of the wave's
+//     strip, so the NI operands a lane needs at one k are NI consecutive floats of one row (one ds_read_b128 for
+//     NI = 4) and the NI results it holds per row are consecutive too (one 16-byte store).
+//   * a filter bank (FilterB), whose k runs contiguously per column, is kept as k-quads like A:
+//       B quad (q, n) = B[4q .. 4q+3][n]      at  Bs[q][b_slot(n)];  block ni takes columns 32*ni + li.
+// Every VALU instruction costs the matrix pipe 3-5 cycles (measured: a wave's VALU and MFMA work do not overlap), so
+// the K loop is kept as free of address arithmetic and data shuffling as the layouts allow.
 //
 // Ragged edges: rows >= M and columns >= N are read from clamped (valid) addresses and never stored; only the last,
 // partial K step zero-fills (both operands, so that 0 * Inf cannot appear).  No padded copies exist anywhere.
@@ -174,6 +180,7 @@ __device__ __forceinline__ float relu_by_sign(float v) {
 struct DenseOut {
     int ld;
     bool relu = false;
+    bool vec = false;      // every row of the result starts 16-byte aligned: runs of consecutive columns go out as one store
     __device__ __forceinline__ size_t offset(int m) const { return (size_t)m * ld; }
     __device__ __forceinline__ float finish(float v) const { return relu ? relu_by_sign(v) : v; }
 };
@@ -182,6 +189,7 @@ struct TensorOut {
     size_t row_stride;
     bool dense;      // row_stride == Wout*dpitch: pixel m simply starts at m*dpitch, no division needed
     bool relu = false;
+    static constexpr bool vec = false;
     __device__ __forceinline__ float finish(float v) const { return relu ? relu_by_sign(v) : v; }
     __device__ __forceinline__ size_t offset(int m) const {
         if (dense) return (size_t)m * dpitch;
@@ -197,21 +205,29 @@ struct TensorOut {
 //   load<S, TAIL>(stage, tid, ks, bn0)           fetch this thread's share of B[k0 .. k0+BK) x [bn0 .. bn0+BN)
 //   store<S>(plane, stage, tid)                  write it to the LDS planes as k-quads at [q][b_slot(n)]
 // ---------------------------------------------------------------------------------------------------------------
-// B as a row-major K x N matrix: a thread takes a 4(k) x 4(n) block with four 16-byte row loads (consecutive lanes
-// -> consecutive column groups, so a wave reads whole rows) and transposes it in registers into four k-quads.
+// B as a row-major K x N matrix.  Staging copies 16-byte pieces of rows straight through: task t of a K step is
+// row t / (BN/4), column group t % (BN/4), so a wave reads and writes whole kilobytes of consecutive addresses.  Rows
+// are BN + 8 floats apart in LDS: the two half-waves of a fragment read touch rows 4 apart, and 4*(BN+8) floats puts
+// them on opposite halves of the 64 banks.
 template <bool VEC>
 struct DenseB {
     const float* B;
     int ldb, N, K;
     size_t batch_stride;
+    static constexpr bool ROW_MAJOR_LDS = true;
     __device__ __forceinline__ void select_batch(int b) { B += (size_t)b * batch_stride; }
     __device__ __forceinline__ void set_k_end(int k_end) { K = k_end; }
     template <class S>
-    static constexpr int tasks() { return S::KQ * (S::BN / 4); }
+    static constexpr int row_floats() { return S::BN + 8; }
     template <class S>
-    static constexpr int passes() { return (tasks<S>() + S::NT - 1) / S::NT; }
+    static constexpr int lds_floats() { return S::BK * row_floats<S>(); }      // one buffer
     template <class S>
-    static constexpr int quads() { return 4 * passes<S>(); }
+    static constexpr int quads() {
+        static_assert((S::BK * S::BN / 4) % S::NT == 0, "B staging must divide evenly over the threads");
+        return S::BK * S::BN / 4 / S::NT;
+    }
+    template <class S>
+    static constexpr int frag_reads() { return 4; }                           // LDS reads per quad pair: one per k-slot pair
     struct KState {
         int k0;
     };
@@ -226,48 +242,48 @@ struct DenseB {
 
     template <class S, bool TAIL>
     __device__ __forceinline__ void load(f32x4* st, int tid, const KState& ks, int bn0) const {
-        const int k0 = ks.k0;
         constexpr int CG = S::BN / 4;
 #pragma unroll
-        for (int p = 0; p < passes<S>(); ++p) {
+        for (int p = 0; p < quads<S>(); ++p) {
             const int task = tid + p * S::NT;
-            if (tasks<S>() % S::NT != 0 && task >= tasks<S>()) break;
-            const int q = task / CG, cg = task % CG;
-            const int col = bn0 + 4 * cg;
+            const int k = ks.k0 + task / CG, col = bn0 + 4 * (task % CG);
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            if (!TAIL || k < K) {
+                if (VEC) {
+                    const int cc = col <= ldb - 4 ? col : ldb - 4;   // stay inside the pitch; such columns are never stored
+                    v = *reinterpret_cast<const f32x4*>(B + (size_t)k * ldb + cc);
+                } else {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int k = k0 + 4 * q + r;
-                f32x4 v = {0.f, 0.f, 0.f, 0.f};
-                if (!TAIL || k < K) {
-                    if (VEC) {
-                        const int cc = col <= ldb - 4 ? col : ldb - 4;   // stay inside the pitch; such columns are never stored
-                        v = *reinterpret_cast<const f32x4*>(B + (size_t)k * ldb + cc);
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (col + e < N) v[e] = B[(size_t)k * ldb + col + e];
-                    }
+                    for (int e = 0; e < 4; ++e)
+                        if (col + e < N) v[e] = B[(size_t)k * ldb + col + e];
                 }
-                st[4 * p + r] = v;
             }
+            st[p] = v;
         }
     }
     template <class S>
-    __device__ __forceinline__ void store(f32x4* plane, const f32x4* st, int tid) const {
+    __device__ __forceinline__ void store(float* buf, const f32x4* st, int tid) const {
         constexpr int CG = S::BN / 4;
 #pragma unroll
-        for (int p = 0; p < passes<S>(); ++p) {
+        for (int p = 0; p < quads<S>(); ++p) {
             const int task = tid + p * S::NT;
-            if (tasks<S>() % S::NT != 0 && task >= tasks<S>()) break;
-            const int q = task / CG, cg = task % CG;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int n = 4 * cg + j;
-                f32x4 t = {st[4 * p + 0][j], st[4 * p + 1][j], st[4 * p + 2][j], st[4 * p + 3][j]};
-                plane[q * S::B_ROW + b_slot(n)] = t;
-            }
+            *reinterpret_cast<f32x4*>(buf + (task / CG) * row_floats<S>() + 4 * (task % CG)) = st[p];
         }
     }
+    // operands of quad pair s for this lane: frag[e][ni] = B[k(s, e, lh)][wn0 + NI*li + ni], k = 8s + 4lh + e
+    template <class S>
+    __device__ __forceinline__ void read_frags(const float* buf, int s, int lh, int li, int wn0, float (*frag)[S::NI]) const {
+        typedef float vec_t __attribute__((ext_vector_type(S::NI)));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const vec_t v = *reinterpret_cast<const vec_t*>(buf + (8 * s + 4 * lh + e) * row_floats<S>() + wn0 + S::NI * li);
+#pragma unroll
+            for (int ni = 0; ni < S::NI; ++ni) frag[e][ni] = v[ni];
+        }
+    }
+    // column (relative to the wave's strip) held by lane li in block ni
+    template <class S>
+    __device__ __forceinline__ static int strip_col(int ni, int li) { return S::NI * li + ni; }
 };
 
 // B as a bank of N filters, filter n holding its taps channel-innermost: column n of the lowered GEMM is filter n and
@@ -278,8 +294,13 @@ struct FilterB {
     size_t filt_stride, filt_row_stride;
     __device__ __forceinline__ void select_batch(int) {}
     __device__ __forceinline__ void set_k_end(int k_end) { K = k_end; }
+    static constexpr bool ROW_MAJOR_LDS = false;
     template <class S>
     static constexpr int quads() { return S::KQ * S::BN / S::NT; }
+    template <class S>
+    static constexpr int lds_floats() { return 4 * S::KQ * S::B_ROW; }          // one buffer
+    template <class S>
+    static constexpr int frag_reads() { return S::NI; }                        // one k-quad per 32-column block
     typedef TapWalk KState;       // every quad of a thread has the same k-quad index q = tid % KQ (NT is a multiple of KQ)
     template <class S>
     __device__ __forceinline__ KState k_state(int tid, int k_begin) const {
@@ -308,7 +329,8 @@ struct FilterB {
         }
     }
     template <class S>
-    __device__ __forceinline__ void store(f32x4* plane, const f32x4* st, int tid) const {
+    __device__ __forceinline__ void store(float* buf, const f32x4* st, int tid) const {
+        f32x4* plane = reinterpret_cast<f32x4*>(buf);
 #pragma unroll
         for (int j = 0; j < quads<S>(); ++j) {
             const int id = tid + j * S::NT;
@@ -316,6 +338,19 @@ struct FilterB {
             plane[q * S::B_ROW + b_slot(n)] = st[j];
         }
     }
+    // operands of quad pair s for this lane: frag[e][ni] = B[8s + 4lh + e][wn0 + 32*ni + li]
+    template <class S>
+    __device__ __forceinline__ void read_frags(const float* buf, int s, int lh, int li, int wn0, float (*frag)[S::NI]) const {
+        const f32x4* plane = reinterpret_cast<const f32x4*>(buf) + (2 * s + lh) * S::B_ROW;
+#pragma unroll
+        for (int ni = 0; ni < S::NI; ++ni) {
+            const f32x4 v = plane[b_slot(wn0 + ni * 32 + li)];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) frag[e][ni] = v[e];
+        }
+    }
+    template <class S>
+    __device__ __forceinline__ static int strip_col(int ni, int li) { return 32 * ni + li; }
 };
 
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int WAVES_PER_SIMD_ = 1,
@@ -338,9 +373,12 @@ struct SgemmShape {
     // branches -- a divergent skip would split the loop body into basic blocks and undo its instruction schedule.
     static constexpr int A_STAGED_ROWS = A_PASSES * (NT / KQ);
     static constexpr int A_ROW = A_STAGED_ROWS + 2;           // quads per A plane (planes 2 slots out of step mod 8)
-    static constexpr int B_ROW = BN + 2;                      // quads per B plane
+    static constexpr int B_ROW = BN + 2;                      // quads per B plane (k-quad layout only)
     static constexpr bool A_PARTIAL = (BM * KQ) % NT != 0;
-    static constexpr size_t LDS_BYTES = 2 * (size_t)KQ * (A_ROW + B_ROW) * sizeof(f32x4);
+    template <class BSrc>
+    static constexpr size_t lds_bytes() {
+        return 2 * ((size_t)KQ * A_ROW * sizeof(f32x4) + (size_t)BSrc::template lds_floats<SgemmShape>() * sizeof(float));
+    }
     static_assert(BM % (WAVES_M * 32) == 0 && BN % (WAVES_N * 32) == 0, "wave tile must be whole 32x32 blocks");
     static_assert(BK % 8 == 0, "a K step is whole quad pairs");
     static_assert(NT % KQ == 0, "A staging: KQ lanes per row");
@@ -369,7 +407,8 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, NT = S::NT, KQ = S::KQ, MI = S::MI, NI = S::NI;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     f32x4* As = reinterpret_cast<f32x4*>(lds_raw);                       // [2][KQ][A_ROW]
-    f32x4* Bs = As + 2 * KQ * S::A_ROW;                                  // [2][KQ][B_ROW]
+    float* Bs = reinterpret_cast<float*>(As + 2 * KQ * S::A_ROW);        // [2][layout of the B source]
+    constexpr int B_BUF = BSrc::template lds_floats<S>();
 
     const TileCoord tc = xcd_grouped_tile(blockIdx.x, tiles_m, tiles_n, group_m);
     const int bm0 = tc.tm * BM, bn0 = tc.tn * BN;
@@ -419,7 +458,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
             const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
             Ab[a_q * S::A_ROW + a_r + p * A_RSTEP] = a_keep[SET][p] ? a_stage[SET][p] : zero;
         }
-        b_src.template store<S>(Bs + buf * KQ * S::B_ROW, b_stage[SET], tid);
+        b_src.template store<S>(Bs + buf * B_BUF, b_stage[SET], tid);
     };
 
     f32x16 acc[MI][NI];
@@ -430,33 +469,31 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
 
-    // Fragments of one quad pair s: per 32-row / 32-column block one float4 = four consecutive k of this lane's k-slot.
-    auto read_frags = [&](int buf, int s, f32x4* af, f32x4* bf) {
+    // Fragments of one quad pair s: A, per 32-row block one float4 = four consecutive k of this lane's k-slot; B, per
+    // k of the pair (e) and block (ni) one float, fetched as the B source's LDS layout dictates.
+    typedef float BFrag[4][NI];
+    auto read_frags = [&](int buf, int s, f32x4* af, BFrag& bf) {
         const f32x4* Ab = As + buf * KQ * S::A_ROW;
-        const f32x4* Bb = Bs + buf * KQ * S::B_ROW;
         const int q = 2 * s + lh;
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) af[mi] = Ab[q * S::A_ROW + wm0 + mi * 32 + li];
-#pragma unroll
-        for (int ni = 0; ni < NI; ++ni) {
-            const int n = wn0 + ni * 32 + li;
-            bf[ni] = Bb[q * S::B_ROW + b_slot(n)];
-        }
+        b_src.template read_frags<S>(Bs + buf * B_BUF, s, lh, li, wn0, bf);
     };
     // MFMAs number lo .. hi-1 of a quad pair, in the order (e, mi, ni); a full pair is 4*MI*NI of them.
     constexpr int PAIR_MFMAS = 4 * MI * NI;
-    auto mfma_range = [&](const f32x4* af, const f32x4* bf, auto lo_tag, auto hi_tag) {
+    auto mfma_range = [&](const f32x4* af, const BFrag& bf, auto lo_tag, auto hi_tag) {
         constexpr int LO = decltype(lo_tag)::value, HI = decltype(hi_tag)::value;
 #pragma unroll
         for (int i = LO; i < HI; ++i) {
             const int e = i / (MI * NI), mi = (i / NI) % MI, ni = i % NI;
-            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[mi][e], bf[ni][e], acc[mi][ni], 0, 0, 0);
+            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[mi][e], bf[e][ni], acc[mi][ni], 0, 0, 0);
         }
     };
     auto compute_stage = [&](int buf) {      // unpipelined: used for the peeled steps only
 #pragma unroll
         for (int s = 0; s < KQ / 2; ++s) {
-            f32x4 af[MI], bf[NI];
+            f32x4 af[MI];
+            BFrag bf;
             read_frags(buf, s, af, bf);
             mfma_range(af, bf, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
         }
@@ -486,9 +523,10 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
 
     static_assert(KQ == 4, "the pipelined loop is written for two quad pairs per K step");
     constexpr int VMEM_OPS = S::A_PASSES + B_QUADS;     // global loads per thread and step
-    constexpr int FRAG_OPS = MI + NI;                   // ds_read_b128 per quad pair
+    constexpr int FRAG_OPS = MI + BSrc::template frag_reads<S>();   // LDS reads per quad pair
     constexpr int WRITE_OPS = S::A_PASSES + B_QUADS;    // ds_write_b128 per thread and step
-    f32x4 af0[MI], bf0[NI], af1[MI], bf1[NI];
+    f32x4 af0[MI], af1[MI];
+    BFrag bf0, bf1;
 
     // Steady state of one K step t (fragments of its first quad pair are in af0/bf0):
     //   pair 0 MFMAs   interleaved with: global loads of step t+SETS, LDS reads of pair 1
@@ -580,7 +618,8 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         }
     }
 
-    // ---- epilogue: each lane holds column li of its 32-wide block; a half-wave writes 128 contiguous bytes.
+    // ---- epilogue.  Lane li holds, per row, the columns strip_col(ni, li) of its wave's strip: NI consecutive ones when B
+    // came from a row-major matrix (one vector store per row where alignment and the edge allow), 32 apart otherwise.
     // dst = A*B + C adds C here (C may alias dst: every element is read and written by the same lane).
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
@@ -590,11 +629,23 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
             if (m < M) {
                 float* drow = D + out.offset(m);
                 const float* crow = HAS_C ? Cin + (size_t)m * ldc : nullptr;
+                const bool add_c = HAS_C && (!SPLIT_K || blockIdx.z == 0);
+                if (BSrc::ROW_MAJOR_LDS && !SPLIT_K && NI > 1) {
+                    const int n0 = bn0 + wn0 + NI * li;
+                    if (out.vec && n0 + NI <= N) {
+                        typedef float vec_t __attribute__((ext_vector_type(NI)));
+                        vec_t v;
+#pragma unroll
+                        for (int ni = 0; ni < NI; ++ni) v[ni] = out.finish(add_c ? acc[mi][ni][r] + crow[n0 + ni] : acc[mi][ni][r]);
+                        *reinterpret_cast<vec_t*>(drow + n0) = v;
+                        continue;
+                    }
+                }
 #pragma unroll
                 for (int ni = 0; ni < NI; ++ni) {
-                    const int n = bn0 + wn0 + ni * 32 + li;
+                    const int n = bn0 + wn0 + BSrc::template strip_col<S>(ni, li);
                     if (n < N) {
-                        const float v = (HAS_C && (!SPLIT_K || blockIdx.z == 0)) ? acc[mi][ni][r] + crow[n] : acc[mi][ni][r];
+                        const float v = add_c ? acc[mi][ni][r] + crow[n] : acc[mi][ni][r];
                         if (SPLIT_K) unsafeAtomicAdd(drow + n, v);      // hardware fp32 add in L2
                         else drow[n] = out.finish(v);
                     }

@@ -14,7 +14,7 @@ CASES = [  # H, W, C, N, kh, kw, flag
 ]
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("case", CASES)
 def test_integer_exact(gpu, oracle, case, variant):
     H, W, C, N, kh, kw, flag = case
@@ -48,7 +48,7 @@ def test_config4_224x224x64_128_filters(gpu, oracle):
     # accurate enough for a scale
     scale = oracle.conv2_chain(np.abs(src), np.abs(filt), 1).astype(np.float64)
     K = 3 * 3 * 64
-    for variant in (0, 1, 2, 3, 4):
+    for variant in (0, 1, 2, 3, 4, 7):
         got = gpu_conv(src, filt, 1, variant=variant)
         err = float(np.max(np.abs(got.astype(np.float64) - ref) / scale))
         print("conv 224x224x64 (*) 128x3x3x64 variant %d: max |x-r|/sum|a||b| = %.3e (bound %.3e)" %
