@@ -199,7 +199,9 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
         for (int b = 0; b + 1 < KS; ++b) {
 #pragma unroll
             for (int i = 0; i < BLK; ++i) {
-                if (i < FRAG_READS) read_one((b & 1) ? f0 : f1, stg, b + 1, i);
+                constexpr int RPS = (FRAG_READS + BLK - 1) / BLK;      // reads per MFMA slot, front-loaded
+#pragma unroll
+                for (int r = i * RPS; r < (i + 1) * RPS && r < FRAG_READS; ++r) read_one((b & 1) ? f0 : f1, stg, b + 1, r);
                 mfma_one((b & 1) ? f1 : f0, i);
                 DECX_PIN();
             }
