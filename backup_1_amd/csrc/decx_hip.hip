@@ -261,8 +261,13 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
     const long Ml = (long)Hout * Wout, Kl = (long)kh * kw * dpitch;
     if (Ml > 0x7fffffffL || Kl > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large\n");
     const int M = (int)Ml, K = (int)Kl;
-    Im2colA a{src, H, W, dpitch, kh, kw, flag ? kh / 2 : 0, flag ? kw / 2 : 0, Wout, M, K, src_row_stride};
-    FilterB b{filt, N, K, dpitch, kw, filt_stride, filt_row_stride};
+    // the loaders address both tensors with 32-bit byte offsets through buffer resources
+    const size_t src_bytes = ((size_t)(H - 1) * src_row_stride + (size_t)W * dpitch) * sizeof(float);
+    const size_t filt_bytes = ((size_t)(N - 1) * filt_stride + (size_t)(kh - 1) * filt_row_stride + (size_t)kw * dpitch) * sizeof(float);
+    if (src_bytes >= 0x80000000ull || filt_bytes >= 0x80000000ull)
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "source tensor and filter bank must each stay below 2 GiB\n");
+    Im2colA a{src, H, W, dpitch, kh, kw, flag ? kh / 2 : 0, flag ? kw / 2 : 0, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
+    FilterB b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
     TensorOut out{Wout, dst_dpitch, dst_row_stride, dst_row_stride == (size_t)Wout * dst_dpitch, relu};
     Batch one;
     one.stream = g_rt.stream;

@@ -48,37 +48,56 @@ namespace decx_hip {
 // need no fold: consecutive slots are read, and the planes are 2 slots out of step for the staging stores.
 __device__ __forceinline__ int b_slot(int n) { return n ^ ((n >> 3) & 3); }
 
-// A K step of dk as an increment of the im2col position (c, kj, ki): dk = (dki*kw + dkj)*dpitch + dc.  Worked out once
-// per kernel so that advancing is a handful of adds and selects.
+// 16 bytes through a buffer resource: offsets at or beyond the resource's size read as zeros, which is how taps
+// outside the image, rows of a ragged last tile and the K tail are zero-filled without a select per element.
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+constexpr unsigned kOutOfRange = 0x80000000u;      // resources are kept below 2 GiB
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ f32x4 buffer_load_quad(__amdgpu_buffer_rsrc_t rsrc, unsigned byte_offset) {
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)byte_offset, 0, 0));
+}
+
+// A K step of dk as an increment of the im2col position (c, kj, ki): dk = (dki*kw + dkj)*dpitch + dc, and of the byte
+// offset of that position inside a tensor whose rows are row_stride floats apart.  Worked out once per kernel so that
+// advancing is a handful of adds and selects.
 struct TapStep {
     int dk, dc, dkj, dki;
-    __device__ __forceinline__ static TapStep make(int dk, int dpitch, int kw) {
+    int step_bytes;      // offset change of the raw increments
+    int wrap_bytes;      // extra change when kj wraps into the next tensor row (a c -> kj carry changes nothing: the
+                         // channels of consecutive taps of one row are contiguous)
+    __device__ __forceinline__ static TapStep make(int dk, int dpitch, int kw, int row_stride) {
         const int taps = dk / dpitch, rows = taps / kw;
-        return TapStep{dk, dk - taps * dpitch, taps - rows * kw, rows};
+        const int dc = dk - taps * dpitch, dkj = taps - rows * kw;
+        return TapStep{dk, dc, dkj, rows, 4 * (rows * row_stride + dkj * dpitch + dc), 4 * (row_stride - kw * dpitch)};
     }
 };
 
-// Position of one k index inside the im2col ordering k = (ki*kw + kj)*dpitch + c.  Decoded once (two integer
-// divisions), then advanced by whole K steps without divisions, loops or branches (control flow inside the K loop
-// would split its body into basic blocks and undo the instruction schedule).
+// Position of one k index inside the im2col ordering k = (ki*kw + kj)*dpitch + c, with its byte offset
+// 4*(ki*row_stride + kj*dpitch + c).  Decoded once (two integer divisions), then advanced by whole K steps without
+// divisions, loops or branches (control flow inside the K loop would split its body into basic blocks and undo the
+// instruction schedule).
 struct TapWalk {
-    int k, c, ki, kj;
-    __device__ __forceinline__ void init(int k_, int dpitch, int kw) {
+    int k, c, ki, kj, off;
+    __device__ __forceinline__ void init(int k_, int dpitch, int kw, int row_stride) {
         k = k_;
         const int tap = k_ / dpitch;
         c = k_ - tap * dpitch;
         ki = tap / kw;
         kj = tap - ki * kw;
+        off = 4 * (ki * row_stride + kj * dpitch + c);
     }
     __device__ __forceinline__ void advance(const TapStep& st, int dpitch, int kw) {
         k += st.dk;
         c += st.dc;
-        const int carry_c = c >= dpitch ? 1 : 0;          // c < 2*dpitch: one carry at most
+        const bool carry_c = c >= dpitch;                 // c < 2*dpitch: one carry at most
         c -= carry_c ? dpitch : 0;
-        kj += st.dkj + carry_c;
-        const int carry_kj = kj >= kw ? 1 : 0;            // kj <= 2*kw - 1: one carry at most
+        kj += st.dkj + (carry_c ? 1 : 0);
+        const bool carry_kj = kj >= kw;                   // kj <= 2*kw - 1: one carry at most
         kj -= carry_kj ? kw : 0;
-        ki += st.dki + carry_kj;
+        ki += st.dki + (carry_kj ? 1 : 0);
+        off += st.step_bytes + (carry_kj ? st.wrap_bytes : 0);
     }
 };
 
@@ -130,42 +149,43 @@ struct DenseA {
 };
 
 // The im2col view of a channel-innermost tensor: row m = (y, x) of the output, column k = (ki*kw + kj)*dpitch + c.
-// Per row the element offset of its top-left tap is kept; per K step one tap offset is added to it, so a load costs
-// two coordinate adds, two unsigned range checks and one 64-bit add.
+// Everything is 32-bit byte-offset arithmetic against one buffer resource (tensors stay below 2 GiB): per row the offset
+// of its top-left tap is kept, per K step the tap's offset is added, and a tap outside the image gets an out-of-range
+// offset instead, which the hardware answers with zeros.
 struct Im2colA {
     const float* src;
     int H, W, dpitch, kh, kw, oy, ox, Wout, Mtot, K;
-    size_t row_stride;
+    int row_stride;            // floats between image rows
+    unsigned bytes;            // extent of the tensor
     __device__ __forceinline__ void select_batch(int) {}
     __device__ __forceinline__ void set_k_end(int k_end) { K = k_end; }
     struct RowState {
         int y, x;          // output pixel shifted by (-oy, -ox): the image position of tap (0, 0)
-        long base;         // y*row_stride + x*dpitch (may be negative: it is only used together with an in-image tap)
+        int base;          // 4*(y*row_stride + x*dpitch); may be negative, only used together with an in-image tap
     };
     __device__ __forceinline__ RowState row_state(int m) const {
         if (m >= Mtot) m = Mtot - 1;
         RowState rs;
         rs.y = m / Wout - oy;
         rs.x = m % Wout - ox;
-        rs.base = (long)rs.y * (long)row_stride + (long)rs.x * dpitch;
+        rs.base = 4 * (rs.y * row_stride + rs.x * dpitch);
         return rs;
     }
     typedef TapWalk KState;
+    typedef TapStep KStep;
     __device__ __forceinline__ KState k_state(int k) const {
         KState ks;
-        ks.init(k, dpitch, kw);
+        ks.init(k, dpitch, kw, row_stride);
         return ks;
     }
-    typedef TapStep KStep;
-    __device__ __forceinline__ KStep k_step(int dk) const { return TapStep::make(dk, dpitch, kw); }
+    __device__ __forceinline__ KStep k_step(int dk) const { return TapStep::make(dk, dpitch, kw, row_stride); }
     __device__ __forceinline__ void advance(KState& ks, const KStep& st) const { ks.advance(st, dpitch, kw); }
     template <bool TAIL>
     __device__ __forceinline__ f32x4 load(const RowState& rs, const KState& ks, bool& keep) const {
-        // K = kh*kw*dpitch is a multiple of 4: quads never straddle it.  A tap outside the image (or k >= K, TAIL only)
-        // reads the tensor's first quad instead and is zeroed by the caller.
-        const long tap_off = (long)ks.ki * (long)row_stride + (long)(ks.kj * dpitch + ks.c);
-        keep = (unsigned)(rs.y + ks.ki) < (unsigned)H && (unsigned)(rs.x + ks.kj) < (unsigned)W && (!TAIL || ks.k < K);
-        return *reinterpret_cast<const f32x4*>(src + (keep ? rs.base + tap_off : 0L));
+        // K = kh*kw*dpitch is a multiple of 4: quads never straddle it
+        const bool inside = (unsigned)(rs.y + ks.ki) < (unsigned)H && (unsigned)(rs.x + ks.kj) < (unsigned)W && (!TAIL || ks.k < K);
+        keep = true;
+        return buffer_load_quad(make_rsrc(src, bytes), inside ? (unsigned)(rs.base + ks.off) : kOutOfRange);
     }
 };
 
@@ -235,7 +255,7 @@ struct DenseB {
         int dk;
     };
     template <class S>
-    __device__ __forceinline__ KState k_state(int tid, int k_begin) const { return KState{k_begin}; }
+    __device__ __forceinline__ KState k_state(int tid, int k_begin, int bn0) const { return KState{k_begin}; }
     template <class S>
     __device__ __forceinline__ KStep k_step() const { return KStep{S::BK}; }
     __device__ __forceinline__ void advance(KState& ks, const KStep& st) const { ks.k0 += st.dk; }
@@ -288,45 +308,53 @@ struct DenseB {
 
 // B as a bank of N filters, filter n holding its taps channel-innermost: column n of the lowered GEMM is filter n and
 // four consecutive k (same tap, four channels) are already contiguous in memory, so a k-quad is one 16-byte load.
+// Same 32-bit offsets against a buffer resource as Im2colA (the bank stays below 2 GiB).
 struct FilterB {
     const float* filt;
     int N, K, dpitch, kw;
-    size_t filt_stride, filt_row_stride;
+    int filt_stride, filt_row_stride;      // floats between filters / between tap rows of one filter
+    unsigned bytes;
+    static constexpr bool ROW_MAJOR_LDS = false;
     __device__ __forceinline__ void select_batch(int) {}
     __device__ __forceinline__ void set_k_end(int k_end) { K = k_end; }
-    static constexpr bool ROW_MAJOR_LDS = false;
     template <class S>
     static constexpr int quads() { return S::KQ * S::BN / S::NT; }
     template <class S>
     static constexpr int lds_floats() { return 4 * S::KQ * S::B_ROW; }          // one buffer
     template <class S>
     static constexpr int frag_reads() { return S::NI; }                        // one k-quad per 32-column block
-    typedef TapWalk KState;       // every quad of a thread has the same k-quad index q = tid % KQ (NT is a multiple of KQ)
-    template <class S>
-    __device__ __forceinline__ KState k_state(int tid, int k_begin) const {
-        KState ks;
-        ks.init(k_begin + 4 * (tid % S::KQ), dpitch, kw);
-        return ks;
-    }
+    // every quad of a thread has the same k-quad index q = tid % KQ (NT is a multiple of KQ): one walk serves them all;
+    // what differs is the filter, whose byte offset is worked out once
+    template <int QUADS>
+    struct KStateT {
+        TapWalk walk;
+        int filter_base[QUADS];
+    };
     typedef TapStep KStep;
     template <class S>
-    __device__ __forceinline__ KStep k_step() const { return TapStep::make(S::BK, dpitch, kw); }
-    __device__ __forceinline__ void advance(KState& ks, const KStep& st) const { ks.advance(st, dpitch, kw); }
-
-    template <class S, bool TAIL>
-    __device__ __forceinline__ void load(f32x4* st, int tid, const KState& ks, int bn0) const {
+    __device__ __forceinline__ KStateT<quads<S>()> k_state(int tid, int k_begin, int bn0) const {
         static_assert((S::KQ * S::BN) % S::NT == 0 && S::NT % S::KQ == 0, "filter staging must divide evenly");
-        const bool k_ok = !TAIL || ks.k < K;
-        const size_t tap_off = k_ok ? (size_t)ks.ki * filt_row_stride + (size_t)ks.kj * dpitch + ks.c : 0;
+        KStateT<quads<S>()> ks;
+        ks.walk.init(k_begin + 4 * (tid % S::KQ), dpitch, kw, filt_row_stride);
 #pragma unroll
         for (int j = 0; j < quads<S>(); ++j) {
-            const int id = tid + j * S::NT;
-            int n = bn0 + id / S::KQ;
+            int n = bn0 + (tid + j * S::NT) / S::KQ;
             if (n >= N) n = N - 1;
-            f32x4 v = *reinterpret_cast<const f32x4*>(filt + (size_t)n * filt_stride + tap_off);
-            if (TAIL && !k_ok) v = f32x4{0.f, 0.f, 0.f, 0.f};
-            st[j] = v;
+            ks.filter_base[j] = 4 * n * filt_stride;
         }
+        return ks;
+    }
+    template <class S>
+    __device__ __forceinline__ KStep k_step() const { return TapStep::make(S::BK, dpitch, kw, filt_row_stride); }
+    template <class KS>
+    __device__ __forceinline__ void advance(KS& ks, const KStep& st) const { ks.walk.advance(st, dpitch, kw); }
+
+    template <class S, bool TAIL, class KS>
+    __device__ __forceinline__ void load(f32x4* st, int tid, const KS& ks, int bn0) const {
+        const bool k_ok = !TAIL || ks.walk.k < K;
+#pragma unroll
+        for (int j = 0; j < quads<S>(); ++j)
+            st[j] = buffer_load_quad(make_rsrc(filt, bytes), k_ok ? (unsigned)(ks.filter_base[j] + ks.walk.off) : kOutOfRange);
     }
     template <class S>
     __device__ __forceinline__ void store(float* buf, const f32x4* st, int tid) const {
@@ -435,7 +463,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
     bool a_keep[SETS][S::A_PASSES];
     f32x4 b_stage[SETS][B_QUADS];
     typename ASrc::KState a_ks = a_src.k_state(k_begin + 4 * a_q);   // this thread's k-quad of the next K step to fetch
-    typename BSrc::KState b_ks = b_src.template k_state<S>(tid, k_begin);
+    auto b_ks = b_src.template k_state<S>(tid, k_begin, bn0);
     const typename ASrc::KStep a_step = a_src.k_step(BK);
     const typename BSrc::KStep b_step = b_src.template k_step<S>();
 
