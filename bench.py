@@ -27,7 +27,7 @@ PEAK_HBM_GBPS = 8000.0              # MI355X HBM3E
 # HBM-side bytes per launch of the headline kernel (fp32 8192^3), from the FETCH_SIZE / WRITE_SIZE counter runs
 # summarised in profiles/hbm_traffic_fetch_write_size.txt (read factor 2.0, write factor 1.0 against a copy kernel).
 # Counters cannot be read from inside this script; the figure is only reported for the workload it was measured on.
-MEASURED_TRAFFIC_BYTES_FP32_8192 = 3.755e9
+MEASURED_TRAFFIC_BYTES_FP32_8192 = 3.765e9
 
 
 def log(msg):
@@ -63,8 +63,9 @@ def bench_sgemm(capi, workloads, M, K, N, steps, warmup, seed, dist="uniform"):
     launch = lambda: capi.sgemm(dA.ptr, lda, dB.ptr, ldb, dD.ptr, ldd, M, N, K, blocking=False)
     wall, ev = time_launches(capi, launch, steps, warmup)
     flops = 2.0 * M * N * K
+    med, mn = per_launch_stats(capi, launch, 10)
     return {"ms_wall": wall, "ms_kernel": ev, "tflops": flops / (wall * 1e-3) / 1e12, "tflops_kernel": flops / (ev * 1e-3) / 1e12,
-            "flops": flops, "A": A, "B": B}
+            "flops": flops, "A": A, "B": B, "ms_median": med, "ms_min": mn}
 
 
 def bench_hgemm(capi, workloads, n, steps, warmup, seed):
@@ -89,6 +90,106 @@ def bench_conv(capi, workloads, steps, warmup):
     wall, ev = time_launches(capi, launch, steps, warmup)
     flops = 2.0 * H * W * N * kh * kw * C
     return {"ms_wall": wall, "ms_kernel": ev, "tflops": flops / (wall * 1e-3) / 1e12, "tflops_kernel": flops / (ev * 1e-3) / 1e12}
+
+
+def per_launch_stats(capi, launch, reps):
+    """Each launch timed on its own between two HIP events: (median ms, min ms)."""
+    ms = []
+    for _ in range(reps):
+        capi.timer_start()
+        launch()
+        ms.append(capi.timer_stop())
+    ms.sort()
+    return ms[len(ms) // 2], ms[0]
+
+
+class PinnedArray:
+    """Host memory from decx_hip_host_malloc viewed as a numpy array (what Page_Locked DECX containers hold)."""
+
+    def __init__(self, capi, shape, dtype):
+        import ctypes
+        self.capi, self.nbytes = capi, int(np.prod(shape)) * np.dtype(dtype).itemsize
+        p = ctypes.c_void_p()
+        capi.check(capi.lib().decx_hip_host_malloc(ctypes.byref(p), self.nbytes))
+        self.ptr = p.value
+        self.array = np.ctypeslib.as_array((ctypes.c_byte * self.nbytes).from_address(self.ptr)).view(dtype).reshape(shape)
+
+    def free(self):
+        self.array = None
+        self.capi.check(self.capi.lib().decx_hip_host_free(self.ptr))
+
+
+def bench_host_resident_gemm(capi, A, B, reps):
+    """de::cuda::GEMM(Matrix<float>...) equivalent (GEMM.h:56-131): pinned host operands, H2D of A and B, kernel, D2H of
+    the result -- the PCIe-inclusive figure.  Device buffers keep the host pitch; none of it is padded."""
+    M, K = A.shape
+    N = B.shape[1]
+    hA, hB, hD = PinnedArray(capi, (M, K), np.float32), PinnedArray(capi, (K, N), np.float32), PinnedArray(capi, (M, N), np.float32)
+    hA.array[:], hB.array[:] = A, B
+    dA, dB, dD = capi.DeviceBuffer(M * K * 4), capi.DeviceBuffer(K * N * 4), capi.DeviceBuffer(M * N * 4)
+    L = capi.lib()
+    best = None
+    for _ in range(reps + 1):
+        t0 = time.perf_counter()
+        capi.check(L.decx_hip_memcpy2d(dA.ptr, K * 4, hA.ptr, K * 4, K * 4, M, capi.H2D))
+        capi.check(L.decx_hip_memcpy2d(dB.ptr, N * 4, hB.ptr, N * 4, N * 4, K, capi.H2D))
+        capi.sgemm(dA.ptr, K, dB.ptr, N, dD.ptr, N, M, N, K)
+        capi.check(L.decx_hip_memcpy2d(hD.ptr, N * 4, dD.ptr, N * 4, N * 4, M, capi.D2H))
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    for h in (hA, hB, hD): h.free()
+    return {"ms": best * 1e3, "tflops": 2.0 * M * N * K / best / 1e12, "pcie_bytes": 4.0 * (M * K + K * N + M * N)}
+
+
+def bench_host_resident_conv(capi, workloads, reps):
+    """de::cuda::Conv2_MK_im2col(Tensor, TensorArray, Tensor) equivalent (conv2_mk_im2col.h:278-306): upload the
+    tensor and the filters, fused kernel, download the result."""
+    H = W = 224; C = 64; N = 128; kh = kw = 3
+    src, filt = workloads.conv_case()
+    hS, hF, hD = PinnedArray(capi, (H, W, C), np.float32), PinnedArray(capi, (N, kh, 4, C), np.float32), PinnedArray(capi, (H, W, N), np.float32)
+    hS.array[:] = src
+    hF.array[:] = 0
+    hF.array[:, :, :kw, :] = filt
+    dS, dF, dD = capi.DeviceBuffer(hS.nbytes), capi.DeviceBuffer(hF.nbytes), capi.DeviceBuffer(hD.nbytes)
+    L = capi.lib()
+    best = None
+    for _ in range(reps + 1):
+        t0 = time.perf_counter()
+        capi.check(L.decx_hip_memcpy(dS.ptr, hS.ptr, hS.nbytes, capi.H2D))
+        capi.check(L.decx_hip_memcpy(dF.ptr, hF.ptr, hF.nbytes, capi.H2D))
+        capi.conv2_im2col(dS.ptr, H, W, C, W * C, dF.ptr, N, kh, kw, kh * 4 * C, 4 * C, dD.ptr, N, W * N, 1)
+        capi.check(L.decx_hip_memcpy(hD.ptr, dD.ptr, hD.nbytes, capi.D2H))
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    for h in (hS, hF, hD): h.free()
+    return {"ms": best * 1e3, "tflops": 2.0 * H * W * N * kh * kw * C / best / 1e12}
+
+
+def cpu_conv_baseline(workloads):
+    """The reference has no CPU convolution; its CPU equivalent is a host im2col in the reference's k order followed by
+    the restated DECX_cpu thread-pool SGEMM on the 50176 x 576 x 128 lowered problem."""
+    import oracle
+    H = W = 224; C = 64; N = 128; kh = kw = 3
+    src, filt = workloads.conv_case()
+    padded = np.zeros((H + 2, W + 2, C), np.float32)
+    cols = np.zeros((H * W, kh * kw * C), np.float32)
+    out = np.zeros((H * W, N), np.float32)
+    Bm = np.ascontiguousarray(filt.reshape(N, kh * kw * C).T)
+    best = None
+    for _ in range(2):
+        t0 = time.perf_counter()
+        padded[1:-1, 1:-1] = src
+        for ki in range(kh):
+            for kj in range(kw):
+                cols[:, (ki * kw + kj) * C:(ki * kw + kj + 1) * C] = padded[ki:ki + H, kj:kj + W].reshape(H * W, C)
+        t1 = time.perf_counter()
+        oracle.decx_cpu_sgemm(cols, Bm, out=out)
+        t2 = time.perf_counter()
+        if best is None or t2 - t0 < best[0]: best = (t2 - t0, t1 - t0, t2 - t1)
+    flops = 2.0 * H * W * N * kh * kw * C
+    return {"tflops": round(flops / best[0] / 1e12, 4), "ms": round(best[0] * 1e3, 2), "im2col_ms": round(best[1] * 1e3, 2),
+            "sgemm_ms": round(best[2] * 1e3, 2), "sgemm_tflops": round(flops / best[2] / 1e12, 4),
+            "what": "numpy im2col (reference k order, single thread) + restated DECX_cpu SGEMM on 50176x576x128, best of 2"}
 
 
 def bench_relu(capi, workloads, steps, warmup):
@@ -149,7 +250,7 @@ def main():
     ap.add_argument("--size", type=int, default=8192, help="square size of the headline fp32 GEMM")
     ap.add_argument("--sgemm-variant", type=int, default=0, help="force a fp32 tile shape (0 = automatic)")
     ap.add_argument("--hgemm-variant", type=int, default=0, help="force a fp16 tile shape (0 = automatic)")
-    ap.add_argument("--only", default="", help="comma list of: headline,fp16,sq4096,ragged,conv,relu,cpu (default all)")
+    ap.add_argument("--only", default="", help="comma list of: headline,fp16,sq4096,ragged,conv,relu,host,cpu (default all)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); --gpus %d is not supported. "
@@ -215,8 +316,19 @@ def main():
             capi.check(capi.lib().decx_hip_copy_kernel(dst.ptr, src.ptr, nbytes))
         also["copy_1GiB"] = {"bytes_read": nbytes, "bytes_written": nbytes}
 
+    if want("host"):
+        r = bench_host_resident_gemm(capi, head["A"], head["B"], 2)
+        also["host_resident_gemm_%d_pcie_inclusive" % n] = {"tflops": round(r["tflops"], 2), "ms_per_call": round(r["ms"], 2),
+                                                            "pcie_bytes": r["pcie_bytes"]}
+        log("host-resident GEMM %d^3 (H2D + kernel + D2H): %.1f ms -> %.1f TFLOP/s" % (n, r["ms"], r["tflops"]))
+        r = bench_host_resident_conv(capi, workloads, 5)
+        also["host_resident_conv_pcie_inclusive"] = {"tflops": round(r["tflops"], 2), "ms_per_call": round(r["ms"], 3)}
+        log("host-resident conv (H2D + kernel + D2H): %.3f ms -> %.1f TFLOP/s" % (r["ms"], r["tflops"]))
+
     cpu = None
     if want("cpu"):
+        also["cpu_conv_baseline"] = cpu_conv_baseline(workloads)
+        log("cpu conv baseline: %.1f ms" % also["cpu_conv_baseline"]["ms"])
         log("cpu baseline (oracle port of the DECX_cpu thread-pool SGEMM) ...")
         cpu = cpu_baseline(head["A"], head["B"], rows=min(n, 3072))
         log("  %.4f TFLOP/s on %d cores" % (cpu["value"], cpu["cores"]))
@@ -233,7 +345,8 @@ def main():
                      "frac": round(achieved / PEAK_FP32_MATRIX_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES_FP32_8192 if (n == 8192 and args.sgemm_variant in (0, 7)) else None,
                      "kernel": "sgemm_tile_kernel", "flop_per_launch": head["flops"],
-                     "avg_launch_ms_hip_events": round(head["ms_kernel"], 4)},
+                     "avg_launch_ms_hip_events": round(head["ms_kernel"], 4),
+                     "single_launch_ms_median": round(head["ms_median"], 4), "single_launch_ms_min": round(head["ms_min"], 4)},
         "cpu_baseline": cpu,
         "also": also,
     }
