@@ -142,6 +142,8 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //   7: 256x256x16, 4x2 waves of  64x128   -- two waves per SIMD: the matrix pipe takes the next MFMA from the other wave
 //         while one wave issues its loads and LDS traffic (a lone wave leaves ~3.5 idle cycles between 64-cycle MFMAs);
 //         the default for large problems, 1-2 % ahead of shape 1
+//   8:  64x64x16,  2x2 waves of  32x32    -- small problems: 1024^3 has only 64 tiles of 128x128 for 256 CUs
+//   9: 128x64x16,  2x2 waves of  64x32
 //   5, 6: shapes 3 and 4 compiled for one wave per SIMD (512 registers, two staging sets) -- for launches that put at
 //         most one workgroup on a CU anyway, where a second resident workgroup cannot be what hides the load latency
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
@@ -151,14 +153,20 @@ typedef SgemmShape<224, 128, 16, 1, 4, 2> SShape224;
 typedef SgemmShape<256, 128, 16, 2, 2, 1> SShapeTallSolo;
 typedef SgemmShape<224, 128, 16, 1, 4, 1> SShape224Solo;
 typedef SgemmShape<256, 256, 16, 4, 2, 2, 2> SShapeBig8;
+typedef SgemmShape<64, 64, 16, 2, 2, 4> SShapeTiny;      // 2x2 waves of 32x32
+typedef SgemmShape<128, 64, 16, 2, 2, 4> SShapeTiny2;    // 2x2 waves of 64x32
 
-// Tile shape by a small cost model: a CU works through ceil(tiles / CUs) tiles one after another, a tile costs its area
-// divided by how well that shape keeps the matrix pipe busy (measured on 8192^3, relative to shape 1).
-int pick_sgemm_variant(int M, int N, int batch) {
-    if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 7) return g_rt.sgemm_variant;
+// Tile shape by a small cost model: a CU works through ceil(tiles / CUs) tiles one after another (tiles that share a CU
+// share its matrix pipe, so residency does not change this), a tile costs its area divided by how well that shape keeps
+// the pipe busy (measured on large squares, relative to shape 7).  The 256x128 and 224x128 shapes come in a
+// two-workgroups-per-CU build, better on short K walks where one tile's prologue and epilogue overlap the other's loop,
+// and a one-wave-per-SIMD build with deeper prefetch, better on long ones.
+int pick_sgemm_variant(int M, int N, int K, int batch) {
+    if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 9) return g_rt.sgemm_variant;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     struct Cand { int variant, bm, bn; double eff; };
-    const Cand cands[] = {{7, 256, 256, 1.00}, {3, 256, 128, 0.93}, {4, 224, 128, 0.83}, {2, 128, 128, 0.89}};
+    const Cand cands[] = {{7, 256, 256, 1.00}, {3, 256, 128, 0.95}, {4, 224, 128, 0.94}, {2, 128, 128, 0.89},
+                          {9, 128, 64, 0.83}, {8, 64, 64, 0.78}};
     int best = 7;
     double best_cost = 0.0;
     for (const Cand& c : cands) {
@@ -166,7 +174,7 @@ int pick_sgemm_variant(int M, int N, int batch) {
         const double cost = (double)((tiles + cus - 1) / cus) * c.bm * c.bn / c.eff;
         if (best_cost == 0.0 || cost < best_cost) {
             best_cost = cost;
-            best = (tiles <= cus && (c.variant == 3 || c.variant == 4)) ? c.variant + 2 : c.variant;
+            best = ((tiles <= cus || K >= 1024) && (c.variant == 3 || c.variant == 4)) ? c.variant + 2 : c.variant;
         }
     }
     return best;
@@ -182,6 +190,8 @@ int dispatch_sgemm(int variant, const ASrc& a, const BSrc& b, const float* Cin, 
         case 5: return launch_sgemm_tile<SShapeTallSolo>(a, b, Cin, ldc, D, out, M, N, K, batch);
         case 6: return launch_sgemm_tile<SShape224Solo>(a, b, Cin, ldc, D, out, M, N, K, batch);
         case 7: return launch_sgemm_tile<SShapeBig8>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 8: return launch_sgemm_tile<SShapeTiny>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 9: return launch_sgemm_tile<SShapeTiny2>(a, b, Cin, ldc, D, out, M, N, K, batch);
         default: return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K, batch);
     }
 }
@@ -202,7 +212,7 @@ int check_gemm_args(const void* A, int lda, const void* B, int ldb, const void* 
 int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
                   int N, int K, const Batch& batch, bool relu = false) {
     if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
-    const int variant = pick_sgemm_variant(M, N, batch.count);
+    const int variant = pick_sgemm_variant(M, N, K, batch.count);
     const bool vec_a = aligned16(A) && lda % 4 == 0 && batch.stride_a % 4 == 0;
     const bool vec_b = aligned16(B) && ldb % 4 == 0 && ldb >= 4 && batch.stride_b % 4 == 0;
     DenseOut out{ldd, relu, aligned16(D) && ldd % 4 == 0 && batch.stride_d % 4 == 0};
@@ -272,7 +282,7 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
     Batch one;
     one.stream = g_rt.stream;
     // a bias is the "+ C" operand with row stride 0: every output pixel adds the same N values
-    return dispatch_sgemm(pick_sgemm_variant(M, N, 1), a, b, bias, 0, dst, out, M, N, K, one);
+    return dispatch_sgemm(pick_sgemm_variant(M, N, K, 1), a, b, bias, 0, dst, out, M, N, K, one);
 }
 
 // ---------------------------------------------------------------------------------------------------------------

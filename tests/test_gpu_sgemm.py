@@ -27,7 +27,7 @@ SHAPES = [(1, 1, 1), (3, 5, 7), (31, 17, 33), (32, 16, 32), (128, 16, 128), (129
           (300, 70, 500), (257, 1500, 255), (64, 8, 1000), (1000, 3, 64), (513, 129, 259)]
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9])
 @pytest.mark.parametrize("shape", SHAPES)
 def test_integer_exact_all_tiles(gpu, shape, variant):
     M, K, N = shape
@@ -45,7 +45,7 @@ def test_unaligned_pitch_uses_elementwise_loader(gpu, shape):
     assert np.array_equal(gpu_sgemm(A, B, align=1), exact_int_product(A, B))
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9])
 def test_a_times_b_plus_c(gpu, oracle, variant):
     M, K, N = 200, 150, 300
     A, B, C = workloads.small_ints((M, K), 21), workloads.small_ints((K, N), 22), workloads.small_ints((M, N), 23, -100, 100)
