@@ -294,6 +294,9 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
 //   3: 256x256x32, 2x2 waves of 128x128, 4-stage LDS-DMA pipeline
 //   4: 256x256x64, 2x2 waves of 128x128, 2-stage LDS-DMA pipeline (whole 128-byte lines of A per row and step)
 //   5: 256x256x32, 2x2 waves of 128x128, 5-stage LDS-DMA pipeline
+//   8: 128x128x64, 2x2 waves of 64x64, 2-stage LDS-DMA pipeline (64 KB of LDS: two workgroups per CU) -- mid-size problems
+//   9: as 8 with 3 stages (one workgroup per CU) -- small problems
+//  10: 256x128x64, 2x2 waves of 128x64, 2-stage LDS-DMA pipeline
 //   6: as 4 with 4x2 waves of 64x128 (two waves per SIMD)
 //   7: as 4 with 2x4 waves of 128x64 (two waves per SIMD) -- the default for large problems: the chip is power-capped on
 //      this kernel (MFMA busy x clock stays ~1.27 GHz-equivalents whatever the schedule), and this one is 1 % ahead
@@ -304,6 +307,9 @@ typedef HgemmDmaShape<256, 256, 64, 2, 2, 2> HShapeDma64;
 typedef HgemmDmaShape<256, 256, 32, 2, 2, 5> HShapeDma5;
 typedef HgemmDmaShape<256, 256, 64, 4, 2, 2> HShapeDma64W8a;     // 8 waves, 64x128 each
 typedef HgemmDmaShape<256, 256, 64, 2, 4, 2> HShapeDma64W8b;     // 8 waves, 128x64 each
+typedef HgemmDmaShape<128, 128, 64, 2, 2, 2> HShapeDmaSmall;     // 4 waves, 64x64 each, 64 KB of LDS: two workgroups per CU
+typedef HgemmDmaShape<128, 128, 64, 2, 2, 3> HShapeDmaSmall3;
+typedef HgemmDmaShape<256, 128, 64, 2, 2, 2> HShapeDmaTall;      // 4 waves, 128x64 each
 
 template <class S, bool VEC>
 int launch_hgemm_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
@@ -358,15 +364,23 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
                      batch.stride_b % 8 == 0;
     if (!vec) return launch_hgemm_tile<HShapeSmall, false>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     int variant = g_rt.hgemm_variant;
-    if (variant < 1 || variant > 7) {
-        const int cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
-        variant = ((long)cdiv(M, 256) * cdiv(N, 256) * batch.count * 10 >= (long)cus * 8) ? 7 : 2;
+    if (variant < 1 || variant > 10) {
+        // same cost model as the fp32 picker: rounds of tiles per CU x tile area / measured shape efficiency
+        const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+        const long big = (long)cdiv(M, 256) * cdiv(N, 256) * batch.count, small = (long)cdiv(M, 128) * cdiv(N, 128) * batch.count;
+        const double cost_big = (double)((big + cus - 1) / cus) * 65536.0;
+        const double cost_small = (double)((small + cus - 1) / cus) * 16384.0 / 0.75;
+        // the small tile with three LDS stages holds one workgroup per CU: only worth it when there is at most one to hold
+        variant = cost_big <= cost_small ? 7 : (small <= cus ? 9 : 8);
     }
     if (variant == 3) return launch_hgemm_dma_tile<HShapeDma>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     if (variant == 4) return launch_hgemm_dma_tile<HShapeDma64>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     if (variant == 5) return launch_hgemm_dma_tile<HShapeDma5>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     if (variant == 6) return launch_hgemm_dma_tile<HShapeDma64W8a>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     if (variant == 7) return launch_hgemm_dma_tile<HShapeDma64W8b>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 8) return launch_hgemm_dma_tile<HShapeDmaSmall>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 9) return launch_hgemm_dma_tile<HShapeDmaSmall3>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 10) return launch_hgemm_dma_tile<HShapeDmaTall>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     if (variant == 1) return launch_hgemm_tile<HShapeBig, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     return launch_hgemm_tile<HShapeSmall, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
 }
