@@ -482,6 +482,86 @@ int gemm3_host_pipeline(const T* hA, int lda, size_t plane_a, const T* hB, int l
     return 0;
 }
 
+// One GEMM on HOST-resident matrices (the Matrix<T> overloads of de::cuda::GEMM, GEMM.h:56-131, :139-228): the result's
+// rows are cut into panels, and the upload of A's panel p+1, the kernel on panel p and the download of result panel p-1
+// overlap on three streams.  B goes up first, whole.  Device copies keep the host pitches.  Overlap needs pinned host
+// memory (decx_hip_host_malloc); pageable memory works but serialises.
+template <typename T, class Enqueue>
+int gemm_host_pipeline(const T* hA, int lda, const T* hB, int ldb, const T* hC, int ldc, T* hD, int ldd, int M, int N, int K,
+                       Enqueue enqueue) {
+    if (!g_rt.is_init) return need_init();
+    if (!hA || !hB || !hD) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "null matrix pointer\n");
+    if (M <= 0 || N <= 0 || K <= 0) return fail(DECX_HIP_FAIL_DIMS, "Matrix Dims don't match each other");
+    if (lda < K || ldb < N || ldd < N || (hC && ldc < N))
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "leading dimension smaller than the row length\n");
+    // panels of whole 256-row tiles, big enough to fill the chip (>= 2048 rows x N), at most 16 of them
+    int panel_rows = 2048;
+    while ((long)cdiv(M, panel_rows) > 16) panel_rows *= 2;
+    const int panels = cdiv(M, panel_rows);
+    T *dA = nullptr, *dB = nullptr, *dD = nullptr;
+    hipStream_t s_up = nullptr, s_down = nullptr;
+    hipEvent_t b_up = nullptr, up[16] = {}, done[16] = {};
+    int rc = 0;
+    auto cleanup = [&] {
+        (void)hipDeviceSynchronize();
+        if (dA) (void)hipFree(dA);
+        if (dB) (void)hipFree(dB);
+        if (dD) (void)hipFree(dD);
+        if (b_up) (void)hipEventDestroy(b_up);
+        for (int p = 0; p < 16; ++p) {
+            if (up[p]) (void)hipEventDestroy(up[p]);
+            if (done[p]) (void)hipEventDestroy(done[p]);
+        }
+        if (s_up) (void)hipStreamDestroy(s_up);
+        if (s_down) (void)hipStreamDestroy(s_down);
+    };
+#define PIPE_TRY(expr)                                   \
+    do {                                                 \
+        hipError_t e_ = (expr);                          \
+        if (e_ != hipSuccess) { rc = hip_fail(e_, #expr); cleanup(); return rc; } \
+    } while (0)
+    if (hipMalloc(&dA, (size_t)M * lda * sizeof(T)) != hipSuccess || hipMalloc(&dB, (size_t)K * ldb * sizeof(T)) != hipSuccess ||
+        hipMalloc(&dD, (size_t)M * ldd * sizeof(T)) != hipSuccess) {
+        (void)hipGetLastError();
+        cleanup();
+        return fail(DECX_HIP_FAIL_ALLOCATION, "Fail to allocate memory\n");
+    }
+    PIPE_TRY(hipStreamCreateWithFlags(&s_up, hipStreamNonBlocking));
+    PIPE_TRY(hipStreamCreateWithFlags(&s_down, hipStreamNonBlocking));
+    PIPE_TRY(hipEventCreateWithFlags(&b_up, hipEventDisableTiming));
+    for (int p = 0; p < panels; ++p) {
+        PIPE_TRY(hipEventCreateWithFlags(&up[p], hipEventDisableTiming));
+        PIPE_TRY(hipEventCreateWithFlags(&done[p], hipEventDisableTiming));
+    }
+    PIPE_TRY(hipMemcpy2DAsync(dB, (size_t)ldb * sizeof(T), hB, (size_t)ldb * sizeof(T), (size_t)N * sizeof(T), K,
+                              hipMemcpyHostToDevice, s_up));
+    PIPE_TRY(hipEventRecord(b_up, s_up));
+    PIPE_TRY(hipStreamWaitEvent(g_rt.stream, b_up, 0));
+    for (int p = 0; p < panels; ++p) {
+        const int r0 = p * panel_rows, rows = (M - r0 < panel_rows) ? M - r0 : panel_rows;
+        PIPE_TRY(hipMemcpy2DAsync(dA + (size_t)r0 * lda, (size_t)lda * sizeof(T), hA + (size_t)r0 * lda, (size_t)lda * sizeof(T),
+                                  (size_t)K * sizeof(T), rows, hipMemcpyHostToDevice, s_up));
+        if (hC)   // C goes into the result buffer and is accumulated onto in place, as the reference does (GEMM.h:196-206)
+            PIPE_TRY(hipMemcpy2DAsync(dD + (size_t)r0 * ldd, (size_t)ldd * sizeof(T), hC + (size_t)r0 * ldc, (size_t)ldc * sizeof(T),
+                                      (size_t)N * sizeof(T), rows, hipMemcpyHostToDevice, s_up));
+        PIPE_TRY(hipEventRecord(up[p], s_up));
+        PIPE_TRY(hipStreamWaitEvent(g_rt.stream, up[p], 0));
+        Batch one;
+        one.stream = g_rt.stream;
+        rc = enqueue(dA + (size_t)r0 * lda, dB, hC ? dD + (size_t)r0 * ldd : nullptr, dD + (size_t)r0 * ldd, rows, one);
+        if (rc) { cleanup(); return rc; }
+        PIPE_TRY(hipEventRecord(done[p], g_rt.stream));
+        PIPE_TRY(hipStreamWaitEvent(s_down, done[p], 0));
+        PIPE_TRY(hipMemcpy2DAsync(hD + (size_t)r0 * ldd, (size_t)ldd * sizeof(T), dD + (size_t)r0 * ldd, (size_t)ldd * sizeof(T),
+                                  (size_t)N * sizeof(T), rows, hipMemcpyDeviceToHost, s_down));
+    }
+    PIPE_TRY(hipStreamSynchronize(s_down));
+    PIPE_TRY(hipStreamSynchronize(g_rt.stream));
+#undef PIPE_TRY
+    cleanup();
+    return 0;
+}
+
 // Plain streaming copy, 16 bytes per lane and iteration: the known-size kernel that hardware traffic counters
 // (FETCH_SIZE / WRITE_SIZE) are calibrated against.
 __global__ __launch_bounds__(256) void copy_kernel(f32x4* __restrict__ dst, const f32x4* __restrict__ src, size_t quads) {
@@ -728,6 +808,21 @@ int decx_hip_gemm3_host_f16(const uint16_t* hA, int lda, size_t plane_a, const u
                                          [&](const uint16_t* a, const uint16_t* b, const uint16_t* c, uint16_t* d, const Batch& one) {
                                              return hgemm_enqueue(a, lda, b, ldb, c, ldd, d, ldd, M, N, K, one);
                                          });
+}
+
+int decx_hip_gemm_host_f32(const float* hA, int lda, const float* hB, int ldb, const float* hC, int ldc, float* hD, int ldd,
+                           int M, int N, int K) {
+    return gemm_host_pipeline<float>(hA, lda, hB, ldb, hC, ldc, hD, ldd, M, N, K,
+                                     [&](const float* a, const float* b, const float* c, float* d, int rows, const Batch& one) {
+                                         return sgemm_enqueue(a, lda, b, ldb, c, ldd, d, ldd, rows, N, K, one);
+                                     });
+}
+int decx_hip_gemm_host_f16(const uint16_t* hA, int lda, const uint16_t* hB, int ldb, const uint16_t* hC, int ldc, uint16_t* hD,
+                           int ldd, int M, int N, int K) {
+    return gemm_host_pipeline<uint16_t>(hA, lda, hB, ldb, hC, ldc, hD, ldd, M, N, K,
+                                        [&](const uint16_t* a, const uint16_t* b, const uint16_t* c, uint16_t* d, int rows, const Batch& one) {
+                                            return hgemm_enqueue(a, lda, b, ldb, c, ldd, d, ldd, rows, N, K, one);
+                                        });
 }
 
 int decx_hip_conv2_im2col_f32_async(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt,

@@ -50,6 +50,19 @@ template <> struct GemmCall<de::Half> {
     }
 };
 
+template <typename T> struct HostGemmCall;
+template <> struct HostGemmCall<float> {
+    static int run(const float* A, int lda, const float* B, int ldb, const float* C, int ldc, float* D, int ldd, int M,
+                   int N, int K) { return decx_hip_gemm_host_f32(A, lda, B, ldb, C, ldc, D, ldd, M, N, K); }
+};
+template <> struct HostGemmCall<de::Half> {
+    static int run(const de::Half* A, int lda, const de::Half* B, int ldb, const de::Half* C, int ldc, de::Half* D, int ldd,
+                   int M, int N, int K) {
+        return decx_hip_gemm_host_f16(reinterpret_cast<const uint16_t*>(A), lda, reinterpret_cast<const uint16_t*>(B), ldb,
+                                      reinterpret_cast<const uint16_t*>(C), ldc, reinterpret_cast<uint16_t*>(D), ldd, M, N, K);
+    }
+};
+
 template <typename T>
 de::DH gemm_host(de::Matrix<T>& A_, de::Matrix<T>& B_, de::Matrix<T>* C_, de::Matrix<T>& dst_) {
     auto* A = dynamic_cast<decx::_Matrix<T>*>(&A_);
@@ -62,30 +75,11 @@ de::DH gemm_host(de::Matrix<T>& A_, de::Matrix<T>& B_, de::Matrix<T>* C_, de::Ma
     if (C && (C->width != B->width || C->height != A->height))                            // GEMM.h:154-157
         return de::DH{decx::DECX_FAIL_DimsNotMatching, kMDims};
     const int M = (int)A->height, K = (int)A->width, N = (int)B->width;
-    // C may be the same object as dst: read it before dst is re-constructed
-    DeviceTemp dA, dB, dD;
-    if (dA.alloc(A->total_bytes) || dB.alloc(B->total_bytes)) return alloc_fail();
-    int rc = decx_hip_memcpy2d(dA.ptr, (size_t)A->pitch * sizeof(T), A->Mat.ptr, (size_t)A->pitch * sizeof(T),
-                               (size_t)K * sizeof(T), M, DECX_HIP_H2D);
-    if (rc) return from_status(rc);
-    rc = decx_hip_memcpy2d(dB.ptr, (size_t)B->pitch * sizeof(T), B->Mat.ptr, (size_t)B->pitch * sizeof(T),
-                           (size_t)N * sizeof(T), K, DECX_HIP_H2D);
-    if (rc) return from_status(rc);
-    const uint pitch_d = decx::ceil_to((uint)N, decx::matrix_align<T>());
-    if (dD.alloc((size_t)pitch_d * M * sizeof(T))) return alloc_fail();
-    if (C) {   // the reference uploads C into the dst device buffer and accumulates in place (GEMM.h:196-206)
-        rc = decx_hip_memcpy2d(dD.ptr, (size_t)pitch_d * sizeof(T), C->Mat.ptr, (size_t)C->pitch * sizeof(T),
-                               (size_t)N * sizeof(T), M, DECX_HIP_H2D);
-        if (rc) return from_status(rc);
-    }
-    if (!dst->re_construct((uint)N, (uint)M, decx::Page_Locked)) return alloc_fail();     // GEMM.h:73
-    rc = GemmCall<T>::run(static_cast<const T*>(dA.ptr), (int)A->pitch, static_cast<const T*>(dB.ptr), (int)B->pitch,
-                          C ? static_cast<const T*>(dD.ptr) : nullptr, (int)pitch_d, static_cast<T*>(dD.ptr), (int)pitch_d,
-                          M, N, K);
-    if (rc) return from_status(rc);
-    rc = decx_hip_memcpy2d(dst->Mat.ptr, (size_t)dst->pitch * sizeof(T), dD.ptr, (size_t)pitch_d * sizeof(T),
-                           (size_t)N * sizeof(T), M, DECX_HIP_D2H);                        // only the valid columns, GEMM.h:119-120
-    return from_status(rc);
+    // dst takes its size from the operands (GEMM.h:73); when C is the same object it already has it and keeps its data
+    if (!dst->re_construct((uint)N, (uint)M, decx::Page_Locked)) return alloc_fail();
+    // allocation, uploads, kernel and download, pipelined over row panels, all below the C ABI
+    return from_status(HostGemmCall<T>::run(A->Mat.ptr, (int)A->pitch, B->Mat.ptr, (int)B->pitch, C ? C->Mat.ptr : nullptr,
+                                            C ? (int)C->pitch : 0, dst->Mat.ptr, (int)dst->pitch, M, N, K));
 }
 
 template <typename T>

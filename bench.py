@@ -120,21 +120,17 @@ class PinnedArray:
 
 
 def bench_host_resident_gemm(capi, A, B, reps):
-    """de::cuda::GEMM(Matrix<float>...) equivalent (GEMM.h:56-131): pinned host operands, H2D of A and B, kernel, D2H of
-    the result -- the PCIe-inclusive figure.  Device buffers keep the host pitch; none of it is padded."""
+    """de::cuda::GEMM(Matrix<float>...) equivalent (GEMM.h:56-131) through decx_hip_gemm_host_f32: pinned host operands,
+    device allocation, uploads, kernel and download (pipelined over row panels) -- the PCIe-inclusive figure."""
     M, K = A.shape
     N = B.shape[1]
     hA, hB, hD = PinnedArray(capi, (M, K), np.float32), PinnedArray(capi, (K, N), np.float32), PinnedArray(capi, (M, N), np.float32)
     hA.array[:], hB.array[:] = A, B
-    dA, dB, dD = capi.DeviceBuffer(M * K * 4), capi.DeviceBuffer(K * N * 4), capi.DeviceBuffer(M * N * 4)
     L = capi.lib()
     best = None
     for _ in range(reps + 1):
         t0 = time.perf_counter()
-        capi.check(L.decx_hip_memcpy2d(dA.ptr, K * 4, hA.ptr, K * 4, K * 4, M, capi.H2D))
-        capi.check(L.decx_hip_memcpy2d(dB.ptr, N * 4, hB.ptr, N * 4, N * 4, K, capi.H2D))
-        capi.sgemm(dA.ptr, K, dB.ptr, N, dD.ptr, N, M, N, K)
-        capi.check(L.decx_hip_memcpy2d(hD.ptr, N * 4, dD.ptr, N * 4, N * 4, M, capi.D2H))
+        capi.check(L.decx_hip_gemm_host_f32(hA.ptr, K, hB.ptr, N, None, 0, hD.ptr, N, M, N, K))
         dt = time.perf_counter() - t0
         best = dt if best is None else min(best, dt)
     for h in (hA, hB, hD): h.free()

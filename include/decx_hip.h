@@ -112,6 +112,17 @@ int decx_hip_hgemm_f32acc_batched(const uint16_t* A, int lda, size_t stride_a, c
                                   const uint16_t* Cin, int ldc, size_t stride_c, uint16_t* D, int ldd, size_t stride_d, int M,
                                   int N, int K, int batch);
 
+/* de::cuda::GEMM(Matrix<T>& A, B, [C,] dst) on HOST-resident matrices (GEMM.h:56-131, :139-228; decx::sGEMM_part /
+ * hGEMM_part, GEMM3_macros.h:65-134): everything between the caller's host buffers -- device allocation, uploads, the
+ * kernel, the download -- without the reference's padded device copies (GEMM.h:80-104).  The rows of the result are
+ * processed in panels so that the upload of the next panel of A, the kernel and the download of the previous result
+ * panel overlap (the reference runs them back to back on one stream).  hA, hB, hC (nullable, may equal hD), hD are
+ * HOST pointers; pinned memory (decx_hip_host_malloc) is needed for the overlap, pageable memory works serially. */
+int decx_hip_gemm_host_f32(const float* hA, int lda, const float* hB, int ldb, const float* hC, int ldc, float* hD, int ldd,
+                           int M, int N, int K);
+int decx_hip_gemm_host_f16(const uint16_t* hA, int lda, const uint16_t* hB, int ldb, const uint16_t* hC, int ldc, uint16_t* hD,
+                           int ldd, int M, int N, int K);
+
 /* de::cuda::GEMM3(MatrixArray<T>& A, B, [C,] dst) on HOST-resident arrays (GEMM3.h:40-300): the reference's pipeline of
  * GEMM3_macros.h:140-374 -- upload of matrix i+1, kernel on matrix i and download of result i-1 overlap on three
  * streams with two device buffer sets.  hA, hB, hC (nullable), hD are HOST pointers (pinned memory overlaps best);

@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 
 from backup_1_amd import workloads
-from gpu_helpers import gpu_sgemm, rel_err_vs_abs_scale
+from gpu_helpers import gpu_sgemm, rel_err_vs_abs_scale, pitched
 
 pytestmark = pytest.mark.gpu
 
@@ -174,6 +174,40 @@ def test_gemm3_host_pipeline(gpu):
     assert np.array_equal(D, want.astype(np.float32))
     gpu.check(L.decx_hip_gemm3_host_f32(p(A), K, M * K, p(B), N, K * N, p(C), N, M * N, p(D), N, M * N, M, N, K, count))
     assert np.array_equal(D, (want + C).astype(np.float32))
+
+
+@pytest.mark.parametrize("shape", [(96, 40, 120), (2048 + 300, 72, 264), (5000, 33, 100)])
+def test_host_resident_gemm_pipeline(gpu, shape):
+    # decx_hip_gemm_host_f32: pitched host matrices in, pitched host matrix out; M above 2048 runs several row panels
+    M, K, N = shape
+    A, B = workloads.small_ints((M, K), 91), workloads.small_ints((K, N), 92)
+    C = workloads.small_ints((M, N), 93, -50, 50)
+    Ab, lda = pitched(A, 8)
+    Bb, ldb = pitched(B, 8)
+    Cb, ldc = pitched(C, 8)
+    ldd = ldc
+    Db = np.full((M, ldd), -5.0, np.float32)
+    L = gpu.lib()
+    p = lambda a: a.ctypes.data
+    want = (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32)
+    gpu.check(L.decx_hip_gemm_host_f32(p(Ab), lda, p(Bb), ldb, None, 0, p(Db), ldd, M, N, K))
+    assert np.array_equal(Db[:, :N], want) and np.all(Db[:, N:] == -5.0)
+    gpu.check(L.decx_hip_gemm_host_f32(p(Ab), lda, p(Bb), ldb, p(Cb), ldc, p(Db), ldd, M, N, K))
+    assert np.array_equal(Db[:, :N], want + C)
+    Db[:, :N] = C                                          # C and dst the same host matrix
+    gpu.check(L.decx_hip_gemm_host_f32(p(Ab), lda, p(Bb), ldb, p(Db), ldd, p(Db), ldd, M, N, K))
+    assert np.array_equal(Db[:, :N], want + C) and np.all(Db[:, N:] == -5.0)
+    assert L.decx_hip_gemm_host_f32(p(Ab), K - 1, p(Bb), ldb, None, 0, p(Db), ldd, M, N, K) == 0x0d
+
+
+def test_host_resident_gemm_pipeline_fp16(gpu, oracle):
+    M, K, N = 2048 + 100, 64, 144
+    A, B = workloads.small_ints((M, K), 94, -3, 3), workloads.small_ints((K, N), 95, -3, 3)
+    Ah, Bh = oracle.float_to_half(A), oracle.float_to_half(B)
+    D = np.zeros((M, N), np.uint16)
+    p = lambda a: a.ctypes.data
+    gpu.check(gpu.lib().decx_hip_gemm_host_f16(p(Ah), K, p(Bh), N, None, 0, p(D), N, M, N, K))
+    assert np.array_equal(oracle.half_to_float(D), (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32))
 
 
 def _splitk(gpu, A, B, C=None, splits=0, inplace=False):
