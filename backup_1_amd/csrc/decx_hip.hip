@@ -276,13 +276,20 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
     const size_t filt_bytes = ((size_t)(N - 1) * filt_stride + (size_t)(kh - 1) * filt_row_stride + (size_t)kw * dpitch) * sizeof(float);
     if (src_bytes >= 0x80000000ull || filt_bytes >= 0x80000000ull)
         return fail(DECX_HIP_FAIL_ERROR_PARAMS, "source tensor and filter bank must each stay below 2 GiB\n");
-    Im2colA a{src, H, W, dpitch, kh, kw, flag ? kh / 2 : 0, flag ? kw / 2 : 0, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
-    FilterB b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
     TensorOut out{Wout, dst_dpitch, dst_row_stride, dst_row_stride == (size_t)Wout * dst_dpitch, relu};
     Batch one;
     one.stream = g_rt.stream;
+    const int variant = pick_sgemm_variant(M, N, K, 1);
+    const int oy = flag ? kh / 2 : 0, ox = flag ? kw / 2 : 0;
     // a bias is the "+ C" operand with row stride 0: every output pixel adds the same N values
-    return dispatch_sgemm(pick_sgemm_variant(M, N, K, 1), a, b, bias, 0, dst, out, M, N, K, one);
+    if (dpitch % 8 == 0) {       // the 8 consecutive k of a staging task never straddle a tap
+        Im2colA<true> a{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
+        FilterB<true> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
+        return dispatch_sgemm(variant, a, b, bias, 0, dst, out, M, N, K, one);
+    }
+    Im2colA<false> a{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
+    FilterB<false> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
+    return dispatch_sgemm(variant, a, b, bias, 0, dst, out, M, N, K, one);
 }
 
 // ---------------------------------------------------------------------------------------------------------------

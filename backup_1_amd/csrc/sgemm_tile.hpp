@@ -6,18 +6,23 @@
 //
 // Staging: global -> registers -> LDS, two LDS buffers, one barrier per K step; the loads run one or two K steps ahead
 // of the MFMAs.  A is kept in LDS as float4 "k-quads":
-//   A quad (q, m) = A[m][4q .. 4q+3]          at  As[q][m]             (plane rows 2 slots out of step mod 8, which
+//   A quad (p, m) = A[m][8s+par+{0,2,4,6}], p = 2s+par,  at  As[p][m]  (plane rows 2 slots out of step mod 8, which
 //                                                                       keeps the staging stores off each other's banks)
-// so that one ds_read_b128 per 32-row block feeds four MFMAs.  The MFMA's two k-slots (lanes 0-31 / 32-63) take
-// quads 2s and 2s+1: within a quad pair the products are summed in the order k = 8s+e (lanes 0-31) and 8s+4+e
-// (lanes 32-63), e = 0..3 -- a fixed permutation of k inside each group of 8, applied identically to A and B.
+// so that one ds_read_b128 per 32-row block feeds four MFMAs.
+// Summation order.  v_mfma_f32_32x32x2_f32 computes, per output element, fma(a1, b1, fma(a0, b0, c)) with operand 0 from
+// lanes 0-31 and operand 1 from lanes 32-63 (checked bit for bit on the hardware), i.e. it IS two steps of the
+// reference's single-accumulator fused chain.  The k indices are therefore laid out so that every output sees them in
+// ascending order: of each group of 8 consecutive k (8s .. 8s+7) the even ones go to plane 2s, the odd ones to plane
+// 2s+1 (de-interleaved while staging), lanes 0-31 read plane 2s and lanes 32-63 plane 2s+1, and MFMA e of the group
+// multiplies k = 8s+2e and 8s+2e+1.  The result equals fmaf over k = 0 .. K-1 from a single accumulator -- the
+// arithmetic of every fp32 path of the reference -- bit for bit, whatever the tile shape.
 // B has two LDS layouts, chosen by its source:
 //   * a row-major K x N matrix (DenseB) stays row-major, Bs[k][n], exactly as loaded -- no transpose, no VALU work.
 //     The wave's 32x32 blocks then take INTERLEAVED columns: lane li of block ni owns column NI*li + ni of the wave's
 //     strip, so the NI operands a lane needs at one k are NI consecutive floats of one row (one ds_read_b128 for
 //     NI = 4) and the NI results it holds per row are consecutive too (one 16-byte store).
 //   * a filter bank (FilterB), whose k runs contiguously per column, is kept as k-quads like A:
-//       B quad (q, n) = B[4q .. 4q+3][n]      at  Bs[q][b_slot(n)];  block ni takes columns 32*ni + li.
+//       B quad (p, n) = B[8s+par+{0,2,4,6}][n] at  Bs[p][b_slot(n)];  block ni takes columns 32*ni + li.
 // Every VALU instruction costs the matrix pipe 3-5 cycles (measured: a wave's VALU and MFMA work do not overlap), so
 // the K loop is kept as free of address arithmetic and data shuffling as the layouts allow.
 //
@@ -99,6 +104,18 @@ struct TapWalk {
         ki += st.dki + (carry_kj ? 1 : 0);
         off += st.step_bytes + (carry_kj ? st.wrap_bytes : 0);
     }
+    // the position 4 further on (c and dpitch are multiples of 4, so c + 4 never exceeds dpitch)
+    __device__ __forceinline__ TapWalk next_quad(const TapStep& st, int dpitch, int kw) const {
+        TapWalk w;
+        w.k = k + 4;
+        const bool carry_c = c + 4 >= dpitch;
+        w.c = carry_c ? 0 : c + 4;
+        const bool carry_kj = carry_c && kj + 1 >= kw;
+        w.kj = carry_c ? (carry_kj ? 0 : kj + 1) : kj;
+        w.ki = ki + (carry_kj ? 1 : 0);
+        w.off = off + 16 + (carry_kj ? st.wrap_bytes : 0);
+        return w;
+    }
 };
 
 template <bool VEC>
@@ -120,15 +137,20 @@ struct DenseA {
     __device__ __forceinline__ KState k_state(int k) const { return KState{k}; }
     __device__ __forceinline__ KStep k_step(int dk) const { return KStep{dk}; }
     __device__ __forceinline__ void advance(KState& ks, const KStep& st) const { ks.k += st.dk; }
+    // the 8 consecutive k of one staging task: two quads
+    template <bool TAIL>
+    __device__ __forceinline__ void load_pair(const RowState& rs, const KState& ks, const KStep&, f32x4& lo, f32x4& hi) const {
+        lo = load<TAIL>(rs, ks);
+        hi = load<TAIL>(rs, KState{ks.k + 4});
+    }
     __device__ __forceinline__ RowState row_state(int m) const {
         RowState rs;
         rs.row = A + (size_t)(m < M ? m : M - 1) * lda;
         return rs;
     }
     template <bool TAIL>
-    __device__ __forceinline__ f32x4 load(const RowState& rs, const KState& ks, bool& keep) const {
+    __device__ __forceinline__ f32x4 load(const RowState& rs, const KState& ks) const {
         const int k = ks.k;
-        keep = true;
         f32x4 v = {0.f, 0.f, 0.f, 0.f};
         if (VEC) {
             if (!TAIL) {
@@ -152,6 +174,9 @@ struct DenseA {
 // Everything is 32-bit byte-offset arithmetic against one buffer resource (tensors stay below 2 GiB): per row the offset
 // of its top-left tap is kept, per K step the tap's offset is added, and a tap outside the image gets an out-of-range
 // offset instead, which the hardware answers with zeros.
+// PAIRED (dpitch % 8 == 0): the two quads of a staging task (8 consecutive k) always lie in the same tap, so one bounds
+// check and one offset serve both; otherwise the second quad's position is derived from the first.
+template <bool PAIRED>
 struct Im2colA {
     const float* src;
     int H, W, dpitch, kh, kw, oy, ox, Wout, Mtot, K;
@@ -181,11 +206,17 @@ struct Im2colA {
     __device__ __forceinline__ KStep k_step(int dk) const { return TapStep::make(dk, dpitch, kw, row_stride); }
     __device__ __forceinline__ void advance(KState& ks, const KStep& st) const { ks.advance(st, dpitch, kw); }
     template <bool TAIL>
-    __device__ __forceinline__ f32x4 load(const RowState& rs, const KState& ks, bool& keep) const {
-        // K = kh*kw*dpitch is a multiple of 4: quads never straddle it
+    __device__ __forceinline__ unsigned quad_offset(const RowState& rs, const KState& ks) const {
+        // K = kh*kw*dpitch is a multiple of 4 (of 8 when PAIRED): quads (pairs) never straddle it
         const bool inside = (unsigned)(rs.y + ks.ki) < (unsigned)H && (unsigned)(rs.x + ks.kj) < (unsigned)W && (!TAIL || ks.k < K);
-        keep = true;
-        return buffer_load_quad(make_rsrc(src, bytes), inside ? (unsigned)(rs.base + ks.off) : kOutOfRange);
+        return inside ? (unsigned)(rs.base + ks.off) : kOutOfRange;
+    }
+    template <bool TAIL>
+    __device__ __forceinline__ void load_pair(const RowState& rs, const KState& ks, const KStep& st, f32x4& lo, f32x4& hi) const {
+        const unsigned o = quad_offset<TAIL>(rs, ks);
+        lo = buffer_load_quad(make_rsrc(src, bytes), o);
+        if (PAIRED) hi = buffer_load_quad(make_rsrc(src, bytes), o + 16u);      // out of range stays out of range
+        else hi = buffer_load_quad(make_rsrc(src, bytes), quad_offset<TAIL>(rs, ks.next_quad(st, dpitch, kw)));
     }
 };
 
@@ -198,6 +229,7 @@ __device__ __forceinline__ float relu_by_sign(float v) {
 // Result addressing: dense matrices (row m at m*ld) or the convolution's output tensor (pixel (y,x) at
 // y*row_stride + x*dpitch).  relu: apply relu_by_sign to every result element before it is stored.
 struct DenseOut {
+    static constexpr bool PRELOAD_C = true;      // "+ C" enters the accumulators before the K walk
     int ld;
     bool relu = false;
     bool vec = false;      // every row of the result starts 16-byte aligned: runs of consecutive columns go out as one store
@@ -210,6 +242,7 @@ struct TensorOut {
     bool dense;      // row_stride == Wout*dpitch: pixel m simply starts at m*dpitch, no division needed
     bool relu = false;
     static constexpr bool vec = false;
+    static constexpr bool PRELOAD_C = false;     // the "+ C" operand is a bias row, added to the finished sum
     __device__ __forceinline__ float finish(float v) const { return relu ? relu_by_sign(v) : v; }
     __device__ __forceinline__ size_t offset(int m) const {
         if (dense) return (size_t)m * dpitch;
@@ -227,8 +260,8 @@ struct TensorOut {
 // ---------------------------------------------------------------------------------------------------------------
 // B as a row-major K x N matrix.  Staging copies 16-byte pieces of rows straight through: task t of a K step is
 // row t / (BN/4), column group t % (BN/4), so a wave reads and writes whole kilobytes of consecutive addresses.  Rows
-// are BN + 8 floats apart in LDS: the two half-waves of a fragment read touch rows 4 apart, and 4*(BN+8) floats puts
-// them on opposite halves of the 64 banks.
+// are BN + 8 floats apart in LDS (BN + 32 when a lane reads a single float, where both half-waves of a fragment read,
+// touching adjacent rows, are serviced together and have to land on opposite halves of the 64 banks).
 template <bool VEC>
 struct DenseB {
     const float* B;
@@ -238,7 +271,7 @@ struct DenseB {
     __device__ __forceinline__ void select_batch(int b) { B += (size_t)b * batch_stride; }
     __device__ __forceinline__ void set_k_end(int k_end) { K = k_end; }
     template <class S>
-    static constexpr int row_floats() { return S::BN + 8; }
+    static constexpr int row_floats() { return S::BN + (S::NI == 1 ? 32 : 8); }
     template <class S>
     static constexpr int lds_floats() { return S::BK * row_floats<S>(); }      // one buffer
     template <class S>
@@ -261,7 +294,7 @@ struct DenseB {
     __device__ __forceinline__ void advance(KState& ks, const KStep& st) const { ks.k0 += st.dk; }
 
     template <class S, bool TAIL>
-    __device__ __forceinline__ void load(f32x4* st, int tid, const KState& ks, int bn0) const {
+    __device__ __forceinline__ void load(f32x4* st, int tid, const KState& ks, int bn0, const KStep&) const {
         constexpr int CG = S::BN / 4;
 #pragma unroll
         for (int p = 0; p < quads<S>(); ++p) {
@@ -290,13 +323,13 @@ struct DenseB {
             *reinterpret_cast<f32x4*>(buf + (task / CG) * row_floats<S>() + 4 * (task % CG)) = st[p];
         }
     }
-    // operands of quad pair s for this lane: frag[e][ni] = B[k(s, e, lh)][wn0 + NI*li + ni], k = 8s + 4lh + e
+    // operands of k-group s for this lane: frag[e][ni] = B[k(s, e, lh)][wn0 + NI*li + ni], k = 8s + 2e + lh
     template <class S>
     __device__ __forceinline__ void read_frags(const float* buf, int s, int lh, int li, int wn0, float (*frag)[S::NI]) const {
         typedef float vec_t __attribute__((ext_vector_type(S::NI)));
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const vec_t v = *reinterpret_cast<const vec_t*>(buf + (8 * s + 4 * lh + e) * row_floats<S>() + wn0 + S::NI * li);
+            const vec_t v = *reinterpret_cast<const vec_t*>(buf + (8 * s + 2 * e + lh) * row_floats<S>() + wn0 + S::NI * li);
 #pragma unroll
             for (int ni = 0; ni < S::NI; ++ni) frag[e][ni] = v[ni];
         }
@@ -308,7 +341,8 @@ struct DenseB {
 
 // B as a bank of N filters, filter n holding its taps channel-innermost: column n of the lowered GEMM is filter n and
 // four consecutive k (same tap, four channels) are already contiguous in memory, so a k-quad is one 16-byte load.
-// Same 32-bit offsets against a buffer resource as Im2colA (the bank stays below 2 GiB).
+// Same 32-bit offsets against a buffer resource as Im2colA (the bank stays below 2 GiB), same meaning of PAIRED.
+template <bool PAIRED>
 struct FilterB {
     const float* filt;
     int N, K, dpitch, kw;
@@ -317,28 +351,32 @@ struct FilterB {
     static constexpr bool ROW_MAJOR_LDS = false;
     __device__ __forceinline__ void select_batch(int) {}
     __device__ __forceinline__ void set_k_end(int k_end) { K = k_end; }
+    // a staging task is 8 consecutive k (one k-group s) of one filter n: two 16-byte loads, de-interleaved into the
+    // even-k and odd-k planes.  Task id = tid + j*NT: group s = id % GROUPS, filter (id / GROUPS) % BN -- when there are
+    // more threads than tasks the surplus repeats earlier tasks, which is harmless and keeps the loop branch-free.
     template <class S>
-    static constexpr int quads() { return S::KQ * S::BN / S::NT; }
+    static constexpr int tasks() { return (S::BN * (S::KQ / 2) + S::NT - 1) / S::NT; }
+    template <class S>
+    static constexpr int quads() { return 2 * tasks<S>(); }
     template <class S>
     static constexpr int lds_floats() { return 4 * S::KQ * S::B_ROW; }          // one buffer
     template <class S>
     static constexpr int frag_reads() { return S::NI; }                        // one k-quad per 32-column block
-    // every quad of a thread has the same k-quad index q = tid % KQ (NT is a multiple of KQ): one walk serves them all;
-    // what differs is the filter, whose byte offset is worked out once
-    template <int QUADS>
+    template <int TASKS>
     struct KStateT {
-        TapWalk walk;
-        int filter_base[QUADS];
+        TapWalk walk;                 // the first quad of this thread's k-group (the same group for all its tasks)
+        int filter_base[TASKS];       // byte offset of each task's filter
     };
     typedef TapStep KStep;
     template <class S>
-    __device__ __forceinline__ KStateT<quads<S>()> k_state(int tid, int k_begin, int bn0) const {
-        static_assert((S::KQ * S::BN) % S::NT == 0 && S::NT % S::KQ == 0, "filter staging must divide evenly");
-        KStateT<quads<S>()> ks;
-        ks.walk.init(k_begin + 4 * (tid % S::KQ), dpitch, kw, filt_row_stride);
+    __device__ __forceinline__ KStateT<tasks<S>()> k_state(int tid, int k_begin, int bn0) const {
+        constexpr int G = S::KQ / 2;
+        static_assert(S::NT % G == 0, "every task of a thread must fall into the same k-group");
+        KStateT<tasks<S>()> ks;
+        ks.walk.init(k_begin + 8 * (tid % G), dpitch, kw, filt_row_stride);
 #pragma unroll
-        for (int j = 0; j < quads<S>(); ++j) {
-            int n = bn0 + (tid + j * S::NT) / S::KQ;
+        for (int j = 0; j < tasks<S>(); ++j) {
+            int n = bn0 + ((tid + j * S::NT) / G) % S::BN;
             if (n >= N) n = N - 1;
             ks.filter_base[j] = 4 * n * filt_stride;
         }
@@ -350,23 +388,40 @@ struct FilterB {
     __device__ __forceinline__ void advance(KS& ks, const KStep& st) const { ks.walk.advance(st, dpitch, kw); }
 
     template <class S, bool TAIL, class KS>
-    __device__ __forceinline__ void load(f32x4* st, int tid, const KS& ks, int bn0) const {
-        const bool k_ok = !TAIL || ks.walk.k < K;
+    __device__ __forceinline__ void load(f32x4* st, int tid, const KS& ks, int bn0, const KStep& step) const {
+        const bool ok0 = !TAIL || ks.walk.k < K;
+        if (PAIRED) {
 #pragma unroll
-        for (int j = 0; j < quads<S>(); ++j)
-            st[j] = buffer_load_quad(make_rsrc(filt, bytes), k_ok ? (unsigned)(ks.filter_base[j] + ks.walk.off) : kOutOfRange);
+            for (int j = 0; j < tasks<S>(); ++j) {
+                const unsigned o = ok0 ? (unsigned)(ks.filter_base[j] + ks.walk.off) : kOutOfRange;
+                st[2 * j] = buffer_load_quad(make_rsrc(filt, bytes), o);
+                st[2 * j + 1] = buffer_load_quad(make_rsrc(filt, bytes), o + 16u);
+            }
+        } else {
+            const TapWalk second = ks.walk.next_quad(step, dpitch, kw);
+            const bool ok1 = !TAIL || second.k < K;
+#pragma unroll
+            for (int j = 0; j < tasks<S>(); ++j) {
+                st[2 * j] = buffer_load_quad(make_rsrc(filt, bytes), ok0 ? (unsigned)(ks.filter_base[j] + ks.walk.off) : kOutOfRange);
+                st[2 * j + 1] = buffer_load_quad(make_rsrc(filt, bytes), ok1 ? (unsigned)(ks.filter_base[j] + second.off) : kOutOfRange);
+            }
+        }
     }
     template <class S>
     __device__ __forceinline__ void store(float* buf, const f32x4* st, int tid) const {
+        constexpr int G = S::KQ / 2;
         f32x4* plane = reinterpret_cast<f32x4*>(buf);
 #pragma unroll
-        for (int j = 0; j < quads<S>(); ++j) {
+        for (int j = 0; j < tasks<S>(); ++j) {
             const int id = tid + j * S::NT;
-            const int q = id % S::KQ, n = id / S::KQ;
-            plane[q * S::B_ROW + b_slot(n)] = st[j];
+            const int s = id % G, n = (id / G) % S::BN;
+            const f32x4 even = {st[2 * j][0], st[2 * j][2], st[2 * j + 1][0], st[2 * j + 1][2]};
+            const f32x4 odd = {st[2 * j][1], st[2 * j][3], st[2 * j + 1][1], st[2 * j + 1][3]};
+            plane[(2 * s) * S::B_ROW + b_slot(n)] = even;
+            plane[(2 * s + 1) * S::B_ROW + b_slot(n)] = odd;
         }
     }
-    // operands of quad pair s for this lane: frag[e][ni] = B[8s + 4lh + e][wn0 + 32*ni + li]
+    // operands of k-group s for this lane: frag[e][ni] = B[8s + 2e + lh][wn0 + 32*ni + li] (plane 2s+lh, element e)
     template <class S>
     __device__ __forceinline__ void read_frags(const float* buf, int s, int lh, int li, int wn0, float (*frag)[S::NI]) const {
         const f32x4* plane = reinterpret_cast<const f32x4*>(buf) + (2 * s + lh) * S::B_ROW;
@@ -395,21 +450,24 @@ struct SgemmShape {
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     static constexpr int MI = WM / 32, NI = WN / 32;
     static constexpr int KQ = BK / 4;                         // k-quads per step
-    static constexpr int A_PASSES = (BM * KQ + NT - 1) / NT;  // float4 global loads of A per thread per step
-    // When BM*KQ is not a multiple of NT the last pass covers rows past BM: they are staged like any other (loaded from
-    // the tile's first row, stored to plane rows BM .. A_STAGED_ROWS-1 that no wave reads), which keeps the K loop free of
-    // branches -- a divergent skip would split the loop body into basic blocks and undo its instruction schedule.
-    static constexpr int A_STAGED_ROWS = A_PASSES * (NT / KQ);
+    static constexpr int KGROUPS = KQ / 2;                    // groups of 8 consecutive k per step
+    // An A staging task is one k-group of one row (two float4 loads); a thread takes A_TASKS of them per step.
+    // When BM*KGROUPS is not a multiple of NT the last pass covers rows past BM: they are staged like any other (loaded
+    // from the tile's first row, stored to plane rows BM .. A_STAGED_ROWS-1 that no wave reads), which keeps the K loop
+    // free of branches -- a divergent skip would split the loop body into basic blocks and undo its instruction schedule.
+    static constexpr int A_TASKS = (BM * KGROUPS + NT - 1) / NT;
+    static constexpr int A_PASSES = 2 * A_TASKS;              // float4 global loads of A per thread per step
+    static constexpr int A_STAGED_ROWS = A_TASKS * (NT / KGROUPS);
     static constexpr int A_ROW = A_STAGED_ROWS + 2;           // quads per A plane (planes 2 slots out of step mod 8)
     static constexpr int B_ROW = BN + 2;                      // quads per B plane (k-quad layout only)
-    static constexpr bool A_PARTIAL = (BM * KQ) % NT != 0;
+    static constexpr bool A_PARTIAL = (BM * KGROUPS) % NT != 0;
     template <class BSrc>
     static constexpr size_t lds_bytes() {
         return 2 * ((size_t)KQ * A_ROW * sizeof(f32x4) + (size_t)BSrc::template lds_floats<SgemmShape>() * sizeof(float));
     }
     static_assert(BM % (WAVES_M * 32) == 0 && BN % (WAVES_N * 32) == 0, "wave tile must be whole 32x32 blocks");
     static_assert(BK % 8 == 0, "a K step is whole quad pairs");
-    static_assert(NT % KQ == 0, "A staging: KQ lanes per row");
+    static_assert(NT % KGROUPS == 0, "A staging: KGROUPS lanes per row");
 };
 
 // SPLIT_K: blockIdx.z selects a K range of k_split_len (a multiple of BK); every range adds its partial products to dst
@@ -446,12 +504,13 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
     const int li = lane & 31, lh = lane >> 5;
 
     // ---- staging assignment -------------------------------------------------------------------------------
-    // A: KQ consecutive lanes cover one row's BK floats (one 16-byte quad each)
-    const int a_q = tid % KQ, a_r = tid / KQ;
-    constexpr int A_RSTEP = NT / KQ;
-    typename ASrc::RowState a_rs[S::A_PASSES];
+    // A: KGROUPS consecutive lanes cover one row's BK floats, 8 consecutive k (two 16-byte quads) each
+    constexpr int G = S::KGROUPS;
+    const int a_s = tid % G, a_r = tid / G;
+    constexpr int A_RSTEP = NT / G;
+    typename ASrc::RowState a_rs[S::A_TASKS];
 #pragma unroll
-    for (int p = 0; p < S::A_PASSES; ++p) {
+    for (int p = 0; p < S::A_TASKS; ++p) {
         const int r = a_r + p * A_RSTEP;
         a_rs[p] = a_src.row_state(bm0 + (S::A_PARTIAL && r >= BM ? 0 : r));
     }
@@ -460,9 +519,8 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
     constexpr int B_QUADS = BSrc::template quads<S>();
     constexpr int SETS = S::STAGE_SETS;
     f32x4 a_stage[SETS][S::A_PASSES];
-    bool a_keep[SETS][S::A_PASSES];
     f32x4 b_stage[SETS][B_QUADS];
-    typename ASrc::KState a_ks = a_src.k_state(k_begin + 4 * a_q);   // this thread's k-quad of the next K step to fetch
+    typename ASrc::KState a_ks = a_src.k_state(k_begin + 8 * a_s);   // first quad of this thread's k-group in the next step to fetch
     auto b_ks = b_src.template k_state<S>(tid, k_begin, bn0);
     const typename ASrc::KStep a_step = a_src.k_step(BK);
     const typename BSrc::KStep b_step = b_src.template k_step<S>();
@@ -472,23 +530,30 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         constexpr int SET = decltype(set_tag)::value;
         constexpr bool TAIL = decltype(tail_tag)::value;
 #pragma unroll
-        for (int p = 0; p < S::A_PASSES; ++p) a_stage[SET][p] = a_src.template load<TAIL>(a_rs[p], a_ks, a_keep[SET][p]);
-        b_src.template load<S, TAIL>(b_stage[SET], tid, b_ks, bn0);
+        for (int p = 0; p < S::A_TASKS; ++p)
+            a_src.template load_pair<TAIL>(a_rs[p], a_ks, a_step, a_stage[SET][2 * p], a_stage[SET][2 * p + 1]);
+        b_src.template load<S, TAIL>(b_stage[SET], tid, b_ks, bn0, b_step);
         a_src.advance(a_ks, a_step);
         b_src.advance(b_ks, b_step);
     };
 
+    // A's 8 consecutive k are de-interleaved on the way: even k to plane 2s, odd k to plane 2s+1
     auto store_stage = [&](auto set_tag, int buf) {
         constexpr int SET = decltype(set_tag)::value;
         f32x4* Ab = As + buf * KQ * S::A_ROW;
 #pragma unroll
-        for (int p = 0; p < S::A_PASSES; ++p) {
-            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-            Ab[a_q * S::A_ROW + a_r + p * A_RSTEP] = a_keep[SET][p] ? a_stage[SET][p] : zero;
+        for (int p = 0; p < S::A_TASKS; ++p) {
+            const f32x4 lo = a_stage[SET][2 * p], hi = a_stage[SET][2 * p + 1];
+            const f32x4 even = {lo[0], lo[2], hi[0], hi[2]}, odd = {lo[1], lo[3], hi[1], hi[3]};
+            Ab[(2 * a_s) * S::A_ROW + a_r + p * A_RSTEP] = even;
+            Ab[(2 * a_s + 1) * S::A_ROW + a_r + p * A_RSTEP] = odd;
         }
         b_src.template store<S>(Bs + buf * B_BUF, b_stage[SET], tid);
     };
 
+    // Accumulators start at zero, or at C for dst = A*B + C on dense matrices: the reference's chain starts from C
+    // (GEMM.cuh:223), and starting anywhere else would round differently.  A convolution's bias is added at the end.
+    constexpr bool PRELOAD_C = HAS_C && Out::PRELOAD_C;
     f32x16 acc[MI][NI];
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
@@ -496,6 +561,19 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
+    if (PRELOAD_C && (!SPLIT_K || blockIdx.z == 0)) {
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni) {
+                    const int n = bn0 + wn0 + BSrc::template strip_col<S>(ni, li);
+                    if (m < M && n < N) acc[mi][ni][r] = Cin[(size_t)m * ldc + n];
+                }
+            }
+    }
 
     // Fragments of one quad pair s: A, per 32-row block one float4 = four consecutive k of this lane's k-slot; B, per
     // k of the pair (e) and block (ni) one float, fetched as the B source's LDS layout dictates.
@@ -657,7 +735,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
             if (m < M) {
                 float* drow = D + out.offset(m);
                 const float* crow = HAS_C ? Cin + (size_t)m * ldc : nullptr;
-                const bool add_c = HAS_C && (!SPLIT_K || blockIdx.z == 0);
+                const bool add_c = HAS_C && !PRELOAD_C && (!SPLIT_K || blockIdx.z == 0);
                 if (BSrc::ROW_MAJOR_LDS && !SPLIT_K && NI > 1) {
                     const int n0 = bn0 + wn0 + NI * li;
                     if (out.vec && n0 + NI <= N) {

@@ -72,7 +72,10 @@ int decx_hip_sync(void);
  * and, between the H2D / D2H copies, the kernel step of the host-matrix overloads (decx::sGEMM_part,
  * GEMM3_macros.h:65-78).  Replaces cu_GEMM_fp32_spec / _ABC_spec (GEMM.cuh:31, :206) and the ragged variants
  * (GEMM_nonuniform.cuh:32-693).
- *   D[i*ldd + j] = Cin[i*ldc + j] + sum_k A[i*lda + k] * B[k*ldb + j],  0<=i<M, 0<=j<N, 0<=k<K, fp32 throughout.
+ *   D[i*ldd + j] = Cin[i*ldc + j] + sum_k A[i*lda + k] * B[k*ldb + j],  0<=i<M, 0<=j<N, 0<=k<K, fp32 throughout,
+ * evaluated exactly as the reference's kernels do: one accumulator per element, started at Cin (or 0) and updated by
+ * a fused multiply-add for k = 0, 1, ..., K-1 (GEMM_kernel_def.cuh:33-55, GEMM.cuh:83-92, :223).  The result is
+ * therefore bit-identical to the reference's and does not depend on the tile shape chosen.
  * M, N, K are arbitrary positive sizes: ragged edges are handled inside the kernel, no padded copies are made.
  * Cin may alias D.  Fast path needs A, B 16-byte aligned with lda, ldb multiples of 4 (always true for DECX
  * containers, whose pitch is a multiple of 8 floats, Matrix.h:24-27); otherwise a slower element-wise loader runs. */
@@ -146,7 +149,8 @@ int decx_hip_gemm3_host_f16(const uint16_t* hA, int lda, size_t plane_a, const u
  *   dst  : dst(y,x,n) at dst + y*dst_row_stride + x*dst_dpitch + n;
  *   flag : DECX_HIP_CONV_ZERO_COMPENSATE -> H x W outputs, input taken as 0 outside the image;
  *          DECX_HIP_CONV_NO_COMPENSATE   -> (H-2*(kh/2)) x (W-2*(kw/2)) outputs;  anything else -> DECX_HIP_FAIL_ERROR_FLAG.
- *   dst(y,x,n) = sum over k = (ki*kw + kj)*dpitch + c of src(y+ki-oy, x+kj-ox, c) * filt(n,ki,kj,c),
+ *   dst(y,x,n) = sum over k = (ki*kw + kj)*dpitch + c, ascending, one fused accumulator (eq_GEMM.cuh:65-74, :172-193),
+ *                of src(y+ki-oy, x+kj-ox, c) * filt(n,ki,kj,c),
  *   (oy,ox) = (kh/2, kw/2) for ZERO_COMPENSATE, (0,0) otherwise: cross-correlation, stride 1 (im2col.cuh:150-163).
  * Channels c in [C, dpitch) are read like any other, so the containers' zero padding must be zero.
  * Columns x >= W_out of a dst row (the wpitch padding) are not written. */
@@ -197,8 +201,8 @@ int decx_hip_timer_stop(float* milliseconds);
 const char* decx_hip_last_error(void);
 
 /* Tile-shape override for experiments: 0 = automatic choice by problem shape; other values select a fixed
- * kernel variant (see the table in backup_1_amd/csrc/decx_hip.hip).  Returns the previous value.  Results never depend on it
- * beyond fp32 summation order. */
+ * kernel variant (see the table in backup_1_amd/csrc/decx_hip.hip).  Returns the previous value.  fp32 results never depend on
+ * it (every shape walks k in the same order); fp16 results can differ in the last bit of the fp32 sum. */
 int decx_hip_set_sgemm_variant(int variant);
 int decx_hip_set_hgemm_variant(int variant);
 
