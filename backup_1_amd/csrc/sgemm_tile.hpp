@@ -64,6 +64,38 @@ __device__ __forceinline__ f32x4 buffer_load_quad(__amdgpu_buffer_rsrc_t rsrc, u
     return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)byte_offset, 0, 0));
 }
 
+// Two floats from any two registers to two consecutive-pair LDS dwords: halves 0 and 1 fill dwords (0,1) and (2,3) of a
+// 16-byte quad.  This is how 8 consecutive k are de-interleaved into an even-k and an odd-k quad without first gathering
+// the values into consecutive registers (which costs a register move per float, and every VALU instruction takes cycles
+// from the matrix pipe).  Issued from inline asm: the compiler does not count these stores in its LDS wait counts, which
+// is safe (a wait computed without them only ever waits for more), and the barrier code waits for lgkmcnt(0) itself.
+template <int HALF>
+__device__ __forceinline__ void lds_write_pair(unsigned byte_addr, float x, float y) {
+    if (HALF == 0) asm volatile("ds_write2_b32 %0, %1, %2 offset0:0 offset1:1" : : "v"(byte_addr), "v"(x), "v"(y) : "memory");
+    else asm volatile("ds_write2_b32 %0, %1, %2 offset0:2 offset1:3" : : "v"(byte_addr), "v"(x), "v"(y) : "memory");
+}
+// 8 consecutive k held as two quads (lo = k0..k3, hi = k4..k7); part 0, 1: even k to the quad at even_addr; 2, 3: odd k
+template <int PART>
+__device__ __forceinline__ void lds_write_deinterleaved(unsigned even_addr, unsigned odd_addr, const f32x4& lo, const f32x4& hi) {
+    if (PART == 0) lds_write_pair<0>(even_addr, lo[0], lo[2]);
+    if (PART == 1) lds_write_pair<1>(even_addr, hi[0], hi[2]);
+    if (PART == 2) lds_write_pair<0>(odd_addr, lo[1], lo[3]);
+    if (PART == 3) lds_write_pair<1>(odd_addr, hi[1], hi[3]);
+}
+__device__ __forceinline__ unsigned lds_byte_address(const void* p) {
+    return (unsigned)(size_t)(__attribute__((address_space(3))) const char*)p;
+}
+// Workgroup barrier that first waits for this wave's own LDS traffic, stated explicitly because the compiler's wait
+// counting does not see the inline-asm stores above.
+__device__ __forceinline__ void lds_sync() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
 // A K step of dk as an increment of the im2col position (c, kj, ki): dk = (dki*kw + dkj)*dpitch + dc, and of the byte
 // offset of that position inside a tensor whose rows are row_stride floats apart.  Worked out once per kernel so that
 // advancing is a handful of adds and selects.
@@ -288,7 +320,7 @@ struct DenseB {
         int dk;
     };
     template <class S>
-    __device__ __forceinline__ KState k_state(int tid, int k_begin, int bn0) const { return KState{k_begin}; }
+    __device__ __forceinline__ KState k_state(int tid, int k_begin, int bn0, const float*) const { return KState{k_begin}; }
     template <class S>
     __device__ __forceinline__ KStep k_step() const { return KStep{S::BK}; }
     __device__ __forceinline__ void advance(KState& ks, const KStep& st) const { ks.k0 += st.dk; }
@@ -314,14 +346,14 @@ struct DenseB {
             st[p] = v;
         }
     }
+    // LDS store instructions per thread and step, and store number W of them (W a compile-time tag)
     template <class S>
-    __device__ __forceinline__ void store(float* buf, const f32x4* st, int tid) const {
-        constexpr int CG = S::BN / 4;
-#pragma unroll
-        for (int p = 0; p < quads<S>(); ++p) {
-            const int task = tid + p * S::NT;
-            *reinterpret_cast<f32x4*>(buf + (task / CG) * row_floats<S>() + 4 * (task % CG)) = st[p];
-        }
+    static constexpr int writes() { return quads<S>(); }
+    template <class S, class KS, class WTag>
+    __device__ __forceinline__ void write_one(float* buf0, int buf, const f32x4* st, int tid, const KS&, WTag) const {
+        constexpr int CG = S::BN / 4, W = WTag::value;
+        const int task = tid + W * S::NT;
+        *reinterpret_cast<f32x4*>(buf0 + buf * lds_floats<S>() + (task / CG) * row_floats<S>() + 4 * (task % CG)) = st[W];
     }
     // operands of k-group s for this lane: frag[e][ni] = B[k(s, e, lh)][wn0 + NI*li + ni], k = 8s + 2e + lh
     template <class S>
@@ -366,19 +398,28 @@ struct FilterB {
     struct KStateT {
         TapWalk walk;                 // the first quad of this thread's k-group (the same group for all its tasks)
         int filter_base[TASKS];       // byte offset of each task's filter
+        unsigned store_addr[2][TASKS][2];   // LDS byte address of each task's even-k / odd-k quad, per buffer
     };
     typedef TapStep KStep;
     template <class S>
-    __device__ __forceinline__ KStateT<tasks<S>()> k_state(int tid, int k_begin, int bn0) const {
+    __device__ __forceinline__ KStateT<tasks<S>()> k_state(int tid, int k_begin, int bn0, const float* lds_buf0) const {
         constexpr int G = S::KQ / 2;
         static_assert(S::NT % G == 0, "every task of a thread must fall into the same k-group");
         KStateT<tasks<S>()> ks;
         ks.walk.init(k_begin + 8 * (tid % G), dpitch, kw, filt_row_stride);
+        const unsigned base = lds_byte_address(lds_buf0);
 #pragma unroll
         for (int j = 0; j < tasks<S>(); ++j) {
-            int n = bn0 + ((tid + j * S::NT) / G) % S::BN;
+            const int id = tid + j * S::NT;
+            const int s = id % G, col = (id / G) % S::BN;
+            int n = bn0 + col;
             if (n >= N) n = N - 1;
             ks.filter_base[j] = 4 * n * filt_stride;
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int par = 0; par < 2; ++par)
+                    ks.store_addr[b][j][par] = base + 4u * (unsigned)(b * lds_floats<S>()) + 16u * (unsigned)((2 * s + par) * S::B_ROW + b_slot(col));
         }
         return ks;
     }
@@ -408,18 +449,12 @@ struct FilterB {
         }
     }
     template <class S>
-    __device__ __forceinline__ void store(float* buf, const f32x4* st, int tid) const {
-        constexpr int G = S::KQ / 2;
-        f32x4* plane = reinterpret_cast<f32x4*>(buf);
-#pragma unroll
-        for (int j = 0; j < tasks<S>(); ++j) {
-            const int id = tid + j * S::NT;
-            const int s = id % G, n = (id / G) % S::BN;
-            const f32x4 even = {st[2 * j][0], st[2 * j][2], st[2 * j + 1][0], st[2 * j + 1][2]};
-            const f32x4 odd = {st[2 * j][1], st[2 * j][3], st[2 * j + 1][1], st[2 * j + 1][3]};
-            plane[(2 * s) * S::B_ROW + b_slot(n)] = even;
-            plane[(2 * s + 1) * S::B_ROW + b_slot(n)] = odd;
-        }
+    static constexpr int writes() { return 4 * tasks<S>(); }
+    template <class S, class KS, class WTag>
+    __device__ __forceinline__ void write_one(float*, int buf, const f32x4* st, int tid, const KS& ks, WTag) const {
+        constexpr int W = WTag::value, J = W / 4;
+        lds_write_deinterleaved<W % 4>(buf ? ks.store_addr[1][J][0] : ks.store_addr[0][J][0],
+                                       buf ? ks.store_addr[1][J][1] : ks.store_addr[0][J][1], st[2 * J], st[2 * J + 1]);
     }
     // operands of k-group s for this lane: frag[e][ni] = B[8s + 2e + lh][wn0 + 32*ni + li] (plane 2s+lh, element e)
     template <class S>
@@ -521,7 +556,16 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
     f32x4 a_stage[SETS][S::A_PASSES];
     f32x4 b_stage[SETS][B_QUADS];
     typename ASrc::KState a_ks = a_src.k_state(k_begin + 8 * a_s);   // first quad of this thread's k-group in the next step to fetch
-    auto b_ks = b_src.template k_state<S>(tid, k_begin, bn0);
+    auto b_ks = b_src.template k_state<S>(tid, k_begin, bn0, Bs);
+    // LDS byte addresses of this thread's A staging stores: [buffer][task][even-k plane, odd-k plane]
+    unsigned a_waddr[2][S::A_TASKS][2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int p = 0; p < S::A_TASKS; ++p)
+#pragma unroll
+            for (int par = 0; par < 2; ++par)
+                a_waddr[b][p][par] = lds_byte_address(As) + 16u * (unsigned)(b * KQ * S::A_ROW + (2 * a_s + par) * S::A_ROW + a_r + p * A_RSTEP);
     const typename ASrc::KStep a_step = a_src.k_step(BK);
     const typename BSrc::KStep b_step = b_src.template k_step<S>();
 
@@ -537,18 +581,21 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         b_src.advance(b_ks, b_step);
     };
 
-    // A's 8 consecutive k are de-interleaved on the way: even k to plane 2s, odd k to plane 2s+1
-    auto store_stage = [&](auto set_tag, int buf) {
-        constexpr int SET = decltype(set_tag)::value;
-        f32x4* Ab = As + buf * KQ * S::A_ROW;
-#pragma unroll
-        for (int p = 0; p < S::A_TASKS; ++p) {
-            const f32x4 lo = a_stage[SET][2 * p], hi = a_stage[SET][2 * p + 1];
-            const f32x4 even = {lo[0], lo[2], hi[0], hi[2]}, odd = {lo[1], lo[3], hi[1], hi[3]};
-            Ab[(2 * a_s) * S::A_ROW + a_r + p * A_RSTEP] = even;
-            Ab[(2 * a_s + 1) * S::A_ROW + a_r + p * A_RSTEP] = odd;
+    // LDS store number W of a step (A's first, then B's).  A's 8 consecutive k are de-interleaved on the way: even k to
+    // plane 2s, odd k to plane 2s+1.
+    constexpr int A_WRITES = 4 * S::A_TASKS, B_WRITES = BSrc::template writes<S>(), WRITE_OPS = A_WRITES + B_WRITES;
+    auto write_one = [&](auto set_tag, int buf, auto w_tag) {
+        constexpr int SET = decltype(set_tag)::value, W = decltype(w_tag)::value;
+        if constexpr (W < A_WRITES) {
+            constexpr int P = W / 4;
+            lds_write_deinterleaved<W % 4>(buf ? a_waddr[1][P][0] : a_waddr[0][P][0], buf ? a_waddr[1][P][1] : a_waddr[0][P][1],
+                                           a_stage[SET][2 * P], a_stage[SET][2 * P + 1]);
+        } else {
+            b_src.template write_one<S>(Bs, buf, b_stage[SET], tid, b_ks, std::integral_constant<int, W - A_WRITES>{});
         }
-        b_src.template store<S>(Bs + buf * B_BUF, b_stage[SET], tid);
+    };
+    auto store_stage = [&](auto set_tag, int buf) {
+        static_for<0, WRITE_OPS>([&](auto w_tag) { write_one(set_tag, buf, w_tag); });
     };
 
     // Accumulators start at zero, or at C for dst = A*B + C on dense matrices: the reference's chain starts from C
@@ -619,7 +666,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
     if (full_steps > 0) load_stage(Set0{}, std::false_type{});
     else load_stage(Set0{}, std::true_type{});
     store_stage(Set0{}, 0);
-    __syncthreads();
+    lds_sync();
     if constexpr (SETS == 2) {
         if (T > 1) {
             if (full_steps > 1) load_stage(Set1{}, std::false_type{});
@@ -630,7 +677,6 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
     static_assert(KQ == 4, "the pipelined loop is written for two quad pairs per K step");
     constexpr int VMEM_OPS = S::A_PASSES + B_QUADS;     // global loads per thread and step
     constexpr int FRAG_OPS = MI + BSrc::template frag_reads<S>();   // LDS reads per quad pair
-    constexpr int WRITE_OPS = S::A_PASSES + B_QUADS;    // ds_write_b128 per thread and step
     f32x4 af0[MI], af1[MI];
     BFrag bf0, bf1;
 
@@ -660,18 +706,16 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
 
         constexpr int LATE = MI * NI < PAIR_MFMAS / 4 ? MI * NI : PAIR_MFMAS / 4;   // MFMAs kept for after the barrier
         constexpr int EARLY = PAIR_MFMAS - LATE;
-        // step t+1 sits in the other set when there are two; buffer buf^1 was last read before the previous barrier
-        store_stage(std::integral_constant<int, SETS == 2 ? 1 - SET : 0>{}, buf ^ 1);
-        mfma_range(af1, bf1, std::integral_constant<int, 0>{}, std::integral_constant<int, EARLY>{});
-        constexpr int G1 = (EARLY / 2) / WRITE_OPS > 0 ? (EARLY / 2) / WRITE_OPS : 1;
-        __builtin_amdgcn_sched_group_barrier(0x008, EARLY - G1 * WRITE_OPS, 1);
-#pragma unroll
-        for (int i = 0; i < WRITE_OPS; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x002, 4, 1);
-            __builtin_amdgcn_sched_group_barrier(0x200, 1, 1);
-            __builtin_amdgcn_sched_group_barrier(0x008, G1, 1);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+        // step t+1 sits in the other set when there are two; buffer buf^1 was last read before the previous barrier.
+        // Its LDS stores are spread evenly between the MFMAs, each placement pinned (the de-interleaving stores are
+        // inline asm, which the scheduling-group masks cannot name).
+        typedef std::integral_constant<int, SETS == 2 ? 1 - SET : 0> StoreSet;
+        static_for<0, WRITE_OPS>([&](auto w_tag) {
+            constexpr int W = decltype(w_tag)::value;
+            write_one(StoreSet{}, buf ^ 1, w_tag);
+            mfma_range(af1, bf1, std::integral_constant<int, W * EARLY / WRITE_OPS>{}, std::integral_constant<int, (W + 1) * EARLY / WRITE_OPS>{});
+            __builtin_amdgcn_sched_barrier(0);
+        });
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
         read_frags(buf ^ 1, 0, af0, bf0);
@@ -705,7 +749,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
             if (t + 1 < T) {
                 if (buf == 0) store_stage(Set1{}, 1);
                 else store_stage(Set0{}, 0);
-                __syncthreads();
+                lds_sync();
             }
         }
     } else {
@@ -719,7 +763,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
             compute_stage(buf);
             if (t + 1 < T) {
                 store_stage(Set0{}, buf ^ 1);
-                __syncthreads();
+                lds_sync();
             }
         }
     }
