@@ -27,7 +27,7 @@ PEAK_HBM_GBPS = 8000.0              # MI355X HBM3E
 # HBM-side bytes per launch of the headline kernel (fp32 8192^3), from the FETCH_SIZE / WRITE_SIZE counter runs
 # summarised in profiles/hbm_traffic_fetch_write_size.txt (read factor 2.0, write factor 1.0 against a copy kernel).
 # Counters cannot be read from inside this script; the figure is only reported for the workload it was measured on.
-MEASURED_TRAFFIC_BYTES_FP32_8192 = 3.765e9
+MEASURED_TRAFFIC_BYTES_FP32_8192 = 3.773e9
 
 
 def log(msg):
