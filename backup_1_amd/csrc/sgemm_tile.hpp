@@ -6,8 +6,7 @@
 //
 // Staging: global -> registers -> LDS, two LDS buffers, one barrier per K step; the loads run one or two K steps ahead
 // of the MFMAs.  A is kept in LDS as float4 "k-quads":
-//   A quad (p, m) = A[m][8s+par+{0,2,4,6}], p = 2s+par,  at  As[p][m]  (plane rows 2 slots out of step mod 8, which
-//                                                                       keeps the staging stores off each other's banks)
+//   A quad (p, m) = A[m][8s+par+{0,2,4,6}], p = 2s+par,  at  As[p][m]
 // so that one ds_read_b128 per 32-row block feeds four MFMAs.
 // Summation order.  v_mfma_f32_32x32x2_f32 computes, per output element, fma(a1, b1, fma(a0, b0, c)) with operand 0 from
 // lanes 0-31 and operand 1 from lanes 32-63 (checked bit for bit on the hardware), i.e. it IS two steps of the
@@ -23,8 +22,9 @@
 //     NI = 4) and the NI results it holds per row are consecutive too (one 16-byte store).
 //   * a filter bank (FilterB), whose k runs contiguously per column, is kept as k-quads like A:
 //       B quad (p, n) = B[8s+par+{0,2,4,6}][n] at  Bs[p][b_slot(n)];  block ni takes columns 32*ni + li.
-// Every VALU instruction costs the matrix pipe 3-5 cycles (measured: a wave's VALU and MFMA work do not overlap), so
-// the K loop is kept as free of address arithmetic and data shuffling as the layouts allow.
+// Every instruction that is not an MFMA costs the matrix pipe cycles (measured: 3-8 per VALU instruction; a wave's VALU
+// and MFMA work do not overlap), so the K loop is kept as free of address arithmetic and data shuffling as the layouts
+// allow, and two waves share a SIMD where the registers permit (a lone wave leaves ~3.5 idle cycles between MFMAs).
 //
 // Ragged edges: rows >= M and columns >= N are read from clamped (valid) addresses and never stored; only the last,
 // partial K step zero-fills (both operands, so that 0 * Inf cannot appear).  No padded copies exist anywhere.
@@ -37,20 +37,19 @@ namespace decx_hip {
 // ---------------------------------------------------------------------------------------------------------------
 // A-operand sources.  Interface:
 //   RowState row_state(int m)                       per-row values that do not change along K
-//   KState k_state(k) / advance(ks, dk)             position of a k-quad, moved on by whole K steps
-//   template<bool TAIL> f32x4 load(rs, ks, keep)    A[m][k..k+3] read from an always-valid address; the caller replaces
-//                                                   the quad by zeros when keep comes back false (deferred, so that the
-//                                                   load itself stays branch-free and nothing waits on it early);
-//                                                   TAIL additionally zero-fills elements with k >= K
-//   size_t out_offset(int m)                        where row m of the result starts, in elements
+//   KState k_state(k) / KStep k_step(dk) / advance(ks, step)
+//                                                   position of the first quad of a k-group (8 consecutive k), moved on
+//                                                   by whole K steps
+//   template<bool TAIL> load_pair(rs, ks, step, lo, hi)
+//                                                   A[m][k..k+3] and A[m][k+4..k+7], branch-free; what lies outside the
+//                                                   operand (image border, K tail when TAIL) comes back as zeros
 // ---------------------------------------------------------------------------------------------------------------
 // Slot of column n inside a B plane: bits 3-4 of n are folded onto bits 0-1.
 // Measured on gfx950 (two active lanes hitting the same banks, SQ_LDS_BANK_CONFLICT): ds_read_b128 services a wave in
 // four phases -- lanes {0-3, 12-15, 20-23, 24-27} and {4-11, 16-19, 28-31} of each half-wave -- and a phase is
 // conflict-free when its 16-byte accesses fall into distinct slots mod 16; ds_write_b128 goes in eight phases of 8
 // consecutive lanes, conflict-free when the slots are distinct mod 8.  With this fold the fragment reads (32
-// consecutive columns per half-wave) and the staging stores (every 4th column per instruction) both qualify.  Rows of A
-// need no fold: consecutive slots are read, and the planes are 2 slots out of step for the staging stores.
+// consecutive columns per half-wave) qualify.  Rows of A need no fold: consecutive slots are read.
 __device__ __forceinline__ int b_slot(int n) { return n ^ ((n >> 3) & 3); }
 
 // 16 bytes through a buffer resource: offsets at or beyond the resource's size read as zeros, which is how taps
@@ -285,10 +284,17 @@ struct TensorOut {
 
 // ---------------------------------------------------------------------------------------------------------------
 // B-operand sources.  Interface (S = SgemmShape):
+//   ROW_MAJOR_LDS, lds_floats<S>()               which LDS layout the source keeps, and the size of one buffer of it
 //   quads<S>()                                   staging registers (float4) per thread and K step
-//   KState k_state<S>(tid, k_begin) / advance<S>(ks)   position of the K step to fetch next
-//   load<S, TAIL>(stage, tid, ks, bn0)           fetch this thread's share of B[k0 .. k0+BK) x [bn0 .. bn0+BN)
-//   store<S>(plane, stage, tid)                  write it to the LDS planes as k-quads at [q][b_slot(n)]
+//   k_state<S>(tid, k_begin, bn0, lds_buf0) / k_step<S>() / advance(ks, step)
+//                                                position of the K step to fetch next (plus whatever per-thread
+//                                                constants the source wants to keep: filter offsets, LDS addresses)
+//   load<S, TAIL>(stage, tid, ks, bn0, step)     fetch this thread's share of B[k0 .. k0+BK) x [bn0 .. bn0+BN)
+//   writes<S>() / write_one<S>(buf0, buf, stage, tid, ks, W)
+//                                                LDS store instructions per thread and step, and the W-th of them
+//   frag_reads<S>() / read_frags<S>(buf, s, lh, li, wn0, frag)
+//                                                LDS reads per k-group, and the operands of k-group s for this lane
+//   strip_col<S>(ni, li)                         column (within the wave's strip) that lane li holds in block ni
 // ---------------------------------------------------------------------------------------------------------------
 // B as a row-major K x N matrix.  Staging copies 16-byte pieces of rows straight through: task t of a K step is
 // row t / (BN/4), column group t % (BN/4), so a wave reads and writes whole kilobytes of consecutive addresses.  Rows
