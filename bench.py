@@ -331,7 +331,10 @@ def main():
 
     achieved = head["tflops_kernel"]
     line = {
-        "metric": "GEMM TFLOP/s at 8192^3 fp32 (fraction of MI355X fp32 matrix peak under roofline.frac; fp16 and conv under also)",
+        # the metric's name as the baseline file spells it; `value` is its first component (fp32 8192^3), the fraction of
+        # peak is roofline.frac, and the fp16 and conv components are under `also`
+        "metric": "GEMM TFLOP/s at 8192\u00b3 fp32 & fp16 + % of MI355X matrix peak; conv TFLOP/s",
+        "metric_note": "value = fp32 8192^3 GEMM; % of peak = roofline.frac; fp16 8192^3 and conv under also",
         "value": round(head["tflops"], 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(head["ms_wall"], 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
