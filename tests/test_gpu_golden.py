@@ -1,0 +1,42 @@
+"""The GPU path against the committed fixtures of tests/golden/ alone (no oracle at run time): fp32 GEMM, A*B + C, the
+convolution in both border modes and the ReLU family must reproduce the frozen bit patterns."""
+import os
+
+import numpy as np
+import pytest
+
+from backup_1_amd import capi
+from gpu_helpers import gpu_conv, gpu_sgemm
+
+pytestmark = pytest.mark.gpu
+
+V = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "chain_vectors.npz"))
+
+
+def same_bits(a, b):
+    nan = np.isnan(b)
+    return np.array_equal(np.isnan(a), nan) and np.array_equal(a[~nan].view(np.uint32), b[~nan].view(np.uint32))
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9])
+def test_gemm_and_conv_reproduce_the_fixtures(gpu, variant):
+    assert same_bits(gpu_sgemm(V["gemm_A"], V["gemm_B"], variant=variant), V["gemm_AB"])
+    assert same_bits(gpu_sgemm(V["gemm_A"], V["gemm_B"], C=V["gemm_C"], variant=variant), V["gemm_AB_plus_C"])
+    assert same_bits(gpu_conv(V["conv_src"], V["conv_filt"], 1, variant=variant), V["conv_same"])
+    assert same_bits(gpu_conv(V["conv_src"], V["conv_filt"], 0, variant=variant), V["conv_valid"])
+
+
+def test_relu_family_reproduces_the_fixtures(gpu):
+    x, g = V["relu_x"], V["relu_g"]
+    n = x.size
+    L = gpu.lib()
+    d_x, d_y, d_g, d_gx = (capi.DeviceBuffer.from_numpy(x), capi.DeviceBuffer(n * 4), capi.DeviceBuffer.from_numpy(g),
+                           capi.DeviceBuffer(n * 4))
+    d_map = capi.DeviceBuffer(n // 8)
+    gpu.check(L.decx_hip_relu_f32(d_x.ptr, d_y.ptr, n))
+    assert same_bits(d_y.download((n,), np.float32), V["relu_forward"])
+    gpu.check(L.decx_hip_relu_f32_rec(d_x.ptr, d_y.ptr, d_map.ptr, n))
+    assert same_bits(d_y.download((n,), np.float32), V["relu_forward"])
+    assert np.array_equal(d_map.download((n // 8,), np.uint8), V["relu_rec_map"])
+    gpu.check(L.decx_hip_relu_f32_backward(d_g.ptr, d_gx.ptr, d_map.ptr, n))
+    assert same_bits(d_gx.download((n,), np.float32), V["relu_backward"])

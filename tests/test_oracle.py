@@ -4,6 +4,9 @@ Every check here is something the oracle's own formula does not restate: the ref
 exact integer arithmetic, closed forms, an exact-rational model of the fused chain, numpy's independent
 float16 / float64 routines.
 """
+import json
+import os
+
 import numpy as np
 import pytest
 
@@ -301,3 +304,38 @@ def test_relu_backward_identities(oracle):
     assert np.all(oracle.relu_backward(g, np.zeros_like(ones)) == 0)
     # backward with the map of x applied to x itself reproduces forward
     assert np.array_equal(oracle.relu_backward(x, rec).view(np.uint32), oracle.relu(x).view(np.uint32))
+
+
+# ---- committed fixtures (tests/golden/): the reference-held known answer as data, and frozen oracle outputs -------
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def test_reference_known_answer_fixture(oracle):
+    with open(os.path.join(GOLDEN, "reference_known_answer.json")) as f:
+        known = json.load(f)
+    K = known["K"]
+    A, B, printed, closed = workloads.known_answer_pattern(8, K, 24)      # every row and column is the same: a slab will do
+    assert printed == known["printed_expectation_float32"] and closed == known["closed_form"]
+    got = oracle.sgemm_chain(A, B)
+    assert np.all(got == got[0, 0])
+    assert abs(float(got[0, 0]) - known["closed_form"]) / known["closed_form"] < 1e-5 * np.sqrt(K)
+    assert abs(float(got[0, 0]) - known["printed_expectation_float32"]) / known["closed_form"] < 1e-5 * np.sqrt(K)
+
+
+def test_oracle_reproduces_the_frozen_vectors(oracle):
+    v = np.load(os.path.join(GOLDEN, "chain_vectors.npz"))
+    same = lambda a, b: np.array_equal(np.isnan(a), np.isnan(b)) and np.array_equal(a[~np.isnan(a)].view(np.uint32), b[~np.isnan(b)].view(np.uint32))
+    assert same(oracle.sgemm_chain(v["gemm_A"], v["gemm_B"], fast=False), v["gemm_AB"])
+    assert same(oracle.sgemm_chain(v["gemm_A"], v["gemm_B"], fast=True), v["gemm_AB"])
+    assert same(oracle.sgemm_chain(v["gemm_A"], v["gemm_B"], v["gemm_C"]), v["gemm_AB_plus_C"])
+    assert same(oracle.decx_cpu_sgemm(v["gemm_A"], v["gemm_B"]), v["gemm_AB"])
+    assert same(oracle.conv2_chain(v["conv_src"], v["conv_filt"], 1), v["conv_same"])
+    assert same(oracle.conv2_chain(v["conv_src"], v["conv_filt"], 0), v["conv_valid"])
+    assert same(oracle.relu(v["relu_x"]), v["relu_forward"])
+    fwd, rec = oracle.relu_rec(v["relu_x"])
+    assert same(fwd, v["relu_forward"]) and np.array_equal(rec, v["relu_rec_map"])
+    assert same(oracle.relu_backward(v["relu_g"], rec), v["relu_backward"])
+    assert np.array_equal(oracle.float_to_half(v["half_in"]), v["half_bits"])
+    with np.errstate(over="ignore"):          # 65520 rounds to +inf, as it must
+        assert np.array_equal(v["half_bits"], v["half_in"].astype(np.float16).view(np.uint16))  # numpy's own RNE agrees
+    assert same(oracle.half_to_float(v["half_bits"]), v["half_back"])
