@@ -1,0 +1,46 @@
+"""Seeded sweep over random small problems: every combination of ragged M / N / K (including K shorter than one, two or
+three K steps, which take the peeled paths of the pipelined loop), pitch padding, tile shape, "+ C" and the ReLU epilogue
+must reproduce the oracle's fused chain bit for bit; random convolutions likewise."""
+import numpy as np
+import pytest
+
+from backup_1_amd import workloads
+from gpu_helpers import gpu_conv, gpu_sgemm
+
+pytestmark = pytest.mark.gpu
+
+
+def bits(a):
+    return np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_gemms_bit_exact(gpu, oracle, seed):
+    rng = np.random.Generator(np.random.PCG64(7000 + seed))
+    for case in range(10):
+        M, N = int(rng.integers(1, 420)), int(rng.integers(1, 420))
+        K = int(rng.choice([int(rng.integers(1, 70)), int(rng.integers(1, 700))]))
+        variant = int(rng.integers(0, 10))
+        align = int(rng.choice([8, 8, 4, 1]))          # DECX pitch, a 16-byte pitch, an unaligned pitch
+        with_c, relu = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        A, B = workloads.normal((M, K), 100 * seed + case), workloads.normal((K, N), 100 * seed + case + 50)
+        C = workloads.normal((M, N), 100 * seed + case + 77) if with_c else None
+        ref = oracle.sgemm_chain(A, B, C)
+        if relu:
+            ref = oracle.relu(ref)
+        got = gpu_sgemm(A, B, C=C, align=align, variant=variant, relu=relu)
+        assert np.array_equal(bits(got), bits(ref)), (M, K, N, variant, align, with_c, relu)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_convolutions_bit_exact(gpu, oracle, seed):
+    rng = np.random.Generator(np.random.PCG64(8000 + seed))
+    for case in range(6):
+        kh, kw = int(rng.choice([1, 3, 5, 7])), int(rng.choice([1, 3, 5, 7]))
+        H, W = int(rng.integers(kh, 40)), int(rng.integers(kw, 40))
+        C, N = int(rng.integers(1, 40)), int(rng.integers(1, 150))
+        flag, variant = int(rng.integers(0, 2)), int(rng.integers(0, 10))
+        src = workloads.normal((H, W, C), 300 * seed + case)
+        filt = workloads.normal((N, kh, kw, C), 300 * seed + case + 150)
+        ref = oracle.conv2_chain(src, filt, flag)
+        assert np.array_equal(bits(gpu_conv(src, filt, flag, variant=variant)), bits(ref)), (H, W, C, N, kh, kw, flag, variant)
