@@ -142,6 +142,7 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //   7: 256x256x16, 4x2 waves of  64x128   -- two waves per SIMD: the matrix pipe takes the next MFMA from the other wave
 //         while one wave issues its loads and LDS traffic (a lone wave leaves ~3.5 idle cycles between 64-cycle MFMAs);
 //         the default for large problems, 1-2 % ahead of shape 1
+//  10: 224x256x16, 1x8 waves of 224x32    -- two waves per SIMD like 7; 7/8 of its tile, for tile counts that 7 rounds badly
 //   8:  64x64x16,  2x2 waves of  32x32    -- small problems: 1024^3 has only 64 tiles of 128x128 for 256 CUs
 //   9: 128x64x16,  2x2 waves of  64x32
 //   5, 6: shapes 3 and 4 compiled for one wave per SIMD (512 registers, two staging sets) -- for launches that put at
@@ -153,6 +154,7 @@ typedef SgemmShape<224, 128, 16, 1, 4, 2> SShape224;
 typedef SgemmShape<256, 128, 16, 2, 2, 1> SShapeTallSolo;
 typedef SgemmShape<224, 128, 16, 1, 4, 1> SShape224Solo;
 typedef SgemmShape<256, 256, 16, 4, 2, 2, 2> SShapeBig8;
+typedef SgemmShape<224, 256, 16, 1, 8, 2, 2> SShape224Wide;   // 8 waves of 224x32, two per SIMD
 typedef SgemmShape<64, 64, 16, 2, 2, 4> SShapeTiny;      // 2x2 waves of 32x32
 typedef SgemmShape<128, 64, 16, 2, 2, 4> SShapeTiny2;    // 2x2 waves of 64x32
 
@@ -162,10 +164,10 @@ typedef SgemmShape<128, 64, 16, 2, 2, 4> SShapeTiny2;    // 2x2 waves of 64x32
 // two-workgroups-per-CU build, better on short K walks where one tile's prologue and epilogue overlap the other's loop,
 // and a one-wave-per-SIMD build with deeper prefetch, better on long ones.
 int pick_sgemm_variant(int M, int N, int K, int batch) {
-    if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 9) return g_rt.sgemm_variant;
+    if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) return g_rt.sgemm_variant;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     struct Cand { int variant, bm, bn; double eff; };
-    const Cand cands[] = {{7, 256, 256, 1.00}, {3, 256, 128, 0.95}, {4, 224, 128, 0.94}, {2, 128, 128, 0.89},
+    const Cand cands[] = {{7, 256, 256, 1.00}, {10, 224, 256, 0.96}, {3, 256, 128, 0.95}, {4, 224, 128, 0.94}, {2, 128, 128, 0.89},
                           {9, 128, 64, 0.83}, {8, 64, 64, 0.78}};
     int best = 7;
     double best_cost = 0.0;
@@ -192,6 +194,7 @@ int dispatch_sgemm(int variant, const ASrc& a, const BSrc& b, const float* Cin, 
         case 7: return launch_sgemm_tile<SShapeBig8>(a, b, Cin, ldc, D, out, M, N, K, batch);
         case 8: return launch_sgemm_tile<SShapeTiny>(a, b, Cin, ldc, D, out, M, N, K, batch);
         case 9: return launch_sgemm_tile<SShapeTiny2>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 10: return launch_sgemm_tile<SShape224Wide>(a, b, Cin, ldc, D, out, M, N, K, batch);
         default: return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K, batch);
     }
 }

@@ -15,7 +15,7 @@ CASES = [  # H, W, C, N, kh, kw, flag
 ]
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10])
 @pytest.mark.parametrize("case", CASES)
 def test_integer_exact(gpu, oracle, case, variant):
     H, W, C, N, kh, kw, flag = case
