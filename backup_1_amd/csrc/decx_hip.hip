@@ -134,19 +134,19 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
     return launch_sgemm_tile_c<S, ASrc, BSrc, Out, false>(a, b, Cin, ldc, D, out, M, N, K, batch);
 }
 
-// Tile shapes (variant numbers of decx_hip_set_sgemm_variant):
-//   1: 256x256x16, 2x2 waves of 128x128   -- large problems, highest reuse per LDS byte
-//   2: 128x128x16, 2x2 waves of  64x64    -- small problems, several workgroups per CU
+// Tile shapes (variant numbers of decx_hip_set_sgemm_variant; results are identical for all of them):
+//   1: 256x256x16, 2x2 waves of 128x128   -- one wave per SIMD, highest reuse per LDS byte
+//   2: 128x128x16, 2x2 waves of  64x64    -- mid-size problems, several workgroups per CU
 //   3: 256x128x16, 2x2 waves of 128x64    -- narrow N
 //   4: 224x128x16, 1x4 waves of 224x32    -- 7/8 of shape 3 per tile: fills more CUs when M/256 tiles leave many idle
+//   5, 6: shapes 3 and 4 compiled for one wave per SIMD (512 registers, two staging sets) -- for long K walks and for
+//         launches that put at most one workgroup on a CU anyway
 //   7: 256x256x16, 4x2 waves of  64x128   -- two waves per SIMD: the matrix pipe takes the next MFMA from the other wave
 //         while one wave issues its loads and LDS traffic (a lone wave leaves ~3.5 idle cycles between 64-cycle MFMAs);
 //         the default for large problems, 1-2 % ahead of shape 1
-//  10: 224x256x16, 1x8 waves of 224x32    -- two waves per SIMD like 7; 7/8 of its tile, for tile counts that 7 rounds badly
 //   8:  64x64x16,  2x2 waves of  32x32    -- small problems: 1024^3 has only 64 tiles of 128x128 for 256 CUs
 //   9: 128x64x16,  2x2 waves of  64x32
-//   5, 6: shapes 3 and 4 compiled for one wave per SIMD (512 registers, two staging sets) -- for launches that put at
-//         most one workgroup on a CU anyway, where a second resident workgroup cannot be what hides the load latency
+//  10: 224x256x16, 1x8 waves of 224x32    -- two waves per SIMD like 7; 7/8 of its tile, for tile counts that 7 rounds badly
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
 typedef SgemmShape<128, 128, 16, 2, 2, 2> SShapeSmall;
 typedef SgemmShape<256, 128, 16, 2, 2, 2> SShapeTall;
