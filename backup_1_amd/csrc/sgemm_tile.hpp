@@ -669,16 +669,17 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
     typedef std::integral_constant<int, 0> Set0;
     typedef std::integral_constant<int, 1> Set1;
 
+    // prologue: the loads of steps 0 and 1 go out back to back, so the tile pays one global round trip, not two
     if (full_steps > 0) load_stage(Set0{}, std::false_type{});
     else load_stage(Set0{}, std::true_type{});
-    store_stage(Set0{}, 0);
-    lds_sync();
     if constexpr (SETS == 2) {
         if (T > 1) {
             if (full_steps > 1) load_stage(Set1{}, std::false_type{});
             else load_stage(Set1{}, std::true_type{});
         }
     }
+    store_stage(Set0{}, 0);
+    lds_sync();
 
     static_assert(KQ == 4, "the pipelined loop is written for two quad pairs per K step");
     constexpr int VMEM_OPS = S::A_PASSES + B_QUADS;     // global loads per thread and step
