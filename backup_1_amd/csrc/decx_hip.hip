@@ -11,6 +11,7 @@
 #include "hgemm_dma_tile.hpp"
 #include "hgemm_tile.hpp"
 #include "sgemm_tile.hpp"
+#include "sgemm_chain16.hpp"
 
 using namespace decx_hip;
 
@@ -147,6 +148,9 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //   8:  64x64x16,  2x2 waves of  32x32    -- small problems: 1024^3 has only 64 tiles of 128x128 for 256 CUs
 //   9: 128x64x16,  2x2 waves of  64x32
 //  10: 224x256x16, 1x8 waves of 224x32    -- two waves per SIMD like 7; 7/8 of its tile, for tile counts that 7 rounds badly
+// and, for dense GEMM only, the one-wave-per-16x16-block kernel of sgemm_chain16.hpp:
+//  11:  32x32x64,  2x2 computing + 4 moving waves, two workgroups per CU -- results too small to fill the chip with tiles
+//  12:  16x16x64,  1 computing + 2 moving waves -- at most one 16x16 block per CU: the fastest a single chain can walk K
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
 typedef SgemmShape<128, 128, 16, 2, 2, 2> SShapeSmall;
 typedef SgemmShape<256, 128, 16, 2, 2, 2> SShapeTall;
@@ -212,6 +216,20 @@ int check_gemm_args(const void* A, int lda, const void* B, int ldb, const void* 
     return 0;
 }
 
+// One wave per 16x16 block (sgemm_chain16.hpp): for results with few tiles and a long K.
+template <class S>
+int launch_sgemm_chain16(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
+                         int N, int K, const Batch& batch, bool relu) {
+    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    const long total = (long)tiles_m * tiles_n;
+    if (total > 0x7fffffffL || batch.count > 65535) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
+    auto kern = Cin ? sgemm_chain16_kernel<S, true> : sgemm_chain16_kernel<S, false>;
+    hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), 0, batch.stream, A, lda, B, ldb, Cin,
+                       ldc, D, ldd, M, N, K, tiles_n, relu, batch.stride_a, batch.stride_b, batch.stride_c, batch.stride_d);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
                   int N, int K, const Batch& batch, bool relu = false) {
     if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
@@ -219,6 +237,17 @@ int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float*
     const bool vec_a = aligned16(A) && lda % 4 == 0 && batch.stride_a % 4 == 0;
     const bool vec_b = aligned16(B) && ldb % 4 == 0 && ldb >= 4 && batch.stride_b % 4 == 0;
     DenseOut out{ldd, relu, aligned16(D) && ldd % 4 == 0 && batch.stride_d % 4 == 0};
+    if (vec_a && vec_b) {
+        // Small results go to the one-wave-per-block kernel (measured: ahead of the tiles up to about ten 32x32 tiles per
+        // CU -- 1536x1536 on 256 CUs -- whatever K is; 1.5x at 1024x8192x1024, 9x at 64x65536x1024).  All paths give
+        // the same bits, so this is a choice of speed only.
+        const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+        const long blocks16 = (long)cdiv(M, 16) * cdiv(N, 16) * batch.count, tiles32 = (long)cdiv(M, 32) * cdiv(N, 32) * batch.count;
+        int chain = g_rt.sgemm_variant == 11 || g_rt.sgemm_variant == 12 ? g_rt.sgemm_variant : 0;
+        if (g_rt.sgemm_variant < 1 || g_rt.sgemm_variant > 12) chain = blocks16 <= cus ? 12 : (tiles32 <= 10 * cus ? 11 : 0);
+        if (chain == 11) return launch_sgemm_chain16<Chain16<2, 4, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+        if (chain == 12) return launch_sgemm_chain16<Chain16<1, 8, 2>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+    }
     if (vec_a && vec_b) {
         DenseA<true> a{A, lda, M, K, batch.stride_a};
         DenseB<true> b{B, ldb, N, K, batch.stride_b};

@@ -1,0 +1,261 @@
+// fp32 GEMM for problems with few output tiles and a long K: one wave per 16x16 block of the result.
+//
+// Every output of the reference is one fused multiply-add chain over ascending k, and a chain cannot be cut into
+// parallel pieces without changing its rounding.  What bounds a long, thin problem (say 64 x 65536 x 1024) is then how
+// fast ONE accumulator can walk K.  v_mfma_f32_16x16x4_f32 consumes four k per instruction -- per output element
+// fma(a3,b3, fma(a2,b2, fma(a1,b1, fma(a0,b0, c)))) with k-slot s taken from lanes 16s .. 16s+15 (checked bit for bit on
+// the hardware) -- and dependent instructions issue back to back every 32 cycles, i.e. 8 cycles per k, four times the
+// pace of the 32x32x2 form the big tiles use.  The big tiles win on everything else (16 times the reuse per operand
+// byte), so this kernel is only chosen when the result has too few tiles to fill the chip anyway.
+//
+// Nothing but the MFMAs may sit on that chain, and on this hardware every other instruction does: measured per chunk of
+// 16 MFMAs (518 cycles alone), the wave's own eight 16-byte LDS reads add 55 cycles, and with loads, LDS stores and
+// address arithmetic in the same wave the chunk took 970 -- the sum of everybody's issue time, bank conflicts or not.
+// Instructions of ANOTHER wave on the same SIMD cost the chain about as much (+210 cycles for the 25 instructions that
+// stage a chunk); only a wave on another SIMD is free.  So the work is split by role.  Computing waves do per chunk of
+// 64 k the 16 MFMAs and the 8 LDS reads of the next chunk's operands, nothing else; moving waves bring the data: global
+// memory -> DEPTH register sets -> LDS, DEPTH chunks ahead.  Three LDS buffers: while chunk c is computed from
+// registers, chunk c+1 is read from one buffer and chunk c+2 written into another; one barrier per chunk (free: the
+// moving waves are always early).  Two shapes:
+//   T = 1: a 16x16 tile, one computing wave and two moving waves -- three waves on three different SIMDs of a CU, so
+//          the chain runs undisturbed: for results of at most one block per CU (241 ns per chunk, against 218 for bare
+//          MFMAs);
+//   T = 2: a 32x32 tile, 2x2 computing waves and four moving waves, one of each per SIMD: half the staging work per
+//          block (A and B tiles are shared) but it runs on the computing waves' SIMDs: for more blocks than CUs.  Built
+//          with 4 register sets for 128 registers, so that two workgroups share a CU and one's MFMAs fill the gaps
+//          the other's staging leaves.
+//
+// Lane (r, s) of a computing wave feeds row r (of A) or column r (of B) of its block and k-slot s; so that its operands
+// for the 16 MFMAs of a chunk (k = 4j + s, j = 0..15) are 16 consecutive floats -- four 16-byte reads -- the chunk lies in
+// LDS as  As[s][row][j]  and  Bs[s][col][j]  with lines of 20 floats (16 lanes of a 16-byte read then cover all banks).
+// The moving waves scatter each loaded quad into that layout with ds_write2 pairs; quads are dealt to lanes, and B's
+// planes padded by 4 floats, so that the 32 lanes of one store pass fall on 32 different banks.  The k order inside an
+// instruction (slot 0..3) and across instructions (j) is ascending, so results are bit-identical to
+// sgemm_tile_kernel's and to the reference's chain.
+//
+// Loads never run past the last whole chunk: the fetch pointers stop advancing there (later refills fetch that chunk
+// again and are never used), which keeps the loop free of bounds checks.  A ragged last chunk is fetched with masks once,
+// at the start, into registers of its own, and computed after the loop.
+#pragma once
+#include "sgemm_tile.hpp"
+
+namespace decx_hip {
+
+template <int T, int DEPTH_, int WAVES_PER_SIMD_>
+struct Chain16 {
+    static_assert(T == 1 || T == 2, "tiles of 1x1 or 2x2 blocks");
+    static constexpr int WAVES_PER_SIMD = WAVES_PER_SIMD_;           // what the register budget is cut for
+    static constexpr int BM = 16 * T, BN = 16 * T, BK = 64;
+    static constexpr int COMPUTE_WAVES = T * T, MOVE_THREADS = 128 * T;
+    static constexpr int NT = 64 * COMPUTE_WAVES + MOVE_THREADS;     // computing waves first, then the moving waves
+    static constexpr int DEPTH = DEPTH_;                             // register sets: chunks of K in flight from global memory (even)
+    static constexpr int LINE = 20;                                  // floats per (k-slot, row or column) line in LDS: 16 + 4
+    static constexpr int A_PLANE = BM * LINE, B_PLANE = BN * LINE + 4;   // floats per k-slot plane
+    static constexpr int A_FLOATS = 4 * A_PLANE, B_FLOATS = 4 * B_PLANE;
+    static constexpr int LDS_BUFFERS = 3;
+    static constexpr size_t LDS_BYTES = LDS_BUFFERS * (size_t)(A_FLOATS + B_FLOATS) * sizeof(float);
+};
+
+// two floats to LDS, OFF0 and OFF1 dwords past byte_addr (each below 256)
+template <int OFF0, int OFF1>
+__device__ __forceinline__ void lds_write2(unsigned byte_addr, float x, float y) {
+    asm volatile("ds_write2_b32 %0, %1, %2 offset0:%3 offset1:%4" : : "v"(byte_addr), "v"(x), "v"(y), "n"(OFF0), "n"(OFF1) : "memory");
+}
+// the same with offsets in units of 64 dwords
+template <int OFF0, int OFF1>
+__device__ __forceinline__ void lds_write2_st64(unsigned byte_addr, float x, float y) {
+    asm volatile("ds_write2st64_b32 %0, %1, %2 offset0:%3 offset1:%4" : : "v"(byte_addr), "v"(x), "v"(y), "n"(OFF0), "n"(OFF1) : "memory");
+}
+
+template <class S, bool HAS_C>
+__global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_chain16_kernel(const float* __restrict__ A, int lda,
+                                                                    const float* __restrict__ B, int ldb, const float* Cin,
+                                                                    int ldc, float* D, int ldd, int M, int N, int K,
+                                                                    int tiles_n, bool relu, size_t a_batch_stride,
+                                                                    size_t b_batch_stride, size_t c_batch_stride,
+                                                                    size_t d_batch_stride) {
+    constexpr int T = S::BM / 16;
+    constexpr int DEPTH = S::DEPTH;
+    static_assert(DEPTH % 2 == 0 && DEPTH >= 2, "set and fragment indices repeat with period DEPTH");
+    static_assert(S::A_PLANE % 64 == 0 && S::LINE == 20, "the store offsets below are written for these strides");
+    A += (size_t)blockIdx.y * a_batch_stride;
+    B += (size_t)blockIdx.y * b_batch_stride;
+    if (HAS_C) Cin += (size_t)blockIdx.y * c_batch_stride;
+    D += (size_t)blockIdx.y * d_batch_stride;
+    __shared__ __attribute__((aligned(16))) float lds[S::LDS_BUFFERS * (S::A_FLOATS + S::B_FLOATS)];
+    float* As = lds;                                     // [3][4 slots][BM][LINE]
+    float* Bs = lds + S::LDS_BUFFERS * S::A_FLOATS;      // [3][4 slots][BN][LINE] (+4 per plane)
+
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int bm0 = ((int)blockIdx.x / tiles_n) * S::BM, bn0 = ((int)blockIdx.x % tiles_n) * S::BN;
+    const int chunks = (K + S::BK - 1) / S::BK, full_chunks = K / S::BK;
+    typedef std::integral_constant<int, 0> I0;
+    typedef std::integral_constant<int, 1> I1;
+
+    // Both roles run the same sequence of barriers: one after the prologue (when there is a whole chunk), one per whole
+    // chunk, one for a ragged last chunk.
+    if (wave >= S::COMPUTE_WAVES) {
+        // =============================== moving waves ===============================
+        // per chunk two quads of A (row, 4 consecutive k) and two of B (k, 4 consecutive columns) per thread; quad 2p is
+        // A's, 2p + 1 is B's.  32 consecutive lanes hold, of A, 16 quads of rows r and r + 4 (banks 20 r + kq and 16
+        // further), of B, 16 consecutive k of two neighbouring column quads (banks 4 (k % 4) + k / 4 and 16 further).
+        const int pt = tid - 64 * S::COMPUTE_WAVES;
+        const float* src[4];
+        unsigned dst[4];                          // LDS byte address, buffer 0, of element 0 of the quad
+        int a_k[2], b_k[2];                       // k of the quad inside its chunk (first element for A)
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            const int q = pt + p * S::MOVE_THREADS, rest = q / 32;
+            const int row = rest % 4 + 4 * ((q / 16) % 2) + 8 * (rest / 4), kq = q % 16;
+            int m = bm0 + row;
+            if (m >= M) m = M - 1;                // rows past the end are computed and never stored
+            a_k[p] = 4 * kq;
+            src[2 * p] = A + (size_t)m * lda + 4 * kq;
+            dst[2 * p] = lds_byte_address(As) + 4u * (unsigned)(row * S::LINE + kq);      // element e: plane e, j = kq
+            const int k = 16 * (rest % 4) + q % 16, cq = 2 * (rest / 4) + (q / 16) % 2;
+            int col = bn0 + 4 * cq;
+            if (col > ldb - 4) col = ldb - 4;     // stay inside the pitch; such columns are never stored
+            b_k[p] = k;
+            src[2 * p + 1] = B + (size_t)k * ldb + col;
+            dst[2 * p + 1] = lds_byte_address(Bs) + 4u * (unsigned)((k % 4) * S::B_PLANE + (4 * cq) * S::LINE + k / 4);   // element e: line 4cq + e
+        }
+        auto store_quad = [&](const f32x4& v, auto quad_tag, int buf) {
+            constexpr int Q = decltype(quad_tag)::value;
+            if constexpr (Q % 2 == 0) {
+                const unsigned addr = dst[Q] + (unsigned)buf * (S::A_FLOATS * 4u);
+                lds_write2_st64<0, S::A_PLANE / 64>(addr, v[0], v[1]);
+                lds_write2_st64<2 * S::A_PLANE / 64, 3 * S::A_PLANE / 64>(addr, v[2], v[3]);
+            } else {
+                const unsigned addr = dst[Q] + (unsigned)buf * (S::B_FLOATS * 4u);
+                lds_write2<0, S::LINE>(addr, v[0], v[1]);
+                lds_write2<2 * S::LINE, 3 * S::LINE>(addr, v[2], v[3]);
+            }
+        };
+
+        // the ragged last chunk, fetched first (it is the only load with per-lane conditions)
+        f32x4 tail_stage[4];
+        if (chunks > full_chunks) {
+            const int k0 = full_chunks * S::BK;
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                f32x4 va = {0.f, 0.f, 0.f, 0.f}, vb = {0.f, 0.f, 0.f, 0.f};
+                const int ka = k0 + a_k[p], kb = k0 + b_k[p];
+                if (ka < K) {
+                    va = *reinterpret_cast<const f32x4*>(src[2 * p] + k0);       // lda % 4 == 0 keeps the quad inside the pitch
+                    if (ka + 1 >= K) va[1] = 0.f;
+                    if (ka + 2 >= K) va[2] = 0.f;
+                    if (ka + 3 >= K) va[3] = 0.f;
+                }
+                if (kb < K) vb = *reinterpret_cast<const f32x4*>(src[2 * p + 1] + (size_t)k0 * ldb);
+                tail_stage[2 * p] = va;
+                tail_stage[2 * p + 1] = vb;
+            }
+        }
+
+        // DEPTH register sets: chunk x travels through set x % DEPTH, fetched DEPTH chunks ahead of its use
+        f32x4 stage[DEPTH][4];
+        int fetch_chunk = 0;                      // the chunk the fetch pointers stand on
+        auto fetch = [&](auto set_tag) {
+            constexpr int SET = decltype(set_tag)::value;
+            const bool more = fetch_chunk + 1 < full_chunks;      // the pointers stop on the last whole chunk
+            const long a_step = more ? S::BK : 0, b_step = more ? (long)S::BK * ldb : 0;
+            fetch_chunk += more ? 1 : 0;
+            static_for<0, 4>([&](auto q_tag) {
+                constexpr int Q = decltype(q_tag)::value;
+                stage[SET][Q] = *reinterpret_cast<const f32x4*>(src[Q]);
+                src[Q] += (Q % 2 == 0) ? a_step : b_step;
+            });
+        };
+        if (full_chunks > 0) {
+            // chunks 0 .. DEPTH-1 are fetched; chunks 0 and 1 go to LDS buffers 0 and 1 and their sets are refilled
+            static_for<0, DEPTH>([&](auto d) { fetch(d); });
+            static_for<0, 4>([&](auto q) { store_quad(stage[0][decltype(q)::value], q, 0); });
+            static_for<0, 4>([&](auto q) { store_quad(stage[1][decltype(q)::value], q, 1); });
+            lds_sync();
+            fetch(I0{});
+            fetch(I1{});
+            // while chunk c is computed: chunk c+2 goes into buffer (c+2) % 3 (it held chunk c-1, which nobody reads any
+            // more), and once the stores have left the registers, the set is refilled with chunk c+2+DEPTH
+            int buf_store = 2;
+            auto chunk = [&](auto d) {
+                constexpr int SET = (decltype(d)::value + 2) % DEPTH;
+                static_for<0, 4>([&](auto q) { store_quad(stage[SET][decltype(q)::value], q, buf_store); });
+                lds_sync();
+                fetch(std::integral_constant<int, SET>{});
+                buf_store = buf_store == 2 ? 0 : buf_store + 1;
+            };
+            int c0 = 0;
+            for (; c0 + DEPTH <= full_chunks; c0 += DEPTH) static_for<0, DEPTH>([&](auto d) { chunk(d); });
+            // c0 is a multiple of DEPTH, so the set indices continue with the same period
+            static_for<0, DEPTH>([&](auto d) {
+                if (c0 + decltype(d)::value < full_chunks) chunk(d);
+            });
+        }
+        if (chunks > full_chunks) {
+            // every computing wave is past the last barrier and has all its LDS reads back: any buffer is free
+            static_for<0, 4>([&](auto q) { store_quad(tail_stage[decltype(q)::value], q, 0); });
+            lds_sync();
+        }
+        return;
+    }
+
+    // =============================== computing waves ===============================
+    const int wm0 = (wave / T) * 16, wn0 = (wave % T) * 16;
+    const int lr = lane % 16, ls = lane / 16;     // row (of A) or column (of B) inside the block, and k-slot
+    // accumulators: lane holds D[4*ls + r][lr] of its block, r = 0..3; the chain starts at C when there is one
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    const int n_out = bn0 + wn0 + lr;
+    if (HAS_C) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int m = bm0 + wm0 + 4 * ls + r;
+            if (m < M && n_out < N) acc[r] = Cin[(size_t)m * ldc + n_out];
+        }
+    }
+    const float* a_frag = As + ls * S::A_PLANE + (wm0 + lr) * S::LINE;       // this lane's 16 operands of a chunk, buffer 0
+    const float* b_frag = Bs + ls * S::B_PLANE + (wn0 + lr) * S::LINE;
+    f32x4 av[2][4], bv[2][4];
+    // read R (0..3: A, 4..7: B) of the eight 16-byte operand reads of a chunk in LDS buffer buf, into fragment set F
+    auto read_one = [&](auto f_tag, auto r_tag, int buf) {
+        constexpr int F = decltype(f_tag)::value, R = decltype(r_tag)::value;
+        if constexpr (R < 4) av[F][R] = reinterpret_cast<const f32x4*>(a_frag + buf * S::A_FLOATS)[R];
+        else bv[F][R - 4] = reinterpret_cast<const f32x4*>(b_frag + buf * S::B_FLOATS)[R - 4];
+    };
+    if (full_chunks > 0) {
+        lds_sync();
+        static_for<0, 8>([&](auto r) { read_one(I0{}, r, 0); });
+        // chunk c: its operands are in fragment set c % 2; buffer (c+1) % 3 holds chunk c+1 since the previous barrier
+        int buf_next = 1;
+        auto chunk = [&](auto d) {
+            constexpr int NOW = decltype(d)::value & 1;
+            typedef std::integral_constant<int, NOW ^ 1> Next;
+            static_for<0, 16>([&](auto j_tag) {
+                constexpr int J = decltype(j_tag)::value;
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[NOW][J / 4][J % 4], bv[NOW][J / 4][J % 4], acc, 0, 0, 0);
+                if constexpr (J < 8) read_one(Next{}, j_tag, buf_next);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            lds_sync();
+            __builtin_amdgcn_sched_barrier(0);
+            buf_next = buf_next == 2 ? 0 : buf_next + 1;
+        };
+        int c0 = 0;
+        for (; c0 + DEPTH <= full_chunks; c0 += DEPTH) static_for<0, DEPTH>([&](auto d) { chunk(d); });
+        static_for<0, DEPTH>([&](auto d) {
+            if (c0 + decltype(d)::value < full_chunks) chunk(d);
+        });
+    }
+    if (chunks > full_chunks) {
+        lds_sync();
+        static_for<0, 8>([&](auto r) { read_one(I0{}, r, 0); });
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[0][j / 4][j % 4], bv[0][j / 4][j % 4], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int m = bm0 + wm0 + 4 * ls + r;
+        if (m < M && n_out < N) D[(size_t)m * ldd + n_out] = relu ? relu_by_sign(acc[r]) : acc[r];
+    }
+}
+
+}  // namespace decx_hip

@@ -268,8 +268,10 @@ DH GEMM_Long_Lr(GPU_Matrix<float>& A_, GPU_Matrix<float>& B_, GPU_Matrix<float>&
     if (A->width != B->height) return DH{decx::DECX_FAIL_DimsNotMatching, kGemmDims};
     if (!dst->re_construct(B->width, A->height))
         return dst->last_status == DECX_HIP_FAIL_ALLOCATION ? alloc_fail() : from_status(dst->last_status);
-    return from_status(decx_hip_sgemm_splitk(A->Mat.ptr, (int)A->pitch, B->Mat.ptr, (int)B->pitch, nullptr, 0, dst->Mat.ptr,
-                                             (int)dst->pitch, (int)A->height, (int)B->width, (int)A->width, 0));
+    // the reference's long-K kernel is one fused chain per output like every other (GEMM_long_linear_region.cuh:35-55):
+    // decx_hip_sgemm follows it bit for bit and sends results this small to its one-wave-per-block kernel
+    return from_status(decx_hip_sgemm(A->Mat.ptr, (int)A->pitch, B->Mat.ptr, (int)B->pitch, nullptr, 0, dst->Mat.ptr,
+                                      (int)dst->pitch, (int)A->height, (int)B->width, (int)A->width));
 }
 
 DH GEMM3(MatrixArray<float>& A, MatrixArray<float>& B, MatrixArray<float>& dst) { return gemm3_host<float>(A, B, nullptr, dst); }

@@ -265,14 +265,14 @@ static void gemm_long_lr() {
     de::Matrix<float>& A = de::CreateMatrixRef<float>(K, M, 0);
     de::Matrix<float>& B = de::CreateMatrixRef<float>(N, K, 0);
     de::Matrix<float>& R = de::CreateMatrixRef<float>(N, M, 0);
-    fill(A, small_int); fill(B, small_int);
+    fill(A, unif); fill(B, unif);
     de::GPU_Matrix<float>& dA = de::CreateGPUMatrixRef<float>(K, M);
     de::GPU_Matrix<float>& dB = de::CreateGPUMatrixRef<float>(N, K);
     de::GPU_Matrix<float>& dD = de::CreateGPUMatrixRef<float>();
     dA.Load_from_host(A); dB.Load_from_host(B);
     CHECK(de::cuda::GEMM_Long_Lr(dA, dB, dD).error_type == decx::DECX_SUCCESS && dD.Width() == (uint)N && dD.Height() == (uint)M);
     dD.Load_to_host(R);
-    CHECK(dense(R) == chain(A, B));               // integer data: exact whatever the order of the K ranges
+    CHECK(dense(R) == chain(A, B));               // real-valued data: the reference's fused chain over all of K, bit for bit
     de::GPU_Matrix<float>& dBad = de::CreateGPUMatrixRef<float>(N, K + 8);
     CHECK(de::cuda::GEMM_Long_Lr(dA, dBad, dD).error_type == decx::DECX_FAIL_DimsNotMatching);
 }
