@@ -22,7 +22,7 @@ SYMBOLS = [
     "decx_hip_conv2_im2col_f32", "decx_hip_conv2_im2col_f32_async", "decx_hip_timer_start", "decx_hip_timer_stop",
     "decx_hip_last_error", "decx_hip_set_sgemm_variant", "decx_hip_set_hgemm_variant", "decx_hip_copy_kernel",
     "decx_hip_sgemm_splitk", "decx_hip_sgemm_batched", "decx_hip_hgemm_f32acc_batched", "decx_hip_gemm3_host_f32", "decx_hip_gemm3_host_f16",
-    "decx_hip_conv2_im2col_f32_fused", "decx_hip_sgemm_relu", "decx_hip_relu_f32", "decx_hip_relu_f32_async",
+    "decx_hip_conv2_im2col_f32_fused", "decx_hip_conv2_im2col_f16", "decx_hip_conv2_im2col_f16_async", "decx_hip_sgemm_relu", "decx_hip_relu_f32", "decx_hip_relu_f32_async",
     "decx_hip_relu_f32_rec", "decx_hip_relu_f32_backward", "decx_hip_gemm_host_f32", "decx_hip_gemm_host_f16",
 ]
 
@@ -65,6 +65,8 @@ def lib():
             "decx_hip_gemm3_host_f32": ([P, I, Z, P, I, Z, P, I, Z, P, I, Z, I, I, I, I], I),
             "decx_hip_gemm3_host_f16": ([P, I, Z, P, I, Z, P, I, Z, P, I, Z, I, I, I, I], I),
             "decx_hip_conv2_im2col_f32_fused": ([P, I, I, I, Z, P, I, I, I, Z, Z, P, I, Z, I, P, I], I),
+            "decx_hip_conv2_im2col_f16": ([P, I, I, I, Z, P, I, I, I, Z, Z, P, I, Z, I, P, I], I),
+            "decx_hip_conv2_im2col_f16_async": ([P, I, I, I, Z, P, I, I, I, Z, Z, P, I, Z, I, P, I], I),
             "decx_hip_sgemm_relu": ([P, I, P, I, P, I, P, I, I, I, I], I),
             "decx_hip_gemm_host_f32": ([P, I, P, I, P, I, P, I, I, I, I], I),
             "decx_hip_gemm_host_f16": ([P, I, P, I, P, I, P, I, I, I, I], I),

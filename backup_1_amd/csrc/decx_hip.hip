@@ -12,6 +12,7 @@
 #include "hgemm_tile.hpp"
 #include "sgemm_tile.hpp"
 #include "sgemm_chain16.hpp"
+#include "hconv_tile.hpp"
 
 using namespace decx_hip;
 
@@ -422,6 +423,60 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
     if (variant == 10) return launch_hgemm_dma_tile<HShapeDmaTall>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     if (variant == 1) return launch_hgemm_tile<HShapeBig, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     return launch_hgemm_tile<HShapeSmall, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+}
+
+// fp16 convolution (hconv_tile.hpp).  Strides and pitches in halves, as the binary16 containers hold them.
+typedef HconvShape<128, 128, 2, 2> HconvSquare;      // 2x2 waves of 64x64
+typedef HconvShape<256, 128, 4, 2> HconvTall;        // 4x2 waves of 64x64, two per SIMD: half the filter reads per pixel
+int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_stride, const uint16_t* filt, int N, int kh,
+                  int kw, size_t filt_stride, size_t filt_row_stride, uint16_t* dst, int dst_dpitch, size_t dst_row_stride,
+                  int flag, const uint16_t* bias, bool relu) {
+    if (!g_rt.is_init) return need_init();
+    if (flag != DECX_HIP_CONV_NO_COMPENSATE && flag != DECX_HIP_CONV_ZERO_COMPENSATE)
+        return fail(DECX_HIP_FAIL_ERROR_FLAG, "This flag is meaningless in current context\n");   // core/error.h:67
+    if (!src || !filt || !dst) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "null tensor pointer\n");
+    if (H <= 0 || W <= 0 || N <= 0 || kh <= 0 || kw <= 0 || dpitch <= 0)
+        return fail(DECX_HIP_FAIL_DIMS, "Tensor Dims don't match each other");
+    if (dpitch % 8 != 0 || src_row_stride % 8 != 0 || filt_stride % 8 != 0 || filt_row_stride % 8 != 0 || !aligned16(src) ||
+        !aligned16(filt))
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "tensors must be 16-byte aligned with channel pitch a multiple of 8\n");
+    const int Hout = flag ? H : H - 2 * (kh / 2), Wout = flag ? W : W - 2 * (kw / 2);
+    if (Hout <= 0 || Wout <= 0) return fail(DECX_HIP_FAIL_DIMS, "kernel larger than the image\n");
+    if (src_row_stride < (size_t)W * dpitch || filt_row_stride < (size_t)kw * dpitch ||
+        filt_stride < (size_t)(kh - 1) * filt_row_stride + (size_t)kw * dpitch || dst_dpitch < N ||
+        dst_row_stride < (size_t)Wout * dst_dpitch)
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "stride smaller than the extent it spans\n");
+    const long Ml = (long)Hout * Wout, Kl = (long)kh * kw * dpitch;
+    if (Ml > 0x7fffffffL || Kl > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large\n");
+    const int M = (int)Ml, Kw = (int)(Kl / 2);
+    // the loaders address both tensors with 32-bit byte offsets through buffer resources
+    const size_t src_bytes = ((size_t)(H - 1) * src_row_stride + (size_t)W * dpitch) * 2;
+    const size_t filt_bytes = ((size_t)(N - 1) * filt_stride + (size_t)(kh - 1) * filt_row_stride + (size_t)kw * dpitch) * 2;
+    if (src_bytes >= 0x80000000ull || filt_bytes >= 0x80000000ull)
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "source tensor and filter bank must each stay below 2 GiB\n");
+    const int oy = flag ? kh / 2 : 0, ox = flag ? kw / 2 : 0;
+    HalfImage img{src, H, W, kh, kw, oy, ox, Wout, M, dpitch / 2, (int)(src_row_stride / 2), (unsigned)src_bytes};
+    HalfFilters fb{filt, N, dpitch / 2, kw, (int)(filt_stride / 2), (int)(filt_row_stride / 2), (unsigned)filt_bytes};
+    HalfTensorOut out{reinterpret_cast<_Float16*>(dst), Wout, dst_dpitch, dst_row_stride, reinterpret_cast<const _Float16*>(bias), relu};
+    const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+    // the tall tile when its workgroups still fill the chip twice over
+    const bool tall = (long)cdiv(M, 256) * cdiv(N, 128) >= 2 * cus;
+    const int bm = tall ? 256 : 128, tiles_n = cdiv(N, 128);
+    const long total = (long)cdiv(M, bm) * tiles_n;
+    if (total > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
+    if (tall) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hconv_tile_kernel<HconvTall>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)HconvTall::LDS_BYTES));
+        hipLaunchKernelGGL(hconv_tile_kernel<HconvTall>, dim3((unsigned)total), dim3(HconvTall::NT), HconvTall::LDS_BYTES,
+                           g_rt.stream, img, fb, out, M, N, Kw, tiles_n);
+    } else {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hconv_tile_kernel<HconvSquare>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)HconvSquare::LDS_BYTES));
+        hipLaunchKernelGGL(hconv_tile_kernel<HconvSquare>, dim3((unsigned)total), dim3(HconvSquare::NT), HconvSquare::LDS_BYTES,
+                           g_rt.stream, img, fb, out, M, N, Kw, tiles_n);
+    }
+    HIP_TRY(hipGetLastError());
+    return 0;
 }
 
 Batch single_on_library_stream() {
@@ -882,6 +937,19 @@ int decx_hip_conv2_im2col_f32_fused(const float* src, int H, int W, int dpitch, 
                                     int dst_dpitch, size_t dst_row_stride, int flag, const float* bias, int relu) {
     return finish(conv_enqueue(src, H, W, dpitch, src_row_stride, filt, N, kh, kw, filt_stride, filt_row_stride, dst,
                                dst_dpitch, dst_row_stride, flag, bias, relu != 0));
+}
+
+int decx_hip_conv2_im2col_f16_async(const uint16_t* src, int H, int W, int dpitch, size_t src_row_stride, const uint16_t* filt,
+                                    int N, int kh, int kw, size_t filt_stride, size_t filt_row_stride, uint16_t* dst,
+                                    int dst_dpitch, size_t dst_row_stride, int flag, const uint16_t* bias, int relu) {
+    return hconv_enqueue(src, H, W, dpitch, src_row_stride, filt, N, kh, kw, filt_stride, filt_row_stride, dst, dst_dpitch,
+                         dst_row_stride, flag, bias, relu != 0);
+}
+int decx_hip_conv2_im2col_f16(const uint16_t* src, int H, int W, int dpitch, size_t src_row_stride, const uint16_t* filt, int N,
+                              int kh, int kw, size_t filt_stride, size_t filt_row_stride, uint16_t* dst, int dst_dpitch,
+                              size_t dst_row_stride, int flag, const uint16_t* bias, int relu) {
+    return finish(hconv_enqueue(src, H, W, dpitch, src_row_stride, filt, N, kh, kw, filt_stride, filt_row_stride, dst,
+                                dst_dpitch, dst_row_stride, flag, bias, relu != 0));
 }
 
 int decx_hip_relu_f32(const float* src, float* dst, size_t n) { return finish(relu_enqueue<0>(src, dst, nullptr, n)); }

@@ -92,6 +92,20 @@ def bench_conv(capi, workloads, steps, warmup):
     return {"ms_wall": wall, "ms_kernel": ev, "tflops": flops / (wall * 1e-3) / 1e12, "tflops_kernel": flops / (ev * 1e-3) / 1e12}
 
 
+def bench_hconv(capi, workloads, steps, warmup):
+    """config 4 in binary16 with fp32 accumulation (decx_hip_conv2_im2col_f16_async); same flop count as bench_conv."""
+    H = W = 224; C = 64; N = 128; kh = kw = 3
+    src, filt = workloads.conv_case()
+    fb = np.zeros((N, kh, 4, C), np.float16); fb[:, :, :kw, :] = filt.astype(np.float16)
+    dS, dF = capi.DeviceBuffer.from_numpy(src.astype(np.float16).view(np.uint16)), capi.DeviceBuffer.from_numpy(fb.view(np.uint16))
+    dD = capi.DeviceBuffer(H * W * N * 2)
+    launch = lambda: capi.check(capi.lib().decx_hip_conv2_im2col_f16_async(
+        dS.ptr, H, W, C, W * C, dF.ptr, N, kh, kw, kh * 4 * C, 4 * C, dD.ptr, N, W * N, 1, None, 0))
+    wall, ev = time_launches(capi, launch, steps, warmup)
+    flops = 2.0 * H * W * N * kh * kw * C
+    return {"ms_wall": wall, "ms_kernel": ev, "tflops": flops / (wall * 1e-3) / 1e12, "tflops_kernel": flops / (ev * 1e-3) / 1e12}
+
+
 def per_launch_stats(capi, launch, reps):
     """Each launch timed on its own between two HIP events: (median ms, min ms)."""
     ms = []
@@ -306,6 +320,13 @@ def main():
             "tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
             "frac_of_fp32_matrix_peak": round(r["tflops_kernel"] / PEAK_FP32_MATRIX_TFLOPS, 4)}
         log("conv: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+
+    if want("conv"):
+        r = bench_hconv(capi, workloads, side_steps, side_warmup)
+        also["fp16_conv_224x224x64_128f3x3_f32acc_fused_im2col"] = {
+            "tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
+            "frac_of_fp16_dense_peak": round(r["tflops_kernel"] / PEAK_FP16_MATRIX_TFLOPS, 4)}
+        log("fp16 conv: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
 
     if want("relu"):
         r = bench_relu(capi, workloads, side_steps, side_warmup)

@@ -174,6 +174,22 @@ int decx_hip_conv2_im2col_f32_async(const float* src, int H, int W, int dpitch, 
 int decx_hip_conv2_im2col_f32_fused(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt,
                                     int N, int kh, int kw, size_t filt_stride, size_t filt_row_stride, float* dst,
                                     int dst_dpitch, size_t dst_row_stride, int flag, const float* bias, int relu);
+
+/* The same convolution on binary16 tensors with fp32 accumulation: the fp16 twin of the entry points above, named as a
+ * next step beside them; the reference itself has no binary16 im2col convolution (convolution/CUDA/im2col/ holds fp32
+ * only), its binary16 containers fix the layout: de::Tensor<de::Half> / de::TensorArray<de::Half> pad the channel
+ * pitch to a multiple of 8 halves and the width pitch to a multiple of 4 (classes/Tensor.h:214-235,
+ * classes/TensorArray.h:232-256; device twins classes/GPU_Tensor.h:201-222, classes/GPU_TensorArray.h:234-257).
+ * All strides and pitches in halves; dpitch % 8 == 0; src and filt 16-byte aligned.  Same index arithmetic, flags and
+ * error codes as decx_hip_conv2_im2col_f32.  Products are accumulated in fp32 (in the matrix instruction's order),
+ * then   dst(y,x,n) = half( relu( sum + float(bias[n]) ) )   with bias (N halves on the device) and relu optional (NULL / 0),
+ * rounded to binary16, nearest even, once.  Checked against fp64 arithmetic on the binary16 inputs to 2e-3 relative. */
+int decx_hip_conv2_im2col_f16(const uint16_t* src, int H, int W, int dpitch, size_t src_row_stride, const uint16_t* filt, int N,
+                              int kh, int kw, size_t filt_stride, size_t filt_row_stride, uint16_t* dst, int dst_dpitch,
+                              size_t dst_row_stride, int flag, const uint16_t* bias, int relu);
+int decx_hip_conv2_im2col_f16_async(const uint16_t* src, int H, int W, int dpitch, size_t src_row_stride, const uint16_t* filt,
+                                    int N, int kh, int kw, size_t filt_stride, size_t filt_row_stride, uint16_t* dst,
+                                    int dst_dpitch, size_t dst_row_stride, int flag, const uint16_t* bias, int relu);
 /* decx_hip_sgemm followed by de::nn::ReLU_f on the result, in one kernel: D = relu(A*B + Cin). */
 int decx_hip_sgemm_relu(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
                         int N, int K);

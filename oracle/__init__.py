@@ -43,6 +43,8 @@ def lib():
         L.oracle_decx_cpu_sgemm.restype = I
         L.oracle_conv2_chain.argtypes = [P, I, I, I, L_, P, I, I, I, L_, L_, P, I, L_, I, I]
         L.oracle_conv2_chain.restype = I
+        L.oracle_conv2_f64_f16.argtypes = [P, I, I, I, L_, P, I, I, I, L_, L_, P, P, I, I]
+        L.oracle_conv2_f64_f16.restype = I
         L.oracle_float_to_half.argtypes = [P, P, L_]
         L.oracle_float_to_half.restype = None
         L.oracle_half_to_float.argtypes = [P, P, L_]
@@ -180,6 +182,28 @@ def gemm_f64_rows_f32(A, B, rows, nthreads=0):
     ab = np.empty((len(rows), N), dtype=np.float64)
     lib().oracle_gemm_f64_rows_f32(_p(A), _ld(A), _p(B), _ld(B), _p(rows), len(rows), _p(out), _p(ab), N, K, nthreads)
     return out, ab
+
+
+def conv2_f64_f16(src_bits, filt_bits, flag, nthreads=0):
+    """fp64 convolution of binary16 tensors given as uint16 bit patterns: src (H, W, dpitch), filt (N, kh, kw, dpitch),
+    strides as in conv2_chain.  Returns (out, scale), both (H_out, W_out, N) float64: the sums of products and of their
+    absolute values.  flag 1 = same size with zero border, flag 0 = valid region."""
+    src = np.asarray(src_bits)
+    filt = np.asarray(filt_bits)
+    assert src.dtype == np.uint16 and filt.dtype == np.uint16
+    H, W, dp = src.shape
+    N, kh, kw, dp2 = filt.shape
+    assert dp == dp2
+    assert src.strides[2] == 2 and src.strides[1] == 2 * dp
+    assert filt.strides[3] == 2 and filt.strides[2] == 2 * dp
+    Hout, Wout = (H, W) if flag == 1 else (H - 2 * (kh // 2), W - 2 * (kw // 2))
+    out = np.zeros((max(Hout, 0), max(Wout, 0), N), dtype=np.float64)
+    scale = np.zeros_like(out)
+    rc = lib().oracle_conv2_f64_f16(_p(src), H, W, dp, src.strides[0] // 2, _p(filt), N, kh, kw, filt.strides[0] // 2,
+                                    filt.strides[1] // 2, _p(out), _p(scale), flag, nthreads)
+    if rc != 0:
+        raise ValueError("oracle_conv2_f64_f16 rejected its arguments (flag %r)" % (flag,))
+    return out, scale
 
 
 def relu(x):

@@ -26,6 +26,10 @@
 //   oracle_conv2_chain        : all-ones closed form (tap counts), impulse response = reversed filter slices,
 //                               fp64 7-loop brute force on tiny shapes, integer-exact vs int64.
 //   oracle_gemm_f64_rows_f16  : integer-exact vs int64, numpy float64 matmul on random data.
+//   oracle_conv2_f64_f16      : fp64 arithmetic on binary16 tensors, the yardstick of the fp16 convolution (the reference has
+//                               none to restate; indexing as oracle_conv2_chain): numpy float16 -> float64 conversion
+//                               plus a 7-loop brute force, all-ones tap counts, impulse response, equality with
+//                               oracle_conv2_chain on integer data, padded strides.
 //   oracle_float_to_half/back : numpy float16 casts (independent RNE implementation), IEEE known values.
 //   oracle_relu_f32[_rec|_backward] : restate srcs/nn/operators/ReLU.h:57-165 (value times float(sign bit clear); one
 //                               map byte per 8 floats).  The reference holds no test vectors for them; pinned by
@@ -392,6 +396,55 @@ int oracle_conv2_chain(const float* src, int H, int W, int dpitch, long src_row_
                 std::memset(acc.data(), 0, sizeof(float) * N);
                 for (int k = 0; k < K; ++k) row_fma(patch[k], Wt.data() + (size_t)k * N, acc.data(), N);
                 std::memcpy(dst + (size_t)y * dst_row_stride + (size_t)x * dst_dpitch, acc.data(), sizeof(float) * N);
+            }
+    });
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Convolution of binary16 tensors in fp64: what the fp16 convolution (fp32 accumulate) is checked against, as the fp16
+// GEMM is against oracle_gemm_f64_rows_f16.  Same index arithmetic as oracle_conv2_chain (k = (ki*kw + kj)*dpitch + c,
+// cross-correlation, im2col.cuh:150-163; flag as conv2_mk_im2col.h:63-66, :173-176); all strides in halves.
+// out[(y*W_out + x)*N + n] = sum of products, scale[...] = sum of |products| (the denominator of the relative error).
+// The reference has no binary16 im2col convolution, so there is no reference arithmetic to restate beyond the indexing.
+// ---------------------------------------------------------------------------------------------------------------
+static inline float h2f(uint16_t h);      // defined with the conversions below
+int oracle_conv2_f64_f16(const uint16_t* src, int H, int W, int dpitch, long src_row_stride, const uint16_t* filt, int N,
+                         int kh, int kw, long filt_stride, long filt_row_stride, double* out, double* scale, int flag,
+                         int nthreads) {
+    if (flag != 0 && flag != 1) return -1;
+    int Hout = flag ? H : H - 2 * (kh / 2), Wout = flag ? W : W - 2 * (kw / 2);
+    if (Hout <= 0 || Wout <= 0 || N <= 0 || dpitch <= 0) return -1;
+    int oy = flag ? kh / 2 : 0, ox = flag ? kw / 2 : 0;
+    int K = kh * kw * dpitch;
+    std::vector<double> Wt((size_t)K * N);
+    for (int n = 0; n < N; ++n)
+        for (int ki = 0; ki < kh; ++ki)
+            for (int kj = 0; kj < kw; ++kj)
+                for (int c = 0; c < dpitch; ++c)
+                    Wt[(size_t)((ki * kw + kj) * dpitch + c) * N + n] =
+                        (double)h2f(filt[(size_t)n * filt_stride + (size_t)ki * filt_row_stride + (size_t)kj * dpitch + c]);
+    parallel_ranges(nthreads, Hout, [&](long lo, long hi) {
+        std::vector<double> patch(K);
+        for (long y = lo; y < hi; ++y)
+            for (int x = 0; x < Wout; ++x) {
+                for (int ki = 0; ki < kh; ++ki)
+                    for (int kj = 0; kj < kw; ++kj) {
+                        long sy = y + ki - oy, sx = x + kj - ox;
+                        double* p = patch.data() + (size_t)(ki * kw + kj) * dpitch;
+                        const bool inside = sy >= 0 && sy < H && sx >= 0 && sx < W;
+                        for (int c = 0; c < dpitch; ++c)
+                            p[c] = inside ? (double)h2f(src[(size_t)sy * src_row_stride + (size_t)sx * dpitch + c]) : 0.0;
+                    }
+                double* o = out + ((size_t)y * Wout + x) * N;
+                double* sc = scale + ((size_t)y * Wout + x) * N;
+                for (int n = 0; n < N; ++n) o[n] = sc[n] = 0.0;
+                for (int k = 0; k < K; ++k) {
+                    const double a = patch[k];
+                    if (a == 0.0) continue;
+                    const double* w = Wt.data() + (size_t)k * N;
+                    for (int n = 0; n < N; ++n) { o[n] += a * w[n]; sc[n] += std::fabs(a * w[n]); }
+                }
             }
     });
     return 0;

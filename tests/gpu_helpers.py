@@ -120,6 +120,42 @@ def gpu_conv(src, filt, flag, variant=0, bias=None, relu=False):
     return out[:Hout, :Wout, :N].copy()
 
 
+def half_tensor_storage(t16, pad_bits=0x7e00):
+    """(H, W, C) float16 -> the reference's binary16 Tensor storage [H][ceil4(W)][ceil8(C)] (Tensor.h:214-235) as uint16
+    bit patterns: channel padding zero, width padding filled with pad_bits (a NaN by default)."""
+    H, W, C = t16.shape
+    wp, dp = (W + 3) // 4 * 4, (C + 7) // 8 * 8
+    buf = np.full((H, wp, dp), pad_bits, dtype=np.uint16)
+    buf[:, :W, :] = 0
+    buf[:, :W, :C] = t16.view(np.uint16)
+    return buf, wp, dp
+
+
+def gpu_hconv(src16, filt16, flag, bias16=None, relu=False):
+    """fp16 convolution through the C ABI: src16 (H, W, C), filt16 (N, kh, kw, C), bias16 (N,) float16 arrays.
+    Returns (dst float16 (H_out, W_out, N), the image storage, the filter storage) -- the storages, as uint16 views
+    without their width padding, are what the oracle is fed."""
+    H, W, C = src16.shape
+    N, kh, kw, _ = filt16.shape
+    sbuf, swp, dp = half_tensor_storage(src16)
+    fwp = (kw + 3) // 4 * 4
+    fb = np.full((N, kh, fwp, dp), 0x7e00, dtype=np.uint16)
+    fb[:, :, :kw, :] = 0
+    fb[:, :, :kw, :C] = filt16.view(np.uint16)
+    Hout, Wout = (H, W) if flag == 1 else (H - 2 * (kh // 2), W - 2 * (kw // 2))
+    Ho, Wo = max(Hout, 1), max(Wout, 1)
+    dwp, ddp = (Wo + 3) // 4 * 4, (N + 7) // 8 * 8
+    sentinel = np.full((Ho, dwp, ddp), 0xd610, dtype=np.uint16)          # -97.0
+    dS, dF, dD = (capi.DeviceBuffer.from_numpy(sbuf), capi.DeviceBuffer.from_numpy(fb),
+                  capi.DeviceBuffer.from_numpy(sentinel))
+    dB = capi.DeviceBuffer.from_numpy(np.asarray(bias16, dtype=np.float16).view(np.uint16)) if bias16 is not None else None
+    capi.check(capi.lib().decx_hip_conv2_im2col_f16(dS.ptr, H, W, dp, swp * dp, dF.ptr, N, kh, kw, kh * fwp * dp, fwp * dp,
+                                                    dD.ptr, ddp, dwp * ddp, flag, dB.ptr if dB else None, 1 if relu else 0))
+    out = dD.download((Ho, dwp, ddp), np.uint16)
+    assert np.all(out[:, Wout:, :] == 0xd610) and np.all(out[:, :, N:] == 0xd610), "kernel wrote into dst padding"
+    return out[:Hout, :Wout, :N].copy().view(np.float16), sbuf[:, :W], fb[:, :, :kw]
+
+
 def rel_err_vs_abs_scale(got, ref, scale):
     """max |got - ref| / sum_k |a||b|: the relative-error definition used for the fp32 / fp16 tolerances (a bound
     any correct summation order satisfies, and well-defined where the reference value itself is near zero)."""

@@ -1,0 +1,112 @@
+"""fp16 convolution (decx_hip_conv2_im2col_f16, backup_1_amd/csrc/hconv_tile.hpp) through the C ABI.
+
+The reference has no binary16 im2col convolution to compare bits with; the bar is the fp16 rule of this build: fp32
+accumulation, at most 2e-3 relative to fp64 arithmetic on the same binary16 inputs (relative to sum |a||b|, plus the
+half-ulp of the final rounding to binary16), and exact results wherever binary16 can hold them (small integers)."""
+import numpy as np
+import pytest
+
+from backup_1_amd import capi, workloads
+from gpu_helpers import gpu_hconv
+
+pytestmark = pytest.mark.gpu
+
+TOL = 2e-3
+
+
+def check_against_f64(oracle, got16, sbuf, fb, flag, bias16=None, relu=False):
+    ref, scale = oracle.conv2_f64_f16(sbuf, fb, flag)
+    if bias16 is not None:
+        b = np.asarray(bias16, np.float16).astype(np.float64)
+        ref = ref + b[None, None, :]
+        scale = scale + np.abs(b)[None, None, :]
+    if relu:
+        ref = np.maximum(ref, 0.0)
+    got = got16.astype(np.float64)
+    # fp32 accumulation error relative to sum |a||b|, and the one rounding to binary16 relative to the value itself
+    bound = TOL * scale + 2.0 ** -11 * np.abs(ref) + 2.0 ** -24
+    assert np.all(np.isfinite(got))
+    worst = np.max(np.abs(got - ref) / np.maximum(bound, 1e-300))
+    assert worst <= 1.0, worst
+    acc_err = np.max((np.abs(got - ref) - 2.0 ** -11 * np.abs(ref) - 2.0 ** -24) / np.maximum(scale, 1e-300))
+    return max(acc_err, 0.0)
+
+
+CASES = [(20, 22, 8, 6, 3, 3), (9, 13, 3, 2, 3, 3), (16, 16, 64, 128, 3, 3), (33, 17, 24, 130, 1, 1), (12, 40, 16, 5, 5, 3),
+         (40, 12, 40, 7, 3, 5), (7, 7, 8, 1, 7, 7), (64, 48, 32, 200, 3, 3)]
+
+
+@pytest.mark.parametrize("flag", [1, 0])
+@pytest.mark.parametrize("case", CASES)
+def test_small_integers_are_exact(gpu, oracle, case, flag):
+    # |values| <= 2, at most 8 taps... products summed stay below 2048, where binary16 holds every integer
+    H, W, C, N, kh, kw = case
+    if flag == 0 and (H <= 2 * (kh // 2) or W <= 2 * (kw // 2)):
+        pytest.skip("no valid region")
+    src = workloads.small_ints((H, W, C), 801, -1, 1).astype(np.float16)
+    filt = workloads.small_ints((N, kh, kw, C), 802, -1, 1).astype(np.float16)
+    got, sbuf, fb = gpu_hconv(src, filt, flag)
+    ref, scale = oracle.conv2_f64_f16(sbuf, fb, flag)
+    assert scale.max() < 2048
+    assert np.array_equal(got.astype(np.float64), ref)
+
+
+@pytest.mark.parametrize("flag", [1, 0])
+@pytest.mark.parametrize("case", CASES)
+def test_real_values_within_tolerance(gpu, oracle, case, flag):
+    H, W, C, N, kh, kw = case
+    if flag == 0 and (H <= 2 * (kh // 2) or W <= 2 * (kw // 2)):
+        pytest.skip("no valid region")
+    src = workloads.uniform_01((H, W, C), 811).astype(np.float16)
+    filt = workloads.normal((N, kh, kw, C), 812, sigma=0.05).astype(np.float16)
+    got, sbuf, fb = gpu_hconv(src, filt, flag)
+    assert check_against_f64(oracle, got, sbuf, fb, flag) < TOL
+
+
+def test_all_ones_counts_taps_and_impulse_returns_the_reversed_filter(gpu):
+    H, W, C, N = 11, 14, 16, 4
+    got, _, _ = gpu_hconv(np.ones((H, W, C), np.float16), np.ones((N, 3, 3, C), np.float16), 1)
+    assert np.all(got[1:-1, 1:-1] == 9 * C) and np.all(got[0, 1:-1] == 6 * C) and np.all(got[-1, -1] == 4 * C)
+    filt = workloads.normal((N, 3, 5, C), 821).astype(np.float16)
+    src = np.zeros((H, W, C), np.float16)
+    src[5, 6, 3] = 1.0
+    got, _, _ = gpu_hconv(src, filt, 1)
+    for di in (-1, 0, 1):
+        for dj in (-2, -1, 0, 1, 2):
+            assert np.array_equal(got[5 - di, 6 - dj, :].view(np.uint16), filt[:, 1 + di, 2 + dj, 3].view(np.uint16))
+    got[4:7, 4:9] = 0
+    assert not got.any()
+
+
+def test_bias_and_relu_in_the_epilogue(gpu, oracle):
+    H, W, C, N = 30, 26, 24, 70
+    src = workloads.normal((H, W, C), 831).astype(np.float16)
+    filt = workloads.normal((N, 3, 3, C), 832, sigma=0.1).astype(np.float16)
+    bias = workloads.normal((N,), 833).astype(np.float16)
+    for b, r in ((bias, False), (None, True), (bias, True)):
+        got, sbuf, fb = gpu_hconv(src, filt, 1, bias16=b, relu=r)
+        check_against_f64(oracle, got, sbuf, fb, 1, bias16=b, relu=r)
+        if r:
+            assert not np.any(got.astype(np.float64) < 0)
+    # ReLU by sign as in nn/operators/ReLU.h:57-82: a negative sum becomes -0.0
+    got, _, _ = gpu_hconv(-np.ones((4, 4, 8), np.float16), np.ones((1, 1, 1, 8), np.float16), 1, relu=True)
+    assert np.all(got.view(np.uint16) == 0x8000)
+
+
+def test_headline_shape_sampled(gpu, oracle):
+    # 224x224x64 image, 128 filters 3x3x64, same size: the fp32 conv config in binary16
+    src = workloads.uniform_01((224, 224, 64), 841).astype(np.float16)
+    filt = workloads.normal((128, 3, 3, 64), 842, sigma=0.05).astype(np.float16)
+    got, sbuf, fb = gpu_hconv(src, filt, 1)
+    assert check_against_f64(oracle, got, sbuf, fb, 1) < TOL
+
+
+def test_error_codes(gpu):
+    L = capi.lib()
+    d = capi.DeviceBuffer(1 << 16)
+    args = lambda **kw: [kw.get("src", d.ptr), 8, 8, kw.get("dpitch", 8), 64, d.ptr, 4, 3, 3, 3 * 4 * 8, 4 * 8, d.ptr, 8, 64,
+                         kw.get("flag", 1), None, 0]
+    assert L.decx_hip_conv2_im2col_f16(*args(flag=7)) == 0x0b          # DECX_FAIL_ErrorFlag
+    assert L.decx_hip_conv2_im2col_f16(*args(dpitch=4)) == 0x0d    # channel pitch not a multiple of 8
+    assert L.decx_hip_conv2_im2col_f16(*args(src=None)) == 0x0d
+    assert L.decx_hip_conv2_im2col_f16(*args()) == 0

@@ -225,6 +225,53 @@ def test_conv_strided_containers_and_bad_flag(oracle):
 
 
 # ---------------------------------------------------------------- fp16 ----------------------------------------
+# ---------------------------------------------------------------- fp16 convolution, fp64 arithmetic ------------
+@pytest.mark.parametrize("case", [(6, 7, 8, 3, 3, 3, 1), (6, 7, 8, 3, 3, 3, 0), (5, 9, 16, 2, 5, 3, 1), (8, 8, 8, 5, 1, 1, 1),
+                                  (9, 6, 8, 2, 3, 5, 0)])
+def test_conv_f64_of_halves_vs_bruteforce_and_numpy_float16(oracle, case):
+    # pins oracle_conv2_f64_f16: numpy's own float16 -> float64 conversion and a 7-loop brute force fix values and indexing
+    H, W, C, N, kh, kw, flag = case
+    src = workloads.uniform_01((H, W, C), 71).astype(np.float16)
+    filt = workloads.normal((N, kh, kw, C), 72, sigma=0.5).astype(np.float16)
+    got, scale = oracle.conv2_f64_f16(src.view(np.uint16), filt.view(np.uint16), flag)
+    want = _conv_bruteforce_f64(src.astype(np.float64), filt.astype(np.float64), flag)
+    np.testing.assert_allclose(got, want, rtol=1e-13, atol=1e-13)
+    want_scale = _conv_bruteforce_f64(np.abs(src).astype(np.float64), np.abs(filt).astype(np.float64), flag)
+    np.testing.assert_allclose(scale, want_scale, rtol=1e-13, atol=1e-13)
+    # integer data: equals the fp32 chain oracle exactly (two independent index walks)
+    si, fi = workloads.small_ints((H, W, C), 73, -4, 4), workloads.small_ints((N, kh, kw, C), 74, -4, 4)
+    g2, _ = oracle.conv2_f64_f16(si.astype(np.float16).view(np.uint16), fi.astype(np.float16).view(np.uint16), flag)
+    assert np.array_equal(g2, oracle.conv2_chain(si, fi, flag).astype(np.float64))
+
+
+def test_conv_f64_of_halves_closed_forms_and_strides(oracle):
+    H, W, C, N = 7, 9, 8, 3
+    ones = np.ones((H, W, C), np.float16).view(np.uint16)
+    fones = np.ones((N, 3, 3, C), np.float16).view(np.uint16)
+    d, sc = oracle.conv2_f64_f16(ones, fones, 1)
+    assert np.all(d[1:-1, 1:-1] == 9 * C) and np.all(d[0, 1:-1] == 6 * C) and np.all(d[0, 0] == 4 * C) and np.array_equal(d, sc)
+    v, _ = oracle.conv2_f64_f16(ones, fones, 0)
+    assert v.shape == (H - 2, W - 2, N) and np.all(v == 9 * C)
+    # impulse: cross-correlation, so the response is the filter reversed in space
+    filt = workloads.normal((N, 3, 5, C), 75).astype(np.float16)
+    src = np.zeros((H, W, C), np.float16)
+    src[3, 4, 2] = 1.0
+    d, _ = oracle.conv2_f64_f16(src.view(np.uint16), filt.view(np.uint16), 1)
+    for di in (-1, 0, 1):
+        for dj in (-2, -1, 0, 1, 2):
+            assert np.array_equal(d[3 - di, 4 - dj, :], filt[:, 1 + di, 2 + dj, 2].astype(np.float64))
+    # padded containers (row stride of the image, tap-row stride of the filters) and the flag check
+    sbuf = np.zeros((H, W + 3, C), np.float16)
+    sbuf[:, :W] = workloads.uniform_01((H, W, C), 76).astype(np.float16)
+    fbuf = np.zeros((N, 3, 4, C), np.float16)
+    fbuf[:, :, :3] = workloads.normal((N, 3, 3, C), 77).astype(np.float16)
+    got, _ = oracle.conv2_f64_f16(sbuf.view(np.uint16)[:, :W], fbuf.view(np.uint16)[:, :, :3], 1)
+    want, _ = oracle.conv2_f64_f16(np.ascontiguousarray(sbuf[:, :W]).view(np.uint16), np.ascontiguousarray(fbuf[:, :, :3]).view(np.uint16), 1)
+    assert np.array_equal(got, want)
+    with pytest.raises(ValueError):
+        oracle.conv2_f64_f16(ones, fones, 2)
+
+
 def test_half_conversion_matches_numpy_and_ieee(oracle):
     known = {1.0: 0x3C00, -2.0: 0xC000, 65504.0: 0x7BFF, 65520.0: 0x7C00, 65519.99: 0x7BFF, 5.9604645e-8: 0x0001,
              2.9802322e-8: 0x0000, 0.0: 0x0000, 1.0009765625: 0x3C01, 1.00048828125: 0x3C00, 1.00146484375: 0x3C02,
