@@ -426,8 +426,8 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
 }
 
 // fp16 convolution (hconv_tile.hpp).  Strides and pitches in halves, as the binary16 containers hold them.
-typedef HconvShape<128, 128, 2, 2> HconvSquare;      // 2x2 waves of 64x64
-typedef HconvShape<256, 128, 4, 2> HconvTall;        // 4x2 waves of 64x64, two per SIMD: half the filter reads per pixel
+typedef HconvShape<128, 128, 2, 2, 4> HconvSquare;   // 2x2 waves of 64x64
+typedef HconvShape<256, 128, 4, 2, 4> HconvTall;     // 4x2 waves of 64x64, two per SIMD: half the filter reads per pixel
 int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_stride, const uint16_t* filt, int N, int kh,
                   int kw, size_t filt_stride, size_t filt_row_stride, uint16_t* dst, int dst_dpitch, size_t dst_row_stride,
                   int flag, const uint16_t* bias, bool relu) {
