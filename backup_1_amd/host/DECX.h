@@ -133,7 +133,7 @@ public:
     virtual ~MatrixArray() {}
 };
 
-// classes/GPU_Tensor.h:19-47.  Device-resident tensor with the host Tensor's layout (dpitch = ceil4(depth),
+// classes/GPU_Tensor.h:19-47.  Device-resident tensor with the host Tensor's layout (dpitch = ceil4(depth) for 4-byte and ceil8(depth) for 2-byte elements,
 // wpitch = ceil4(width)).
 template <typename T>
 class GPU_Tensor {
@@ -166,7 +166,7 @@ public:
 };
 
 // factories: classes/Matrix.h:430-476, GPU_Matrix.h:361-435, Tensor.h:401-463, TensorArray.h:440-474.
-// Instantiated for float and de::Half (Matrix, GPU_Matrix) and float (Tensor, TensorArray).
+// Instantiated for float and de::Half.
 template <typename T> Matrix<T>& CreateMatrixRef();
 template <typename T> Matrix<T>* CreateMatrixPtr();
 template <typename T> Matrix<T>& CreateMatrixRef(const uint width, const uint height, const int store_type);
@@ -190,7 +190,7 @@ template <typename T> MatrixArray<T>* CreateMatrixArrayPtr();
 template <typename T> MatrixArray<T>& CreateMatrixArrayRef(uint width, uint height, uint MatrixNum, const int flag);
 template <typename T> MatrixArray<T>* CreateMatrixArrayPtr(uint width, uint height, uint MatrixNum, const int flag);
 
-// classes/GPU_Tensor.h:385-397, GPU_TensorArray.h (same pattern); instantiated for float
+// classes/GPU_Tensor.h:385-397, GPU_TensorArray.h (same pattern); instantiated for float and de::Half
 template <typename T> GPU_Tensor<T>& CreateGPUTensorRef();
 template <typename T> GPU_Tensor<T>* CreateGPUTensorPtr();
 template <typename T> GPU_Tensor<T>& CreateGPUTensorRef(const uint width, const uint height, const uint depth);
@@ -230,6 +230,11 @@ DH Conv2_MK_im2col(Tensor<float>& src, TensorArray<float>& kernel, Tensor<float>
 // GPU_TensorArray containers, classes/GPU_Tensor.h and GPU_TensorArray.h, are what it would take).  dst is
 // (re)constructed to the output size; no host copies are made.
 DH Conv2_MK_im2col(GPU_Tensor<float>& src, GPU_TensorArray<float>& kernel, GPU_Tensor<float>& dst, const int flag);
+// The same convolution on binary16 containers (de::Tensor<de::Half> etc., channel pitch a multiple of 8: classes/Tensor.h:214-235,
+// TensorArray.h:232-256, GPU_Tensor.h:201-222, GPU_TensorArray.h:234-257), accumulated in fp32.  The reference declares
+// the containers but no binary16 im2col convolution; these overloads are what it would look like.
+DH Conv2_MK_im2col(Tensor<Half>& src, TensorArray<Half>& kernel, Tensor<Half>& dst, const int flag);
+DH Conv2_MK_im2col(GPU_Tensor<Half>& src, GPU_TensorArray<Half>& kernel, GPU_Tensor<Half>& dst, const int flag);
 }  // namespace cuda
 
 namespace nn {

@@ -219,13 +219,21 @@ template MatrixArray<Half>* CreateMatrixArrayPtr<Half>();
 template MatrixArray<Half>& CreateMatrixArrayRef<Half>(uint, uint, uint, const int);
 template MatrixArray<Half>* CreateMatrixArrayPtr<Half>(uint, uint, uint, const int);
 template GPU_Tensor<float>& CreateGPUTensorRef<float>();
+template GPU_Tensor<Half>& CreateGPUTensorRef<Half>();
 template GPU_Tensor<float>* CreateGPUTensorPtr<float>();
+template GPU_Tensor<Half>* CreateGPUTensorPtr<Half>();
 template GPU_Tensor<float>& CreateGPUTensorRef<float>(const uint, const uint, const uint);
+template GPU_Tensor<Half>& CreateGPUTensorRef<Half>(const uint, const uint, const uint);
 template GPU_Tensor<float>* CreateGPUTensorPtr<float>(const uint, const uint, const uint);
+template GPU_Tensor<Half>* CreateGPUTensorPtr<Half>(const uint, const uint, const uint);
 template GPU_TensorArray<float>& CreateGPUTensorArrayRef<float>();
+template GPU_TensorArray<Half>& CreateGPUTensorArrayRef<Half>();
 template GPU_TensorArray<float>* CreateGPUTensorArrayPtr<float>();
+template GPU_TensorArray<Half>* CreateGPUTensorArrayPtr<Half>();
 template GPU_TensorArray<float>& CreateGPUTensorArrayRef<float>(const uint, const uint, const uint, const uint);
+template GPU_TensorArray<Half>& CreateGPUTensorArrayRef<Half>(const uint, const uint, const uint, const uint);
 template GPU_TensorArray<float>* CreateGPUTensorArrayPtr<float>(const uint, const uint, const uint, const uint);
+template GPU_TensorArray<Half>* CreateGPUTensorArrayPtr<Half>(const uint, const uint, const uint, const uint);
 
 #define DECX_INSTANTIATE_MATRIX(T)                                                     \
     template Matrix<T>& CreateMatrixRef<T>();                                          \
@@ -240,13 +248,21 @@ DECX_INSTANTIATE_MATRIX(float)
 DECX_INSTANTIATE_MATRIX(Half)
 DECX_INSTANTIATE_MATRIX(uchar)
 template Tensor<float>& CreateTensorRef<float>();
+template Tensor<Half>& CreateTensorRef<Half>();
 template Tensor<float>* CreateTensorPtr<float>();
+template Tensor<Half>* CreateTensorPtr<Half>();
 template Tensor<float>& CreateTensorRef<float>(const uint, const uint, const uint, const int);
+template Tensor<Half>& CreateTensorRef<Half>(const uint, const uint, const uint, const int);
 template Tensor<float>* CreateTensorPtr<float>(const uint, const uint, const uint, const int);
+template Tensor<Half>* CreateTensorPtr<Half>(const uint, const uint, const uint, const int);
 template TensorArray<float>& CreateTensorArrayRef<float>();
+template TensorArray<Half>& CreateTensorArrayRef<Half>();
 template TensorArray<float>* CreateTensorArrayPtr<float>();
+template TensorArray<Half>* CreateTensorArrayPtr<Half>();
 template TensorArray<float>& CreateTensorArrayRef<float>(const uint, const uint, const uint, const uint, const int);
+template TensorArray<Half>& CreateTensorArrayRef<Half>(const uint, const uint, const uint, const uint, const int);
 template TensorArray<float>* CreateTensorArrayPtr<float>(const uint, const uint, const uint, const uint, const int);
+template TensorArray<Half>* CreateTensorArrayPtr<Half>(const uint, const uint, const uint, const uint, const int);
 
 // ---- GEMM ---------------------------------------------------------------------------------------------------
 namespace cuda {
@@ -280,26 +296,49 @@ DH GEMM3(MatrixArray<float>& A, MatrixArray<float>& B, MatrixArray<float>& C, Ma
 DH GEMM3(MatrixArray<Half>& A, MatrixArray<Half>& B, MatrixArray<Half>& C, MatrixArray<Half>& dst) { return gemm3_host<Half>(A, B, &C, dst); }
 
 // ---- convolution ----------------------------------------------------------------------------------------------
-DH Conv2_MK_im2col(Tensor<float>& src_, TensorArray<float>& kernel_, Tensor<float>& dst_, const int flag) {
-    auto* src = dynamic_cast<decx::_Tensor<float>*>(&src_);
-    auto* ker = dynamic_cast<decx::_TensorArray<float>*>(&kernel_);
-    auto* dst = dynamic_cast<decx::_Tensor<float>*>(&dst_);
-    if (!src || !ker || !dst) return DH{decx::DECX_FAIL_ErrorParams, kNotFactory};
-    if (!decx_hip_is_init()) return not_init();                                           // conv2_mk_im2col.h:285-289
+namespace {
+template <typename T> struct ConvCall;
+template <> struct ConvCall<float> {
+    static int run(const float* src, int H, int W, int dpitch, size_t src_row, const float* filt, int N, int kh, int kw,
+                   size_t filt_stride, size_t filt_row, float* dst, int dst_dpitch, size_t dst_row, int flag) {
+        return decx_hip_conv2_im2col_f32(src, H, W, dpitch, src_row, filt, N, kh, kw, filt_stride, filt_row, dst, dst_dpitch,
+                                         dst_row, flag);
+    }
+};
+template <> struct ConvCall<Half> {
+    static int run(const Half* src, int H, int W, int dpitch, size_t src_row, const Half* filt, int N, int kh, int kw,
+                   size_t filt_stride, size_t filt_row, Half* dst, int dst_dpitch, size_t dst_row, int flag) {
+        return decx_hip_conv2_im2col_f16(reinterpret_cast<const uint16_t*>(src), H, W, dpitch, src_row,
+                                         reinterpret_cast<const uint16_t*>(filt), N, kh, kw, filt_stride, filt_row,
+                                         reinterpret_cast<uint16_t*>(dst), dst_dpitch, dst_row, flag, nullptr, 0);
+    }
+};
+
+// what both container flavours check before anything is allocated (conv2_mk_im2col.h:285-289, :63-66, :173-176)
+DH conv_precheck(uint src_depth, uint ker_depth, int H, int W, int kh, int kw, int flag, int& Hout, int& Wout) {
+    if (!decx_hip_is_init()) return not_init();
     if (flag != decx::de_conv_no_compensate && flag != decx::de_conv_zero_compensate) {
         static char msg[] = "This flag is meaningless in current context\n";              // core/error.h:67
         return DH{decx::DECX_FAIL_ErrorFlag, msg};
     }
-    if (src->depth != ker->depth) {
-        static char msg[] = "Tensor Dims don't match each other";
-        return DH{decx::DECX_FAIL_DimsNotMatching, msg};
-    }
+    static char dims_msg[] = "Tensor Dims don't match each other";
+    if (src_depth != ker_depth) return DH{decx::DECX_FAIL_DimsNotMatching, dims_msg};
+    Hout = flag ? H : H - 2 * (kh / 2);
+    Wout = flag ? W : W - 2 * (kw / 2);
+    if (Hout <= 0 || Wout <= 0) return DH{decx::DECX_FAIL_DimsNotMatching, dims_msg};
+    return ok();
+}
+
+template <typename T>
+DH conv_host(Tensor<T>& src_, TensorArray<T>& kernel_, Tensor<T>& dst_, const int flag) {
+    auto* src = dynamic_cast<decx::_Tensor<T>*>(&src_);
+    auto* ker = dynamic_cast<decx::_TensorArray<T>*>(&kernel_);
+    auto* dst = dynamic_cast<decx::_Tensor<T>*>(&dst_);
+    if (!src || !ker || !dst) return DH{decx::DECX_FAIL_ErrorParams, kNotFactory};
     const int H = (int)src->height, W = (int)src->width, kh = (int)ker->height, kw = (int)ker->width;
-    const int Hout = flag ? H : H - 2 * (kh / 2), Wout = flag ? W : W - 2 * (kw / 2);     // conv2_mk_im2col.h:63-66, :173-176
-    if (Hout <= 0 || Wout <= 0) {
-        static char msg[] = "Tensor Dims don't match each other";
-        return DH{decx::DECX_FAIL_DimsNotMatching, msg};
-    }
+    int Hout = 0, Wout = 0;
+    DH pre = conv_precheck(src->depth, ker->depth, H, W, kh, kw, flag, Hout, Wout);
+    if (pre.error_type != decx::DECX_SUCCESS) return pre;
     if (!dst->re_construct((uint)Wout, (uint)Hout, ker->tensor_num, decx::Page_Locked)) return alloc_fail();   // :178
     DeviceTemp dS, dK, dD;
     if (dS.alloc(src->total_bytes) || dK.alloc(ker->total_bytes) || dD.alloc(dst->total_bytes)) return alloc_fail();
@@ -309,33 +348,42 @@ DH Conv2_MK_im2col(Tensor<float>& src_, TensorArray<float>& kernel_, Tensor<floa
     if (rc) return from_status(rc);
     rc = decx_hip_memset(dD.ptr, 0, dst->total_bytes);   // the width / channel padding of dst stays zero
     if (rc) return from_status(rc);
-    rc = decx_hip_conv2_im2col_f32(static_cast<const float*>(dS.ptr), H, W, (int)src->dpitch, src->dp_x_wp,
-                                   static_cast<const float*>(dK.ptr), (int)ker->tensor_num, kh, kw, ker->_gap, ker->dp_x_wp,
-                                   static_cast<float*>(dD.ptr), (int)dst->dpitch, dst->dp_x_wp, flag);
+    rc = ConvCall<T>::run(static_cast<const T*>(dS.ptr), H, W, (int)src->dpitch, src->dp_x_wp, static_cast<const T*>(dK.ptr),
+                          (int)ker->tensor_num, kh, kw, ker->_gap, ker->dp_x_wp, static_cast<T*>(dD.ptr), (int)dst->dpitch,
+                          dst->dp_x_wp, flag);
     if (rc) return from_status(rc);
     return from_status(decx_hip_memcpy(dst->Tens.ptr, dD.ptr, dst->total_bytes, DECX_HIP_D2H));   // :266
 }
 
-DH Conv2_MK_im2col(GPU_Tensor<float>& src_, GPU_TensorArray<float>& kernel_, GPU_Tensor<float>& dst_, const int flag) {
-    auto* src = dynamic_cast<decx::_GPU_Tensor<float>*>(&src_);
-    auto* ker = dynamic_cast<decx::_GPU_TensorArray<float>*>(&kernel_);
-    auto* dst = dynamic_cast<decx::_GPU_Tensor<float>*>(&dst_);
+template <typename T>
+DH conv_device(GPU_Tensor<T>& src_, GPU_TensorArray<T>& kernel_, GPU_Tensor<T>& dst_, const int flag) {
+    auto* src = dynamic_cast<decx::_GPU_Tensor<T>*>(&src_);
+    auto* ker = dynamic_cast<decx::_GPU_TensorArray<T>*>(&kernel_);
+    auto* dst = dynamic_cast<decx::_GPU_Tensor<T>*>(&dst_);
     if (!src || !ker || !dst) return DH{decx::DECX_FAIL_ErrorParams, kNotFactory};
-    if (!decx_hip_is_init()) return not_init();
-    if (flag != decx::de_conv_no_compensate && flag != decx::de_conv_zero_compensate) {
-        static char msg[] = "This flag is meaningless in current context\n";
-        return DH{decx::DECX_FAIL_ErrorFlag, msg};
-    }
-    static char dims_msg[] = "Tensor Dims don't match each other";
-    if (src->depth != ker->depth) return DH{decx::DECX_FAIL_DimsNotMatching, dims_msg};
     const int H = (int)src->height, W = (int)src->width, kh = (int)ker->height, kw = (int)ker->width;
-    const int Hout = flag ? H : H - 2 * (kh / 2), Wout = flag ? W : W - 2 * (kw / 2);
-    if (Hout <= 0 || Wout <= 0) return DH{decx::DECX_FAIL_DimsNotMatching, dims_msg};
+    int Hout = 0, Wout = 0;
+    DH pre = conv_precheck(src->depth, ker->depth, H, W, kh, kw, flag, Hout, Wout);
+    if (pre.error_type != decx::DECX_SUCCESS) return pre;
     if (!dst->re_construct((uint)Wout, (uint)Hout, ker->tensor_num))
         return dst->last_status == DECX_HIP_FAIL_ALLOCATION ? alloc_fail() : from_status(dst->last_status);
-    return from_status(decx_hip_conv2_im2col_f32(src->Tens.ptr, H, W, (int)src->dpitch, src->dp_x_wp, ker->TensArr.ptr,
-                                                 (int)ker->tensor_num, kh, kw, ker->_gap, ker->dp_x_wp, dst->Tens.ptr,
-                                                 (int)dst->dpitch, dst->dp_x_wp, flag));
+    return from_status(ConvCall<T>::run(src->Tens.ptr, H, W, (int)src->dpitch, src->dp_x_wp, ker->TensArr.ptr,
+                                        (int)ker->tensor_num, kh, kw, ker->_gap, ker->dp_x_wp, dst->Tens.ptr,
+                                        (int)dst->dpitch, dst->dp_x_wp, flag));
+}
+}  // namespace
+
+DH Conv2_MK_im2col(Tensor<float>& src, TensorArray<float>& kernel, Tensor<float>& dst, const int flag) {
+    return conv_host<float>(src, kernel, dst, flag);
+}
+DH Conv2_MK_im2col(GPU_Tensor<float>& src, GPU_TensorArray<float>& kernel, GPU_Tensor<float>& dst, const int flag) {
+    return conv_device<float>(src, kernel, dst, flag);
+}
+DH Conv2_MK_im2col(Tensor<Half>& src, TensorArray<Half>& kernel, Tensor<Half>& dst, const int flag) {
+    return conv_host<Half>(src, kernel, dst, flag);
+}
+DH Conv2_MK_im2col(GPU_Tensor<Half>& src, GPU_TensorArray<Half>& kernel, GPU_Tensor<Half>& dst, const int flag) {
+    return conv_device<Half>(src, kernel, dst, flag);
 }
 }  // namespace cuda
 

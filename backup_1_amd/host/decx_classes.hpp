@@ -189,7 +189,7 @@ public:
         depth = d;
         _store_type = store_type;
         wpitch = ceil_to(w, 4);
-        dpitch = ceil_to(d, 4);
+        dpitch = ceil_to(d, sizeof(T) == 2 ? 8 : 4);     // _TENSOR_ALIGN_4B_ = 4, _TENSOR_ALIGN_2B_ = 8 (classes/Tensor.h:21-23)
         dp_x_wp = (size_t)dpitch * wpitch;
         element_num = (size_t)d * w * h;
         _element_num = (size_t)h * dp_x_wp;
@@ -249,7 +249,7 @@ public:
         tensor_num = n;
         _store_type = store_type;
         wpitch = ceil_to(w, 4);
-        dpitch = ceil_to(d, 4);
+        dpitch = ceil_to(d, sizeof(T) == 2 ? 8 : 4);     // _TENSOR_ALIGN_4B_ = 4, _TENSOR_ALIGN_2B_ = 8 (classes/Tensor.h:21-23)
         dp_x_wp = (size_t)dpitch * wpitch;
         _gap = dp_x_wp * h;
         element_num = (size_t)d * w * h * n;
@@ -357,7 +357,7 @@ public:
         height = h;
         depth = d;
         wpitch = ceil_to(w, 4);
-        dpitch = ceil_to(d, 4);
+        dpitch = ceil_to(d, sizeof(T) == 2 ? 8 : 4);     // _TENSOR_ALIGN_4B_ = 4, _TENSOR_ALIGN_2B_ = 8 (classes/Tensor.h:21-23)
         dp_x_wp = (size_t)dpitch * wpitch;
         element_num = (size_t)d * w * h;
         _element_num = (size_t)h * dp_x_wp;
@@ -421,7 +421,7 @@ public:
         depth = d;
         tensor_num = n;
         wpitch = ceil_to(w, 4);
-        dpitch = ceil_to(d, 4);
+        dpitch = ceil_to(d, sizeof(T) == 2 ? 8 : 4);     // _TENSOR_ALIGN_4B_ = 4, _TENSOR_ALIGN_2B_ = 8 (classes/Tensor.h:21-23)
         dp_x_wp = (size_t)dpitch * wpitch;
         _gap = dp_x_wp * h;
         element_num = (size_t)d * w * h * n;

@@ -17,6 +17,9 @@ void oracle_sgemm_chain_fast(const float* A, long lda, const float* B, long ldb,
 int oracle_conv2_chain(const float* src, int H, int W, int dpitch, long src_row_stride, const float* filt, int N, int kh,
                        int kw, long filt_stride, long filt_row_stride, float* dst, int dst_dpitch, long dst_row_stride,
                        int flag, int nthreads);
+int oracle_conv2_f64_f16(const uint16_t* src, int H, int W, int dpitch, long src_row_stride, const uint16_t* filt, int N,
+                         int kh, int kw, long filt_stride, long filt_row_stride, double* out, double* scale, int flag,
+                         int nthreads);
 void oracle_gemm_f64_rows_f16(const uint16_t* A, long lda, const uint16_t* B, long ldb, const int* rows, int nrows,
                               double* out, double* abs_out, int N, int K, int nthreads);
 }
@@ -401,6 +404,51 @@ static void conv_device_resident() {
     dsrc.release(); dker.release(); ddst.release(); src.release(); ker.release();
 }
 
+static void conv_half_containers() {
+    // binary16 containers: channel pitch ceil8 (Tensor.h:214-235), fp32 accumulation, checked against fp64 on the same halves
+    const int H = 30, W = 26, C = 12, N = 10, kh = 3, kw = 3;
+    de::Tensor<de::Half>& src = de::CreateTensorRef<de::Half>(W, H, C, 0);
+    de::TensorArray<de::Half>& ker = de::CreateTensorArrayRef<de::Half>(kw, kh, C, N, 0);
+    for (int y = 0; y < H; ++y) for (int x = 0; x < W; ++x) for (int c = 0; c < C; ++c) src.index(y, x, c) = de::Float2Half(unif());
+    for (int n = 0; n < N; ++n) for (int i = 0; i < kh; ++i) for (int j = 0; j < kw; ++j) for (int c = 0; c < C; ++c)
+        ker.index(i, j, c, n) = de::Float2Half(0.1f * unif());
+    const long dp = &src.index(0, 1, 0) - &src.index(0, 0, 0), s_row = &src.index(1, 0, 0) - &src.index(0, 0, 0);
+    const long k_gap = &ker.index(0, 0, 0, 1) - &ker.index(0, 0, 0, 0), k_row = &ker.index(1, 0, 0, 0) - &ker.index(0, 0, 0, 0);
+    CHECK(dp == 16 && s_row == 16 * 28 && k_row == 16 * 4 && k_gap == 16 * 4 * 3);
+    de::GPU_Tensor<de::Half>& dsrc = de::CreateGPUTensorRef<de::Half>(W, H, C);
+    de::GPU_TensorArray<de::Half>& dker = de::CreateGPUTensorArrayRef<de::Half>(kw, kh, C, N);
+    de::GPU_Tensor<de::Half>& ddst = de::CreateGPUTensorRef<de::Half>();
+    dsrc.Load_from_host(src); dker.Load_from_host(ker);
+    for (int flag = 0; flag < 2; ++flag) {
+        const int Ho = flag ? H : H - 2, Wo = flag ? W : W - 2;
+        std::vector<double> ref((size_t)Ho * Wo * N), scale(ref.size());
+        CHECK(oracle_conv2_f64_f16(reinterpret_cast<const uint16_t*>(&src.index(0, 0, 0)), H, W, (int)dp, s_row,
+                                   reinterpret_cast<const uint16_t*>(&ker.index(0, 0, 0, 0)), N, kh, kw, k_gap, k_row, ref.data(),
+                                   scale.data(), flag, 0) == 0);
+        de::Tensor<de::Half>& host_out = de::CreateTensorRef<de::Half>();
+        CHECK(de::cuda::Conv2_MK_im2col(src, ker, host_out, flag).error_type == decx::DECX_SUCCESS);
+        CHECK(de::cuda::Conv2_MK_im2col(dsrc, dker, ddst, flag).error_type == decx::DECX_SUCCESS);
+        CHECK(host_out.Width() == (uint)Wo && host_out.Height() == (uint)Ho && host_out.Depth() == (uint)N);
+        CHECK(ddst.Width() == (uint)Wo && ddst.Height() == (uint)Ho && ddst.Depth() == (uint)N);
+        de::Tensor<de::Half>& dev_out = de::CreateTensorRef<de::Half>(Wo, Ho, N, 0);
+        ddst.Load_to_host(dev_out);
+        double worst = 0.0;
+        bool same = true;
+        for (int y = 0; y < Ho; ++y) for (int x = 0; x < Wo; ++x) for (int n = 0; n < N; ++n) {
+            const size_t i = ((size_t)y * Wo + x) * N + n;
+            const double got = de::Half2Float(host_out.index(y, x, n));
+            const double err = (std::fabs(got - ref[i]) - std::fabs(ref[i]) / 2048.0) / (scale[i] + 1e-30);   // minus the final rounding
+            if (err > worst) worst = err;
+            same = same && host_out.index(y, x, n).val == dev_out.index(y, x, n).val;
+        }
+        CHECK(worst < 2e-3);
+        CHECK(same);                                   // host-tensor and device-resident flavours run the same kernel
+        host_out.release(); dev_out.release();
+    }
+    CHECK(de::cuda::Conv2_MK_im2col(dsrc, dker, ddst, 5).error_type == decx::DECX_FAIL_ErrorFlag);
+    dsrc.release(); dker.release(); ddst.release(); src.release(); ker.release();
+}
+
 static void conv_flavours_and_flags() {
     conv_case(20, 22, 8, 6, 3, 3, decx::de_conv_zero_compensate);
     conv_case(20, 22, 8, 6, 3, 3, decx::de_conv_no_compensate);
@@ -429,6 +477,7 @@ int main(int argc, char** argv) {
         RUN(gemm_fp16_flavours);
         RUN(conv_flavours_and_flags);
         RUN(conv_device_resident);
+        RUN(conv_half_containers);
         RUN(gemm3_matrix_arrays);
         RUN(gemm_long_lr);
         RUN(nn_relu_family);

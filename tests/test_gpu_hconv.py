@@ -101,6 +101,20 @@ def test_headline_shape_sampled(gpu, oracle):
     assert check_against_f64(oracle, got, sbuf, fb, 1) < TOL
 
 
+def test_many_pixels_take_the_tall_tile(gpu, oracle):
+    # more than two 256-pixel tiles per CU: the 256x128 tile shape of hconv_enqueue
+    H, W, C, N = 384, 400, 8, 9
+    src = workloads.normal((H, W, C), 851).astype(np.float16)
+    filt = workloads.normal((N, 3, 3, C), 852, sigma=0.2).astype(np.float16)
+    got, sbuf, fb = gpu_hconv(src, filt, 1)
+    assert check_against_f64(oracle, got, sbuf, fb, 1) < TOL
+    si = workloads.small_ints((H, W, C), 853, -2, 2).astype(np.float16)
+    fi = workloads.small_ints((N, 3, 3, C), 854, -2, 2).astype(np.float16)
+    got, sbuf, fb = gpu_hconv(si, fi, 0)
+    ref, _ = oracle.conv2_f64_f16(sbuf, fb, 0)
+    assert np.array_equal(got.astype(np.float64), ref)
+
+
 def test_error_codes(gpu):
     L = capi.lib()
     d = capi.DeviceBuffer(1 << 16)
