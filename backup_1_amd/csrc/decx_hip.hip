@@ -459,22 +459,25 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
     HalfFilters fb{filt, N, dpitch / 2, kw, (int)(filt_stride / 2), (int)(filt_row_stride / 2), (unsigned)filt_bytes};
     HalfTensorOut out{reinterpret_cast<_Float16*>(dst), Wout, dst_dpitch, dst_row_stride, reinterpret_cast<const _Float16*>(bias), relu};
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
-    // the tall tile when its workgroups still fill the chip twice over
-    const bool tall = (long)cdiv(M, 256) * cdiv(N, 128) >= 2 * cus;
+    // the tall tile (half the filter traffic per pixel) once its workgroups cover most of the chip: measured 4 % ahead at
+    // 196 tiles on 256 CUs, where the square tile has 392
+    const bool tall = (long)cdiv(M, 256) * cdiv(N, 128) >= 3 * cus / 4;
     const int bm = tall ? 256 : 128, tiles_n = cdiv(N, 128);
     const long total = (long)cdiv(M, bm) * tiles_n;
     if (total > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
-    if (tall) {
-        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hconv_tile_kernel<HconvTall>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)HconvTall::LDS_BYTES));
-        hipLaunchKernelGGL(hconv_tile_kernel<HconvTall>, dim3((unsigned)total), dim3(HconvTall::NT), HconvTall::LDS_BYTES,
-                           g_rt.stream, img, fb, out, M, N, Kw, tiles_n);
-    } else {
-        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hconv_tile_kernel<HconvSquare>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)HconvSquare::LDS_BYTES));
-        hipLaunchKernelGGL(hconv_tile_kernel<HconvSquare>, dim3((unsigned)total), dim3(HconvSquare::NT), HconvSquare::LDS_BYTES,
-                           g_rt.stream, img, fb, out, M, N, Kw, tiles_n);
-    }
+    // a K step of 64 halves inside one tap: the tap walk runs on the scalar unit (hconv_tile.hpp)
+    const bool tap_uniform = dpitch % 64 == 0;
+    auto launch = [&](auto kern, auto shape) -> hipError_t {
+        typedef decltype(shape) S;
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, out, M, N, Kw, tiles_n);
+        return hipSuccess;
+    };
+    if (tall && tap_uniform) HIP_TRY(launch(hconv_tile_kernel<HconvTall, true>, HconvTall{}));
+    else if (tall) HIP_TRY(launch(hconv_tile_kernel<HconvTall, false>, HconvTall{}));
+    else if (tap_uniform) HIP_TRY(launch(hconv_tile_kernel<HconvSquare, true>, HconvSquare{}));
+    else HIP_TRY(launch(hconv_tile_kernel<HconvSquare, false>, HconvSquare{}));
     HIP_TRY(hipGetLastError());
     return 0;
 }

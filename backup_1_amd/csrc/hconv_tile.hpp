@@ -78,7 +78,10 @@ __device__ __forceinline__ void small_divmod(int m, int d, float rcp_d, int& quo
     rem = r;
 }
 
-template <class S>
+// TAP_UNIFORM (channel pitch a multiple of 64 halves, i.e. of a K step): a K step lies inside one tap, so the walk over
+// (tap row, tap column, channel) is the same for every lane up to a constant and runs on the scalar unit; a load then
+// costs the vector unit one add (plus the column check of an image load), and a filter load nothing at all.
+template <class S, bool TAP_UNIFORM>
 __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, HalfFilters fb, HalfTensorOut out, int M, int N,
                                                            int Kw /* K in words */, int tiles_n) {
     constexpr int BM = S::BM, BN = S::BN, NT = S::NT, U = S::U, MI = S::MI, NI = S::NI;
@@ -118,11 +121,19 @@ __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, Hal
         if (n >= N) n = N - 1;
         b_base[p] = 4 * n * fb.filt_stride_w;
     }
-    TapWalk wa, wb;                                                   // position of this thread's unit: in the image, in a filter
-    wa.init(4 * q, img.dpitch_w, img.kw, img.row_stride_w);
-    wb.init(4 * q, fb.dpitch_w, fb.kw, fb.row_stride_w);
+    // position of this thread's unit in the image and in a filter; with TAP_UNIFORM the walk starts at unit 0 for all
+    // lanes (scalar registers) and the lane's own 16 q bytes are part of its base offsets
+    TapWalk wa, wb;
+    wa.init(TAP_UNIFORM ? 0 : 4 * q, img.dpitch_w, img.kw, img.row_stride_w);
+    wb.init(TAP_UNIFORM ? 0 : 4 * q, fb.dpitch_w, fb.kw, fb.row_stride_w);
     const TapStep sa = TapStep::make(S::BK / 2, img.dpitch_w, img.kw, img.row_stride_w);
     const TapStep sb = TapStep::make(S::BK / 2, fb.dpitch_w, fb.kw, fb.row_stride_w);
+    if (TAP_UNIFORM) {
+#pragma unroll
+        for (int p = 0; p < S::A_PASSES; ++p) a_base[p] += 16 * q;
+#pragma unroll
+        for (int p = 0; p < S::B_PASSES; ++p) b_base[p] += 16 * q;
+    }
 
     // LDS addresses.  Unit (row, u) of a buffer lies at row*U + (u ^ ((row / 2) % U)) (a_unit_slot); rows that are a
     // multiple of 16 apart share the swizzle term, so per lane it is one value for all staging passes and one for all
@@ -141,17 +152,32 @@ __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, Hal
     u32x4 a_stage[DEPTH][S::A_PASSES], b_stage[DEPTH][S::B_PASSES];
     auto load_stage = [&](auto set_tag) {
         constexpr int SET = decltype(set_tag)::value;
-        const bool k_ok = wa.k < Kw;                                  // a unit never straddles the end of K (K % 8 == 0 halves)
+        if constexpr (TAP_UNIFORM) {
+            // Rows above and below the image need no test: their offsets are negative or past the end of the tensor.  K
+            // is a whole number of steps here; the loads that run past it fetch something that is never used.
 #pragma unroll
-        for (int p = 0; p < S::A_PASSES; ++p) {
-            const bool inside = k_ok && (unsigned)(a_y[p] + wa.ki) < (unsigned)img.H && (unsigned)(a_x[p] + wa.kj) < (unsigned)img.W;
-            const f32x4 v = buffer_load_quad(make_rsrc(img.src, img.bytes), inside ? (unsigned)(a_base[p] + wa.off) : kOutOfRange);
-            a_stage[SET][p] = __builtin_bit_cast(u32x4, v);
-        }
+            for (int p = 0; p < S::A_PASSES; ++p) {
+                const bool inside = (unsigned)(a_x[p] + wa.kj) < (unsigned)img.W;
+                const unsigned off = inside ? (unsigned)(a_base[p] + wa.off) : kOutOfRange;
+                a_stage[SET][p] = __builtin_bit_cast(u32x4, buffer_load_quad(make_rsrc(img.src, img.bytes), off));
+            }
 #pragma unroll
-        for (int p = 0; p < S::B_PASSES; ++p) {
-            const f32x4 v = buffer_load_quad(make_rsrc(fb.filt, fb.bytes), k_ok ? (unsigned)(b_base[p] + wb.off) : kOutOfRange);
-            b_stage[SET][p] = __builtin_bit_cast(u32x4, v);
+            for (int p = 0; p < S::B_PASSES; ++p)
+                b_stage[SET][p] = __builtin_bit_cast(
+                    u32x4, __builtin_amdgcn_raw_buffer_load_b128(make_rsrc(fb.filt, fb.bytes), b_base[p], wb.off, 0));
+        } else {
+            const bool k_ok = wa.k < Kw;                              // a unit never straddles the end of K (K % 8 == 0 halves)
+#pragma unroll
+            for (int p = 0; p < S::A_PASSES; ++p) {
+                const bool inside = k_ok && (unsigned)(a_y[p] + wa.ki) < (unsigned)img.H && (unsigned)(a_x[p] + wa.kj) < (unsigned)img.W;
+                const f32x4 v = buffer_load_quad(make_rsrc(img.src, img.bytes), inside ? (unsigned)(a_base[p] + wa.off) : kOutOfRange);
+                a_stage[SET][p] = __builtin_bit_cast(u32x4, v);
+            }
+#pragma unroll
+            for (int p = 0; p < S::B_PASSES; ++p) {
+                const f32x4 v = buffer_load_quad(make_rsrc(fb.filt, fb.bytes), k_ok ? (unsigned)(b_base[p] + wb.off) : kOutOfRange);
+                b_stage[SET][p] = __builtin_bit_cast(u32x4, v);
+            }
         }
         wa.advance(sa, img.dpitch_w, img.kw);
         wb.advance(sb, fb.dpitch_w, fb.kw);

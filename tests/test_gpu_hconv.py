@@ -33,7 +33,7 @@ def check_against_f64(oracle, got16, sbuf, fb, flag, bias16=None, relu=False):
 
 
 CASES = [(20, 22, 8, 6, 3, 3), (9, 13, 3, 2, 3, 3), (16, 16, 64, 128, 3, 3), (33, 17, 24, 130, 1, 1), (12, 40, 16, 5, 5, 3),
-         (40, 12, 40, 7, 3, 5), (7, 7, 8, 1, 7, 7), (64, 48, 32, 200, 3, 3)]
+         (40, 12, 40, 7, 3, 5), (7, 7, 8, 1, 7, 7), (64, 48, 32, 200, 3, 3), (10, 12, 128, 20, 3, 3), (9, 70, 64, 3, 1, 5)]
 
 
 @pytest.mark.parametrize("flag", [1, 0])
@@ -102,7 +102,7 @@ def test_headline_shape_sampled(gpu, oracle):
 
 
 def test_many_pixels_take_the_tall_tile(gpu, oracle):
-    # more than two 256-pixel tiles per CU: the 256x128 tile shape of hconv_enqueue
+    # enough 256-pixel tiles to cover most CUs: the 256x128 tile shape of hconv_enqueue
     H, W, C, N = 384, 400, 8, 9
     src = workloads.normal((H, W, C), 851).astype(np.float16)
     filt = workloads.normal((N, 3, 3, C), 852, sigma=0.2).astype(np.float16)
