@@ -90,7 +90,9 @@ __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, Hal
     unsigned char* As = lds_raw;                              // [2][A_UNITS] units of 16 bytes
     unsigned char* Bs = lds_raw + 2 * A_BYTES;                // [2][B_UNITS]
 
-    const int bm0 = ((int)blockIdx.x / tiles_n) * BM, bn0 = ((int)blockIdx.x % tiles_n) * BN;
+    // each XCD gets one contiguous run of tiles: neighbouring tiles share their halo rows in that XCD's L2
+    const TileCoord tc = xcd_grouped_tile((int)blockIdx.x, (int)gridDim.x / tiles_n, tiles_n, 8);
+    const int bm0 = tc.tm * BM, bn0 = tc.tn * BN;
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
     const int wm0 = (wave / S::WAVES_N) * S::WM, wn0 = (wave % S::WAVES_N) * S::WN;
     const int li = lane & 31, lh = lane >> 5;
