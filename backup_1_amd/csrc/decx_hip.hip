@@ -152,6 +152,7 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 // and, for dense GEMM only, the one-wave-per-16x16-block kernel of sgemm_chain16.hpp:
 //  11:  32x32x64,  2x2 computing + 4 moving waves, two workgroups per CU -- results too small to fill the chip with tiles
 //  12:  16x16x64,  1 computing + 2 moving waves -- at most one 16x16 block per CU: the fastest a single chain can walk K
+//  13:  64x64x64,  8 computing waves of two blocks each + 4 moving waves -- results of about one such tile per CU (1024^2)
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
 typedef SgemmShape<128, 128, 16, 2, 2, 2> SShapeSmall;
 typedef SgemmShape<256, 128, 16, 2, 2, 2> SShapeTall;
@@ -225,8 +226,9 @@ int launch_sgemm_chain16(const float* A, int lda, const float* B, int ldb, const
     const long total = (long)tiles_m * tiles_n;
     if (total > 0x7fffffffL || batch.count > 65535) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
     auto kern = Cin ? sgemm_chain16_kernel<S, true> : sgemm_chain16_kernel<S, false>;
-    hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), 0, batch.stream, A, lda, B, ldb, Cin,
-                       ldc, D, ldd, M, N, K, tiles_n, relu, batch.stride_a, batch.stride_b, batch.stride_c, batch.stride_d);
+    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+    hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::LDS_BYTES, batch.stream, A, lda, B, ldb,
+                       Cin, ldc, D, ldd, M, N, K, tiles_n, relu, batch.stride_a, batch.stride_b, batch.stride_c, batch.stride_d);
     HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -240,14 +242,21 @@ int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float*
     DenseOut out{ldd, relu, aligned16(D) && ldd % 4 == 0 && batch.stride_d % 4 == 0};
     if (vec_a && vec_b) {
         // Small results go to the one-wave-per-block kernel (measured: ahead of the tiles up to about ten 32x32 tiles per
-        // CU -- 1536x1536 on 256 CUs -- whatever K is; 1.5x at 1024x8192x1024, 9x at 64x65536x1024).  All paths give
+        // CU -- 1536x1536 on 256 CUs -- whatever K is; 1.7x at 1024x8192x1024, 9x at 64x65536x1024).  All paths give
         // the same bits, so this is a choice of speed only.
         const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
         const long blocks16 = (long)cdiv(M, 16) * cdiv(N, 16) * batch.count, tiles32 = (long)cdiv(M, 32) * cdiv(N, 32) * batch.count;
-        int chain = g_rt.sgemm_variant == 11 || g_rt.sgemm_variant == 12 ? g_rt.sgemm_variant : 0;
-        if (g_rt.sgemm_variant < 1 || g_rt.sgemm_variant > 12) chain = blocks16 <= cus ? 12 : (tiles32 <= 10 * cus ? 11 : 0);
-        if (chain == 11) return launch_sgemm_chain16<Chain16<2, 4, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
-        if (chain == 12) return launch_sgemm_chain16<Chain16<1, 8, 2>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+        int chain = g_rt.sgemm_variant >= 11 && g_rt.sgemm_variant <= 13 ? g_rt.sgemm_variant : 0;
+        if (g_rt.sgemm_variant < 1 || g_rt.sgemm_variant > 13) {
+            // 32x32 tiles share a CU two at a time, 64x64 tiles take one each and cost 1.78 times a pair (measured at
+            // 1024x8192x1024: 0.153 ms for one round of 64x64 tiles, 0.171 ms for two rounds of 32x32 pairs)
+            const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch.count;
+            const double cost64 = 1.78 * (double)((tiles64 + cus - 1) / cus), pairs = (double)tiles32 / (2.0 * cus);
+            chain = blocks16 <= cus ? 12 : tiles32 > 10 * cus ? 0 : cost64 < (pairs > 1.0 ? pairs : 1.0) ? 13 : 11;
+        }
+        if (chain == 11) return launch_sgemm_chain16<Chain16<2, 1, 4, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+        if (chain == 12) return launch_sgemm_chain16<Chain16<1, 1, 8, 2>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+        if (chain == 13) return launch_sgemm_chain16<Chain16<4, 2, 2, 3>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
     }
     if (vec_a && vec_b) {
         DenseA<true> a{A, lda, M, K, batch.stride_a};

@@ -23,7 +23,10 @@
 //   T = 2: a 32x32 tile, 2x2 computing waves and four moving waves, one of each per SIMD: half the staging work per
 //          block (A and B tiles are shared) but it runs on the computing waves' SIMDs: for more blocks than CUs.  Built
 //          with 4 register sets for 128 registers, so that two workgroups share a CU and one's MFMAs fill the gaps
-//          the other's staging leaves.
+//          the other's staging leaves;
+//   T = 4: a 64x64 tile, eight computing waves of two blocks each (two chains per wave, interleaved, one set of A
+//          operands for both) and four moving waves: a quarter of the staging work per block, and four chains per SIMD
+//          keep its matrix pipe busy while one of them waits: for results of about one such tile per CU and more.
 //
 // Lane (r, s) of a computing wave feeds row r (of A) or column r (of B) of its block and k-slot s; so that its operands
 // for the 16 MFMAs of a chunk (k = 4j + s, j = 0..15) are 16 consecutive floats -- four 16-byte reads -- the chunk lies in
@@ -41,19 +44,23 @@
 
 namespace decx_hip {
 
-template <int T, int DEPTH_, int WAVES_PER_SIMD_>
+// T x T blocks of 16x16 per workgroup tile; a computing wave owns NB blocks that lie side by side (NB independent chains,
+// interleaved, sharing the A operands); DEPTH_ register sets; WAVES_PER_SIMD_ is what the register budget is cut for.
+template <int T, int NB_, int DEPTH_, int WAVES_PER_SIMD_>
 struct Chain16 {
-    static_assert(T == 1 || T == 2, "tiles of 1x1 or 2x2 blocks");
-    static constexpr int WAVES_PER_SIMD = WAVES_PER_SIMD_;           // what the register budget is cut for
-    static constexpr int BM = 16 * T, BN = 16 * T, BK = 64;
-    static constexpr int COMPUTE_WAVES = T * T, MOVE_THREADS = 128 * T;
+    static_assert((T == 1 || T == 2 || T == 4) && T % NB_ == 0, "tiles of 1x1, 2x2 or 4x4 blocks");
+    static constexpr int WAVES_PER_SIMD = WAVES_PER_SIMD_;
+    static constexpr int BM = 16 * T, BN = 16 * T, BK = 64, NB = NB_;
+    static constexpr int COMPUTE_WAVES = T * T / NB, MOVE_THREADS = T == 1 ? 128 : 256;
     static constexpr int NT = 64 * COMPUTE_WAVES + MOVE_THREADS;     // computing waves first, then the moving waves
+    static constexpr int PA = 16 * BM / MOVE_THREADS, PB = 16 * BN / MOVE_THREADS;   // quads of A and of B per moving thread and chunk
     static constexpr int DEPTH = DEPTH_;                             // register sets: chunks of K in flight from global memory (even)
     static constexpr int LINE = 20;                                  // floats per (k-slot, row or column) line in LDS: 16 + 4
     static constexpr int A_PLANE = BM * LINE, B_PLANE = BN * LINE + 4;   // floats per k-slot plane
     static constexpr int A_FLOATS = 4 * A_PLANE, B_FLOATS = 4 * B_PLANE;
     static constexpr int LDS_BUFFERS = 3;
     static constexpr size_t LDS_BYTES = LDS_BUFFERS * (size_t)(A_FLOATS + B_FLOATS) * sizeof(float);
+    static_assert(16 * BM % MOVE_THREADS == 0 && NT <= 1024, "staging divides evenly");
 };
 
 // two floats to LDS, OFF0 and OFF1 dwords past byte_addr (each below 256)
@@ -74,15 +81,14 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_chain16_kernel
                                                                     int tiles_n, bool relu, size_t a_batch_stride,
                                                                     size_t b_batch_stride, size_t c_batch_stride,
                                                                     size_t d_batch_stride) {
-    constexpr int T = S::BM / 16;
-    constexpr int DEPTH = S::DEPTH;
+    constexpr int DEPTH = S::DEPTH, NB = S::NB, PA = S::PA, PB = S::PB, Q_ALL = S::PA + S::PB;
     static_assert(DEPTH % 2 == 0 && DEPTH >= 2, "set and fragment indices repeat with period DEPTH");
     static_assert(S::A_PLANE % 64 == 0 && S::LINE == 20, "the store offsets below are written for these strides");
     A += (size_t)blockIdx.y * a_batch_stride;
     B += (size_t)blockIdx.y * b_batch_stride;
     if (HAS_C) Cin += (size_t)blockIdx.y * c_batch_stride;
     D += (size_t)blockIdx.y * d_batch_stride;
-    __shared__ __attribute__((aligned(16))) float lds[S::LDS_BUFFERS * (S::A_FLOATS + S::B_FLOATS)];
+    extern __shared__ __attribute__((aligned(16))) float lds[];      // LDS_BYTES
     float* As = lds;                                     // [3][4 slots][BM][LINE]
     float* Bs = lds + S::LDS_BUFFERS * S::A_FLOATS;      // [3][4 slots][BN][LINE] (+4 per plane)
 
@@ -96,32 +102,36 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_chain16_kernel
     // chunk, one for a ragged last chunk.
     if (wave >= S::COMPUTE_WAVES) {
         // =============================== moving waves ===============================
-        // per chunk two quads of A (row, 4 consecutive k) and two of B (k, 4 consecutive columns) per thread; quad 2p is
-        // A's, 2p + 1 is B's.  32 consecutive lanes hold, of A, 16 quads of rows r and r + 4 (banks 20 r + kq and 16
+        // per chunk PA quads of A (row, 4 consecutive k) and PB of B (k, 4 consecutive columns) per thread; quads 0 .. PA-1
+        // are A's, the rest B's.  32 consecutive lanes hold, of A, 16 quads of rows r and r + 4 (banks 20 r + kq and 16
         // further), of B, 16 consecutive k of two neighbouring column quads (banks 4 (k % 4) + k / 4 and 16 further).
         const int pt = tid - 64 * S::COMPUTE_WAVES;
-        const float* src[4];
-        unsigned dst[4];                          // LDS byte address, buffer 0, of element 0 of the quad
-        int a_k[2], b_k[2];                       // k of the quad inside its chunk (first element for A)
+        const float* src[Q_ALL];
+        unsigned dst[Q_ALL];                      // LDS byte address, buffer 0, of element 0 of the quad
+        int quad_k[Q_ALL];                        // k of the quad inside its chunk (first element for A)
 #pragma unroll
-        for (int p = 0; p < 2; ++p) {
+        for (int p = 0; p < PA; ++p) {
             const int q = pt + p * S::MOVE_THREADS, rest = q / 32;
             const int row = rest % 4 + 4 * ((q / 16) % 2) + 8 * (rest / 4), kq = q % 16;
             int m = bm0 + row;
             if (m >= M) m = M - 1;                // rows past the end are computed and never stored
-            a_k[p] = 4 * kq;
-            src[2 * p] = A + (size_t)m * lda + 4 * kq;
-            dst[2 * p] = lds_byte_address(As) + 4u * (unsigned)(row * S::LINE + kq);      // element e: plane e, j = kq
+            quad_k[p] = 4 * kq;
+            src[p] = A + (size_t)m * lda + 4 * kq;
+            dst[p] = lds_byte_address(As) + 4u * (unsigned)(row * S::LINE + kq);      // element e: plane e, j = kq
+        }
+#pragma unroll
+        for (int p = 0; p < PB; ++p) {
+            const int q = pt + p * S::MOVE_THREADS, rest = q / 32;
             const int k = 16 * (rest % 4) + q % 16, cq = 2 * (rest / 4) + (q / 16) % 2;
             int col = bn0 + 4 * cq;
             if (col > ldb - 4) col = ldb - 4;     // stay inside the pitch; such columns are never stored
-            b_k[p] = k;
-            src[2 * p + 1] = B + (size_t)k * ldb + col;
-            dst[2 * p + 1] = lds_byte_address(Bs) + 4u * (unsigned)((k % 4) * S::B_PLANE + (4 * cq) * S::LINE + k / 4);   // element e: line 4cq + e
+            quad_k[PA + p] = k;
+            src[PA + p] = B + (size_t)k * ldb + col;
+            dst[PA + p] = lds_byte_address(Bs) + 4u * (unsigned)((k % 4) * S::B_PLANE + (4 * cq) * S::LINE + k / 4);   // element e: line 4cq + e
         }
         auto store_quad = [&](const f32x4& v, auto quad_tag, int buf) {
             constexpr int Q = decltype(quad_tag)::value;
-            if constexpr (Q % 2 == 0) {
+            if constexpr (Q < PA) {
                 const unsigned addr = dst[Q] + (unsigned)buf * (S::A_FLOATS * 4u);
                 lds_write2_st64<0, S::A_PLANE / 64>(addr, v[0], v[1]);
                 lds_write2_st64<2 * S::A_PLANE / 64, 3 * S::A_PLANE / 64>(addr, v[2], v[3]);
@@ -133,44 +143,46 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_chain16_kernel
         };
 
         // the ragged last chunk, fetched first (it is the only load with per-lane conditions)
-        f32x4 tail_stage[4];
+        f32x4 tail_stage[Q_ALL];
         if (chunks > full_chunks) {
             const int k0 = full_chunks * S::BK;
 #pragma unroll
-            for (int p = 0; p < 2; ++p) {
-                f32x4 va = {0.f, 0.f, 0.f, 0.f}, vb = {0.f, 0.f, 0.f, 0.f};
-                const int ka = k0 + a_k[p], kb = k0 + b_k[p];
-                if (ka < K) {
-                    va = *reinterpret_cast<const f32x4*>(src[2 * p] + k0);       // lda % 4 == 0 keeps the quad inside the pitch
-                    if (ka + 1 >= K) va[1] = 0.f;
-                    if (ka + 2 >= K) va[2] = 0.f;
-                    if (ka + 3 >= K) va[3] = 0.f;
+            for (int p = 0; p < Q_ALL; ++p) {
+                f32x4 v = {0.f, 0.f, 0.f, 0.f};
+                const int k = k0 + quad_k[p];
+                if (k < K) {
+                    if (p < PA) {
+                        v = *reinterpret_cast<const f32x4*>(src[p] + k0);        // lda % 4 == 0 keeps the quad inside the pitch
+                        if (k + 1 >= K) v[1] = 0.f;
+                        if (k + 2 >= K) v[2] = 0.f;
+                        if (k + 3 >= K) v[3] = 0.f;
+                    } else {
+                        v = *reinterpret_cast<const f32x4*>(src[p] + (size_t)k0 * ldb);
+                    }
                 }
-                if (kb < K) vb = *reinterpret_cast<const f32x4*>(src[2 * p + 1] + (size_t)k0 * ldb);
-                tail_stage[2 * p] = va;
-                tail_stage[2 * p + 1] = vb;
+                tail_stage[p] = v;
             }
         }
 
         // DEPTH register sets: chunk x travels through set x % DEPTH, fetched DEPTH chunks ahead of its use
-        f32x4 stage[DEPTH][4];
+        f32x4 stage[DEPTH][Q_ALL];
         int fetch_chunk = 0;                      // the chunk the fetch pointers stand on
         auto fetch = [&](auto set_tag) {
             constexpr int SET = decltype(set_tag)::value;
             const bool more = fetch_chunk + 1 < full_chunks;      // the pointers stop on the last whole chunk
             const long a_step = more ? S::BK : 0, b_step = more ? (long)S::BK * ldb : 0;
             fetch_chunk += more ? 1 : 0;
-            static_for<0, 4>([&](auto q_tag) {
+            static_for<0, Q_ALL>([&](auto q_tag) {
                 constexpr int Q = decltype(q_tag)::value;
                 stage[SET][Q] = *reinterpret_cast<const f32x4*>(src[Q]);
-                src[Q] += (Q % 2 == 0) ? a_step : b_step;
+                src[Q] += Q < PA ? a_step : b_step;
             });
         };
         if (full_chunks > 0) {
             // chunks 0 .. DEPTH-1 are fetched; chunks 0 and 1 go to LDS buffers 0 and 1 and their sets are refilled
             static_for<0, DEPTH>([&](auto d) { fetch(d); });
-            static_for<0, 4>([&](auto q) { store_quad(stage[0][decltype(q)::value], q, 0); });
-            static_for<0, 4>([&](auto q) { store_quad(stage[1][decltype(q)::value], q, 1); });
+            static_for<0, Q_ALL>([&](auto q) { store_quad(stage[0][decltype(q)::value], q, 0); });
+            static_for<0, Q_ALL>([&](auto q) { store_quad(stage[1][decltype(q)::value], q, 1); });
             lds_sync();
             fetch(I0{});
             fetch(I1{});
@@ -179,7 +191,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_chain16_kernel
             int buf_store = 2;
             auto chunk = [&](auto d) {
                 constexpr int SET = (decltype(d)::value + 2) % DEPTH;
-                static_for<0, 4>([&](auto q) { store_quad(stage[SET][decltype(q)::value], q, buf_store); });
+                static_for<0, Q_ALL>([&](auto q) { store_quad(stage[SET][decltype(q)::value], q, buf_store); });
                 lds_sync();
                 fetch(std::integral_constant<int, SET>{});
                 buf_store = buf_store == 2 ? 0 : buf_store + 1;
@@ -193,46 +205,52 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_chain16_kernel
         }
         if (chunks > full_chunks) {
             // every computing wave is past the last barrier and has all its LDS reads back: any buffer is free
-            static_for<0, 4>([&](auto q) { store_quad(tail_stage[decltype(q)::value], q, 0); });
+            static_for<0, Q_ALL>([&](auto q) { store_quad(tail_stage[decltype(q)::value], q, 0); });
             lds_sync();
         }
         return;
     }
 
     // =============================== computing waves ===============================
-    const int wm0 = (wave / T) * 16, wn0 = (wave % T) * 16;
-    const int lr = lane % 16, ls = lane / 16;     // row (of A) or column (of B) inside the block, and k-slot
-    // accumulators: lane holds D[4*ls + r][lr] of its block, r = 0..3; the chain starts at C when there is one
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    const int n_out = bn0 + wn0 + lr;
-    if (HAS_C) {
+    constexpr int WAVES_N = S::BN / (16 * NB);
+    const int wm0 = (wave / WAVES_N) * 16, wn0 = (wave % WAVES_N) * 16 * NB;
+    const int lr = lane % 16, ls = lane / 16;     // row (of A) or column (of B) inside a block, and k-slot
+    // accumulators: lane holds D[4*ls + r][lr] of each of its blocks, r = 0..3; the chains start at C when there is one
+    f32x4 acc[NB];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int m = bm0 + wm0 + 4 * ls + r;
-            if (m < M && n_out < N) acc[r] = Cin[(size_t)m * ldc + n_out];
+    for (int b = 0; b < NB; ++b) {
+        acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const int n_out = bn0 + wn0 + 16 * b + lr;
+        if (HAS_C) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = bm0 + wm0 + 4 * ls + r;
+                if (m < M && n_out < N) acc[b][r] = Cin[(size_t)m * ldc + n_out];
+            }
         }
     }
     const float* a_frag = As + ls * S::A_PLANE + (wm0 + lr) * S::LINE;       // this lane's 16 operands of a chunk, buffer 0
-    const float* b_frag = Bs + ls * S::B_PLANE + (wn0 + lr) * S::LINE;
-    f32x4 av[2][4], bv[2][4];
-    // read R (0..3: A, 4..7: B) of the eight 16-byte operand reads of a chunk in LDS buffer buf, into fragment set F
+    const float* b_frag = Bs + ls * S::B_PLANE + (wn0 + lr) * S::LINE;       // block b: 16 lines further per block
+    f32x4 av[2][4], bv[2][NB][4];
+    constexpr int READS = 4 + 4 * NB;             // 16-byte operand reads per chunk: 4 of A, then 4 per block of B
     auto read_one = [&](auto f_tag, auto r_tag, int buf) {
         constexpr int F = decltype(f_tag)::value, R = decltype(r_tag)::value;
         if constexpr (R < 4) av[F][R] = reinterpret_cast<const f32x4*>(a_frag + buf * S::A_FLOATS)[R];
-        else bv[F][R - 4] = reinterpret_cast<const f32x4*>(b_frag + buf * S::B_FLOATS)[R - 4];
+        else bv[F][(R - 4) / 4][(R - 4) % 4] = reinterpret_cast<const f32x4*>(b_frag + buf * S::B_FLOATS + ((R - 4) / 4) * 16 * S::LINE)[(R - 4) % 4];
     };
     if (full_chunks > 0) {
         lds_sync();
-        static_for<0, 8>([&](auto r) { read_one(I0{}, r, 0); });
-        // chunk c: its operands are in fragment set c % 2; buffer (c+1) % 3 holds chunk c+1 since the previous barrier
+        static_for<0, READS>([&](auto r) { read_one(I0{}, r, 0); });
+        // chunk c: its operands are in fragment set c % 2; buffer (c+1) % 3 holds chunk c+1 since the previous barrier.
+        // The NB chains advance in turn; behind each of the first READS MFMAs goes one read of the next chunk's operands.
         int buf_next = 1;
         auto chunk = [&](auto d) {
             constexpr int NOW = decltype(d)::value & 1;
             typedef std::integral_constant<int, NOW ^ 1> Next;
-            static_for<0, 16>([&](auto j_tag) {
-                constexpr int J = decltype(j_tag)::value;
-                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[NOW][J / 4][J % 4], bv[NOW][J / 4][J % 4], acc, 0, 0, 0);
-                if constexpr (J < 8) read_one(Next{}, j_tag, buf_next);
+            static_for<0, 16 * NB>([&](auto i_tag) {
+                constexpr int I = decltype(i_tag)::value, J = I / NB, BLK = I % NB;
+                acc[BLK] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[NOW][J / 4][J % 4], bv[NOW][BLK][J / 4][J % 4], acc[BLK], 0, 0, 0);
+                if constexpr (I < READS) read_one(Next{}, i_tag, buf_next);
                 __builtin_amdgcn_sched_barrier(0);
             });
             lds_sync();
@@ -247,14 +265,21 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_chain16_kernel
     }
     if (chunks > full_chunks) {
         lds_sync();
-        static_for<0, 8>([&](auto r) { read_one(I0{}, r, 0); });
+        static_for<0, READS>([&](auto r) { read_one(I0{}, r, 0); });
 #pragma unroll
-        for (int j = 0; j < 16; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av[0][j / 4][j % 4], bv[0][j / 4][j % 4], acc, 0, 0, 0);
+        for (int j = 0; j < 16; ++j)
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+                acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[0][j / 4][j % 4], bv[0][b][j / 4][j % 4], acc[b], 0, 0, 0);
     }
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int m = bm0 + wm0 + 4 * ls + r;
-        if (m < M && n_out < N) D[(size_t)m * ldd + n_out] = relu ? relu_by_sign(acc[r]) : acc[r];
+    for (int b = 0; b < NB; ++b) {
+        const int n_out = bn0 + wn0 + 16 * b + lr;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int m = bm0 + wm0 + 4 * ls + r;
+            if (m < M && n_out < N) D[(size_t)m * ldd + n_out] = relu ? relu_by_sign(acc[b][r]) : acc[b][r];
+        }
     }
 }
 

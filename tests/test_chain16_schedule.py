@@ -9,7 +9,7 @@ import os
 import pytest
 
 BK = 64                    # Chain16::BK
-DEPTHS = (4, 8)            # Chain16::DEPTH of the two shapes that are built
+DEPTHS = (2, 4, 8)           # Chain16::DEPTH of the two shapes that are built
 
 
 def replay(K, DEPTH):
@@ -72,4 +72,4 @@ def test_kernel_source_has_the_modelled_constants_and_bounds():
     assert "BK = 64" in src and "LDS_BUFFERS = 3" in src
     assert "fetch_chunk + 1 < full_chunks" in src and "c0 + DEPTH <= full_chunks" in src
     launches = open(os.path.join(csrc, "decx_hip.hip")).read()
-    assert "Chain16<2, 4, 4>" in launches and "Chain16<1, 8, 2>" in launches
+    assert "Chain16<2, 1, 4, 4>" in launches and "Chain16<1, 1, 8, 2>" in launches and "Chain16<4, 2, 2, 3>" in launches
