@@ -12,7 +12,9 @@ chain_vectors.npz
     answer, closed forms and an exact-rational model of the fused chain.  They freeze the pinned arithmetic as data, so
     that the GPU tests can compare bit patterns without the oracle and a later change to the oracle cannot go unnoticed:
       gemm_*   37x53 times 53x29 (+ C), normal(0,1);  conv_*  9x11x6 tensor, 5 filters 3x5x6, both border modes;
-      relu_*   special values through forward / record / backward;  half_*  float -> binary16 -> float.
+      relu_*   special values through forward / record / backward;  half_*  float -> binary16 -> float;
+      hconv_*  10x13x8 binary16 tensor, 6 filters 3x3x8 (bit patterns), with the fp64 sums of products and of their
+               absolute values in both border modes;  hgemm_*  33x40 times 40x21 binary16 with fp64 products likewise.
 """
 import json
 import os
@@ -65,6 +67,15 @@ def main():
     v["half_in"] = h
     v["half_bits"] = oracle.float_to_half(h)
     v["half_back"] = oracle.half_to_float(v["half_bits"])
+    hs = workloads.uniform_01((10, 13, 8), 9008).astype(np.float16)
+    hf = workloads.normal((6, 3, 3, 8), 9009, sigma=0.25).astype(np.float16)
+    v["hconv_src_bits"], v["hconv_filt_bits"] = hs.view(np.uint16), hf.view(np.uint16)
+    v["hconv_same_f64"], v["hconv_same_abs"] = oracle.conv2_f64_f16(v["hconv_src_bits"], v["hconv_filt_bits"], 1)
+    v["hconv_valid_f64"], v["hconv_valid_abs"] = oracle.conv2_f64_f16(v["hconv_src_bits"], v["hconv_filt_bits"], 0)
+    ha = oracle.float_to_half(workloads.uniform_pm1((33, 40), 9010))
+    hb = oracle.float_to_half(workloads.uniform_pm1((40, 21), 9011))
+    v["hgemm_A_bits"], v["hgemm_B_bits"] = ha, hb
+    v["hgemm_f64"], v["hgemm_abs"] = oracle.gemm_f64_rows_f16(ha, hb, np.arange(33, dtype=np.int32))
     np.savez(os.path.join(HERE, "chain_vectors.npz"), **v)
     print("wrote reference_known_answer.json and chain_vectors.npz (%d arrays)" % len(v))
 

@@ -386,3 +386,8 @@ def test_oracle_reproduces_the_frozen_vectors(oracle):
     with np.errstate(over="ignore"):          # 65520 rounds to +inf, as it must
         assert np.array_equal(v["half_bits"], v["half_in"].astype(np.float16).view(np.uint16))  # numpy's own RNE agrees
     assert same(oracle.half_to_float(v["half_bits"]), v["half_back"])
+    for flag, name in ((1, "same"), (0, "valid")):
+        out, scale = oracle.conv2_f64_f16(v["hconv_src_bits"], v["hconv_filt_bits"], flag)
+        assert np.array_equal(out, v["hconv_%s_f64" % name]) and np.array_equal(scale, v["hconv_%s_abs" % name])
+    out, scale = oracle.gemm_f64_rows_f16(v["hgemm_A_bits"], v["hgemm_B_bits"], np.arange(33, dtype=np.int32))
+    assert np.array_equal(out, v["hgemm_f64"]) and np.array_equal(scale, v["hgemm_abs"])
