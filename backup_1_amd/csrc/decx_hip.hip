@@ -226,7 +226,14 @@ int launch_sgemm_chain16(const float* A, int lda, const float* B, int ldb, const
     const long total = (long)tiles_m * tiles_n;
     if (total > 0x7fffffffL || batch.count > 65535) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
     auto kern = Cin ? sgemm_chain16_kernel<S, true> : sgemm_chain16_kernel<S, false>;
-    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+    static bool attr_done = false;
+    if (!attr_done) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(sgemm_chain16_kernel<S, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(sgemm_chain16_kernel<S, false>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+        attr_done = true;
+    }
     hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::LDS_BYTES, batch.stream, A, lda, B, ldb,
                        Cin, ldc, D, ldd, M, N, K, tiles_n, relu, batch.stride_a, batch.stride_b, batch.stride_c, batch.stride_d);
     HIP_TRY(hipGetLastError());
@@ -476,17 +483,23 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
     if (total > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
     // a K step of 64 halves inside one tap: the tap walk runs on the scalar unit (hconv_tile.hpp)
     const bool tap_uniform = dpitch % 64 == 0;
-    auto launch = [&](auto kern, auto shape) -> hipError_t {
+    static bool attr_done = false;
+    if (!attr_done) {
+        auto allow = [](const void* kern, size_t bytes) { return hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes); };
+        HIP_TRY(allow(reinterpret_cast<const void*>(hconv_tile_kernel<HconvTall, true>), HconvTall::LDS_BYTES));
+        HIP_TRY(allow(reinterpret_cast<const void*>(hconv_tile_kernel<HconvTall, false>), HconvTall::LDS_BYTES));
+        HIP_TRY(allow(reinterpret_cast<const void*>(hconv_tile_kernel<HconvSquare, true>), HconvSquare::LDS_BYTES));
+        HIP_TRY(allow(reinterpret_cast<const void*>(hconv_tile_kernel<HconvSquare, false>), HconvSquare::LDS_BYTES));
+        attr_done = true;
+    }
+    auto launch = [&](auto kern, auto shape) {
         typedef decltype(shape) S;
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES);
-        if (e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, out, M, N, Kw, tiles_n);
-        return hipSuccess;
     };
-    if (tall && tap_uniform) HIP_TRY(launch(hconv_tile_kernel<HconvTall, true>, HconvTall{}));
-    else if (tall) HIP_TRY(launch(hconv_tile_kernel<HconvTall, false>, HconvTall{}));
-    else if (tap_uniform) HIP_TRY(launch(hconv_tile_kernel<HconvSquare, true>, HconvSquare{}));
-    else HIP_TRY(launch(hconv_tile_kernel<HconvSquare, false>, HconvSquare{}));
+    if (tall && tap_uniform) launch(hconv_tile_kernel<HconvTall, true>, HconvTall{});
+    else if (tall) launch(hconv_tile_kernel<HconvTall, false>, HconvTall{});
+    else if (tap_uniform) launch(hconv_tile_kernel<HconvSquare, true>, HconvSquare{});
+    else launch(hconv_tile_kernel<HconvSquare, false>, HconvSquare{});
     HIP_TRY(hipGetLastError());
     return 0;
 }
