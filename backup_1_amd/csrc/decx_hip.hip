@@ -331,6 +331,11 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
     const int variant = pick_sgemm_variant(M, N, K, 1);
     const int oy = flag ? kh / 2 : 0, ox = flag ? kw / 2 : 0;
     // a bias is the "+ C" operand with row stride 0: every output pixel adds the same N values
+    if (dpitch % 16 == 0) {      // a whole K step inside one tap: the tap walk runs on the scalar unit
+        Im2colAUniform a{{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes}};
+        FilterBUniform b{{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes}};
+        return dispatch_sgemm(variant, a, b, bias, 0, dst, out, M, N, K, one);
+    }
     if (dpitch % 8 == 0) {       // the 8 consecutive k of a staging task never straddle a tap
         Im2colA<true> a{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
         FilterB<true> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};

@@ -251,6 +251,32 @@ struct Im2colA {
     }
 };
 
+// Im2colA for a channel pitch that is a multiple of the K step (16 floats): a K step then lies inside one tap, so the
+// walk over (tap row, tap column, channel) is the same for every lane up to the lane's own 0 or 8 floats and runs on
+// the scalar unit.  Rows above and below the image need no test -- their offsets are negative or past the end of the
+// tensor, and the buffer answers those with zeros -- which leaves one column test per task on the vector unit.
+struct Im2colAUniform : Im2colA<true> {
+    struct KState {
+        TapWalk walk;          // of the K step's first float; held in scalar registers
+        int lane_bytes;        // this lane's offset inside the step
+    };
+    __device__ __forceinline__ KState k_state(int k) const {
+        KState ks;
+        const int lane_k = k & 15;
+        ks.walk.init(__builtin_amdgcn_readfirstlane(k - lane_k), dpitch, kw, row_stride);
+        ks.lane_bytes = 4 * lane_k;
+        return ks;
+    }
+    __device__ __forceinline__ void advance(KState& ks, const KStep& st) const { ks.walk.advance(st, dpitch, kw); }
+    template <bool TAIL>
+    __device__ __forceinline__ void load_pair(const RowState& rs, const KState& ks, const KStep&, f32x4& lo, f32x4& hi) const {
+        const bool inside = (unsigned)(rs.x + ks.walk.kj) < (unsigned)W && (!TAIL || ks.walk.k < K);
+        const unsigned o = inside ? (unsigned)(rs.base + ks.lane_bytes + ks.walk.off) : kOutOfRange;
+        lo = buffer_load_quad(make_rsrc(src, bytes), o);
+        hi = buffer_load_quad(make_rsrc(src, bytes), o + 16u);
+    }
+};
+
 // ReLU exactly as the reference's element-wise kernel computes it (nn/operators/ReLU.h:57-82): the value times
 // float(sign bit clear).  Hence a negative input gives -0.0f, -inf gives NaN, NaN stays NaN.
 __device__ __forceinline__ float relu_by_sign(float v) {
@@ -475,6 +501,31 @@ struct FilterB {
     }
     template <class S>
     __device__ __forceinline__ static int strip_col(int ni, int li) { return 32 * ni + li; }
+};
+
+// FilterB for a channel pitch that is a multiple of the K step, the companion of Im2colAUniform: the walk runs on the
+// scalar unit and enters each load as its scalar offset; the lane's own share (its filter, its 0 or 8 floats inside
+// the step) is a constant vector offset.  A filter load then costs the vector unit nothing.
+struct FilterBUniform : FilterB<true> {
+    template <class S>
+    __device__ __forceinline__ KStateT<tasks<S>()> k_state(int tid, int k_begin, int bn0, const float* lds_buf0) const {
+        constexpr int G = S::KQ / 2;
+        KStateT<tasks<S>()> ks = FilterB<true>::template k_state<S>(tid, k_begin, bn0, lds_buf0);
+        ks.walk.init(__builtin_amdgcn_readfirstlane(k_begin), dpitch, kw, filt_row_stride);
+#pragma unroll
+        for (int j = 0; j < tasks<S>(); ++j) ks.filter_base[j] += 32 * (tid % G);
+        return ks;
+    }
+    template <class S, bool TAIL, class KS>
+    __device__ __forceinline__ void load(f32x4* st, int tid, const KS& ks, int bn0, const KStep&) const {
+        const bool ok = !TAIL || ks.walk.k < K;
+#pragma unroll
+        for (int j = 0; j < tasks<S>(); ++j) {
+            const int v = ok ? ks.filter_base[j] : (int)kOutOfRange;
+            st[2 * j] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(make_rsrc(filt, bytes), v, ks.walk.off, 0));
+            st[2 * j + 1] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(make_rsrc(filt, bytes), v + 16, ks.walk.off, 0));
+        }
+    }
 };
 
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int WAVES_PER_SIMD_ = 1,
