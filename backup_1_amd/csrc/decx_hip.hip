@@ -28,6 +28,8 @@ struct Runtime {
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     int sgemm_variant = 0;
     int hgemm_variant = 0;
+    float* partial = nullptr;      // fp32 workspace of the fp16 split-K path, grown on demand, kept until the process ends
+    size_t partial_bytes = 0;
     int group_m = 8;   // tile-rows per raster group of the XCD-aware tile walk (env DECX_HIP_GROUP_M overrides, for tuning)
 };
 Runtime g_rt;
@@ -389,7 +391,8 @@ int launch_hgemm_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb, co
     hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::LDS_BYTES, batch.stream,
                        reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
                        reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N, K,
-                       tiles_m, tiles_n, group_m, batch.stride_a, batch.stride_b, batch.stride_c, batch.stride_d);
+                       tiles_m, tiles_n, group_m, batch.stride_a, batch.stride_b, batch.stride_c, batch.stride_d,
+                       static_cast<float*>(nullptr), 0);
     HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -418,6 +421,48 @@ int launch_hgemm_dma_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb
     return 0;
 }
 
+// fp16 GEMM whose result has too few tiles to fill the chip while K is long: K is cut into ranges that run as separate
+// workgroups (blockIdx.z) and add their fp32 partial sums to a workspace with atomics; a second kernel adds C and
+// rounds to binary16 once.  fp32 sums in no fixed order: the result can differ in its last bit from run to run, inside
+// the 2e-3 rule of the fp16 path.  (fp32 GEMM never does this: its results are bit-exact chains.)
+int hgemm_splitk_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
+                         int ldd, int M, int N, int K, int splits, hipStream_t stream) {
+    typedef HShapeSmall S;
+    const size_t need = (size_t)M * N * sizeof(float);
+    if (need > g_rt.partial_bytes) {
+        HIP_TRY(hipDeviceSynchronize());           // earlier launches may still use the old workspace
+        if (g_rt.partial) HIP_TRY(hipFree(g_rt.partial));
+        g_rt.partial = nullptr;
+        g_rt.partial_bytes = 0;
+        if (hipMalloc(&g_rt.partial, need) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(DECX_HIP_FAIL_ALLOCATION, "Fail to allocate memory\n");
+        }
+        g_rt.partial_bytes = need;
+    }
+    auto kern = hgemm_tile_kernel<S, true, true>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+        attr_done = true;
+    }
+    const size_t total = (size_t)M * N;
+    const unsigned fill_blocks = (unsigned)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+    hipLaunchKernelGGL(zero_region_kernel, dim3(fill_blocks), dim3(256), 0, stream, g_rt.partial, N, M, N);
+    const int k_split_len = cdiv(cdiv(K, splits), S::BK) * S::BK;
+    splits = cdiv(K, k_split_len);                                                        // no empty range
+    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)splits), dim3(S::NT), S::LDS_BYTES, stream,
+                       reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
+                       static_cast<const _Float16*>(nullptr), 0, reinterpret_cast<_Float16*>(D), ldd, M, N, K, tiles_m, tiles_n,
+                       group_m, (size_t)0, (size_t)0, (size_t)0, (size_t)0, g_rt.partial, k_split_len);
+    hipLaunchKernelGGL(hgemm_split_finish_kernel, dim3(fill_blocks), dim3(256), 0, stream, g_rt.partial,
+                       reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                   int ldd, int M, int N, int K, const Batch& batch) {
     if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
@@ -425,6 +470,22 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
                      batch.stride_b % 8 == 0;
     if (!vec) return launch_hgemm_tile<HShapeSmall, false>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     int variant = g_rt.hgemm_variant;
+    {
+        // few 128x128 tiles and a long K: split K (variant 11 forces it, any other fixed variant switches it off).
+        // Measured: an unsplit tile walks K at 6.7 ns per k; the split path costs 15 us (zero fill, finishing kernel,
+        // atomics) plus 45 ns per k of a range, its register-staged tile being the slower kernel.
+        const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+        const long tiles = (long)cdiv(M, 128) * cdiv(N, 128);
+        long splits = (2 * cus + tiles - 1) / tiles;
+        if (splits > K / 512) splits = K / 512;                        // at least 16 K steps per range
+        if (splits >= 2 && batch.count == 1 && (size_t)M * N <= ((size_t)1 << 26)) {
+            const double t_whole = 0.0067 * K * (double)((tiles + cus - 1) / cus);
+            const double t_split = 15.0 + 0.045 * ((double)K / splits) * (double)((tiles * splits + 2 * cus - 1) / (2 * cus));
+            if (variant == 11 || ((variant < 1 || variant > 11) && t_split < 0.8 * t_whole))
+                return hgemm_splitk_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, (int)splits, batch.stream);
+        }
+        if (variant == 11) variant = 0;
+    }
     if (variant < 1 || variant > 10) {
         // same cost model as the fp32 picker: rounds of tiles per CU x tile area / measured shape efficiency
         const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;

@@ -91,7 +91,11 @@ int decx_hip_sgemm_async(const float* A, int lda, const float* B, int ldb, const
  * Operands and result are IEEE binary16 bit patterns (de::Half{unsigned short val}, classes/classes_util.h:58-63).
  * Products are accumulated in fp32 and rounded to binary16 (nearest even) once, on store; the reference accumulates
  * in binary16 (GEMM_kernel_def.cuh:100-121), which this library deliberately does not reproduce.
- * Fast path needs A, B 16-byte aligned with lda, ldb multiples of 8 (DECX pitch is a multiple of 16 halves). */
+ * Fast path needs A, B 16-byte aligned with lda, ldb multiples of 8 (DECX pitch is a multiple of 16 halves).
+ * Results with very few 128x128 tiles and a long K (say 64 x 65536 x 1024) are computed by K ranges in parallel, whose
+ * fp32 partial sums meet in a workspace the library allocates on first use (M*N floats, kept for later calls; growing
+ * it synchronises the device) and are rounded to binary16 once: the order of the additions is not fixed, so such a
+ * result can differ in its last bit from run to run (never on integer-valued data), within the tolerance above. */
 int decx_hip_hgemm_f32acc(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                           int ldd, int M, int N, int K);
 int decx_hip_hgemm_f32acc_async(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,

@@ -57,6 +57,28 @@ def test_a_times_b_plus_c(gpu):
         assert np.array_equal(gpu_hgemm(to_bits(A), to_bits(B), to_bits(C), variant=variant), want)
 
 
+@pytest.mark.parametrize("shape", [(64, 4096, 200), (40, 20000, 130), (130, 2048, 257), (16, 65536, 64)])
+def test_split_k_for_few_tiles_and_long_k(gpu, oracle, shape):
+    # few 128x128 tiles and K >= 2048: K ranges as separate workgroups, fp32 partial sums in a workspace, one rounding at
+    # the end (variant 0 chooses it, 11 forces it).  Integer data: every partial sum is exact, so the result is the exact
+    # product rounded once, whatever the order; real data: within the fp16 rule against fp64.
+    M, K, N = shape
+    A, B = workloads.small_ints((M, K), 31, -1, 1), workloads.small_ints((K, N), 32, -1, 1)
+    C = workloads.small_ints((M, N), 33, -20, 20)
+    with np.errstate(over="ignore"):
+        want = (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float16).view(np.uint16)
+        want_c = (A.astype(np.float64) @ B.astype(np.float64) + C).astype(np.float16).view(np.uint16)
+    for variant in (0, 11):
+        assert np.array_equal(gpu_hgemm(to_bits(A), to_bits(B), variant=variant), want)
+        assert np.array_equal(gpu_hgemm(to_bits(A), to_bits(B), to_bits(C), variant=variant), want_c)
+    Ar, Br = to_bits(workloads.uniform_pm1((M, K), 34)), to_bits(workloads.uniform_pm1((K, N), 35))
+    rows = np.arange(0, M, 3, dtype=np.int32)
+    ref, scale = oracle.gemm_f64_rows_f16(Ar, Br, rows)
+    for variant in (0, 11, 2):
+        got = from_bits(gpu_hgemm(Ar, Br, variant=variant))[rows]
+        assert np.max((np.abs(got - ref) - np.abs(ref) / 2048.0) / scale) < TOL, variant
+
+
 def test_rounding_to_half_is_nearest_even(gpu):
     # single products that are exact in fp32 and lie exactly half-way between two binary16 numbers
     A = np.array([[683.0], [293.0], [439.0]], dtype=np.float32)
