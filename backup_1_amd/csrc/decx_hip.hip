@@ -363,6 +363,7 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
 //   6: as 4 with 4x2 waves of 64x128 (two waves per SIMD)
 //   7: as 4 with 2x4 waves of 128x64 (two waves per SIMD) -- the default for large problems: the chip is power-capped on
 //      this kernel (MFMA busy x clock stays ~1.27 GHz-equivalents whatever the schedule), and this one is 1 % ahead
+//  11: split-K on shape 2 through an fp32 workspace (hgemm_splitk_enqueue) -- few tiles and a long K
 typedef HgemmShape<256, 256, 32, 2, 2> HShapeBig;
 typedef HgemmShape<128, 128, 32, 2, 2> HShapeSmall;
 typedef HgemmDmaShape<256, 256, 32, 2, 2, 4> HShapeDma;
