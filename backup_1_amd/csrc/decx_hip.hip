@@ -363,7 +363,7 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
 //   6: as 4 with 4x2 waves of 64x128 (two waves per SIMD)
 //   7: as 4 with 2x4 waves of 128x64 (two waves per SIMD) -- the default for large problems: the chip is power-capped on
 //      this kernel (MFMA busy x clock stays ~1.27 GHz-equivalents whatever the schedule), and this one is 1 % ahead
-//  11: split-K on shape 2 through an fp32 workspace (hgemm_splitk_enqueue) -- few tiles and a long K
+//  11: split-K on shape 8 through an fp32 workspace (hgemm_splitk_enqueue) -- few tiles and a long K
 typedef HgemmShape<256, 256, 32, 2, 2> HShapeBig;
 typedef HgemmShape<128, 128, 32, 2, 2> HShapeSmall;
 typedef HgemmDmaShape<256, 256, 32, 2, 2, 4> HShapeDma;
@@ -392,8 +392,7 @@ int launch_hgemm_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb, co
     hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::LDS_BYTES, batch.stream,
                        reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
                        reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N, K,
-                       tiles_m, tiles_n, group_m, batch.stride_a, batch.stride_b, batch.stride_c, batch.stride_d,
-                       static_cast<float*>(nullptr), 0);
+                       tiles_m, tiles_n, group_m, batch.stride_a, batch.stride_b, batch.stride_c, batch.stride_d);
     HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -417,7 +416,8 @@ int launch_hgemm_dma_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb
     hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::LDS_BYTES, batch.stream,
                        reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
                        reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N, K,
-                       tiles_m, tiles_n, group_m, batch.stride_a, batch.stride_b, batch.stride_c, batch.stride_d);
+                       tiles_m, tiles_n, group_m, batch.stride_a, batch.stride_b, batch.stride_c, batch.stride_d,
+                       static_cast<float*>(nullptr), 0);
     HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -428,7 +428,7 @@ int launch_hgemm_dma_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb
 // the 2e-3 rule of the fp16 path.  (fp32 GEMM never does this: its results are bit-exact chains.)
 int hgemm_splitk_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                          int ldd, int M, int N, int K, int splits, hipStream_t stream) {
-    typedef HShapeSmall S;
+    typedef HShapeDmaSmall S;                      // 128x128x64, LDS-DMA staged, two workgroups per CU
     const size_t need = (size_t)M * N * sizeof(float);
     if (need > g_rt.partial_bytes) {
         HIP_TRY(hipDeviceSynchronize());           // earlier launches may still use the old workspace
@@ -441,7 +441,7 @@ int hgemm_splitk_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb,
         }
         g_rt.partial_bytes = need;
     }
-    auto kern = hgemm_tile_kernel<S, true, true>;
+    auto kern = hgemm_dma_kernel<S, false, true>;
     static bool attr_done = false;
     if (!attr_done) {
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
@@ -473,16 +473,18 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
     int variant = g_rt.hgemm_variant;
     {
         // few 128x128 tiles and a long K: split K (variant 11 forces it, any other fixed variant switches it off).
-        // Measured: an unsplit tile walks K at 6.7 ns per k; the split path costs 15 us (zero fill, finishing kernel,
-        // atomics) plus 45 ns per k of a range, its register-staged tile being the slower kernel.
+        // Measured, in us: a tile walks K at 6.7 ns per k (1.6 times that when two workgroups share a CU); a launch costs
+        // about 4, the zero fill and the finishing kernel 9 together, an atomic add to the workspace 3.1 ps.
         const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
         const long tiles = (long)cdiv(M, 128) * cdiv(N, 128);
         long splits = (2 * cus + tiles - 1) / tiles;
-        if (splits > K / 512) splits = K / 512;                        // at least 16 K steps per range
+        if (splits > K / 512) splits = K / 512;                        // at least 8 K steps per range
         if (splits >= 2 && batch.count == 1 && (size_t)M * N <= ((size_t)1 << 26)) {
-            const double t_whole = 0.0067 * K * (double)((tiles + cus - 1) / cus);
-            const double t_split = 15.0 + 0.045 * ((double)K / splits) * (double)((tiles * splits + 2 * cus - 1) / (2 * cus));
-            if (variant == 11 || ((variant < 1 || variant > 11) && t_split < 0.8 * t_whole))
+            const double t_whole = 4.0 + 0.0067 * K * (double)((tiles + cus - 1) / cus);
+            const double share = tiles * splits > cus ? 1.6 : 1.0;
+            const double t_split = 9.0 + 3.1e-6 * M * N * splits +
+                                   0.0067 * ((double)K / splits) * share * (double)((tiles * splits + 2 * cus - 1) / (2 * cus));
+            if (variant == 11 || ((variant < 1 || variant > 11) && t_split < 0.85 * t_whole))
                 return hgemm_splitk_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, (int)splits, batch.stream);
         }
         if (variant == 11) variant = 0;

@@ -50,19 +50,29 @@ __device__ __forceinline__ void wait_dma_then_barrier() {
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" : : "n"(N) : "memory");
 }
 
-template <class S, bool HAS_C>
+// SPLIT_K: blockIdx.z selects a range of K (k_split_len long, a multiple of BK); the tile's fp32 partial sums are added
+// with atomics to a dense M x N fp32 workspace `partial` (zeroed beforehand) instead of being rounded and stored.
+template <class S, bool HAS_C, bool SPLIT_K = false>
 __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __restrict__ A, int lda,
                                                           const _Float16* __restrict__ B, int ldb, const _Float16* Cin,
                                                           int ldc, _Float16* D, int ldd, int M, int N, int K, int tiles_m,
                                                           int tiles_n, int group_m, size_t a_batch_stride,
-                                                          size_t b_batch_stride, size_t c_batch_stride, size_t d_batch_stride) {
+                                                          size_t b_batch_stride, size_t c_batch_stride, size_t d_batch_stride,
+                                                          float* partial, int k_split_len) {
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, NT = S::NT, UA = S::UA, UB = S::UB, MI = S::MI, NI = S::NI;
     constexpr int STAGES = S::STAGES;
+    static_assert(!(SPLIT_K && HAS_C), "C joins a split product in the finishing kernel");
     // blockIdx.y walks a batch of independent problems of the same shape
     A += (size_t)blockIdx.y * a_batch_stride;
     B += (size_t)blockIdx.y * b_batch_stride;
     if (HAS_C) Cin += (size_t)blockIdx.y * c_batch_stride;
     D += (size_t)blockIdx.y * d_batch_stride;
+    if (SPLIT_K) {
+        const int k_begin = (int)blockIdx.z * k_split_len;
+        A += k_begin;                             // a multiple of BK halves: rows keep their 16-byte alignment
+        B += (size_t)k_begin * ldb;
+        K = K - k_begin < k_split_len ? K - k_begin : k_split_len;
+    }
     constexpr int KS = BK / 16;                                // MFMA k-blocks per K step
     constexpr int BLK = MI * NI;                               // MFMAs per k-block
     static_assert(KS >= 2, "the schedule below needs at least two k-blocks per K step");
@@ -317,6 +327,22 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
     }
 #undef DECX_PIN
 
+    if (SPLIT_K) {
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                if (m < M) {
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni) {
+                        const int n = bn0 + wn0 + ni * 32 + li;
+                        if (n < N) unsafeAtomicAdd(partial + (size_t)m * N + n, acc[mi][ni][r]);
+                    }
+                }
+            }
+        return;
+    }
     // ---- epilogue: round once to binary16; dst = A*B + C adds C (as fp32) first ---------------------------------------
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)

@@ -38,28 +38,17 @@ struct HgemmShape {
 __device__ __forceinline__ int a_unit_slot(int m, int q, int UA) { return m * UA + (q ^ ((m / (16 / UA)) % UA)); }
 __device__ __forceinline__ int b_unit_slot(int k, int u, int UB) { return k * UB + (u ^ ((k & 3) << 2)); }
 
-// SPLIT_K: blockIdx.z selects a range of K (k_split_len long, a multiple of BK); the tile's fp32 partial sums are
-// added with atomics to a dense M x N fp32 workspace `partial` (zeroed beforehand) instead of being rounded and stored;
-// hgemm_split_finish_kernel turns the workspace into the binary16 result.
-template <class S, bool VEC, bool SPLIT_K = false>
+template <class S, bool VEC>
 __global__ __launch_bounds__(S::NT) void hgemm_tile_kernel(const _Float16* __restrict__ A, int lda,
                                                            const _Float16* __restrict__ B, int ldb, const _Float16* Cin,
                                                            int ldc, _Float16* D, int ldd, int M, int N, int K,
                                                            int tiles_m, int tiles_n, int group_m, size_t a_batch_stride,
-                                                           size_t b_batch_stride, size_t c_batch_stride, size_t d_batch_stride,
-                                                           float* partial = nullptr, int k_split_len = 0) {
+                                                           size_t b_batch_stride, size_t c_batch_stride, size_t d_batch_stride) {
     // blockIdx.y walks a batch of independent problems of the same shape
     A += (size_t)blockIdx.y * a_batch_stride;
     B += (size_t)blockIdx.y * b_batch_stride;
     if (Cin != nullptr) Cin += (size_t)blockIdx.y * c_batch_stride;
     D += (size_t)blockIdx.y * d_batch_stride;
-    if (SPLIT_K) {
-        const int k_begin = (int)blockIdx.z * k_split_len;
-        A += k_begin;                             // k_split_len % BK == 0 keeps the 16-byte alignment of the rows
-        B += (size_t)k_begin * ldb;
-        K = K - k_begin < k_split_len ? K - k_begin : k_split_len;
-        Cin = nullptr;                            // C joins in the finishing kernel
-    }
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, NT = S::NT, UA = S::UA, UB = S::UB, MI = S::MI, NI = S::NI;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     u32x4* As = reinterpret_cast<u32x4*>(lds_raw);            // [2][A_UNITS]
@@ -218,22 +207,6 @@ __global__ __launch_bounds__(S::NT) void hgemm_tile_kernel(const _Float16* __res
         }
     }
 
-    if (SPLIT_K) {
-#pragma unroll
-        for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-                if (m < M) {
-#pragma unroll
-                    for (int ni = 0; ni < NI; ++ni) {
-                        const int n = bn0 + wn0 + ni * 32 + li;
-                        if (n < N) unsafeAtomicAdd(partial + (size_t)m * N + n, acc[mi][ni][r]);
-                    }
-                }
-            }
-        return;
-    }
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
@@ -250,7 +223,7 @@ __global__ __launch_bounds__(S::NT) void hgemm_tile_kernel(const _Float16* __res
         }
 }
 
-// D = half(partial + C): the end of a split-K product.  partial is dense M x N fp32.
+// D = half(partial + C): the end of a split-K product (hgemm_dma_kernel with SPLIT_K).  partial is dense M x N fp32.
 __global__ __launch_bounds__(256) void hgemm_split_finish_kernel(const float* __restrict__ partial, const _Float16* Cin, int ldc,
                                                                  _Float16* D, int ldd, int M, int N) {
     const size_t total = (size_t)M * N;
