@@ -68,14 +68,15 @@ def bench_sgemm(capi, workloads, M, K, N, steps, warmup, seed, dist="uniform"):
             "flops": flops, "A": A, "B": B, "ms_median": med, "ms_min": mn}
 
 
-def bench_hgemm(capi, workloads, n, steps, warmup, seed):
-    A = workloads.uniform_pm1((n, n), seed).astype(np.float16).view(np.uint16)
-    B = workloads.uniform_pm1((n, n), seed + 1).astype(np.float16).view(np.uint16)
+def bench_hgemm(capi, workloads, n, steps, warmup, seed, shape=None):
+    M, K, N = shape if shape else (n, n, n)
+    A = workloads.uniform_pm1((M, K), seed).astype(np.float16).view(np.uint16)
+    B = workloads.uniform_pm1((K, N), seed + 1).astype(np.float16).view(np.uint16)
     dA, dB = capi.DeviceBuffer.from_numpy(A), capi.DeviceBuffer.from_numpy(B)
-    dD = capi.DeviceBuffer(n * n * 2)
-    launch = lambda: capi.hgemm(dA.ptr, n, dB.ptr, n, dD.ptr, n, n, n, n, blocking=False)
+    dD = capi.DeviceBuffer(M * N * 2)
+    launch = lambda: capi.hgemm(dA.ptr, K, dB.ptr, N, dD.ptr, N, M, N, K, blocking=False)
     wall, ev = time_launches(capi, launch, steps, warmup)
-    flops = 2.0 * n * n * n
+    flops = 2.0 * M * N * K
     return {"ms_wall": wall, "ms_kernel": ev, "tflops": flops / (wall * 1e-3) / 1e12, "tflops_kernel": flops / (ev * 1e-3) / 1e12}
 
 
@@ -309,6 +310,9 @@ def main():
                                                           "ms_of_one_bare_mfma_chain": round(chain_ms, 4)}
         log("fp32 64x65536x1024 (exact chain): %.4f ms -> %.1f TFLOP/s (a bare MFMA chain over K: %.4f ms)"
             % (r["ms_wall"], r["tflops"], chain_ms))
+        r = bench_hgemm(capi, workloads, 0, side_steps, side_warmup, 79, shape=(64, 65536, 1024))
+        also["fp16_long_k_64x65536x1024_split_k"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4)}
+        log("fp16 64x65536x1024 (split-K, fp32 workspace): %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
     if want("ragged"):
         r = bench_sgemm(capi, workloads, 3000, 1500, 4500, side_steps, side_warmup, 4321, dist="normal")
         also["fp32_ragged_3000x1500x4500"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
