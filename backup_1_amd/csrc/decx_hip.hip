@@ -257,11 +257,15 @@ int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float*
         const long blocks16 = (long)cdiv(M, 16) * cdiv(N, 16) * batch.count, tiles32 = (long)cdiv(M, 32) * cdiv(N, 32) * batch.count;
         int chain = g_rt.sgemm_variant >= 11 && g_rt.sgemm_variant <= 13 ? g_rt.sgemm_variant : 0;
         if (g_rt.sgemm_variant < 1 || g_rt.sgemm_variant > 13) {
-            // 32x32 tiles share a CU two at a time, 64x64 tiles take one each and cost 1.78 times a pair (measured at
-            // 1024x8192x1024: 0.153 ms for one round of 64x64 tiles, 0.171 ms for two rounds of 32x32 pairs)
+            // In units of one round of 32x32 tiles (two per CU, 512 on 256 CUs): a round of 64x64 tiles (one per CU) costs
+            // 1.55, further rounds of 32x32 tiles overlap with the first and cost 0.9 each once there is more than
+            // one (measured on squares of 640 .. 2560 at K = 512 and 2048).  Beyond 10 (K < 1024: 4) 32x32 tiles per CU
+            // the 32x32x2 tiles are ahead -- the block-chain kernels have the longer prologue.
             const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch.count;
-            const double cost64 = 1.78 * (double)((tiles64 + cus - 1) / cus), pairs = (double)tiles32 / (2.0 * cus);
-            chain = blocks16 <= cus ? 12 : tiles32 > 10 * cus ? 0 : cost64 < (pairs > 1.0 ? pairs : 1.0) ? 13 : 11;
+            const double cost64 = 1.55 * (double)((tiles64 + cus - 1) / cus), pairs = (double)tiles32 / (2.0 * cus);
+            const double cost32 = pairs <= 1.0 ? 1.0 : 0.9 * (pairs + 0.5);
+            const long tile_limit = (K >= 1024 ? 10 : 4) * cus;
+            chain = blocks16 <= cus ? 12 : tiles32 > tile_limit ? 0 : cost64 < cost32 ? 13 : 11;
         }
         if (chain == 11) return launch_sgemm_chain16<Chain16<2, 1, 4, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
         if (chain == 12) return launch_sgemm_chain16<Chain16<1, 1, 8, 2>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
