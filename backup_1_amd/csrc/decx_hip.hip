@@ -12,6 +12,7 @@
 #include "hgemm_tile.hpp"
 #include "sgemm_tile.hpp"
 #include "sgemm_chain16.hpp"
+#include "conv_chain16.hpp"
 #include "hconv_tile.hpp"
 
 using namespace decx_hip;
@@ -242,6 +243,25 @@ int launch_sgemm_chain16(const float* A, int lda, const float* B, int ldb, const
     return 0;
 }
 
+// Which shape of the one-wave-per-block kernel (sgemm_chain16.hpp) a result of M x N takes, or 0 for the tiles.
+// Measured: ahead of the tiles up to about ten 32x32 tiles per CU -- 1536x1536 on 256 CUs -- 1.7x at 1024x8192x1024, 9x at
+// 64x65536x1024.  All paths give the same bits, so this is a choice of speed only.
+int pick_chain_shape(int M, int N, int K, int batch) {
+    if (g_rt.sgemm_variant >= 11 && g_rt.sgemm_variant <= 13) return g_rt.sgemm_variant;
+    if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) return 0;
+    const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+    const long blocks16 = (long)cdiv(M, 16) * cdiv(N, 16) * batch, tiles32 = (long)cdiv(M, 32) * cdiv(N, 32) * batch;
+    // In units of one round of 32x32 tiles (two per CU, 512 on 256 CUs): a round of 64x64 tiles (one per CU) costs
+    // 1.55, further rounds of 32x32 tiles overlap with the first and cost 0.9 each once there is more than
+    // one (measured on squares of 640 .. 2560 at K = 512 and 2048).  Beyond 10 (K < 1024: 4) 32x32 tiles per CU
+    // the 32x32x2 tiles are ahead -- the block-chain kernels have the longer prologue.
+    const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch;
+    const double cost64 = 1.55 * (double)((tiles64 + cus - 1) / cus), pairs = (double)tiles32 / (2.0 * cus);
+    const double cost32 = pairs <= 1.0 ? 1.0 : 0.9 * (pairs + 0.5);
+    const long tile_limit = (K >= 1024 ? 10 : 4) * cus;
+    return blocks16 <= cus ? 12 : tiles32 > tile_limit ? 0 : cost64 < cost32 ? 13 : 11;
+}
+
 int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
                   int N, int K, const Batch& batch, bool relu = false) {
     if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
@@ -250,23 +270,7 @@ int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float*
     const bool vec_b = aligned16(B) && ldb % 4 == 0 && ldb >= 4 && batch.stride_b % 4 == 0;
     DenseOut out{ldd, relu, aligned16(D) && ldd % 4 == 0 && batch.stride_d % 4 == 0};
     if (vec_a && vec_b) {
-        // Small results go to the one-wave-per-block kernel (measured: ahead of the tiles up to about ten 32x32 tiles per
-        // CU -- 1536x1536 on 256 CUs -- whatever K is; 1.7x at 1024x8192x1024, 9x at 64x65536x1024).  All paths give
-        // the same bits, so this is a choice of speed only.
-        const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
-        const long blocks16 = (long)cdiv(M, 16) * cdiv(N, 16) * batch.count, tiles32 = (long)cdiv(M, 32) * cdiv(N, 32) * batch.count;
-        int chain = g_rt.sgemm_variant >= 11 && g_rt.sgemm_variant <= 13 ? g_rt.sgemm_variant : 0;
-        if (g_rt.sgemm_variant < 1 || g_rt.sgemm_variant > 13) {
-            // In units of one round of 32x32 tiles (two per CU, 512 on 256 CUs): a round of 64x64 tiles (one per CU) costs
-            // 1.55, further rounds of 32x32 tiles overlap with the first and cost 0.9 each once there is more than
-            // one (measured on squares of 640 .. 2560 at K = 512 and 2048).  Beyond 10 (K < 1024: 4) 32x32 tiles per CU
-            // the 32x32x2 tiles are ahead -- the block-chain kernels have the longer prologue.
-            const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch.count;
-            const double cost64 = 1.55 * (double)((tiles64 + cus - 1) / cus), pairs = (double)tiles32 / (2.0 * cus);
-            const double cost32 = pairs <= 1.0 ? 1.0 : 0.9 * (pairs + 0.5);
-            const long tile_limit = (K >= 1024 ? 10 : 4) * cus;
-            chain = blocks16 <= cus ? 12 : tiles32 > tile_limit ? 0 : cost64 < cost32 ? 13 : 11;
-        }
+        const int chain = pick_chain_shape(M, N, K, batch.count);
         if (chain == 11) return launch_sgemm_chain16<Chain16<2, 1, 4, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
         if (chain == 12) return launch_sgemm_chain16<Chain16<1, 1, 8, 2>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
         if (chain == 13) return launch_sgemm_chain16<Chain16<4, 2, 2, 3>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
@@ -305,6 +309,24 @@ int sgemm_splitk_enqueue(const float* A, int lda, const float* B, int ldb, const
     return launch_sgemm_splitk<SShapeSmall>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, splits, k_split_len);
 }
 
+template <class S>
+int launch_conv_chain16(const Im2colA<false>& img, const FilterB<false>& fb, const float* bias, float* dst, const TensorOut& out,
+                        int M, int N, int K) {
+    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    const long total = (long)tiles_m * tiles_n;
+    if (total > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
+    static bool attr_done = false;
+    if (!attr_done) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(conv_chain16_kernel<S>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)S::LDS_BYTES));
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(conv_chain16_kernel<S>, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, bias, dst, out,
+                       M, N, K, tiles_n);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt, int N, int kh,
                  int kw, size_t filt_stride, size_t filt_row_stride, float* dst, int dst_dpitch, size_t dst_row_stride,
                  int flag, const float* bias = nullptr, bool relu = false) {
@@ -337,6 +359,14 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
     const int variant = pick_sgemm_variant(M, N, K, 1);
     const int oy = flag ? kh / 2 : 0, ox = flag ? kw / 2 : 0;
     // a bias is the "+ C" operand with row stride 0: every output pixel adds the same N values
+    // small images: too few tiles for the chip, the one-wave-per-block kernel takes them (conv_chain16.hpp)
+    if (const int chain = pick_chain_shape(M, N, K, 1)) {
+        Im2colA<false> a{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
+        FilterB<false> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
+        if (chain == 11) return launch_conv_chain16<Chain16<2, 1, 4, 4>>(a, b, bias, dst, out, M, N, K);
+        if (chain == 12) return launch_conv_chain16<Chain16<1, 1, 8, 2>>(a, b, bias, dst, out, M, N, K);
+        return launch_conv_chain16<Chain16<4, 2, 2, 3>>(a, b, bias, dst, out, M, N, K);
+    }
     if (dpitch % 16 == 0) {      // a whole K step inside one tap: the tap walk runs on the scalar unit
         Im2colAUniform a{{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes}};
         FilterBUniform b{{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes}};

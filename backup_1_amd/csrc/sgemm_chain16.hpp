@@ -74,6 +74,59 @@ __device__ __forceinline__ void lds_write2_st64(unsigned byte_addr, float x, flo
     asm volatile("ds_write2st64_b32 %0, %1, %2 offset0:%3 offset1:%4" : : "v"(byte_addr), "v"(x), "v"(y), "n"(OFF0), "n"(OFF1) : "memory");
 }
 
+// The computing side of a workgroup: walks the chunks the moving waves put into LDS and returns with the finished
+// accumulators.  full_chunks chunks arrive through the three-buffer pipeline (one barrier after the prologue, one per
+// chunk); if chunks > full_chunks one more, ragged, chunk arrives in buffer 0 behind a barrier of its own.
+template <class S>
+__device__ __forceinline__ void chain16_consume(const float* As, const float* Bs, int wm0, int wn0, int lr, int ls, int full_chunks,
+                                                int chunks, f32x4 (&acc)[S::NB]) {
+    constexpr int DEPTH = S::DEPTH, NB = S::NB;
+    typedef std::integral_constant<int, 0> I0;
+    const float* a_frag = As + ls * S::A_PLANE + (wm0 + lr) * S::LINE;       // this lane's 16 operands of a chunk, buffer 0
+    const float* b_frag = Bs + ls * S::B_PLANE + (wn0 + lr) * S::LINE;       // block b: 16 lines further per block
+    f32x4 av[2][4], bv[2][NB][4];
+    constexpr int READS = 4 + 4 * NB;             // 16-byte operand reads per chunk: 4 of A, then 4 per block of B
+    auto read_one = [&](auto f_tag, auto r_tag, int buf) {
+        constexpr int F = decltype(f_tag)::value, R = decltype(r_tag)::value;
+        if constexpr (R < 4) av[F][R] = reinterpret_cast<const f32x4*>(a_frag + buf * S::A_FLOATS)[R];
+        else bv[F][(R - 4) / 4][(R - 4) % 4] = reinterpret_cast<const f32x4*>(b_frag + buf * S::B_FLOATS + ((R - 4) / 4) * 16 * S::LINE)[(R - 4) % 4];
+    };
+    if (full_chunks > 0) {
+        lds_sync();
+        static_for<0, READS>([&](auto r) { read_one(I0{}, r, 0); });
+        // chunk c: its operands are in fragment set c % 2; buffer (c+1) % 3 holds chunk c+1 since the previous barrier.
+        // The NB chains advance in turn; behind each of the first READS MFMAs goes one read of the next chunk's operands.
+        int buf_next = 1;
+        auto chunk = [&](auto d) {
+            constexpr int NOW = decltype(d)::value & 1;
+            typedef std::integral_constant<int, NOW ^ 1> Next;
+            static_for<0, 16 * NB>([&](auto i_tag) {
+                constexpr int I = decltype(i_tag)::value, J = I / NB, BLK = I % NB;
+                acc[BLK] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[NOW][J / 4][J % 4], bv[NOW][BLK][J / 4][J % 4], acc[BLK], 0, 0, 0);
+                if constexpr (I < READS) read_one(Next{}, i_tag, buf_next);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            lds_sync();
+            __builtin_amdgcn_sched_barrier(0);
+            buf_next = buf_next == 2 ? 0 : buf_next + 1;
+        };
+        int c0 = 0;
+        for (; c0 + DEPTH <= full_chunks; c0 += DEPTH) static_for<0, DEPTH>([&](auto d) { chunk(d); });
+        static_for<0, DEPTH>([&](auto d) {
+            if (c0 + decltype(d)::value < full_chunks) chunk(d);
+        });
+    }
+    if (chunks > full_chunks) {
+        lds_sync();
+        static_for<0, READS>([&](auto r) { read_one(I0{}, r, 0); });
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+                acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[0][j / 4][j % 4], bv[0][b][j / 4][j % 4], acc[b], 0, 0, 0);
+    }
+}
+
 template <class S, bool HAS_C>
 __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_chain16_kernel(const float* __restrict__ A, int lda,
                                                                     const float* __restrict__ B, int ldb, const float* Cin,
@@ -229,49 +282,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_chain16_kernel
             }
         }
     }
-    const float* a_frag = As + ls * S::A_PLANE + (wm0 + lr) * S::LINE;       // this lane's 16 operands of a chunk, buffer 0
-    const float* b_frag = Bs + ls * S::B_PLANE + (wn0 + lr) * S::LINE;       // block b: 16 lines further per block
-    f32x4 av[2][4], bv[2][NB][4];
-    constexpr int READS = 4 + 4 * NB;             // 16-byte operand reads per chunk: 4 of A, then 4 per block of B
-    auto read_one = [&](auto f_tag, auto r_tag, int buf) {
-        constexpr int F = decltype(f_tag)::value, R = decltype(r_tag)::value;
-        if constexpr (R < 4) av[F][R] = reinterpret_cast<const f32x4*>(a_frag + buf * S::A_FLOATS)[R];
-        else bv[F][(R - 4) / 4][(R - 4) % 4] = reinterpret_cast<const f32x4*>(b_frag + buf * S::B_FLOATS + ((R - 4) / 4) * 16 * S::LINE)[(R - 4) % 4];
-    };
-    if (full_chunks > 0) {
-        lds_sync();
-        static_for<0, READS>([&](auto r) { read_one(I0{}, r, 0); });
-        // chunk c: its operands are in fragment set c % 2; buffer (c+1) % 3 holds chunk c+1 since the previous barrier.
-        // The NB chains advance in turn; behind each of the first READS MFMAs goes one read of the next chunk's operands.
-        int buf_next = 1;
-        auto chunk = [&](auto d) {
-            constexpr int NOW = decltype(d)::value & 1;
-            typedef std::integral_constant<int, NOW ^ 1> Next;
-            static_for<0, 16 * NB>([&](auto i_tag) {
-                constexpr int I = decltype(i_tag)::value, J = I / NB, BLK = I % NB;
-                acc[BLK] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[NOW][J / 4][J % 4], bv[NOW][BLK][J / 4][J % 4], acc[BLK], 0, 0, 0);
-                if constexpr (I < READS) read_one(Next{}, i_tag, buf_next);
-                __builtin_amdgcn_sched_barrier(0);
-            });
-            lds_sync();
-            __builtin_amdgcn_sched_barrier(0);
-            buf_next = buf_next == 2 ? 0 : buf_next + 1;
-        };
-        int c0 = 0;
-        for (; c0 + DEPTH <= full_chunks; c0 += DEPTH) static_for<0, DEPTH>([&](auto d) { chunk(d); });
-        static_for<0, DEPTH>([&](auto d) {
-            if (c0 + decltype(d)::value < full_chunks) chunk(d);
-        });
-    }
-    if (chunks > full_chunks) {
-        lds_sync();
-        static_for<0, READS>([&](auto r) { read_one(I0{}, r, 0); });
-#pragma unroll
-        for (int j = 0; j < 16; ++j)
-#pragma unroll
-            for (int b = 0; b < NB; ++b)
-                acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[0][j / 4][j % 4], bv[0][b][j / 4][j % 4], acc[b], 0, 0, 0);
-    }
+    chain16_consume<S>(As, Bs, wm0, wn0, lr, ls, full_chunks, chunks, acc);
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
         const int n_out = bn0 + wn0 + 16 * b + lr;

@@ -163,7 +163,9 @@ int decx_hip_gemm3_host_f16(const uint16_t* hA, int lda, size_t plane_a, const u
  *                of src(y+ki-oy, x+kj-ox, c) * filt(n,ki,kj,c),
  *   (oy,ox) = (kh/2, kw/2) for ZERO_COMPENSATE, (0,0) otherwise: cross-correlation, stride 1 (im2col.cuh:150-163).
  * Channels c in [C, dpitch) are read like any other, so the containers' zero padding must be zero.
- * Columns x >= W_out of a dst row (the wpitch padding) are not written. */
+ * Columns x >= W_out of a dst row (the wpitch padding) are not written.
+ * Small images (few 32x32 tiles of the lowered H_out*W_out x N result) run on a one-wave-per-16x16-block kernel instead
+ * of the big tiles; the result is the same bit for bit. */
 int decx_hip_conv2_im2col_f32(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt, int N,
                               int kh, int kw, size_t filt_stride, size_t filt_row_stride, float* dst, int dst_dpitch,
                               size_t dst_row_stride, int flag);
