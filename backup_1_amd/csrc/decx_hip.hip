@@ -456,6 +456,21 @@ int launch_hgemm_dma_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb
     return 0;
 }
 
+// the fp32 workspace of the fp16 split-K paths: grown on demand, kept until the process ends
+int ensure_partial(size_t need) {
+    if (need <= g_rt.partial_bytes) return 0;
+    HIP_TRY(hipDeviceSynchronize());               // earlier launches may still use the old workspace
+    if (g_rt.partial) HIP_TRY(hipFree(g_rt.partial));
+    g_rt.partial = nullptr;
+    g_rt.partial_bytes = 0;
+    if (hipMalloc(&g_rt.partial, need) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(DECX_HIP_FAIL_ALLOCATION, "Fail to allocate memory\n");
+    }
+    g_rt.partial_bytes = need;
+    return 0;
+}
+
 // fp16 GEMM whose result has too few tiles to fill the chip while K is long: K is cut into ranges that run as separate
 // workgroups (blockIdx.z) and add their fp32 partial sums to a workspace with atomics; a second kernel adds C and
 // rounds to binary16 once.  fp32 sums in no fixed order: the result can differ in its last bit from run to run, inside
@@ -463,18 +478,7 @@ int launch_hgemm_dma_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb
 int hgemm_splitk_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                          int ldd, int M, int N, int K, int splits, hipStream_t stream) {
     typedef HShapeDmaSmall S;                      // 128x128x64, LDS-DMA staged, two workgroups per CU
-    const size_t need = (size_t)M * N * sizeof(float);
-    if (need > g_rt.partial_bytes) {
-        HIP_TRY(hipDeviceSynchronize());           // earlier launches may still use the old workspace
-        if (g_rt.partial) HIP_TRY(hipFree(g_rt.partial));
-        g_rt.partial = nullptr;
-        g_rt.partial_bytes = 0;
-        if (hipMalloc(&g_rt.partial, need) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(DECX_HIP_FAIL_ALLOCATION, "Fail to allocate memory\n");
-        }
-        g_rt.partial_bytes = need;
-    }
+    if (int rc = ensure_partial((size_t)M * N * sizeof(float))) return rc;
     auto kern = hgemm_dma_kernel<S, false, true>;
     static bool attr_done = false;
     if (!attr_done) {
@@ -595,9 +599,53 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
         HIP_TRY(allow(reinterpret_cast<const void*>(hconv_tile_kernel<HconvSquare, false>), HconvSquare::LDS_BYTES));
         attr_done = true;
     }
+    // small image: few tiles and many K steps -> ranges of K steps as separate workgroups, fp32 partial sums in the
+    // workspace, bias / ReLU / rounding in a finishing kernel
+    // Measured model, in us: a workgroup walks a K step of 64 halves in 0.75 us (1.3 x that once two workgroups share a
+    // CU's LDS bandwidth); the split pays 9 us for fill, finishing kernel and a third launch, and 3.1 ps per atomic add.
+    const int all_steps = cdiv(Kw, 32);
+    const long square_tiles = (long)cdiv(M, 128) * tiles_n;
+    int splits = 1;
+    if (!tall && 2 * square_tiles <= cus && all_steps >= 8 && (size_t)M * N <= ((size_t)1 << 26)) {
+        const double t_whole = 4.0 + 0.75 * all_steps;
+        double best = 0.85 * t_whole;
+        const long most = (2 * cus + square_tiles - 1) / square_tiles;
+        for (int s = 2; s <= most && s <= all_steps / 2; ++s) {
+            const double share = square_tiles * s > cus ? 1.3 : 1.0;
+            const double t = 9.0 + 3.1e-6 * M * N * s + 0.75 * share * cdiv(all_steps, s);
+            if (t < best) best = t, splits = s;
+        }
+    }
+    if (splits > 1) {
+        const int steps_per_split = cdiv(all_steps, splits);
+        splits = cdiv(all_steps, steps_per_split);                     // no empty range
+        if (int rc = ensure_partial((size_t)M * N * sizeof(float))) return rc;
+        static bool split_attr_done = false;
+        if (!split_attr_done) {
+            HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hconv_tile_kernel<HconvSquare, true, true>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)HconvSquare::LDS_BYTES));
+            HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hconv_tile_kernel<HconvSquare, false, true>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)HconvSquare::LDS_BYTES));
+            split_attr_done = true;
+        }
+        const size_t count = (size_t)M * N;
+        const unsigned fill_blocks = (unsigned)((count + 255) / 256 < 4096 ? (count + 255) / 256 : 4096);
+        hipLaunchKernelGGL(zero_region_kernel, dim3(fill_blocks), dim3(256), 0, g_rt.stream, g_rt.partial, N, M, N);
+        const dim3 grid((unsigned)total, (unsigned)splits);
+        if (tap_uniform)
+            hipLaunchKernelGGL((hconv_tile_kernel<HconvSquare, true, true>), grid, dim3(HconvSquare::NT), HconvSquare::LDS_BYTES,
+                               g_rt.stream, img, fb, out, M, N, Kw, tiles_n, g_rt.partial, steps_per_split);
+        else
+            hipLaunchKernelGGL((hconv_tile_kernel<HconvSquare, false, true>), grid, dim3(HconvSquare::NT), HconvSquare::LDS_BYTES,
+                               g_rt.stream, img, fb, out, M, N, Kw, tiles_n, g_rt.partial, steps_per_split);
+        hipLaunchKernelGGL(hconv_split_finish_kernel, dim3(fill_blocks), dim3(256), 0, g_rt.stream, g_rt.partial, out, M, N);
+        HIP_TRY(hipGetLastError());
+        return 0;
+    }
     auto launch = [&](auto kern, auto shape) {
         typedef decltype(shape) S;
-        hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, out, M, N, Kw, tiles_n);
+        hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, out, M, N, Kw, tiles_n,
+                           static_cast<float*>(nullptr), 0);
     };
     if (tall && tap_uniform) launch(hconv_tile_kernel<HconvTall, true>, HconvTall{});
     else if (tall) launch(hconv_tile_kernel<HconvTall, false>, HconvTall{});

@@ -81,9 +81,13 @@ __device__ __forceinline__ void small_divmod(int m, int d, float rcp_d, int& quo
 // TAP_UNIFORM (channel pitch a multiple of 64 halves, i.e. of a K step): a K step lies inside one tap, so the walk over
 // (tap row, tap column, channel) is the same for every lane up to a constant and runs on the scalar unit; a load then
 // costs the vector unit one add (plus the column check of an image load), and a filter load nothing at all.
-template <class S, bool TAP_UNIFORM>
+// SPLIT_K (small images: few tiles, many K steps): blockIdx.y selects a range of steps_per_split K steps; the tile's fp32
+// partial sums are added with atomics to a dense M x N fp32 workspace `partial` (zeroed beforehand), and
+// hconv_split_finish_kernel applies bias and ReLU and writes the binary16 tensor.
+template <class S, bool TAP_UNIFORM, bool SPLIT_K = false>
 __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, HalfFilters fb, HalfTensorOut out, int M, int N,
-                                                           int Kw /* K in words */, int tiles_n) {
+                                                           int Kw /* K in words */, int tiles_n, float* partial,
+                                                           int steps_per_split) {
     constexpr int BM = S::BM, BN = S::BN, NT = S::NT, U = S::U, MI = S::MI, NI = S::NI;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     constexpr int A_BYTES = S::A_UNITS * 16, B_BYTES = S::B_UNITS * 16;     // one buffer of either operand
@@ -92,6 +96,9 @@ __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, Hal
 
     // each XCD gets one contiguous run of tiles: neighbouring tiles share their halo rows in that XCD's L2
     const TileCoord tc = xcd_grouped_tile((int)blockIdx.x, (int)gridDim.x / tiles_n, tiles_n, 8);
+    const int all_steps = (Kw + S::BK / 2 - 1) / (S::BK / 2);
+    const int first_step = SPLIT_K ? (int)blockIdx.y * steps_per_split : 0;
+    const int steps = SPLIT_K ? (all_steps - first_step < steps_per_split ? all_steps - first_step : steps_per_split) : all_steps;
     const int bm0 = tc.tm * BM, bn0 = tc.tn * BN;
     const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
     const int wm0 = (wave / S::WAVES_N) * S::WM, wn0 = (wave % S::WAVES_N) * S::WN;
@@ -126,8 +133,8 @@ __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, Hal
     // position of this thread's unit in the image and in a filter; with TAP_UNIFORM the walk starts at unit 0 for all
     // lanes (scalar registers) and the lane's own 16 q bytes are part of its base offsets
     TapWalk wa, wb;
-    wa.init(TAP_UNIFORM ? 0 : 4 * q, img.dpitch_w, img.kw, img.row_stride_w);
-    wb.init(TAP_UNIFORM ? 0 : 4 * q, fb.dpitch_w, fb.kw, fb.row_stride_w);
+    wa.init(first_step * (S::BK / 2) + (TAP_UNIFORM ? 0 : 4 * q), img.dpitch_w, img.kw, img.row_stride_w);
+    wb.init(first_step * (S::BK / 2) + (TAP_UNIFORM ? 0 : 4 * q), fb.dpitch_w, fb.kw, fb.row_stride_w);
     const TapStep sa = TapStep::make(S::BK / 2, img.dpitch_w, img.kw, img.row_stride_w);
     const TapStep sb = TapStep::make(S::BK / 2, fb.dpitch_w, fb.kw, fb.row_stride_w);
     if (TAP_UNIFORM) {
@@ -204,7 +211,6 @@ __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, Hal
             for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
 
     typedef std::integral_constant<int, 0> I0;
-    const int steps = (Kw + S::BK / 2 - 1) / (S::BK / 2);
     static_for<0, DEPTH>([&](auto d) { load_stage(d); });
     static_for<0, PASSES>([&](auto p) { store_pass(I0{}, I0{}, p); });
     __syncthreads();
@@ -231,7 +237,10 @@ __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, Hal
             for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
                 for (int ni = 0; ni < NI; ++ni)
-                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ff[ni], pf[mi], acc[mi][ni], 0, 0, 0);
+                    // split-K keeps the GEMM orientation (pixels as rows): a lane's atomic adds then run along the filters,
+                    // i.e. along consecutive addresses of the workspace
+                    acc[mi][ni] = SPLIT_K ? __builtin_amdgcn_mfma_f32_32x32x16_f16(pf[mi], ff[ni], acc[mi][ni], 0, 0, 0)
+                                          : __builtin_amdgcn_mfma_f32_32x32x16_f16(ff[ni], pf[mi], acc[mi][ni], 0, 0, 0);
             static_for<ks * PASSES / KS, (ks + 1) * PASSES / KS>([&](auto p) { store_pass(NextSet{}, NextBuf{}, p); });
         });
         __syncthreads();
@@ -242,6 +251,22 @@ __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, Hal
             if (t0 + decltype(d)::value < steps) k_step(d);
         });
 
+    if (SPLIT_K) {
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                if (m < M) {
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni) {
+                        const int n = bn0 + wn0 + ni * 32 + li;
+                        if (n < N) unsafeAtomicAdd(partial + (size_t)m * N + n, acc[mi][ni][r]);
+                    }
+                }
+            }
+        return;
+    }
     // Epilogue.  Lane (li, lh) holds for pixel wm0 + 32 mi + li the filters wn0 + 32 ni + 8 j + 4 lh + e (e = 0..3) in
     // acc[mi][ni][4 j + e]: bias, ReLU and one rounding to binary16 per run of four, then through LDS (free now) so that
     // the tile leaves in 16-byte pieces.
@@ -290,6 +315,18 @@ __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, Hal
                 for (int e = 0; e < 8 && n + e < N; ++e) pix[e] = t8[e];
             }
         }
+    }
+}
+
+// dst(pixel m, filter n) = half(relu(partial[m][n] + bias[n])): the end of a split-K convolution.
+__global__ __launch_bounds__(256) void hconv_split_finish_kernel(const float* __restrict__ partial, HalfTensorOut out, int M, int N) {
+    const size_t total = (size_t)M * N;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const int m = (int)(i / N), n = (int)(i - (size_t)m * N);
+        float v = partial[i];
+        if (out.bias != nullptr) v += (float)out.bias[n];
+        if (out.relu) v = relu_by_sign(v);
+        out.dst[(size_t)(m / out.Wout) * out.row_stride + (size_t)(m % out.Wout) * out.dpitch + n] = (_Float16)v;
     }
 }
 

@@ -189,7 +189,10 @@ int decx_hip_conv2_im2col_f32_fused(const float* src, int H, int W, int dpitch, 
  * All strides and pitches in halves; dpitch % 8 == 0; src and filt 16-byte aligned.  Same index arithmetic, flags and
  * error codes as decx_hip_conv2_im2col_f32.  Products are accumulated in fp32 (in the matrix instruction's order),
  * then   dst(y,x,n) = half( relu( sum + float(bias[n]) ) )   with bias (N halves on the device) and relu optional (NULL / 0),
- * rounded to binary16, nearest even, once.  Checked against fp64 arithmetic on the binary16 inputs to 2e-3 relative. */
+ * rounded to binary16, nearest even, once.  Checked against fp64 arithmetic on the binary16 inputs to 2e-3 relative.
+ * Small images with long filters (few 128x128 tiles of the lowered result, many K steps) are computed as ranges of K
+ * that meet in the library's fp32 workspace (the one decx_hip_hgemm uses; grown on demand, kept until the process
+ * ends): calls that take this route must not overlap on one GPU, which the library's single stream guarantees. */
 int decx_hip_conv2_im2col_f16(const uint16_t* src, int H, int W, int dpitch, size_t src_row_stride, const uint16_t* filt, int N,
                               int kh, int kw, size_t filt_stride, size_t filt_row_stride, uint16_t* dst, int dst_dpitch,
                               size_t dst_row_stride, int flag, const uint16_t* bias, int relu);

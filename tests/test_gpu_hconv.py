@@ -115,6 +115,25 @@ def test_many_pixels_take_the_tall_tile(gpu, oracle):
     assert np.array_equal(got.astype(np.float64), ref)
 
 
+@pytest.mark.parametrize("case", [(14, 14, 128, 40, 3, 3), (12, 10, 120, 70, 3, 3), (7, 7, 512, 130, 3, 3), (9, 5, 64, 16, 5, 5)])
+def test_small_images_split_the_walk_over_k(gpu, oracle, case):
+    # few 128-pixel tiles and many K steps: ranges of K steps run as separate workgroups and meet in an fp32 workspace;
+    # bias, ReLU and the rounding happen in the finishing kernel.  Integer data exact, real data within the fp16 rule.
+    H, W, C, N, kh, kw = case
+    si = workloads.small_ints((H, W, C), 861, -1, 1).astype(np.float16)
+    fi = workloads.small_ints((N, kh, kw, C), 862, -1, 1).astype(np.float16)
+    for flag in (1, 0):
+        got, sbuf, fb = gpu_hconv(si, fi, flag)
+        ref, _ = oracle.conv2_f64_f16(sbuf, fb, flag)
+        assert np.array_equal(got.astype(np.float64), ref)
+    src = workloads.normal((H, W, C), 863).astype(np.float16)
+    filt = workloads.normal((N, kh, kw, C), 864, sigma=0.05).astype(np.float16)
+    bias = workloads.normal((N,), 865).astype(np.float16)
+    for b, r in ((None, False), (bias, True)):
+        got, sbuf, fb = gpu_hconv(src, filt, 1, bias16=b, relu=r)
+        assert check_against_f64(oracle, got, sbuf, fb, 1, bias16=b, relu=r) < TOL
+
+
 def test_error_codes(gpu):
     L = capi.lib()
     d = capi.DeviceBuffer(1 << 16)
