@@ -505,8 +505,10 @@ int hgemm_splitk_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb,
 int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                   int ldd, int M, int N, int K, const Batch& batch) {
     if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
+    // the LDS-DMA tiles address a tile's rows with 32-bit byte offsets from the tile's first row: 256 rows of A, 64 of B
+    const bool narrow = (size_t)lda * 256 * sizeof(uint16_t) < ((size_t)1 << 32) && (size_t)ldb * 64 * sizeof(uint16_t) < ((size_t)1 << 32);
     const bool vec = aligned16(A) && aligned16(B) && lda % 8 == 0 && ldb % 8 == 0 && ldb >= 8 && batch.stride_a % 8 == 0 &&
-                     batch.stride_b % 8 == 0;
+                     batch.stride_b % 8 == 0 && narrow;
     if (!vec) return launch_hgemm_tile<HShapeSmall, false>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     int variant = g_rt.hgemm_variant;
     {
