@@ -152,6 +152,8 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //   8:  64x64x16,  2x2 waves of  32x32    -- small problems: 1024^3 has only 64 tiles of 128x128 for 256 CUs
 //   9: 128x64x16,  2x2 waves of  64x32
 //  10: 224x256x16, 1x8 waves of 224x32    -- two waves per SIMD like 7; 7/8 of its tile, for tile counts that 7 rounds badly
+//  14: 192x192x16, 2x2 waves of  96x96    -- dense GEMM only: sizes that 256 and 128 divide into a bad number of tiles
+//         (3072^2 is 144 tiles of 256^2, 576 of 128^2, and exactly 256 of these)
 // and, for dense GEMM only, the one-wave-per-16x16-block kernel of sgemm_chain16.hpp:
 //  11:  32x32x64,  2x2 computing + 4 moving waves, two workgroups per CU -- results too small to fill the chip with tiles
 //  12:  16x16x64,  1 computing + 2 moving waves -- at most one 16x16 block per CU: the fastest a single chain can walk K
@@ -164,6 +166,7 @@ typedef SgemmShape<256, 128, 16, 2, 2, 1> SShapeTallSolo;
 typedef SgemmShape<224, 128, 16, 1, 4, 1> SShape224Solo;
 typedef SgemmShape<256, 256, 16, 4, 2, 2, 2> SShapeBig8;
 typedef SgemmShape<224, 256, 16, 1, 8, 2, 2> SShape224Wide;   // 8 waves of 224x32, two per SIMD
+typedef SgemmShape<192, 192, 16, 2, 2, 1> SShape192;
 typedef SgemmShape<64, 64, 16, 2, 2, 4> SShapeTiny;      // 2x2 waves of 32x32
 typedef SgemmShape<128, 64, 16, 2, 2, 4> SShapeTiny2;    // 2x2 waves of 64x32
 
@@ -172,15 +175,17 @@ typedef SgemmShape<128, 64, 16, 2, 2, 4> SShapeTiny2;    // 2x2 waves of 64x32
 // the pipe busy (measured on large squares, relative to shape 7).  The 256x128 and 224x128 shapes come in a
 // two-workgroups-per-CU build, better on short K walks where one tile's prologue and epilogue overlap the other's loop,
 // and a one-wave-per-SIMD build with deeper prefetch, better on long ones.
-int pick_sgemm_variant(int M, int N, int K, int batch) {
+int pick_sgemm_variant(int M, int N, int K, int batch, bool dense = false) {
     if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) return g_rt.sgemm_variant;
+    if (g_rt.sgemm_variant == 14) return dense ? 14 : 2;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     struct Cand { int variant, bm, bn; double eff; };
     const Cand cands[] = {{7, 256, 256, 1.00}, {10, 224, 256, 0.96}, {3, 256, 128, 0.95}, {4, 224, 128, 0.94}, {2, 128, 128, 0.89},
-                          {9, 128, 64, 0.83}, {8, 64, 64, 0.78}};
+                          {9, 128, 64, 0.83}, {8, 64, 64, 0.78}, {14, 192, 192, 0.93}};
     int best = 7;
     double best_cost = 0.0;
     for (const Cand& c : cands) {
+        if (c.variant == 14 && !dense) continue;
         const long tiles = (long)cdiv(M, c.bm) * cdiv(N, c.bn) * batch;
         const double cost = (double)((tiles + cus - 1) / cus) * c.bm * c.bn / c.eff;
         if (best_cost == 0.0 || cost < best_cost) {
@@ -248,7 +253,7 @@ int launch_sgemm_chain16(const float* A, int lda, const float* B, int ldb, const
 // 64x65536x1024.  All paths give the same bits, so this is a choice of speed only.
 int pick_chain_shape(int M, int N, int K, int batch) {
     if (g_rt.sgemm_variant >= 11 && g_rt.sgemm_variant <= 13) return g_rt.sgemm_variant;
-    if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) return 0;
+    if ((g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) || g_rt.sgemm_variant == 14) return 0;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     const long blocks16 = (long)cdiv(M, 16) * cdiv(N, 16) * batch, tiles32 = (long)cdiv(M, 32) * cdiv(N, 32) * batch;
     // In units of one round of 32x32 tiles (two per CU, 512 on 256 CUs): a round of 64x64 tiles (one per CU) costs
@@ -265,7 +270,7 @@ int pick_chain_shape(int M, int N, int K, int batch) {
 int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
                   int N, int K, const Batch& batch, bool relu = false) {
     if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
-    const int variant = pick_sgemm_variant(M, N, K, batch.count);
+    const int variant = pick_sgemm_variant(M, N, K, batch.count, true);
     const bool vec_a = aligned16(A) && lda % 4 == 0 && batch.stride_a % 4 == 0;
     const bool vec_b = aligned16(B) && ldb % 4 == 0 && ldb >= 4 && batch.stride_b % 4 == 0;
     DenseOut out{ldd, relu, aligned16(D) && ldd % 4 == 0 && batch.stride_d % 4 == 0};
@@ -278,6 +283,7 @@ int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float*
     if (vec_a && vec_b) {
         DenseA<true> a{A, lda, M, K, batch.stride_a};
         DenseB<true> b{B, ldb, N, K, batch.stride_b};
+        if (variant == 14) return launch_sgemm_tile<SShape192>(a, b, Cin, ldc, D, out, M, N, K, batch);
         return dispatch_sgemm(variant, a, b, Cin, ldc, D, out, M, N, K, batch);
     }
     // unaligned operands: element-wise loaders, one tile shape only

@@ -393,9 +393,16 @@ struct DenseB {
         typedef float vec_t __attribute__((ext_vector_type(S::NI)));
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const vec_t v = *reinterpret_cast<const vec_t*>(buf + (8 * s + 2 * e + lh) * row_floats<S>() + wn0 + S::NI * li);
+            const float* at = buf + (8 * s + 2 * e + lh) * row_floats<S>() + wn0 + S::NI * li;
+            if constexpr (S::NI == 3) {
+                // 12-byte runs are not aligned for a vector read; three single reads (lanes 3 floats apart: no bank conflict)
 #pragma unroll
-            for (int ni = 0; ni < S::NI; ++ni) frag[e][ni] = v[ni];
+                for (int ni = 0; ni < 3; ++ni) frag[e][ni] = at[ni];
+            } else {
+                const vec_t v = *reinterpret_cast<const vec_t*>(at);
+#pragma unroll
+                for (int ni = 0; ni < S::NI; ++ni) frag[e][ni] = v[ni];
+            }
         }
     }
     // column (relative to the wave's strip) held by lane li in block ni
@@ -838,7 +845,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
                 float* drow = D + out.offset(m);
                 const float* crow = HAS_C ? Cin + (size_t)m * ldc : nullptr;
                 const bool add_c = HAS_C && !PRELOAD_C && (!SPLIT_K || blockIdx.z == 0);
-                if (BSrc::ROW_MAJOR_LDS && !SPLIT_K && NI > 1) {
+                if (BSrc::ROW_MAJOR_LDS && !SPLIT_K && NI > 1 && NI != 3) {      // runs of 3 floats are not aligned for one store
                     const int n0 = bn0 + wn0 + NI * li;
                     if (out.vec && n0 + NI <= N) {
                         typedef float vec_t __attribute__((ext_vector_type(NI)));

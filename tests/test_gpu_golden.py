@@ -19,7 +19,7 @@ def same_bits(a, b):
     return np.array_equal(np.isnan(a), nan) and np.array_equal(a[~nan].view(np.uint32), b[~nan].view(np.uint32))
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14])
 def test_gemm_and_conv_reproduce_the_fixtures(gpu, variant):
     assert same_bits(gpu_sgemm(V["gemm_A"], V["gemm_B"], variant=variant), V["gemm_AB"])
     assert same_bits(gpu_sgemm(V["gemm_A"], V["gemm_B"], C=V["gemm_C"], variant=variant), V["gemm_AB_plus_C"])
