@@ -9,7 +9,7 @@ import os
 import pytest
 
 BK = 64                    # Chain16::BK
-DEPTHS = (2, 4, 8)           # Chain16::DEPTH of the two shapes that are built
+DEPTHS = (2, 4, 8)           # Chain16::DEPTH of the shapes that are built
 
 
 def replay(K, DEPTH):
