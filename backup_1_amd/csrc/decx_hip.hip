@@ -760,10 +760,14 @@ int gemm3_host_pipeline(const T* hA, int lda, size_t plane_a, const T* hB, int l
     return 0;
 }
 
-// One GEMM on HOST-resident matrices (the Matrix<T> overloads of de::cuda::GEMM, GEMM.h:56-131, :139-228): the result's
-// rows are cut into panels, and the upload of A's panel p+1, the kernel on panel p and the download of result panel p-1
-// overlap on three streams.  B goes up first, whole.  Device copies keep the host pitches.  Overlap needs pinned host
-// memory (decx_hip_host_malloc); pageable memory works but serialises.
+// One GEMM on HOST-resident matrices (the Matrix<T> overloads of de::cuda::GEMM, GEMM.h:56-131, :139-228).  The link to
+// the host is the bottleneck (8192^3 fp32: 0.54 GB up at 57 GB/s = 9.3 ms against 7.3 ms of kernel), so the uploads never
+// pause and the kernel follows them as closely as the data allows: A goes up in row panels, B in column panels, taking
+// turns; a new row panel of A is multiplied at once with all column panels of B already there, a new column panel of B
+// with all row panels of A already there (one GEMM launch each, on sub-matrices of the device copies), and each finished
+// region of the result goes down on a third stream.  Every output is still one whole walk over K: same bits as the
+// device-resident call.  Device copies keep the host pitches.  Overlap needs pinned host memory (decx_hip_host_malloc);
+// pageable memory works but serialises.
 template <typename T, class Enqueue>
 int gemm_host_pipeline(const T* hA, int lda, const T* hB, int ldb, const T* hC, int ldc, T* hD, int ldd, int M, int N, int K,
                        Enqueue enqueue) {
@@ -772,21 +776,24 @@ int gemm_host_pipeline(const T* hA, int lda, const T* hB, int ldb, const T* hC, 
     if (M <= 0 || N <= 0 || K <= 0) return fail(DECX_HIP_FAIL_DIMS, "Matrix Dims don't match each other");
     if (lda < K || ldb < N || ldd < N || (hC && ldc < N))
         return fail(DECX_HIP_FAIL_ERROR_PARAMS, "leading dimension smaller than the row length\n");
-    // panels of whole 256-row tiles, big enough to fill the chip (>= 2048 rows x N), at most 16 of them
-    int panel_rows = 2048;
-    while ((long)cdiv(M, panel_rows) > 16) panel_rows *= 2;
-    const int panels = cdiv(M, panel_rows);
+    // panels of whole 256-wide tiles, at least 1024 wide, at most 8 per operand
+    constexpr int MAX_PANELS = 8, MAX_STEPS = 2 * MAX_PANELS;
+    auto panel_extent = [](int extent) {
+        int p = cdiv(cdiv(extent, MAX_PANELS), 256) * 256;
+        return p < 1024 ? 1024 : p;
+    };
+    const int pm = panel_extent(M), pn = panel_extent(N);
+    const int panels_a = cdiv(M, pm), panels_b = cdiv(N, pn), steps = panels_a + panels_b;
     T *dA = nullptr, *dB = nullptr, *dD = nullptr;
     hipStream_t s_up = nullptr, s_down = nullptr;
-    hipEvent_t b_up = nullptr, up[16] = {}, done[16] = {};
+    hipEvent_t up[MAX_STEPS] = {}, done[MAX_STEPS] = {};
     int rc = 0;
     auto cleanup = [&] {
         (void)hipDeviceSynchronize();
         if (dA) (void)hipFree(dA);
         if (dB) (void)hipFree(dB);
         if (dD) (void)hipFree(dD);
-        if (b_up) (void)hipEventDestroy(b_up);
-        for (int p = 0; p < 16; ++p) {
+        for (int p = 0; p < MAX_STEPS; ++p) {
             if (up[p]) (void)hipEventDestroy(up[p]);
             if (done[p]) (void)hipEventDestroy(done[p]);
         }
@@ -806,32 +813,43 @@ int gemm_host_pipeline(const T* hA, int lda, const T* hB, int ldb, const T* hC, 
     }
     PIPE_TRY(hipStreamCreateWithFlags(&s_up, hipStreamNonBlocking));
     PIPE_TRY(hipStreamCreateWithFlags(&s_down, hipStreamNonBlocking));
-    PIPE_TRY(hipEventCreateWithFlags(&b_up, hipEventDisableTiming));
-    for (int p = 0; p < panels; ++p) {
+    for (int p = 0; p < steps; ++p) {
         PIPE_TRY(hipEventCreateWithFlags(&up[p], hipEventDisableTiming));
         PIPE_TRY(hipEventCreateWithFlags(&done[p], hipEventDisableTiming));
     }
-    PIPE_TRY(hipMemcpy2DAsync(dB, (size_t)ldb * sizeof(T), hB, (size_t)ldb * sizeof(T), (size_t)N * sizeof(T), K,
-                              hipMemcpyHostToDevice, s_up));
-    PIPE_TRY(hipEventRecord(b_up, s_up));
-    PIPE_TRY(hipStreamWaitEvent(g_rt.stream, b_up, 0));
-    for (int p = 0; p < panels; ++p) {
-        const int r0 = p * panel_rows, rows = (M - r0 < panel_rows) ? M - r0 : panel_rows;
-        PIPE_TRY(hipMemcpy2DAsync(dA + (size_t)r0 * lda, (size_t)lda * sizeof(T), hA + (size_t)r0 * lda, (size_t)lda * sizeof(T),
-                                  (size_t)K * sizeof(T), rows, hipMemcpyHostToDevice, s_up));
+    int a_up = 0, b_up = 0;      // panels of A / B on the device (or on their way, in stream order)
+    for (int step = 0; step < steps; ++step) {
+        // whichever operand is behind goes next; A first
+        const bool next_is_a = b_up == panels_b || (a_up < panels_a && (long)a_up * panels_b <= (long)b_up * panels_a);
+        int r0, rows, c0, cols;      // the region of the result that this panel completes the operands of
+        if (next_is_a) {
+            r0 = a_up * pm, rows = M - r0 < pm ? M - r0 : pm;
+            c0 = 0, cols = b_up * pn < N ? b_up * pn : N;
+            PIPE_TRY(hipMemcpy2DAsync(dA + (size_t)r0 * lda, (size_t)lda * sizeof(T), hA + (size_t)r0 * lda, (size_t)lda * sizeof(T),
+                                      (size_t)K * sizeof(T), rows, hipMemcpyHostToDevice, s_up));
+            ++a_up;
+        } else {
+            c0 = b_up * pn, cols = N - c0 < pn ? N - c0 : pn;
+            r0 = 0, rows = a_up * pm < M ? a_up * pm : M;
+            PIPE_TRY(hipMemcpy2DAsync(dB + c0, (size_t)ldb * sizeof(T), hB + c0, (size_t)ldb * sizeof(T), (size_t)cols * sizeof(T), K,
+                                      hipMemcpyHostToDevice, s_up));
+            ++b_up;
+        }
+        if (rows == 0 || cols == 0) continue;      // the very first panel: its partner is not there yet
         if (hC)   // C goes into the result buffer and is accumulated onto in place, as the reference does (GEMM.h:196-206)
-            PIPE_TRY(hipMemcpy2DAsync(dD + (size_t)r0 * ldd, (size_t)ldd * sizeof(T), hC + (size_t)r0 * ldc, (size_t)ldc * sizeof(T),
-                                      (size_t)N * sizeof(T), rows, hipMemcpyHostToDevice, s_up));
-        PIPE_TRY(hipEventRecord(up[p], s_up));
-        PIPE_TRY(hipStreamWaitEvent(g_rt.stream, up[p], 0));
+            PIPE_TRY(hipMemcpy2DAsync(dD + (size_t)r0 * ldd + c0, (size_t)ldd * sizeof(T), hC + (size_t)r0 * ldc + c0,
+                                      (size_t)ldc * sizeof(T), (size_t)cols * sizeof(T), rows, hipMemcpyHostToDevice, s_up));
+        PIPE_TRY(hipEventRecord(up[step], s_up));
+        PIPE_TRY(hipStreamWaitEvent(g_rt.stream, up[step], 0));
         Batch one;
         one.stream = g_rt.stream;
-        rc = enqueue(dA + (size_t)r0 * lda, dB, hC ? dD + (size_t)r0 * ldd : nullptr, dD + (size_t)r0 * ldd, rows, one);
+        T* d_region = dD + (size_t)r0 * ldd + c0;
+        rc = enqueue(dA + (size_t)r0 * lda, dB + c0, hC ? d_region : nullptr, d_region, rows, cols, one);
         if (rc) { cleanup(); return rc; }
-        PIPE_TRY(hipEventRecord(done[p], g_rt.stream));
-        PIPE_TRY(hipStreamWaitEvent(s_down, done[p], 0));
-        PIPE_TRY(hipMemcpy2DAsync(hD + (size_t)r0 * ldd, (size_t)ldd * sizeof(T), dD + (size_t)r0 * ldd, (size_t)ldd * sizeof(T),
-                                  (size_t)N * sizeof(T), rows, hipMemcpyDeviceToHost, s_down));
+        PIPE_TRY(hipEventRecord(done[step], g_rt.stream));
+        PIPE_TRY(hipStreamWaitEvent(s_down, done[step], 0));
+        PIPE_TRY(hipMemcpy2DAsync(hD + (size_t)r0 * ldd + c0, (size_t)ldd * sizeof(T), d_region, (size_t)ldd * sizeof(T),
+                                  (size_t)cols * sizeof(T), rows, hipMemcpyDeviceToHost, s_down));
     }
     PIPE_TRY(hipStreamSynchronize(s_down));
     PIPE_TRY(hipStreamSynchronize(g_rt.stream));
@@ -1091,15 +1109,15 @@ int decx_hip_gemm3_host_f16(const uint16_t* hA, int lda, size_t plane_a, const u
 int decx_hip_gemm_host_f32(const float* hA, int lda, const float* hB, int ldb, const float* hC, int ldc, float* hD, int ldd,
                            int M, int N, int K) {
     return gemm_host_pipeline<float>(hA, lda, hB, ldb, hC, ldc, hD, ldd, M, N, K,
-                                     [&](const float* a, const float* b, const float* c, float* d, int rows, const Batch& one) {
-                                         return sgemm_enqueue(a, lda, b, ldb, c, ldd, d, ldd, rows, N, K, one);
+                                     [&](const float* a, const float* b, const float* c, float* d, int rows, int cols, const Batch& one) {
+                                         return sgemm_enqueue(a, lda, b, ldb, c, ldd, d, ldd, rows, cols, K, one);
                                      });
 }
 int decx_hip_gemm_host_f16(const uint16_t* hA, int lda, const uint16_t* hB, int ldb, const uint16_t* hC, int ldc, uint16_t* hD,
                            int ldd, int M, int N, int K) {
     return gemm_host_pipeline<uint16_t>(hA, lda, hB, ldb, hC, ldc, hD, ldd, M, N, K,
-                                        [&](const uint16_t* a, const uint16_t* b, const uint16_t* c, uint16_t* d, int rows, const Batch& one) {
-                                            return hgemm_enqueue(a, lda, b, ldb, c, ldd, d, ldd, rows, N, K, one);
+                                        [&](const uint16_t* a, const uint16_t* b, const uint16_t* c, uint16_t* d, int rows, int cols, const Batch& one) {
+                                            return hgemm_enqueue(a, lda, b, ldb, c, ldd, d, ldd, rows, cols, K, one);
                                         });
 }
 

@@ -191,9 +191,11 @@ def test_gemm3_host_pipeline(gpu):
     assert np.array_equal(D, (want + C).astype(np.float32))
 
 
-@pytest.mark.parametrize("shape", [(96, 40, 120), (2048 + 300, 72, 264), (5000, 33, 100)])
+@pytest.mark.parametrize("shape", [(96, 40, 120), (2048 + 300, 72, 264), (5000, 33, 100), (2100, 40, 2300), (300, 24, 5000),
+                                   (9000, 16, 3100)])
 def test_host_resident_gemm_pipeline(gpu, shape):
-    # decx_hip_gemm_host_f32: pitched host matrices in, pitched host matrix out; M above 2048 runs several row panels
+    # decx_hip_gemm_host_f32: pitched host matrices in, pitched host matrix out; above 1024 rows of A / columns of B the
+    # operands go up as several panels, and the result is computed and brought back region by region
     M, K, N = shape
     A, B = workloads.small_ints((M, K), 91), workloads.small_ints((K, N), 92)
     C = workloads.small_ints((M, N), 93, -50, 50)
@@ -216,7 +218,7 @@ def test_host_resident_gemm_pipeline(gpu, shape):
 
 
 def test_host_resident_gemm_pipeline_fp16(gpu, oracle):
-    M, K, N = 2048 + 100, 64, 144
+    M, K, N = 2048 + 100, 64, 1024 + 144
     A, B = workloads.small_ints((M, K), 94, -3, 3), workloads.small_ints((K, N), 95, -3, 3)
     Ah, Bh = oracle.float_to_half(A), oracle.float_to_half(B)
     D = np.zeros((M, N), np.uint16)
