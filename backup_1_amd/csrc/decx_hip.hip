@@ -14,6 +14,7 @@
 #include "sgemm_chain16.hpp"
 #include "conv_chain16.hpp"
 #include "hconv_tile.hpp"
+#include "hconv_dma.hpp"
 
 using namespace decx_hip;
 
@@ -404,6 +405,8 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
 //   7: as 4 with 2x4 waves of 128x64 (two waves per SIMD) -- the default for large problems: the chip is power-capped on
 //      this kernel (MFMA busy x clock stays ~1.27 GHz-equivalents whatever the schedule), and this one is 1 % ahead
 //  11: split-K on shape 8 through an fp32 workspace (hgemm_splitk_enqueue) -- few tiles and a long K
+// and, for the fp16 convolution only: 12 keeps its register-staged kernels, 13 takes its LDS-DMA kernel for any image
+// whose channel pitch allows it; either switches its split over K off (experiments and tests)
 typedef HgemmShape<256, 256, 32, 2, 2> HShapeBig;
 typedef HgemmShape<128, 128, 32, 2, 2> HShapeSmall;
 typedef HgemmDmaShape<256, 256, 32, 2, 2, 4> HShapeDma;
@@ -559,6 +562,7 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
 // fp16 convolution (hconv_tile.hpp).  Strides and pitches in halves, as the binary16 containers hold them.
 typedef HconvShape<128, 128, 2, 2, 4> HconvSquare;   // 2x2 waves of 64x64
 typedef HconvShape<256, 128, 4, 2, 4> HconvTall;     // 4x2 waves of 64x64, two per SIMD: half the filter reads per pixel
+typedef HconvDmaShape<256, 128, 4, 2, 3> HconvDma;   // the tall tile fed by LDS-DMA loads, three K steps in LDS
 int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_stride, const uint16_t* filt, int N, int kh,
                   int kw, size_t filt_stride, size_t filt_row_stride, uint16_t* dst, int dst_dpitch, size_t dst_row_stride,
                   int flag, const uint16_t* bias, bool relu) {
@@ -614,7 +618,8 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
     const int all_steps = cdiv(Kw, 32);
     const long square_tiles = (long)cdiv(M, 128) * tiles_n;
     int splits = 1;
-    if (!tall && 2 * square_tiles <= cus && all_steps >= 8 && (size_t)M * N <= ((size_t)1 << 26)) {
+    const bool kernel_forced = g_rt.hgemm_variant == 12 || g_rt.hgemm_variant == 13;      // experiments and tests: no split
+    if (!kernel_forced && !tall && 2 * square_tiles <= cus && all_steps >= 8 && (size_t)M * N <= ((size_t)1 << 26)) {
         const double t_whole = 4.0 + 0.75 * all_steps;
         double best = 0.85 * t_whole;
         const long most = (2 * cus + square_tiles - 1) / square_tiles;
@@ -647,6 +652,20 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
             hipLaunchKernelGGL((hconv_tile_kernel<HconvSquare, false, true>), grid, dim3(HconvSquare::NT), HconvSquare::LDS_BYTES,
                                g_rt.stream, img, fb, out, M, N, Kw, tiles_n, g_rt.partial, steps_per_split);
         hipLaunchKernelGGL(hconv_split_finish_kernel, dim3(fill_blocks), dim3(256), 0, g_rt.stream, g_rt.partial, out, M, N);
+        HIP_TRY(hipGetLastError());
+        return 0;
+    }
+    // hgemm variant 12 keeps the register-staged kernels, 13 takes the LDS-DMA kernel wherever it can run (experiments)
+    if (tap_uniform && g_rt.hgemm_variant != 12 && (tall || g_rt.hgemm_variant == 13)) {
+        static bool dma_attr_done = false;
+        if (!dma_attr_done) {
+            HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hconv_dma_kernel<HconvDma>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)HconvDma::LDS_BYTES));
+            dma_attr_done = true;
+        }
+        const long dma_tiles = (long)cdiv(M, HconvDma::BM) * tiles_n;
+        hipLaunchKernelGGL(hconv_dma_kernel<HconvDma>, dim3((unsigned)dma_tiles), dim3(HconvDma::NT), HconvDma::LDS_BYTES, g_rt.stream,
+                           img, fb, out, M, N, Kw, tiles_n);
         HIP_TRY(hipGetLastError());
         return 0;
     }

@@ -78,6 +78,62 @@ __device__ __forceinline__ void small_divmod(int m, int d, float rcp_d, int& quo
     rem = r;
 }
 
+// Epilogue of the fp16 convolution kernels.  Lane (li, lh) holds for pixel wm0 + 32 mi + li the filters
+// wn0 + 32 ni + 8 j + 4 lh + e (e = 0..3) in acc[mi][ni][4 j + e]: bias, ReLU and one rounding to binary16 per run of
+// four, then through LDS (which must be free: no reader of the operand buffers left, no load into them in flight) so
+// that the tile leaves in 16-byte pieces.
+template <class S, class PixelOf>
+__device__ __forceinline__ void hconv_store_tile(const f32x16 (&acc)[S::MI][S::NI], unsigned char* lds_raw, const HalfTensorOut& out,
+                                                 int M, int N, int bm0, int bn0, int wm0, int wn0, int tid, const PixelOf& pixel_of) {
+    constexpr int BM = S::BM, BN = S::BN, NT = S::NT, MI = S::MI, NI = S::NI;
+    const int lane = tid % kWave, li = lane & 31, lh = lane >> 5;
+    typedef _Float16 f16x4v __attribute__((ext_vector_type(4)));
+    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+    _Float16* tile = reinterpret_cast<_Float16*>(lds_raw);                                   // [BM][OUT_ROW]
+    float* bias_lds = reinterpret_cast<float*>(lds_raw + (size_t)BM * S::OUT_ROW * 2);         // [BN]
+    if (out.bias != nullptr) {
+        for (int i = tid; i < BN; i += NT) bias_lds[i] = bn0 + i < N ? (float)out.bias[bn0 + i] : 0.f;
+        __syncthreads();
+    }
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int n_local = wn0 + ni * 32 + 8 * j + 4 * lh;
+                f32x4 v = {acc[mi][ni][4 * j], acc[mi][ni][4 * j + 1], acc[mi][ni][4 * j + 2], acc[mi][ni][4 * j + 3]};
+                if (out.bias != nullptr) v += *reinterpret_cast<const f32x4*>(bias_lds + n_local);
+                if (out.relu) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = relu_by_sign(v[e]);
+                }
+                const f16x4v h = __builtin_convertvector(v, f16x4v);
+                *reinterpret_cast<u32x2*>(tile + (wm0 + mi * 32 + li) * S::OUT_ROW + n_local) = __builtin_bit_cast(u32x2, h);
+            }
+    __syncthreads();
+    constexpr int UNITS_PER_ROW = BN / 8, OUT_PASSES = BM * UNITS_PER_ROW / NT;
+    // whole 16-byte units when dst allows it (pixel pitch a multiple of 8 halves, 16-byte aligned base), else half by half
+    const bool vec = out.dpitch % 8 == 0 && out.row_stride % 8 == 0 && (reinterpret_cast<size_t>(out.dst) & 15) == 0;
+#pragma unroll
+    for (int p = 0; p < OUT_PASSES; ++p) {
+        const int id = tid + p * NT, row = id / UNITS_PER_ROW, u = id % UNITS_PER_ROW;
+        const int m = bm0 + row, n = bn0 + 8 * u;
+        if (m < M && n < N) {
+            int y, x;
+            pixel_of(m, y, x);
+            _Float16* pix = out.dst + (size_t)y * out.row_stride + (size_t)x * out.dpitch + n;
+            const _Float16* t8 = tile + row * S::OUT_ROW + 8 * u;          // 8-byte aligned
+            if (vec && n + 8 <= N) {
+                const u32x2 lo = *reinterpret_cast<const u32x2*>(t8), hi = *reinterpret_cast<const u32x2*>(t8 + 4);
+                *reinterpret_cast<u32x4*>(pix) = u32x4{lo[0], lo[1], hi[0], hi[1]};
+            } else {
+                for (int e = 0; e < 8 && n + e < N; ++e) pix[e] = t8[e];
+            }
+        }
+    }
+}
+
 // TAP_UNIFORM (channel pitch a multiple of 64 halves, i.e. of a K step): a K step lies inside one tap, so the walk over
 // (tap row, tap column, channel) is the same for every lane up to a constant and runs on the scalar unit; a load then
 // costs the vector unit one add (plus the column check of an image load), and a filter load nothing at all.
@@ -267,55 +323,8 @@ __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, Hal
             }
         return;
     }
-    // Epilogue.  Lane (li, lh) holds for pixel wm0 + 32 mi + li the filters wn0 + 32 ni + 8 j + 4 lh + e (e = 0..3) in
-    // acc[mi][ni][4 j + e]: bias, ReLU and one rounding to binary16 per run of four, then through LDS (free now) so that
-    // the tile leaves in 16-byte pieces.
-    typedef _Float16 f16x4v __attribute__((ext_vector_type(4)));
-    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-    _Float16* tile = reinterpret_cast<_Float16*>(lds_raw);                                   // [BM][OUT_ROW]
-    float* bias_lds = reinterpret_cast<float*>(lds_raw + (size_t)BM * S::OUT_ROW * 2);         // [BN]
     __syncthreads();                                           // everybody is done reading the last operand buffer
-    if (out.bias != nullptr) {
-        for (int i = tid; i < BN; i += NT) bias_lds[i] = bn0 + i < N ? (float)out.bias[bn0 + i] : 0.f;
-        __syncthreads();
-    }
-#pragma unroll
-    for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int n_local = wn0 + ni * 32 + 8 * j + 4 * lh;
-                f32x4 v = {acc[mi][ni][4 * j], acc[mi][ni][4 * j + 1], acc[mi][ni][4 * j + 2], acc[mi][ni][4 * j + 3]};
-                if (out.bias != nullptr) v += *reinterpret_cast<const f32x4*>(bias_lds + n_local);
-                if (out.relu) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] = relu_by_sign(v[e]);
-                }
-                const f16x4v h = __builtin_convertvector(v, f16x4v);
-                *reinterpret_cast<u32x2*>(tile + (wm0 + mi * 32 + li) * S::OUT_ROW + n_local) = __builtin_bit_cast(u32x2, h);
-            }
-    __syncthreads();
-    constexpr int UNITS_PER_ROW = BN / 8, OUT_PASSES = BM * UNITS_PER_ROW / NT;
-    // whole 16-byte units when dst allows it (pixel pitch a multiple of 8 halves, 16-byte aligned base), else half by half
-    const bool vec = out.dpitch % 8 == 0 && out.row_stride % 8 == 0 && (reinterpret_cast<size_t>(out.dst) & 15) == 0;
-#pragma unroll
-    for (int p = 0; p < OUT_PASSES; ++p) {
-        const int id = tid + p * NT, row = id / UNITS_PER_ROW, u = id % UNITS_PER_ROW;
-        const int m = bm0 + row, n = bn0 + 8 * u;
-        if (m < M && n < N) {
-            int y, x;
-            pixel_of(m, y, x);
-            _Float16* pix = out.dst + (size_t)y * out.row_stride + (size_t)x * out.dpitch + n;
-            const _Float16* t8 = tile + row * S::OUT_ROW + 8 * u;          // 8-byte aligned
-            if (vec && n + 8 <= N) {
-                const u32x2 lo = *reinterpret_cast<const u32x2*>(t8), hi = *reinterpret_cast<const u32x2*>(t8 + 4);
-                *reinterpret_cast<u32x4*>(pix) = u32x4{lo[0], lo[1], hi[0], hi[1]};
-            } else {
-                for (int e = 0; e < 8 && n + e < N; ++e) pix[e] = t8[e];
-            }
-        }
-    }
+    hconv_store_tile<S>(acc, lds_raw, out, M, N, bm0, bn0, wm0, wn0, tid, pixel_of);
 }
 
 // dst(pixel m, filter n) = half(relu(partial[m][n] + bias[n])): the end of a split-K convolution.

@@ -131,7 +131,7 @@ def half_tensor_storage(t16, pad_bits=0x7e00):
     return buf, wp, dp
 
 
-def gpu_hconv(src16, filt16, flag, bias16=None, relu=False):
+def gpu_hconv(src16, filt16, flag, bias16=None, relu=False, variant=0):
     """fp16 convolution through the C ABI: src16 (H, W, C), filt16 (N, kh, kw, C), bias16 (N,) float16 arrays.
     Returns (dst float16 (H_out, W_out, N), the image storage, the filter storage) -- the storages, as uint16 views
     without their width padding, are what the oracle is fed."""
@@ -149,8 +149,12 @@ def gpu_hconv(src16, filt16, flag, bias16=None, relu=False):
     dS, dF, dD = (capi.DeviceBuffer.from_numpy(sbuf), capi.DeviceBuffer.from_numpy(fb),
                   capi.DeviceBuffer.from_numpy(sentinel))
     dB = capi.DeviceBuffer.from_numpy(np.asarray(bias16, dtype=np.float16).view(np.uint16)) if bias16 is not None else None
-    capi.check(capi.lib().decx_hip_conv2_im2col_f16(dS.ptr, H, W, dp, swp * dp, dF.ptr, N, kh, kw, kh * fwp * dp, fwp * dp,
-                                                    dD.ptr, ddp, dwp * ddp, flag, dB.ptr if dB else None, 1 if relu else 0))
+    prev = capi.lib().decx_hip_set_hgemm_variant(variant)      # 12 / 13: the register-staged / the LDS-DMA kernel
+    try:
+        capi.check(capi.lib().decx_hip_conv2_im2col_f16(dS.ptr, H, W, dp, swp * dp, dF.ptr, N, kh, kw, kh * fwp * dp, fwp * dp,
+                                                        dD.ptr, ddp, dwp * ddp, flag, dB.ptr if dB else None, 1 if relu else 0))
+    finally:
+        capi.lib().decx_hip_set_hgemm_variant(prev)
     out = dD.download((Ho, dwp, ddp), np.uint16)
     assert np.all(out[:, Wout:, :] == 0xd610) and np.all(out[:, :, N:] == 0xd610), "kernel wrote into dst padding"
     return out[:Hout, :Wout, :N].copy().view(np.float16), sbuf[:, :W], fb[:, :, :kw]

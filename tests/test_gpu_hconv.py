@@ -134,6 +134,32 @@ def test_small_images_split_the_walk_over_k(gpu, oracle, case):
         assert check_against_f64(oracle, got, sbuf, fb, 1, bias16=b, relu=r) < TOL
 
 
+# channel pitch a multiple of 64 halves: a K step lies inside one tap, which is what the LDS-DMA kernel needs.  It is the
+# default from about 200 tiles of 256 pixels on; variant 13 takes it for any image, 12 keeps the register-staged kernel.
+DMA_CASES = [(20, 22, 64, 6, 3, 3), (16, 16, 64, 128, 3, 3), (33, 17, 128, 130, 1, 1), (12, 40, 64, 5, 5, 3), (7, 7, 64, 1, 7, 7),
+             (64, 48, 64, 200, 3, 3), (30, 26, 192, 70, 3, 3), (40, 37, 60, 33, 3, 3)]
+
+
+@pytest.mark.parametrize("variant", [13, 12])
+@pytest.mark.parametrize("flag", [1, 0])
+@pytest.mark.parametrize("case", DMA_CASES)
+def test_dma_kernel_and_register_kernel_on_the_same_cases(gpu, oracle, case, flag, variant):
+    H, W, C, N, kh, kw = case
+    if flag == 0 and (H <= 2 * (kh // 2) or W <= 2 * (kw // 2)):
+        pytest.skip("no valid region")
+    si = workloads.small_ints((H, W, C), 871, -1, 1).astype(np.float16)
+    fi = workloads.small_ints((N, kh, kw, C), 872, -1, 1).astype(np.float16)
+    got, sbuf, fb = gpu_hconv(si, fi, flag, variant=variant)
+    ref, scale = oracle.conv2_f64_f16(sbuf, fb, flag)
+    assert scale.max() < 2048
+    assert np.array_equal(got.astype(np.float64), ref)
+    src = workloads.uniform_01((H, W, C), 873).astype(np.float16)
+    filt = workloads.normal((N, kh, kw, C), 874, sigma=0.05).astype(np.float16)
+    bias = workloads.normal((N,), 875).astype(np.float16)
+    got, sbuf, fb = gpu_hconv(src, filt, flag, bias16=bias, relu=True, variant=variant)
+    assert check_against_f64(oracle, got, sbuf, fb, flag, bias16=bias, relu=True) < TOL
+
+
 def test_error_codes(gpu):
     L = capi.lib()
     d = capi.DeviceBuffer(1 << 16)
