@@ -208,12 +208,13 @@ __global__ __launch_bounds__(S::NT) void hconv_dma_kernel(HalfImage img, HalfFil
 #pragma unroll
     for (int r = 0; r < FRAG_READS; ++r) read_one(f0, 0, 0, r);
     DECX_PIN();
-    int stg = 0;
-    for (int t = 0; t < steps; ++t) {
-        const int next = stg + 1 == STAGES ? 0 : stg + 1;
-        k_step(stg, next, t + 1 < steps);
-        stg = next;
-    }
+    // unrolled over the LDS buffers: the buffer of a step is then a compile-time constant and folds into the offset fields
+    // of its fragment reads
+    for (int t0 = 0; t0 < steps; t0 += STAGES)
+        static_for<0, STAGES>([&](auto d) {
+            constexpr int STG = decltype(d)::value;
+            if (t0 + STG < steps) k_step(STG, (STG + 1) % STAGES, t0 + STG + 1 < steps);
+        });
 #undef DECX_PIN
     // the loads past the end of K still write (zeros) when they land: wait for them before LDS becomes the result tile
     wait_dma_then_barrier<0>();
