@@ -15,6 +15,7 @@
 #include "conv_chain16.hpp"
 #include "hconv_tile.hpp"
 #include "hconv_dma.hpp"
+#include "hconv_taprow.hpp"
 
 using namespace decx_hip;
 
@@ -618,7 +619,7 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
     const int all_steps = cdiv(Kw, 32);
     const long square_tiles = (long)cdiv(M, 128) * tiles_n;
     int splits = 1;
-    const bool kernel_forced = g_rt.hgemm_variant == 12 || g_rt.hgemm_variant == 13;      // experiments and tests: no split
+    const bool kernel_forced = g_rt.hgemm_variant >= 12 && g_rt.hgemm_variant <= 14;      // experiments and tests: no split
     if (!kernel_forced && !tall && 2 * square_tiles <= cus && all_steps >= 8 && (size_t)M * N <= ((size_t)1 << 26)) {
         const double t_whole = 4.0 + 0.75 * all_steps;
         double best = 0.85 * t_whole;
@@ -652,6 +653,24 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
             hipLaunchKernelGGL((hconv_tile_kernel<HconvSquare, false, true>), grid, dim3(HconvSquare::NT), HconvSquare::LDS_BYTES,
                                g_rt.stream, img, fb, out, M, N, Kw, tiles_n, g_rt.partial, steps_per_split);
         hipLaunchKernelGGL(hconv_split_finish_kernel, dim3(fill_blocks), dim3(256), 0, g_rt.stream, g_rt.partial, out, M, N);
+        HIP_TRY(hipGetLastError());
+        return 0;
+    }
+    // 3x3-wide filters: the LDS-DMA kernel that loads a tap row's pixels once for its three taps, if a tile's patch fits
+    // its 320 rows (255 + kw positions plus kw - 1 per image row the tile touches).  hgemm variant 14 takes it for any image.
+    const int rows_touched = (254 + Wout) / Wout + 1;
+    const bool taprow_fits = tap_uniform && kw == HconvTapRowShape::KW && 255 + kw + (kw - 1) * rows_touched <= HconvTapRowShape::PATCH_ROWS &&
+                             (long)H * W < (1L << 22);
+    if (taprow_fits && ((tall && (g_rt.hgemm_variant < 12 || g_rt.hgemm_variant > 13)) || g_rt.hgemm_variant == 14)) {
+        typedef HconvTapRowShape S;
+        static bool taprow_attr_done = false;
+        if (!taprow_attr_done) {
+            HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hconv_taprow_kernel<S>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                        (int)S::LDS_BYTES));
+            taprow_attr_done = true;
+        }
+        const long tiles = (long)cdiv(M, S::BM) * tiles_n;
+        hipLaunchKernelGGL(hconv_taprow_kernel<S>, dim3((unsigned)tiles), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, out, M, N, tiles_n);
         HIP_TRY(hipGetLastError());
         return 0;
     }

@@ -140,7 +140,7 @@ DMA_CASES = [(20, 22, 64, 6, 3, 3), (16, 16, 64, 128, 3, 3), (33, 17, 128, 130, 
              (64, 48, 64, 200, 3, 3), (30, 26, 192, 70, 3, 3), (40, 37, 60, 33, 3, 3)]
 
 
-@pytest.mark.parametrize("variant", [13, 12])
+@pytest.mark.parametrize("variant", [14, 13, 12])
 @pytest.mark.parametrize("flag", [1, 0])
 @pytest.mark.parametrize("case", DMA_CASES)
 def test_dma_kernel_and_register_kernel_on_the_same_cases(gpu, oracle, case, flag, variant):
