@@ -407,7 +407,7 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
 //      this kernel (MFMA busy x clock stays ~1.27 GHz-equivalents whatever the schedule), and this one is 1 % ahead
 //  11: split-K on shape 8 through an fp32 workspace (hgemm_splitk_enqueue) -- few tiles and a long K
 // and, for the fp16 convolution only: 12 keeps its register-staged kernels, 13 takes its LDS-DMA kernel for any image
-// whose channel pitch allows it; either switches its split over K off (experiments and tests)
+// whose channel pitch allows it, 14 its tap-row kernel; each switches its split over K off (experiments and tests)
 typedef HgemmShape<256, 256, 32, 2, 2> HShapeBig;
 typedef HgemmShape<128, 128, 32, 2, 2> HShapeSmall;
 typedef HgemmDmaShape<256, 256, 32, 2, 2, 4> HShapeDma;
@@ -656,23 +656,30 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
         HIP_TRY(hipGetLastError());
         return 0;
     }
-    // 3x3-wide filters: the LDS-DMA kernel that loads a tap row's pixels once for its three taps, if a tile's patch fits
-    // its 320 rows (255 + kw positions plus kw - 1 per image row the tile touches).  hgemm variant 14 takes it for any image.
+    // filters 3, 5 or 7 wide: the LDS-DMA kernel that loads a tap row's pixels once for all of its taps, if a tile's patch
+    // fits its 320 rows (255 + kw positions plus kw - 1 per image row the tile touches).  hgemm variant 14 takes it for
+    // any image.
     const int rows_touched = (254 + Wout) / Wout + 1;
-    const bool taprow_fits = tap_uniform && kw == HconvTapRowShape::KW && 255 + kw + (kw - 1) * rows_touched <= HconvTapRowShape::PATCH_ROWS &&
+    const bool taprow_fits = tap_uniform && (kw == 3 || kw == 5 || kw == 7) && 255 + kw + (kw - 1) * rows_touched <= 320 &&
                              (long)H * W < (1L << 22);
     if (taprow_fits && ((tall && (g_rt.hgemm_variant < 12 || g_rt.hgemm_variant > 13)) || g_rt.hgemm_variant == 14)) {
-        typedef HconvTapRowShape S;
-        static bool taprow_attr_done = false;
-        if (!taprow_attr_done) {
-            HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hconv_taprow_kernel<S>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                        (int)S::LDS_BYTES));
-            taprow_attr_done = true;
-        }
-        const long tiles = (long)cdiv(M, S::BM) * tiles_n;
-        hipLaunchKernelGGL(hconv_taprow_kernel<S>, dim3((unsigned)tiles), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, out, M, N, tiles_n);
-        HIP_TRY(hipGetLastError());
-        return 0;
+        auto launch_taprow = [&](auto shape) -> int {
+            typedef decltype(shape) S;
+            static_assert(S::PATCH_ROWS == 320, "the fit test above is written for this patch");
+            static bool attr_done = false;           // one per shape: the lambda's body is instantiated per S
+            if (!attr_done) {
+                HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hconv_taprow_kernel<S>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            (int)S::LDS_BYTES));
+                attr_done = true;
+            }
+            const long tiles = (long)cdiv(M, S::BM) * tiles_n;
+            hipLaunchKernelGGL(hconv_taprow_kernel<S>, dim3((unsigned)tiles), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, out, M, N, tiles_n);
+            HIP_TRY(hipGetLastError());
+            return 0;
+        };
+        if (kw == 3) return launch_taprow(HconvTapRowShape<3>{});
+        if (kw == 5) return launch_taprow(HconvTapRowShape<5>{});
+        return launch_taprow(HconvTapRowShape<7>{});
     }
     // hgemm variant 12 keeps the register-staged kernels, 13 takes the LDS-DMA kernel wherever it can run (experiments)
     if (tap_uniform && g_rt.hgemm_variant != 12 && (tall || g_rt.hgemm_variant == 13)) {

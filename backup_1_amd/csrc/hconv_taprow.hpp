@@ -18,21 +18,24 @@
 // K is walked in the order (ki, channel block, kj) -- not the order of the other kernels, which for binary16 results
 // (no reference bits to match, fp32 accumulation, one rounding) changes nothing but the last bit of a sum.
 //
-// Pipeline: two patch buffers (80 KB) and a ring of four filter buffers (64 KB).  Step t = 3 s + j (row step s, tap j)
+// Pipeline: two patch buffers (80 KB) and a ring of four filter buffers (64 KB).  Step t = kw s + j (row step s, tap j)
 // computes from patch s % 2 and filter buffer t % 4; its barrier sits inside its last block of MFMAs, after it the filter
 // loads of step t + 4 go out and, when j = kw - 1, the patch loads of row step s + 2.  Loads past the end ask for
 // out-of-range offsets, so the number of loads in flight at each wait only depends on j:
-//   program order of a wave's loads ... B(t+1) | B(t+2) | A(s+1) B(t+3) ...   with A(s+1) issued after step 3(s-1)+2
+//   program order of a wave's loads ... B(t+1) | B(t+2) | A(s+1) B(t+3) ...   with A(s+1) issued after the last tap of row step s-1
 //   j = 0: B(t+1), B(t+2), A(s+1), B(t+3)      need B(t+1)          -> at most 2 + 5 + 2 younger loads outstanding
 //   j = 1: B(t+1), A(s+1), B(t+2), B(t+3)      need B(t+1)          -> 5 + 2 + 2
-//   j = 2: A(s+1), B(t+1), B(t+2), B(t+3)      need A(s+1), B(t+1)  -> 2 + 2
+//   j > 1: A(s+1) .. B(t+1), B(t+2), B(t+3)    need B(t+1), and A(s+1) after the last tap -> 2 + 2
+// (kw = 3, 5 and 7 are built; the patch, the tap and the filter buffer of a step repeat with period 4 kw.)
 #pragma once
 #include "hconv_dma.hpp"
 
 namespace decx_hip {
 
+template <int KW_>
 struct HconvTapRowShape {
-    static constexpr int BM = 256, BN = 128, BK = 64, WAVES_M = 4, WAVES_N = 2, KW = 3;
+    static constexpr int BM = 256, BN = 128, BK = 64, WAVES_M = 4, WAVES_N = 2, KW = KW_;
+    static_assert(KW >= 3 && KW % 2 == 1, "the wait counts of the kernel are derived for odd widths from 3 on");
     static constexpr int NWAVES = WAVES_M * WAVES_N, NT = NWAVES * kWave;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     static constexpr int MI = WM / 32, NI = WN / 32;
@@ -184,7 +187,7 @@ __global__ __launch_bounds__(S::NT) void hconv_taprow_kernel(HalfImage img, Half
     Frags f0, f1;
     static_assert(KS % 2 == 0, "fragment sets must line up across K steps (block 0 always in f0)");
 
-    // Step I of a run of 12 (patch buffer, tap and filter buffer repeat with period 12).  f0 holds the fragments of its first
+    // Step I of a run of 4 kw (patch buffer, tap and filter buffer repeat with that period).  f0 holds the fragments of its first
     // k-block on entry and those of the next step's first k-block on exit.
     auto k_step = [&](auto step_tag, bool has_next) {
         constexpr int I = decltype(step_tag)::value, J = I % KW;
@@ -208,7 +211,7 @@ __global__ __launch_bounds__(S::NT) void hconv_taprow_kernel(HalfImage img, Half
         mfma_one(fl, 0);
         DECX_PIN();
         // what the next step reads has landed (see the table at the top), my reads of this step's buffers are done
-        wait_dma_then_barrier<(J == KW - 1 ? 2 * S::B_LOADS : S::A_LOADS + 2 * S::B_LOADS)>();
+        wait_dma_then_barrier<(J >= 2 ? 2 * S::B_LOADS : S::A_LOADS + 2 * S::B_LOADS)>();
         DECX_PIN();
         // three MFMAs left: between them the refills -- the patch of row step s + 2 after the last tap, the filters of step
         // t + 4 -- and the next step's first fragments
@@ -245,8 +248,8 @@ __global__ __launch_bounds__(S::NT) void hconv_taprow_kernel(HalfImage img, Half
         static_for<0, FRAG_READS>([&](auto r) { read_one(f0, Z{}, Z{}, Z{}, 0, decltype(r)::value); });
     }
     DECX_PIN();
-    for (int t0 = 0; t0 < steps; t0 += 12)
-        static_for<0, 12>([&](auto i) {
+    for (int t0 = 0; t0 < steps; t0 += 4 * KW)
+        static_for<0, 4 * KW>([&](auto i) {
             if (t0 + decltype(i)::value < steps) k_step(i, t0 + decltype(i)::value + 1 < steps);
         });
 #undef DECX_PIN

@@ -135,9 +135,11 @@ def test_small_images_split_the_walk_over_k(gpu, oracle, case):
 
 
 # channel pitch a multiple of 64 halves: a K step lies inside one tap, which is what the LDS-DMA kernel needs.  It is the
-# default from about 200 tiles of 256 pixels on; variant 13 takes it for any image, 12 keeps the register-staged kernel.
+# default from about 200 tiles of 256 pixels on; variant 13 takes it for any image, 12 keeps the register-staged kernel, 14
+# takes the kernel that loads a tap row's pixels once for all of its taps (filters 3, 5 or 7 wide).
 DMA_CASES = [(20, 22, 64, 6, 3, 3), (16, 16, 64, 128, 3, 3), (33, 17, 128, 130, 1, 1), (12, 40, 64, 5, 5, 3), (7, 7, 64, 1, 7, 7),
-             (64, 48, 64, 200, 3, 3), (30, 26, 192, 70, 3, 3), (40, 37, 60, 33, 3, 3)]
+             (64, 48, 64, 200, 3, 3), (30, 26, 192, 70, 3, 3), (40, 37, 60, 33, 3, 3), (40, 44, 64, 20, 5, 5), (36, 60, 64, 9, 7, 7),
+             (300, 20, 128, 140, 3, 5)]
 
 
 @pytest.mark.parametrize("variant", [14, 13, 12])
