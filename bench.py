@@ -80,9 +80,9 @@ def bench_hgemm(capi, workloads, n, steps, warmup, seed, shape=None):
     return {"ms_wall": wall, "ms_kernel": ev, "tflops": flops / (wall * 1e-3) / 1e12, "tflops_kernel": flops / (ev * 1e-3) / 1e12}
 
 
-def bench_conv(capi, workloads, steps, warmup):
-    H = W = 224; C = 64; N = 128; kh = kw = 3
-    src, filt = workloads.conv_case()
+def bench_conv(capi, workloads, steps, warmup, H=224, W=224, C=64, N=128):
+    kh = kw = 3
+    src, filt = workloads.conv_case(H=H, W=W, C=C, N=N)
     fb = np.zeros((N, kh, 4, C), np.float32); fb[:, :, :kw, :] = filt       # TensorArray: wpitch = ceil4(kw)
     dS, dF = capi.DeviceBuffer.from_numpy(src), capi.DeviceBuffer.from_numpy(fb)
     dD = capi.DeviceBuffer(H * W * N * 4)
@@ -93,10 +93,10 @@ def bench_conv(capi, workloads, steps, warmup):
     return {"ms_wall": wall, "ms_kernel": ev, "tflops": flops / (wall * 1e-3) / 1e12, "tflops_kernel": flops / (ev * 1e-3) / 1e12}
 
 
-def bench_hconv(capi, workloads, steps, warmup):
+def bench_hconv(capi, workloads, steps, warmup, H=224, W=224, C=64, N=128):
     """config 4 in binary16 with fp32 accumulation (decx_hip_conv2_im2col_f16_async); same flop count as bench_conv."""
-    H = W = 224; C = 64; N = 128; kh = kw = 3
-    src, filt = workloads.conv_case()
+    kh = kw = 3
+    src, filt = workloads.conv_case(H=H, W=W, C=C, N=N)
     fb = np.zeros((N, kh, 4, C), np.float16); fb[:, :, :kw, :] = filt.astype(np.float16)
     dS, dF = capi.DeviceBuffer.from_numpy(src.astype(np.float16).view(np.uint16)), capi.DeviceBuffer.from_numpy(fb.view(np.uint16))
     dD = capi.DeviceBuffer(H * W * N * 2)
@@ -331,6 +331,19 @@ def main():
             "tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
             "frac_of_fp16_dense_peak": round(r["tflops_kernel"] / PEAK_FP16_MATRIX_TFLOPS, 4)}
         log("fp16 conv: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+        # config 4 is 15 - 75 us of work, a good part of it launch, first loads and the write of the result; the same
+        # kernels on an image that fills the chip for several rounds of tiles show what their K loops sustain
+        big = dict(H=512, W=512, C=256, N=256)
+        r = bench_conv(capi, workloads, side_steps, side_warmup, **big)
+        also["fp32_conv_512x512x256_256f3x3_fused_im2col"] = {
+            "tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
+            "frac_of_fp32_matrix_peak": round(r["tflops_kernel"] / PEAK_FP32_MATRIX_TFLOPS, 4)}
+        log("conv 512x512x256 -> 256: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+        r = bench_hconv(capi, workloads, side_steps, side_warmup, **big)
+        also["fp16_conv_512x512x256_256f3x3_f32acc_fused_im2col"] = {
+            "tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
+            "frac_of_fp16_dense_peak": round(r["tflops_kernel"] / PEAK_FP16_MATRIX_TFLOPS, 4)}
+        log("fp16 conv 512x512x256 -> 256: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
 
     if want("relu"):
         r = bench_relu(capi, workloads, side_steps, side_warmup)
