@@ -99,6 +99,12 @@ def test_headline_shape_sampled(gpu, oracle):
     filt = workloads.normal((128, 3, 3, 64), 842, sigma=0.05).astype(np.float16)
     got, sbuf, fb = gpu_hconv(src, filt, 1)
     assert check_against_f64(oracle, got, sbuf, fb, 1) < TOL
+    # the library's choice is the tap-row kernel; the LDS-DMA and the register-staged kernels must agree with it to the
+    # rounding of the result (they add the same fp32 products in another order)
+    for variant in (12, 13, 14):
+        other, _, _ = gpu_hconv(src, filt, 1, variant=variant)
+        diff = np.abs(other.astype(np.float64) - got.astype(np.float64))
+        assert np.all(diff <= 2.0 ** -9 * np.maximum(np.abs(got.astype(np.float64)), 1.0)), variant
 
 
 def test_many_pixels_take_the_tall_tile(gpu, oracle):
