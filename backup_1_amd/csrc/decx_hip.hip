@@ -658,11 +658,13 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
     }
     // filters 3, 5 or 7 wide: the LDS-DMA kernel that loads a tap row's pixels once for all of its taps, if a tile's patch
     // fits its 320 rows (255 + kw positions plus kw - 1 per image row the tile touches).  hgemm variant 14 takes it for
-    // any image.
+    // any image; its tiles are 64 filters wide when there are no more filters than that.
     const int rows_touched = (254 + Wout) / Wout + 1;
     const bool taprow_fits = tap_uniform && (kw == 3 || kw == 5 || kw == 7) && 255 + kw + (kw - 1) * rows_touched <= 320 &&
                              (long)H * W < (1L << 22);
-    if (taprow_fits && ((tall && (g_rt.hgemm_variant < 12 || g_rt.hgemm_variant > 13)) || g_rt.hgemm_variant == 14)) {
+    const bool narrow = N <= 64;
+    const bool many_tiles = narrow ? (long)cdiv(M, 256) >= 3 * cus / 4 : tall;
+    if (taprow_fits && ((many_tiles && (g_rt.hgemm_variant < 12 || g_rt.hgemm_variant > 13)) || g_rt.hgemm_variant == 14)) {
         auto launch_taprow = [&](auto shape) -> int {
             typedef decltype(shape) S;
             static_assert(S::PATCH_ROWS == 320, "the fit test above is written for this patch");
@@ -672,14 +674,43 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
                                             (int)S::LDS_BYTES));
                 attr_done = true;
             }
-            const long tiles = (long)cdiv(M, S::BM) * tiles_n;
-            hipLaunchKernelGGL(hconv_taprow_kernel<S>, dim3((unsigned)tiles), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, out, M, N, tiles_n);
+            const int tn = cdiv(N, S::BN);
+            const long tiles = (long)cdiv(M, S::BM) * tn;
+            hipLaunchKernelGGL(hconv_taprow_kernel<S>, dim3((unsigned)tiles), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, out, M, N, tn);
             HIP_TRY(hipGetLastError());
             return 0;
         };
+        if (narrow) {      // 8x1 waves of 32 pixels x 64 filters
+            if (kw == 3) return launch_taprow(HconvTapRowShape<3, 64, 8, 1>{});
+            if (kw == 5) return launch_taprow(HconvTapRowShape<5, 64, 8, 1>{});
+            return launch_taprow(HconvTapRowShape<7, 64, 8, 1>{});
+        }
         if (kw == 3) return launch_taprow(HconvTapRowShape<3>{});
         if (kw == 5) return launch_taprow(HconvTapRowShape<5>{});
         return launch_taprow(HconvTapRowShape<7>{});
+    }
+    // at most 64 filters: tiles 64 filters wide (the 128-wide ones would spend half of their MFMAs on filters that do not exist)
+    if (narrow && g_rt.hgemm_variant != 13) {
+        typedef HconvShape<256, 64, 4, 2, 4> TallNarrow;     // 4x2 waves of 64x32
+        typedef HconvShape<128, 64, 2, 2, 4> SquareNarrow;   // 2x2 waves of 64x32
+        const bool tall_narrow = many_tiles;
+        auto launch_narrow = [&](auto kern, auto shape) -> int {
+            typedef decltype(shape) S;
+            static bool attr_done = false;           // one per kernel: the lambda's body is instantiated per argument type
+            if (!attr_done) {
+                HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+                attr_done = true;
+            }
+            const long tiles = cdiv(M, S::BM);
+            hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, out, M, N, Kw, 1,
+                               static_cast<float*>(nullptr), 0);
+            HIP_TRY(hipGetLastError());
+            return 0;
+        };
+        if (tall_narrow && tap_uniform) return launch_narrow(hconv_tile_kernel<TallNarrow, true>, TallNarrow{});
+        if (tall_narrow) return launch_narrow(hconv_tile_kernel<TallNarrow, false>, TallNarrow{});
+        if (tap_uniform) return launch_narrow(hconv_tile_kernel<SquareNarrow, true>, SquareNarrow{});
+        return launch_narrow(hconv_tile_kernel<SquareNarrow, false>, SquareNarrow{});
     }
     // hgemm variant 12 keeps the register-staged kernels, 13 takes the LDS-DMA kernel wherever it can run (experiments)
     if (tap_uniform && g_rt.hgemm_variant != 12 && (tall || g_rt.hgemm_variant == 13)) {

@@ -32,9 +32,9 @@
 
 namespace decx_hip {
 
-template <int KW_>
+template <int KW_, int BN_ = 128, int WAVES_M_ = 4, int WAVES_N_ = 2>
 struct HconvTapRowShape {
-    static constexpr int BM = 256, BN = 128, BK = 64, WAVES_M = 4, WAVES_N = 2, KW = KW_;
+    static constexpr int BM = 256, BN = BN_, BK = 64, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, KW = KW_;
     static_assert(KW >= 3 && KW % 2 == 1, "the wait counts of the kernel are derived for odd widths from 3 on");
     static constexpr int NWAVES = WAVES_M * WAVES_N, NT = NWAVES * kWave;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
@@ -49,7 +49,7 @@ struct HconvTapRowShape {
     static constexpr size_t LDS_BYTES = (size_t)A_BUFFERS * A_BYTES + (size_t)B_BUFFERS * B_BYTES;
     static_assert(PATCH_ROWS % (8 * NWAVES) == 0 && BN % (8 * NWAVES) == 0, "chunks of 8 rows must divide over the waves");
     static_assert(LDS_BYTES >= OUT_BYTES, "the result tile reuses the operand buffers");
-    static_assert(MI == 2 && NI == 2, "the schedule below is written for 4 MFMAs per k-block");
+    static_assert(NWAVES == 8, "256 threads would leave a SIMD with one wave and nothing to overlap its waits with");
 };
 
 template <class S>
@@ -197,49 +197,48 @@ __global__ __launch_bounds__(S::NT) void hconv_taprow_kernel(HalfImage img, Half
         typedef std::integral_constant<int, ((I + 1) / KW) % 2> NextABuf;
         typedef std::integral_constant<int, (I + 1) % KW> NextTap;
         typedef std::integral_constant<int, (I + 1) % 4> NextBBuf;
+        // k-blocks 0 .. KS-2: MFMA i of block b rides with the reads of block b+1 (fragment sets alternate f0, f1)
+        constexpr int RPS = (FRAG_READS + BLK - 1) / BLK;      // reads per MFMA slot, front-loaded
 #pragma unroll
         for (int b = 0; b + 1 < KS; ++b) {
 #pragma unroll
             for (int i = 0; i < BLK; ++i) {
-                read_one((b & 1) ? f0 : f1, ABuf{}, Tap{}, BBuf{}, b + 1, i);      // FRAG_READS == BLK: one read per MFMA
+#pragma unroll
+                for (int r = i * RPS; r < (i + 1) * RPS && r < FRAG_READS; ++r) read_one((b & 1) ? f0 : f1, ABuf{}, Tap{}, BBuf{}, b + 1, r);
                 mfma_one((b & 1) ? f1 : f0, i);
                 DECX_PIN();
             }
         }
         Frags& fl = ((KS - 1) & 1) ? f1 : f0;
         Frags& fn = ((KS - 1) & 1) ? f0 : f1;
-        mfma_one(fl, 0);
-        DECX_PIN();
+        constexpr int PRE = BLK / 4 > 0 ? BLK / 4 : 1;
+#pragma unroll
+        for (int i = 0; i < PRE; ++i) {
+            mfma_one(fl, i);
+            DECX_PIN();
+        }
         // what the next step reads has landed (see the table at the top), my reads of this step's buffers are done
         wait_dma_then_barrier<(J >= 2 ? 2 * S::B_LOADS : S::A_LOADS + 2 * S::B_LOADS)>();
         DECX_PIN();
-        // three MFMAs left: between them the refills -- the patch of row step s + 2 after the last tap, the filters of step
-        // t + 4 -- and the next step's first fragments
-        if constexpr (J == KW - 1) {
-            static_for<0, 3>([&](auto j) { issue_patch_load(ABuf::value, decltype(j)::value); });
-        } else {
-            static_for<0, S::B_LOADS>([&](auto j) { issue_filter_load(BBuf::value, decltype(j)::value); });
+        // between the MFMAs that are left: the refills -- the patch of row step s + 2 after the last tap, then the filters
+        // of step t + 4, in this order -- and the next step's first fragments
+        constexpr int SLOTS = BLK - PRE, REFILLS = (J == KW - 1 ? S::A_LOADS : 0) + S::B_LOADS;
+#pragma unroll
+        for (int i = 0; i < SLOTS; ++i) {
+#pragma unroll
+            for (int l = (i * REFILLS) / SLOTS; l < ((i + 1) * REFILLS) / SLOTS; ++l) {
+                if (l < REFILLS - S::B_LOADS) issue_patch_load(ABuf::value, l);
+                else issue_filter_load(BBuf::value, l - (REFILLS - S::B_LOADS));
+            }
+            if (has_next) {
+#pragma unroll
+                for (int r = (i * FRAG_READS) / SLOTS; r < ((i + 1) * FRAG_READS) / SLOTS; ++r) read_one(fn, NextABuf{}, NextTap{}, NextBBuf{}, 0, r);
+            }
+            mfma_one(fl, PRE + i);
+            DECX_PIN();
         }
-        if (has_next) {
-            read_one(fn, NextABuf{}, NextTap{}, NextBBuf{}, 0, 0);
-            read_one(fn, NextABuf{}, NextTap{}, NextBBuf{}, 0, 1);
-        }
-        mfma_one(fl, 1);
-        DECX_PIN();
-        if constexpr (J == KW - 1) {
-            static_for<3, S::A_LOADS>([&](auto j) { issue_patch_load(ABuf::value, decltype(j)::value); });
-        }
-        if (has_next) read_one(fn, NextABuf{}, NextTap{}, NextBBuf{}, 0, 2);
-        mfma_one(fl, 2);
-        DECX_PIN();
-        if constexpr (J == KW - 1) {
-            static_for<0, S::B_LOADS>([&](auto j) { issue_filter_load(BBuf::value, decltype(j)::value); });
-        }
-        if (has_next) read_one(fn, NextABuf{}, NextTap{}, NextBBuf{}, 0, 3);
-        mfma_one(fl, 3);
-        DECX_PIN();
     };
-    static_assert(FRAG_READS == BLK && BLK == 4 && S::A_LOADS >= 3, "the slots above are written out for these counts");
+    static_assert(BLK >= 2, "the barrier sits between two MFMAs of the last k-block");
 
     // A(0) and B(0) have landed: everything younger (B(1), B(2), A(1), B(3)) may still fly
     wait_dma_then_barrier<S::A_LOADS + 3 * S::B_LOADS>();
