@@ -156,6 +156,8 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //  10: 224x256x16, 1x8 waves of 224x32    -- two waves per SIMD like 7; 7/8 of its tile, for tile counts that 7 rounds badly
 //  14: 192x192x16, 2x2 waves of  96x96    -- dense GEMM only: sizes that 256 and 128 divide into a bad number of tiles
 //         (3072^2 is 144 tiles of 256^2, 576 of 128^2, and exactly 256 of these)
+//  15: 224x128x16, 2x4 waves of 128x32 (upper row) and 96x32 (lower row) -- shape 6 on two waves per SIMD: each SIMD
+//         carries a 4-block and a 3-block wave
 // and, for dense GEMM only, the one-wave-per-16x16-block kernel of sgemm_chain16.hpp:
 //  11:  32x32x64,  2x2 computing + 4 moving waves, two workgroups per CU -- results too small to fill the chip with tiles
 //  12:  16x16x64,  1 computing + 2 moving waves -- at most one 16x16 block per CU: the fastest a single chain can walk K
@@ -169,6 +171,7 @@ typedef SgemmShape<224, 128, 16, 1, 4, 1> SShape224Solo;
 typedef SgemmShape<256, 256, 16, 4, 2, 2, 2> SShapeBig8;
 typedef SgemmShape<224, 256, 16, 1, 8, 2, 2> SShape224Wide;   // 8 waves of 224x32, two per SIMD
 typedef SgemmShape<192, 192, 16, 2, 2, 1> SShape192;
+typedef SgemmShape<224, 128, 16, 2, 4, 2, 2, true> SShape224Split;   // 8 waves, 4 + 3 row blocks per SIMD
 typedef SgemmShape<64, 64, 16, 2, 2, 4> SShapeTiny;      // 2x2 waves of 32x32
 typedef SgemmShape<128, 64, 16, 2, 2, 4> SShapeTiny2;    // 2x2 waves of 64x32
 
@@ -176,9 +179,10 @@ typedef SgemmShape<128, 64, 16, 2, 2, 4> SShapeTiny2;    // 2x2 waves of 64x32
 // share its matrix pipe, so residency does not change this), a tile costs its area divided by how well that shape keeps
 // the pipe busy (measured on large squares, relative to shape 7).  The 256x128 and 224x128 shapes come in a
 // two-workgroups-per-CU build, better on short K walks where one tile's prologue and epilogue overlap the other's loop,
-// and a one-wave-per-SIMD build with deeper prefetch, better on long ones.
+// and a one-workgroup-per-CU build with deeper prefetch, better on long ones (224x128: shape 15, which measured 5-6 %
+// ahead of shape 6 on the 224x224x64 convolution under 128 filters).
 int pick_sgemm_variant(int M, int N, int K, int batch, bool dense = false) {
-    if (g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) return g_rt.sgemm_variant;
+    if ((g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) || g_rt.sgemm_variant == 15) return g_rt.sgemm_variant;
     if (g_rt.sgemm_variant == 14) return dense ? 14 : 2;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     struct Cand { int variant, bm, bn; double eff; };
@@ -192,7 +196,8 @@ int pick_sgemm_variant(int M, int N, int K, int batch, bool dense = false) {
         const double cost = (double)((tiles + cus - 1) / cus) * c.bm * c.bn / c.eff;
         if (best_cost == 0.0 || cost < best_cost) {
             best_cost = cost;
-            best = ((tiles <= cus || K >= 1024) && (c.variant == 3 || c.variant == 4)) ? c.variant + 2 : c.variant;
+            const bool one_per_cu = tiles <= cus || K >= 1024;
+            best = one_per_cu && c.variant == 3 ? 5 : one_per_cu && c.variant == 4 ? 15 : c.variant;
         }
     }
     return best;
@@ -211,6 +216,7 @@ int dispatch_sgemm(int variant, const ASrc& a, const BSrc& b, const float* Cin, 
         case 8: return launch_sgemm_tile<SShapeTiny>(a, b, Cin, ldc, D, out, M, N, K, batch);
         case 9: return launch_sgemm_tile<SShapeTiny2>(a, b, Cin, ldc, D, out, M, N, K, batch);
         case 10: return launch_sgemm_tile<SShape224Wide>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 15: return launch_sgemm_tile<SShape224Split>(a, b, Cin, ldc, D, out, M, N, K, batch);
         default: return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K, batch);
     }
 }
@@ -255,7 +261,7 @@ int launch_sgemm_chain16(const float* A, int lda, const float* B, int ldb, const
 // 64x65536x1024.  All paths give the same bits, so this is a choice of speed only.
 int pick_chain_shape(int M, int N, int K, int batch) {
     if (g_rt.sgemm_variant >= 11 && g_rt.sgemm_variant <= 13) return g_rt.sgemm_variant;
-    if ((g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) || g_rt.sgemm_variant == 14) return 0;
+    if ((g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) || g_rt.sgemm_variant >= 14) return 0;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     const long blocks16 = (long)cdiv(M, 16) * cdiv(N, 16) * batch, tiles32 = (long)cdiv(M, 32) * cdiv(N, 32) * batch;
     // In units of one round of 32x32 tiles (two per CU, 512 on 256 CUs): a round of 64x64 tiles (one per CU) costs

@@ -536,7 +536,7 @@ struct FilterBUniform : FilterB<true> {
 };
 
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int WAVES_PER_SIMD_ = 1,
-          int STAGE_SETS_ = (WAVES_PER_SIMD_ == 1 ? 2 : 1)>
+          int STAGE_SETS_ = (WAVES_PER_SIMD_ == 1 ? 2 : 1), bool UNEVEN_M_ = false>
 struct SgemmShape {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
     static constexpr int WAVES_PER_SIMD = WAVES_PER_SIMD_;   // occupancy the register budget is held to
@@ -546,8 +546,14 @@ struct SgemmShape {
     static constexpr int STAGE_SETS = STAGE_SETS_;
     static_assert(STAGE_SETS == 1 || STAGE_SETS == 2, "one or two K steps of prefetch");
     static constexpr int NT = WAVES_M * WAVES_N * kWave;
-    static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
-    static constexpr int MI = WM / 32, NI = WN / 32;
+    // UNEVEN_M: two rows of waves share an odd number of 32-row blocks, the upper row taking one more than the lower
+    // (224 rows = 4 + 3 blocks).  Waves w and w + WAVES_N land on the same SIMD, so every SIMD carries one wave of
+    // each kind and the same number of MFMAs per K step.
+    static constexpr bool UNEVEN_M = UNEVEN_M_;
+    static constexpr int MI = UNEVEN_M ? (BM / 32 + 1) / 2 : BM / WAVES_M / 32;      // blocks of the upper wave row
+    static constexpr int MI_LOW = UNEVEN_M ? BM / 32 - MI : MI;                      // blocks of the other wave rows
+    static constexpr int WM = MI * 32, WN = BN / WAVES_N;
+    static constexpr int NI = WN / 32;
     static constexpr int KQ = BK / 4;                         // k-quads per step
     static constexpr int KGROUPS = KQ / 2;                    // groups of 8 consecutive k per step
     // An A staging task is one k-group of one row (two float4 loads); a thread takes A_TASKS of them per step.
@@ -564,7 +570,9 @@ struct SgemmShape {
     static constexpr size_t lds_bytes() {
         return 2 * ((size_t)KQ * A_ROW * sizeof(f32x4) + (size_t)BSrc::template lds_floats<SgemmShape>() * sizeof(float));
     }
-    static_assert(BM % (WAVES_M * 32) == 0 && BN % (WAVES_N * 32) == 0, "wave tile must be whole 32x32 blocks");
+    static_assert(UNEVEN_M ? (WAVES_M == 2 && BM % 32 == 0 && MI_LOW >= 1 && WAVES_N % 4 == 0) : BM % (WAVES_M * 32) == 0,
+                  "wave tile must be whole 32x32 blocks");
+    static_assert(BN % (WAVES_N * 32) == 0, "wave tile must be whole 32x32 blocks");
     static_assert(BK % 8 == 0, "a K step is whole quad pairs");
     static_assert(NT % KGROUPS == 0, "A staging: KGROUPS lanes per row");
 };
@@ -589,7 +597,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
     b_src.select_batch(blockIdx.y);
     if (HAS_C) Cin += (size_t)blockIdx.y * c_batch_stride;
     D += (size_t)blockIdx.y * d_batch_stride;
-    constexpr int BM = S::BM, BN = S::BN, BK = S::BK, NT = S::NT, KQ = S::KQ, MI = S::MI, NI = S::NI;
+    constexpr int BM = S::BM, BN = S::BN, BK = S::BK, NT = S::NT, KQ = S::KQ, NI = S::NI;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     f32x4* As = reinterpret_cast<f32x4*>(lds_raw);                       // [2][KQ][A_ROW]
     float* Bs = reinterpret_cast<float*>(As + 2 * KQ * S::A_ROW);        // [2][layout of the B source]
@@ -662,211 +670,223 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         static_for<0, WRITE_OPS>([&](auto w_tag) { write_one(set_tag, buf, w_tag); });
     };
 
-    // Accumulators start at zero, or at C for dst = A*B + C on dense matrices: the reference's chain starts from C
-    // (GEMM.cuh:223), and starting anywhere else would round differently.  A convolution's bias is added at the end.
-    constexpr bool PRELOAD_C = HAS_C && Out::PRELOAD_C;
-    f32x16 acc[MI][NI];
-#pragma unroll
-    for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < NI; ++ni)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
-    if (PRELOAD_C && (!SPLIT_K || blockIdx.z == 0)) {
-#pragma unroll
+    // Everything from here on depends on how many 32-row blocks the wave owns, a compile-time count: one instance of the
+    // K walk and the epilogue per count, chosen per wave below.
+    auto run = [&](auto mi_tag) {
+        constexpr int MI = decltype(mi_tag)::value;
+        // Accumulators start at zero, or at C for dst = A*B + C on dense matrices: the reference's chain starts from C
+        // (GEMM.cuh:223), and starting anywhere else would round differently.  A convolution's bias is added at the end.
+        constexpr bool PRELOAD_C = HAS_C && Out::PRELOAD_C;
+        f32x16 acc[MI][NI];
+    #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-#pragma unroll
-                for (int ni = 0; ni < NI; ++ni) {
-                    const int n = bn0 + wn0 + BSrc::template strip_col<S>(ni, li);
-                    if (m < M && n < N) acc[mi][ni][r] = Cin[(size_t)m * ldc + n];
+    #pragma unroll
+            for (int ni = 0; ni < NI; ++ni)
+    #pragma unroll
+                for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
+        if (PRELOAD_C && (!SPLIT_K || blockIdx.z == 0)) {
+    #pragma unroll
+            for (int mi = 0; mi < MI; ++mi)
+    #pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+    #pragma unroll
+                    for (int ni = 0; ni < NI; ++ni) {
+                        const int n = bn0 + wn0 + BSrc::template strip_col<S>(ni, li);
+                        if (m < M && n < N) acc[mi][ni][r] = Cin[(size_t)m * ldc + n];
+                    }
                 }
+        }
+
+        // Fragments of one quad pair s: A, per 32-row block one float4 = four consecutive k of this lane's k-slot; B, per
+        // k of the pair (e) and block (ni) one float, fetched as the B source's LDS layout dictates.
+        typedef float BFrag[4][NI];
+        auto read_frags = [&](int buf, int s, f32x4* af, BFrag& bf) {
+            const f32x4* Ab = As + buf * KQ * S::A_ROW;
+            const int q = 2 * s + lh;
+    #pragma unroll
+            for (int mi = 0; mi < MI; ++mi) af[mi] = Ab[q * S::A_ROW + wm0 + mi * 32 + li];
+            b_src.template read_frags<S>(Bs + buf * B_BUF, s, lh, li, wn0, bf);
+        };
+        // MFMAs number lo .. hi-1 of a quad pair, in the order (e, mi, ni); a full pair is 4*MI*NI of them.
+        constexpr int PAIR_MFMAS = 4 * MI * NI;
+        auto mfma_range = [&](const f32x4* af, const BFrag& bf, auto lo_tag, auto hi_tag) {
+            constexpr int LO = decltype(lo_tag)::value, HI = decltype(hi_tag)::value;
+    #pragma unroll
+            for (int i = LO; i < HI; ++i) {
+                const int e = i / (MI * NI), mi = (i / NI) % MI, ni = i % NI;
+                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[mi][e], bf[e][ni], acc[mi][ni], 0, 0, 0);
             }
-    }
-
-    // Fragments of one quad pair s: A, per 32-row block one float4 = four consecutive k of this lane's k-slot; B, per
-    // k of the pair (e) and block (ni) one float, fetched as the B source's LDS layout dictates.
-    typedef float BFrag[4][NI];
-    auto read_frags = [&](int buf, int s, f32x4* af, BFrag& bf) {
-        const f32x4* Ab = As + buf * KQ * S::A_ROW;
-        const int q = 2 * s + lh;
-#pragma unroll
-        for (int mi = 0; mi < MI; ++mi) af[mi] = Ab[q * S::A_ROW + wm0 + mi * 32 + li];
-        b_src.template read_frags<S>(Bs + buf * B_BUF, s, lh, li, wn0, bf);
-    };
-    // MFMAs number lo .. hi-1 of a quad pair, in the order (e, mi, ni); a full pair is 4*MI*NI of them.
-    constexpr int PAIR_MFMAS = 4 * MI * NI;
-    auto mfma_range = [&](const f32x4* af, const BFrag& bf, auto lo_tag, auto hi_tag) {
-        constexpr int LO = decltype(lo_tag)::value, HI = decltype(hi_tag)::value;
-#pragma unroll
-        for (int i = LO; i < HI; ++i) {
-            const int e = i / (MI * NI), mi = (i / NI) % MI, ni = i % NI;
-            acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[mi][e], bf[e][ni], acc[mi][ni], 0, 0, 0);
-        }
-    };
-    auto compute_stage = [&](int buf) {      // unpipelined: used for the peeled steps only
-#pragma unroll
-        for (int s = 0; s < KQ / 2; ++s) {
-            f32x4 af[MI];
-            BFrag bf;
-            read_frags(buf, s, af, bf);
-            mfma_range(af, bf, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
-        }
-    };
-
-    // K walk over T steps (the last one partial when K % BK != 0; its loader zero-fills, so computing it is no
-    // different).  Step t lives in LDS buffer t&1.  Two sets: step t came through register set t&1; while it is
-    // computed, step t+2 is fetched into set t&1 (free since step t went to LDS during step t-1) and step t+1 moves from
-    // set (t+1)&1 into the other LDS buffer.  One set: step t+1 is fetched at the start of step t and moved to LDS in its
-    // second half.  The bulk of the steps (all whose fetch is a full step) run the software-pipelined body; the last
-    // few, with the masking loader, run a plain one.
-    const int full_steps = K / BK;
-    const int T = full_steps + (full_steps * BK < K ? 1 : 0);
-    typedef std::integral_constant<int, 0> Set0;
-    typedef std::integral_constant<int, 1> Set1;
-
-    // prologue: the loads of steps 0 and 1 go out back to back, so the tile pays one global round trip, not two
-    if (full_steps > 0) load_stage(Set0{}, std::false_type{});
-    else load_stage(Set0{}, std::true_type{});
-    if constexpr (SETS == 2) {
-        if (T > 1) {
-            if (full_steps > 1) load_stage(Set1{}, std::false_type{});
-            else load_stage(Set1{}, std::true_type{});
-        }
-    }
-    store_stage(Set0{}, 0);
-    lds_sync();
-
-    static_assert(KQ == 4, "the pipelined loop is written for two quad pairs per K step");
-    constexpr int VMEM_OPS = S::A_PASSES + B_QUADS;     // global loads per thread and step
-    constexpr int FRAG_OPS = MI + BSrc::template frag_reads<S>();   // LDS reads per quad pair
-    f32x4 af0[MI], af1[MI];
-    BFrag bf0, bf1;
-
-    // Steady state of one K step t (fragments of its first quad pair are in af0/bf0):
-    //   pair 0 MFMAs   interleaved with: global loads of step t+SETS, LDS reads of pair 1
-    //   pair 1 MFMAs   interleaved with: LDS writes of step t+1 into the other buffer
-    //   barrier, then the LDS reads of step t+1's pair 0 hide behind the last few MFMAs of pair 1.
-    // Every memory instruction sits between MFMAs, so the matrix pipe is never starved by an in-order wait.
-    auto pipelined_step = [&](auto set_tag, int buf) {
-        constexpr int SET = decltype(set_tag)::value;
-        load_stage(set_tag, std::false_type{});
-        read_frags(buf, 1, af1, bf1);
-        mfma_range(af0, bf0, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
-        // scheduling-group masks: 0x002 VALU, 0x008 MFMA, 0x020 VMEM read, 0x100 DS read, 0x200 DS write
-        constexpr int G0 = PAIR_MFMAS / (VMEM_OPS + FRAG_OPS) > 0 ? PAIR_MFMAS / (VMEM_OPS + FRAG_OPS) : 1;
-#pragma unroll
-        for (int i = 0; i < VMEM_OPS; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, G0, 0);
-        }
-#pragma unroll
-        for (int i = 0; i < FRAG_OPS; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, G0, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-
-        constexpr int LATE = MI * NI < PAIR_MFMAS / 4 ? MI * NI : PAIR_MFMAS / 4;   // MFMAs kept for after the barrier
-        constexpr int EARLY = PAIR_MFMAS - LATE;
-        // step t+1 sits in the other set when there are two; buffer buf^1 was last read before the previous barrier.
-        // Its LDS stores are spread evenly between the MFMAs, each placement pinned (the de-interleaving stores are
-        // inline asm, which the scheduling-group masks cannot name).
-        typedef std::integral_constant<int, SETS == 2 ? 1 - SET : 0> StoreSet;
-        static_for<0, WRITE_OPS>([&](auto w_tag) {
-            constexpr int W = decltype(w_tag)::value;
-            write_one(StoreSet{}, buf ^ 1, w_tag);
-            mfma_range(af1, bf1, std::integral_constant<int, W * EARLY / WRITE_OPS>{}, std::integral_constant<int, (W + 1) * EARLY / WRITE_OPS>{});
-            __builtin_amdgcn_sched_barrier(0);
-        });
-        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        __builtin_amdgcn_sched_barrier(0);
-        read_frags(buf ^ 1, 0, af0, bf0);
-        mfma_range(af1, bf1, std::integral_constant<int, EARLY>{}, std::integral_constant<int, PAIR_MFMAS>{});
-        __builtin_amdgcn_sched_group_barrier(0x100, FRAG_OPS, 2);
-        __builtin_amdgcn_sched_group_barrier(0x008, LATE, 2);
-        __builtin_amdgcn_sched_barrier(0);
-    };
-
-    int t = 0;
-    if constexpr (SETS == 2) {
-        if (full_steps > 2) {
-            read_frags(0, 0, af0, bf0);
-            for (; t + 3 < full_steps; t += 2) {      // steps t and t+1 both fetch a full step (t+2, t+3 < full_steps)
-                pipelined_step(Set0{}, 0);
-                pipelined_step(Set1{}, 1);
+        };
+        auto compute_stage = [&](int buf) {      // unpipelined: used for the peeled steps only
+    #pragma unroll
+            for (int s = 0; s < KQ / 2; ++s) {
+                f32x4 af[MI];
+                BFrag bf;
+                read_frags(buf, s, af, bf);
+                mfma_range(af, bf, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
             }
-            if (t + 2 < full_steps) {
-                pipelined_step(Set0{}, 0);
-                ++t;
-            }
-        }
-        // the remaining steps: at most one more fetch, and that one is the partial step
-        for (; t < T; ++t) {
-            const int buf = t & 1;
-            if (t + 2 < T) {
-                if (buf == 0) load_stage(Set0{}, std::true_type{});
+        };
+
+        // K walk over T steps (the last one partial when K % BK != 0; its loader zero-fills, so computing it is no
+        // different).  Step t lives in LDS buffer t&1.  Two sets: step t came through register set t&1; while it is
+        // computed, step t+2 is fetched into set t&1 (free since step t went to LDS during step t-1) and step t+1 moves from
+        // set (t+1)&1 into the other LDS buffer.  One set: step t+1 is fetched at the start of step t and moved to LDS in its
+        // second half.  The bulk of the steps (all whose fetch is a full step) run the software-pipelined body; the last
+        // few, with the masking loader, run a plain one.
+        const int full_steps = K / BK;
+        const int T = full_steps + (full_steps * BK < K ? 1 : 0);
+        typedef std::integral_constant<int, 0> Set0;
+        typedef std::integral_constant<int, 1> Set1;
+
+        // prologue: the loads of steps 0 and 1 go out back to back, so the tile pays one global round trip, not two
+        if (full_steps > 0) load_stage(Set0{}, std::false_type{});
+        else load_stage(Set0{}, std::true_type{});
+        if constexpr (SETS == 2) {
+            if (T > 1) {
+                if (full_steps > 1) load_stage(Set1{}, std::false_type{});
                 else load_stage(Set1{}, std::true_type{});
             }
-            compute_stage(buf);
-            if (t + 1 < T) {
-                if (buf == 0) store_stage(Set1{}, 1);
-                else store_stage(Set0{}, 0);
-                lds_sync();
-            }
         }
-    } else {
-        if (full_steps > 1) {
-            read_frags(0, 0, af0, bf0);
-            for (; t + 1 < full_steps; ++t) pipelined_step(Set0{}, t & 1);   // fetches step t+1, a full one
-        }
-        for (; t < T; ++t) {
-            const int buf = t & 1;
-            if (t + 1 < T) load_stage(Set0{}, std::true_type{});
-            compute_stage(buf);
-            if (t + 1 < T) {
-                store_stage(Set0{}, buf ^ 1);
-                lds_sync();
-            }
-        }
-    }
+        store_stage(Set0{}, 0);
+        lds_sync();
 
-    // ---- epilogue.  Lane li holds, per row, the columns strip_col(ni, li) of its wave's strip: NI consecutive ones when B
-    // came from a row-major matrix (one vector store per row where alignment and the edge allow), 32 apart otherwise.
-    // dst = A*B + C adds C here (C may alias dst: every element is read and written by the same lane).
-#pragma unroll
-    for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-            if (m < M) {
-                float* drow = D + out.offset(m);
-                const float* crow = HAS_C ? Cin + (size_t)m * ldc : nullptr;
-                const bool add_c = HAS_C && !PRELOAD_C && (!SPLIT_K || blockIdx.z == 0);
-                if (BSrc::ROW_MAJOR_LDS && !SPLIT_K && NI > 1 && NI != 3) {      // runs of 3 floats are not aligned for one store
-                    const int n0 = bn0 + wn0 + NI * li;
-                    if (out.vec && n0 + NI <= N) {
-                        typedef float vec_t __attribute__((ext_vector_type(NI)));
-                        vec_t v;
-#pragma unroll
-                        for (int ni = 0; ni < NI; ++ni) v[ni] = out.finish(add_c ? acc[mi][ni][r] + crow[n0 + ni] : acc[mi][ni][r]);
-                        *reinterpret_cast<vec_t*>(drow + n0) = v;
-                        continue;
-                    }
+        static_assert(KQ == 4, "the pipelined loop is written for two quad pairs per K step");
+        constexpr int VMEM_OPS = S::A_PASSES + B_QUADS;     // global loads per thread and step
+        constexpr int FRAG_OPS = MI + BSrc::template frag_reads<S>();   // LDS reads per quad pair
+        f32x4 af0[MI], af1[MI];
+        BFrag bf0, bf1;
+
+        // Steady state of one K step t (fragments of its first quad pair are in af0/bf0):
+        //   pair 0 MFMAs   interleaved with: global loads of step t+SETS, LDS reads of pair 1
+        //   pair 1 MFMAs   interleaved with: LDS writes of step t+1 into the other buffer
+        //   barrier, then the LDS reads of step t+1's pair 0 hide behind the last few MFMAs of pair 1.
+        // Every memory instruction sits between MFMAs, so the matrix pipe is never starved by an in-order wait.
+        auto pipelined_step = [&](auto set_tag, int buf) {
+            constexpr int SET = decltype(set_tag)::value;
+            load_stage(set_tag, std::false_type{});
+            read_frags(buf, 1, af1, bf1);
+            mfma_range(af0, bf0, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
+            // scheduling-group masks: 0x002 VALU, 0x008 MFMA, 0x020 VMEM read, 0x100 DS read, 0x200 DS write
+            constexpr int G0 = PAIR_MFMAS / (VMEM_OPS + FRAG_OPS) > 0 ? PAIR_MFMAS / (VMEM_OPS + FRAG_OPS) : 1;
+    #pragma unroll
+            for (int i = 0; i < VMEM_OPS; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, G0, 0);
+            }
+    #pragma unroll
+            for (int i = 0; i < FRAG_OPS; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, G0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+
+            constexpr int LATE = MI * NI < PAIR_MFMAS / 4 ? MI * NI : PAIR_MFMAS / 4;   // MFMAs kept for after the barrier
+            constexpr int EARLY = PAIR_MFMAS - LATE;
+            // step t+1 sits in the other set when there are two; buffer buf^1 was last read before the previous barrier.
+            // Its LDS stores are spread evenly between the MFMAs, each placement pinned (the de-interleaving stores are
+            // inline asm, which the scheduling-group masks cannot name).
+            typedef std::integral_constant<int, SETS == 2 ? 1 - SET : 0> StoreSet;
+            static_for<0, WRITE_OPS>([&](auto w_tag) {
+                constexpr int W = decltype(w_tag)::value;
+                write_one(StoreSet{}, buf ^ 1, w_tag);
+                mfma_range(af1, bf1, std::integral_constant<int, W * EARLY / WRITE_OPS>{}, std::integral_constant<int, (W + 1) * EARLY / WRITE_OPS>{});
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+            read_frags(buf ^ 1, 0, af0, bf0);
+            mfma_range(af1, bf1, std::integral_constant<int, EARLY>{}, std::integral_constant<int, PAIR_MFMAS>{});
+            __builtin_amdgcn_sched_group_barrier(0x100, FRAG_OPS, 2);
+            __builtin_amdgcn_sched_group_barrier(0x008, LATE, 2);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+
+        int t = 0;
+        if constexpr (SETS == 2) {
+            if (full_steps > 2) {
+                read_frags(0, 0, af0, bf0);
+                for (; t + 3 < full_steps; t += 2) {      // steps t and t+1 both fetch a full step (t+2, t+3 < full_steps)
+                    pipelined_step(Set0{}, 0);
+                    pipelined_step(Set1{}, 1);
                 }
-#pragma unroll
-                for (int ni = 0; ni < NI; ++ni) {
-                    const int n = bn0 + wn0 + BSrc::template strip_col<S>(ni, li);
-                    if (n < N) {
-                        const float v = add_c ? acc[mi][ni][r] + crow[n] : acc[mi][ni][r];
-                        if (SPLIT_K) unsafeAtomicAdd(drow + n, v);      // hardware fp32 add in L2
-                        else drow[n] = out.finish(v);
-                    }
+                if (t + 2 < full_steps) {
+                    pipelined_step(Set0{}, 0);
+                    ++t;
+                }
+            }
+            // the remaining steps: at most one more fetch, and that one is the partial step
+            for (; t < T; ++t) {
+                const int buf = t & 1;
+                if (t + 2 < T) {
+                    if (buf == 0) load_stage(Set0{}, std::true_type{});
+                    else load_stage(Set1{}, std::true_type{});
+                }
+                compute_stage(buf);
+                if (t + 1 < T) {
+                    if (buf == 0) store_stage(Set1{}, 1);
+                    else store_stage(Set0{}, 0);
+                    lds_sync();
+                }
+            }
+        } else {
+            if (full_steps > 1) {
+                read_frags(0, 0, af0, bf0);
+                for (; t + 1 < full_steps; ++t) pipelined_step(Set0{}, t & 1);   // fetches step t+1, a full one
+            }
+            for (; t < T; ++t) {
+                const int buf = t & 1;
+                if (t + 1 < T) load_stage(Set0{}, std::true_type{});
+                compute_stage(buf);
+                if (t + 1 < T) {
+                    store_stage(Set0{}, buf ^ 1);
+                    lds_sync();
                 }
             }
         }
+
+        // ---- epilogue.  Lane li holds, per row, the columns strip_col(ni, li) of its wave's strip: NI consecutive ones when B
+        // came from a row-major matrix (one vector store per row where alignment and the edge allow), 32 apart otherwise.
+        // dst = A*B + C adds C here (C may alias dst: every element is read and written by the same lane).
+    #pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+    #pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                if (m < M) {
+                    float* drow = D + out.offset(m);
+                    const float* crow = HAS_C ? Cin + (size_t)m * ldc : nullptr;
+                    const bool add_c = HAS_C && !PRELOAD_C && (!SPLIT_K || blockIdx.z == 0);
+                    if (BSrc::ROW_MAJOR_LDS && !SPLIT_K && NI > 1 && NI != 3) {      // runs of 3 floats are not aligned for one store
+                        const int n0 = bn0 + wn0 + NI * li;
+                        if (out.vec && n0 + NI <= N) {
+                            typedef float vec_t __attribute__((ext_vector_type(NI)));
+                            vec_t v;
+    #pragma unroll
+                            for (int ni = 0; ni < NI; ++ni) v[ni] = out.finish(add_c ? acc[mi][ni][r] + crow[n0 + ni] : acc[mi][ni][r]);
+                            *reinterpret_cast<vec_t*>(drow + n0) = v;
+                            continue;
+                        }
+                    }
+    #pragma unroll
+                    for (int ni = 0; ni < NI; ++ni) {
+                        const int n = bn0 + wn0 + BSrc::template strip_col<S>(ni, li);
+                        if (n < N) {
+                            const float v = add_c ? acc[mi][ni][r] + crow[n] : acc[mi][ni][r];
+                            if (SPLIT_K) unsafeAtomicAdd(drow + n, v);      // hardware fp32 add in L2
+                            else drow[n] = out.finish(v);
+                        }
+                    }
+                }
+            }
+    };
+    if constexpr (S::UNEVEN_M) {
+        // a branch on the scalar unit: the two wave rows run different instances, with the same sequence of barriers
+        if (__builtin_amdgcn_readfirstlane(wave) < S::WAVES_N) run(std::integral_constant<int, S::MI>{});
+        else run(std::integral_constant<int, S::MI_LOW>{});
+    } else {
+        run(std::integral_constant<int, S::MI>{});
+    }
 }
 
 }  // namespace decx_hip
