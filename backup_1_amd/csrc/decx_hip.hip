@@ -180,7 +180,8 @@ typedef SgemmShape<128, 64, 16, 2, 2, 4> SShapeTiny2;    // 2x2 waves of 64x32
 // the pipe busy (measured on large squares, relative to shape 7).  The 256x128 and 224x128 shapes come in a
 // two-workgroups-per-CU build, better on short K walks where one tile's prologue and epilogue overlap the other's loop,
 // and a one-workgroup-per-CU build with deeper prefetch, better on long ones (224x128: shape 15, which measured 5-6 %
-// ahead of shape 6 on the 224x224x64 convolution under 128 filters).
+// ahead of shape 6 on the 224x224x64 convolution under 128 filters; the same split of the 224x256 tile, and 256x128 on
+// 8 waves of 128x32, measured no better than shapes 10 and 5 and are not built).
 int pick_sgemm_variant(int M, int N, int K, int batch, bool dense = false) {
     if ((g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) || g_rt.sgemm_variant == 15) return g_rt.sgemm_variant;
     if (g_rt.sgemm_variant == 14) return dense ? 14 : 2;

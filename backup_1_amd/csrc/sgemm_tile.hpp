@@ -678,19 +678,19 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         // (GEMM.cuh:223), and starting anywhere else would round differently.  A convolution's bias is added at the end.
         constexpr bool PRELOAD_C = HAS_C && Out::PRELOAD_C;
         f32x16 acc[MI][NI];
-    #pragma unroll
+#pragma unroll
         for (int mi = 0; mi < MI; ++mi)
-    #pragma unroll
+#pragma unroll
             for (int ni = 0; ni < NI; ++ni)
-    #pragma unroll
+#pragma unroll
                 for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
         if (PRELOAD_C && (!SPLIT_K || blockIdx.z == 0)) {
-    #pragma unroll
+#pragma unroll
             for (int mi = 0; mi < MI; ++mi)
-    #pragma unroll
+#pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-    #pragma unroll
+#pragma unroll
                     for (int ni = 0; ni < NI; ++ni) {
                         const int n = bn0 + wn0 + BSrc::template strip_col<S>(ni, li);
                         if (m < M && n < N) acc[mi][ni][r] = Cin[(size_t)m * ldc + n];
@@ -704,7 +704,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         auto read_frags = [&](int buf, int s, f32x4* af, BFrag& bf) {
             const f32x4* Ab = As + buf * KQ * S::A_ROW;
             const int q = 2 * s + lh;
-    #pragma unroll
+#pragma unroll
             for (int mi = 0; mi < MI; ++mi) af[mi] = Ab[q * S::A_ROW + wm0 + mi * 32 + li];
             b_src.template read_frags<S>(Bs + buf * B_BUF, s, lh, li, wn0, bf);
         };
@@ -712,14 +712,14 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         constexpr int PAIR_MFMAS = 4 * MI * NI;
         auto mfma_range = [&](const f32x4* af, const BFrag& bf, auto lo_tag, auto hi_tag) {
             constexpr int LO = decltype(lo_tag)::value, HI = decltype(hi_tag)::value;
-    #pragma unroll
+#pragma unroll
             for (int i = LO; i < HI; ++i) {
                 const int e = i / (MI * NI), mi = (i / NI) % MI, ni = i % NI;
                 acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[mi][e], bf[e][ni], acc[mi][ni], 0, 0, 0);
             }
         };
         auto compute_stage = [&](int buf) {      // unpipelined: used for the peeled steps only
-    #pragma unroll
+#pragma unroll
             for (int s = 0; s < KQ / 2; ++s) {
                 f32x4 af[MI];
                 BFrag bf;
@@ -769,12 +769,12 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
             mfma_range(af0, bf0, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
             // scheduling-group masks: 0x002 VALU, 0x008 MFMA, 0x020 VMEM read, 0x100 DS read, 0x200 DS write
             constexpr int G0 = PAIR_MFMAS / (VMEM_OPS + FRAG_OPS) > 0 ? PAIR_MFMAS / (VMEM_OPS + FRAG_OPS) : 1;
-    #pragma unroll
+#pragma unroll
             for (int i = 0; i < VMEM_OPS; ++i) {
                 __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x008, G0, 0);
             }
-    #pragma unroll
+#pragma unroll
             for (int i = 0; i < FRAG_OPS; ++i) {
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x008, G0, 0);
@@ -848,9 +848,9 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         // ---- epilogue.  Lane li holds, per row, the columns strip_col(ni, li) of its wave's strip: NI consecutive ones when B
         // came from a row-major matrix (one vector store per row where alignment and the edge allow), 32 apart otherwise.
         // dst = A*B + C adds C here (C may alias dst: every element is read and written by the same lane).
-    #pragma unroll
+#pragma unroll
         for (int mi = 0; mi < MI; ++mi)
-    #pragma unroll
+#pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
                 if (m < M) {
@@ -862,13 +862,13 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
                         if (out.vec && n0 + NI <= N) {
                             typedef float vec_t __attribute__((ext_vector_type(NI)));
                             vec_t v;
-    #pragma unroll
+#pragma unroll
                             for (int ni = 0; ni < NI; ++ni) v[ni] = out.finish(add_c ? acc[mi][ni][r] + crow[n0 + ni] : acc[mi][ni][r]);
                             *reinterpret_cast<vec_t*>(drow + n0) = v;
                             continue;
                         }
                     }
-    #pragma unroll
+#pragma unroll
                     for (int ni = 0; ni < NI; ++ni) {
                         const int n = bn0 + wn0 + BSrc::template strip_col<S>(ni, li);
                         if (n < N) {
