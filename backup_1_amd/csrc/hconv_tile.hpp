@@ -328,7 +328,7 @@ __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, Hal
 }
 
 // dst(pixel m, filter n) = half(relu(partial[m][n] + bias[n])): the end of a split-K convolution.
-__global__ __launch_bounds__(256) void hconv_split_finish_kernel(const float* __restrict__ partial, HalfTensorOut out, int M, int N) {
+static __global__ __launch_bounds__(256) void hconv_split_finish_kernel(const float* __restrict__ partial, HalfTensorOut out, int M, int N) {
     const size_t total = (size_t)M * N;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const int m = (int)(i / N), n = (int)(i - (size_t)m * N);

@@ -1,0 +1,163 @@
+// fp16 GEMM with fp32 accumulation: kernel choice and launch (hgemm_dma_tile.hpp, hgemm_tile.hpp), split-K.
+#include "runtime.hpp"
+#include "hgemm_dma_tile.hpp"
+#include "hgemm_tile.hpp"
+
+namespace decx_hip {
+
+// ---------------------------------------------------------------------------------------------------------------
+// fp16 launchers
+// ---------------------------------------------------------------------------------------------------------------
+// Tile shapes (variant numbers of decx_hip_set_hgemm_variant):
+//   1: 256x256x32, 2x2 waves of 128x128, register-staged
+//   2: 128x128x32, 2x2 waves of  64x64, register-staged (also the element-wise loader for unaligned operands)
+//   3: 256x256x32, 2x2 waves of 128x128, 4-stage LDS-DMA pipeline
+//   4: 256x256x64, 2x2 waves of 128x128, 2-stage LDS-DMA pipeline (whole 128-byte lines of A per row and step)
+//   5: 256x256x32, 2x2 waves of 128x128, 5-stage LDS-DMA pipeline
+//   8: 128x128x64, 2x2 waves of 64x64, 2-stage LDS-DMA pipeline (64 KB of LDS: two workgroups per CU) -- mid-size problems
+//   9: as 8 with 3 stages (one workgroup per CU) -- small problems
+//  10: 256x128x64, 2x2 waves of 128x64, 2-stage LDS-DMA pipeline
+//   6: as 4 with 4x2 waves of 64x128 (two waves per SIMD)
+//   7: as 4 with 2x4 waves of 128x64 (two waves per SIMD) -- the default for large problems: the chip is power-capped on
+//      this kernel (MFMA busy x clock stays ~1.27 GHz-equivalents whatever the schedule), and this one is 1 % ahead
+//  11: split-K on shape 8 through an fp32 workspace (hgemm_splitk_enqueue) -- few tiles and a long K
+// and, for the fp16 convolution only: 12 keeps its register-staged kernels, 13 takes its LDS-DMA kernel for any image
+// whose channel pitch allows it, 14 its tap-row kernel; each switches its split over K off (experiments and tests)
+typedef HgemmShape<256, 256, 32, 2, 2> HShapeBig;
+typedef HgemmShape<128, 128, 32, 2, 2> HShapeSmall;
+typedef HgemmDmaShape<256, 256, 32, 2, 2, 4> HShapeDma;
+typedef HgemmDmaShape<256, 256, 64, 2, 2, 2> HShapeDma64;
+typedef HgemmDmaShape<256, 256, 32, 2, 2, 5> HShapeDma5;
+typedef HgemmDmaShape<256, 256, 64, 4, 2, 2> HShapeDma64W8a;     // 8 waves, 64x128 each
+typedef HgemmDmaShape<256, 256, 64, 2, 4, 2> HShapeDma64W8b;     // 8 waves, 128x64 each
+typedef HgemmDmaShape<128, 128, 64, 2, 2, 2> HShapeDmaSmall;     // 4 waves, 64x64 each, 64 KB of LDS: two workgroups per CU
+typedef HgemmDmaShape<128, 128, 64, 2, 2, 3> HShapeDmaSmall3;
+typedef HgemmDmaShape<256, 128, 64, 2, 2, 2> HShapeDmaTall;      // 4 waves, 128x64 each
+
+template <class S, bool VEC>
+int launch_hgemm_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
+                      int ldd, int M, int N, int K, const Batch& batch) {
+    auto kern = hgemm_tile_kernel<S, VEC>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)S::LDS_BYTES));
+        attr_done = true;
+    }
+    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    const long total = (long)tiles_m * tiles_n;
+    if (total > 0x7fffffffL || batch.count > 65535) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
+    const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
+    hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::LDS_BYTES, batch.stream,
+                       reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
+                       reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N, K,
+                       tiles_m, tiles_n, group_m, batch.stride_a, batch.stride_b, batch.stride_c, batch.stride_d);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+template <class S>
+int launch_hgemm_dma_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
+                          uint16_t* D, int ldd, int M, int N, int K, const Batch& batch) {
+    auto kern = Cin ? hgemm_dma_kernel<S, true> : hgemm_dma_kernel<S, false>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hgemm_dma_kernel<S, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hgemm_dma_kernel<S, false>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+        attr_done = true;
+    }
+    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    const long total = (long)tiles_m * tiles_n;
+    if (total > 0x7fffffffL || batch.count > 65535) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
+    const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
+    hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::LDS_BYTES, batch.stream,
+                       reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
+                       reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N, K,
+                       tiles_m, tiles_n, group_m, batch.stride_a, batch.stride_b, batch.stride_c, batch.stride_d,
+                       static_cast<float*>(nullptr), 0);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+// fp16 GEMM whose result has too few tiles to fill the chip while K is long: K is cut into ranges that run as separate
+// workgroups (blockIdx.z) and add their fp32 partial sums to a workspace with atomics; a second kernel adds C and
+// rounds to binary16 once.  fp32 sums in no fixed order: the result can differ in its last bit from run to run, inside
+// the 2e-3 rule of the fp16 path.  (fp32 GEMM never does this: its results are bit-exact chains.)
+int hgemm_splitk_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
+                         int ldd, int M, int N, int K, int splits, hipStream_t stream) {
+    typedef HShapeDmaSmall S;                      // 128x128x64, LDS-DMA staged, two workgroups per CU
+    if (int rc = ensure_partial((size_t)M * N * sizeof(float))) return rc;
+    auto kern = hgemm_dma_kernel<S, false, true>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+        attr_done = true;
+    }
+    const size_t total = (size_t)M * N;
+    const unsigned fill_blocks = (unsigned)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+    enqueue_zero_region(g_rt.partial, N, M, N, stream);
+    const int k_split_len = cdiv(cdiv(K, splits), S::BK) * S::BK;
+    splits = cdiv(K, k_split_len);                                                        // no empty range
+    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)splits), dim3(S::NT), S::LDS_BYTES, stream,
+                       reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
+                       static_cast<const _Float16*>(nullptr), 0, reinterpret_cast<_Float16*>(D), ldd, M, N, K, tiles_m, tiles_n,
+                       group_m, (size_t)0, (size_t)0, (size_t)0, (size_t)0, g_rt.partial, k_split_len);
+    hipLaunchKernelGGL(hgemm_split_finish_kernel, dim3(fill_blocks), dim3(256), 0, stream, g_rt.partial,
+                       reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
+                  int ldd, int M, int N, int K, const Batch& batch) {
+    if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
+    // the LDS-DMA tiles address a tile's rows with 32-bit byte offsets from the tile's first row: 256 rows of A, 64 of B
+    const bool narrow = (size_t)lda * 256 * sizeof(uint16_t) < ((size_t)1 << 32) && (size_t)ldb * 64 * sizeof(uint16_t) < ((size_t)1 << 32);
+    const bool vec = aligned16(A) && aligned16(B) && lda % 8 == 0 && ldb % 8 == 0 && ldb >= 8 && batch.stride_a % 8 == 0 &&
+                     batch.stride_b % 8 == 0 && narrow;
+    if (!vec) return launch_hgemm_tile<HShapeSmall, false>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    int variant = g_rt.hgemm_variant;
+    {
+        // few 128x128 tiles and a long K: split K (variant 11 forces it, any other fixed variant switches it off).
+        // Measured, in us: a tile walks K at 6.7 ns per k (1.6 times that when two workgroups share a CU); a launch costs
+        // about 4, the zero fill and the finishing kernel 9 together, an atomic add to the workspace 3.1 ps.
+        const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+        const long tiles = (long)cdiv(M, 128) * cdiv(N, 128);
+        long splits = (2 * cus + tiles - 1) / tiles;
+        if (splits > K / 512) splits = K / 512;                        // at least 8 K steps per range
+        if (splits >= 2 && batch.count == 1 && (size_t)M * N <= ((size_t)1 << 26)) {
+            const double t_whole = 4.0 + 0.0067 * K * (double)((tiles + cus - 1) / cus);
+            const double share = tiles * splits > cus ? 1.6 : 1.0;
+            const double t_split = 9.0 + 3.1e-6 * M * N * splits +
+                                   0.0067 * ((double)K / splits) * share * (double)((tiles * splits + 2 * cus - 1) / (2 * cus));
+            if (variant == 11 || ((variant < 1 || variant > 11) && t_split < 0.85 * t_whole))
+                return hgemm_splitk_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, (int)splits, batch.stream);
+        }
+        if (variant == 11) variant = 0;
+    }
+    if (variant < 1 || variant > 10) {
+        // same cost model as the fp32 picker: rounds of tiles per CU x tile area / measured shape efficiency
+        const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+        const long big = (long)cdiv(M, 256) * cdiv(N, 256) * batch.count, small = (long)cdiv(M, 128) * cdiv(N, 128) * batch.count;
+        const double cost_big = (double)((big + cus - 1) / cus) * 65536.0;
+        const double cost_small = (double)((small + cus - 1) / cus) * 16384.0 / 0.75;
+        // the small tile with three LDS stages holds one workgroup per CU: only worth it when there is at most one to hold
+        variant = cost_big <= cost_small ? 7 : (small <= cus ? 9 : 8);
+    }
+    if (variant == 3) return launch_hgemm_dma_tile<HShapeDma>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 4) return launch_hgemm_dma_tile<HShapeDma64>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 5) return launch_hgemm_dma_tile<HShapeDma5>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 6) return launch_hgemm_dma_tile<HShapeDma64W8a>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 7) return launch_hgemm_dma_tile<HShapeDma64W8b>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 8) return launch_hgemm_dma_tile<HShapeDmaSmall>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 9) return launch_hgemm_dma_tile<HShapeDmaSmall3>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 10) return launch_hgemm_dma_tile<HShapeDmaTall>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 1) return launch_hgemm_tile<HShapeBig, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    return launch_hgemm_tile<HShapeSmall, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+}
+
+}  // namespace decx_hip

@@ -224,7 +224,7 @@ __global__ __launch_bounds__(S::NT) void hgemm_tile_kernel(const _Float16* __res
 }
 
 // D = half(partial + C): the end of a split-K product (hgemm_dma_kernel with SPLIT_K).  partial is dense M x N fp32.
-__global__ __launch_bounds__(256) void hgemm_split_finish_kernel(const float* __restrict__ partial, const _Float16* Cin, int ldc,
+static __global__ __launch_bounds__(256) void hgemm_split_finish_kernel(const float* __restrict__ partial, const _Float16* Cin, int ldc,
                                                                  _Float16* D, int ldd, int M, int N) {
     const size_t total = (size_t)M * N;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {

@@ -1,0 +1,77 @@
+// State and helpers shared by the translation units of libdecx_hip.so (each .hip file instantiates one family of
+// kernels, so that they compile side by side): the library's runtime record, the status-code helpers, the launch
+// description of a batch and the enqueue functions the C ABI calls.
+#pragma once
+#include "../../include/decx_hip.h"
+
+#include <hip/hip_runtime.h>
+#include <cstddef>
+#include <cstdint>
+
+namespace decx_hip {
+
+struct Runtime {
+    bool is_init = false;
+    int device = -1;
+    int compute_units = 0;
+    int clock_khz = 0;
+    size_t hbm_bytes = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    int sgemm_variant = 0;
+    int hgemm_variant = 0;
+    float* partial = nullptr;      // fp32 workspace of the fp16 split-K path, grown on demand, kept until the process ends
+    size_t partial_bytes = 0;
+    int group_m = 8;   // tile-rows per raster group of the XCD-aware tile walk (env DECX_HIP_GROUP_M overrides, for tuning)
+};
+extern Runtime g_rt;
+
+// sets the calling thread's error string (decx_hip_last_error) and returns `code`
+int fail(int code, const char* fmt, ...);
+int hip_fail(hipError_t e, const char* what);
+
+#define HIP_TRY(expr)                                   \
+    do {                                                \
+        hipError_t e_ = (expr);                         \
+        if (e_ != hipSuccess) return hip_fail(e_, #expr); \
+    } while (0)
+
+int need_init();
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int cdiv(int a, int b) { return (a + b - 1) / b; }
+
+// A batch of `count` independent, equally shaped problems; the strides are in elements between consecutive problems.
+// Every launcher enqueues on `stream`.
+struct Batch {
+    int count = 1;
+    size_t stride_a = 0, stride_b = 0, stride_c = 0, stride_d = 0;
+    hipStream_t stream = nullptr;
+};
+
+int check_gemm_args(const void* A, int lda, const void* B, int ldb, const void* Cin, int ldc, const void* D, int ldd, int M,
+                    int N, int K, const Batch& batch);
+
+// zero-fills the M x N region of a pitched matrix on `stream` (the split-K kernels accumulate into it)
+void enqueue_zero_region(float* D, int ldd, int M, int N, hipStream_t stream);
+
+// the fp32 workspace of the fp16 split-K paths (g_rt.partial): grown on demand, kept until the process ends
+int ensure_partial(size_t need);
+
+// Enqueue functions, one family per translation unit.  Each checks its arguments, picks a kernel and launches it on
+// the given stream (the library's, where none is passed) without waiting.
+int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
+                  int N, int K, const Batch& batch, bool relu = false);
+int sgemm_splitk_enqueue(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
+                         int N, int K, int splits);
+int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt, int N, int kh,
+                 int kw, size_t filt_stride, size_t filt_row_stride, float* dst, int dst_dpitch, size_t dst_row_stride,
+                 int flag, const float* bias = nullptr, bool relu = false);
+int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
+                  int ldd, int M, int N, int K, const Batch& batch);
+int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_stride, const uint16_t* filt, int N, int kh,
+                  int kw, size_t filt_stride, size_t filt_row_stride, uint16_t* dst, int dst_dpitch, size_t dst_row_stride,
+                  int flag, const uint16_t* bias, bool relu);
+
+}  // namespace decx_hip

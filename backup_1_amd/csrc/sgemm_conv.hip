@@ -1,0 +1,81 @@
+// fp32 fused im2col convolution: argument checks, loader and kernel choice, launch (sgemm_tile.hpp, conv_chain16.hpp).
+#include "sgemm_launch.hpp"
+#include "sgemm_chain16.hpp"
+#include "conv_chain16.hpp"
+
+namespace decx_hip {
+
+template <class S>
+int launch_conv_chain16(const Im2colA<false>& img, const FilterB<false>& fb, const float* bias, float* dst, const TensorOut& out,
+                        int M, int N, int K) {
+    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    const long total = (long)tiles_m * tiles_n;
+    if (total > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
+    static bool attr_done = false;
+    if (!attr_done) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(conv_chain16_kernel<S>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)S::LDS_BYTES));
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(conv_chain16_kernel<S>, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, bias, dst, out,
+                       M, N, K, tiles_n);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt, int N, int kh,
+                 int kw, size_t filt_stride, size_t filt_row_stride, float* dst, int dst_dpitch, size_t dst_row_stride,
+                 int flag, const float* bias, bool relu) {
+    if (!g_rt.is_init) return need_init();
+    if (flag != DECX_HIP_CONV_NO_COMPENSATE && flag != DECX_HIP_CONV_ZERO_COMPENSATE)
+        return fail(DECX_HIP_FAIL_ERROR_FLAG, "This flag is meaningless in current context\n");   // core/error.h:67
+    if (!src || !filt || !dst) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "null tensor pointer\n");
+    if (H <= 0 || W <= 0 || N <= 0 || kh <= 0 || kw <= 0 || dpitch <= 0)
+        return fail(DECX_HIP_FAIL_DIMS, "Tensor Dims don't match each other");
+    if (dpitch % 4 != 0 || src_row_stride % 4 != 0 || filt_stride % 4 != 0 || filt_row_stride % 4 != 0 ||
+        !aligned16(src) || !aligned16(filt))
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "tensors must be 16-byte aligned with channel pitch a multiple of 4\n");
+    const int Hout = flag ? H : H - 2 * (kh / 2), Wout = flag ? W : W - 2 * (kw / 2);
+    if (Hout <= 0 || Wout <= 0) return fail(DECX_HIP_FAIL_DIMS, "kernel larger than the image\n");
+    if (src_row_stride < (size_t)W * dpitch || filt_row_stride < (size_t)kw * dpitch ||
+        filt_stride < (size_t)(kh - 1) * filt_row_stride + (size_t)kw * dpitch || dst_dpitch < N ||
+        dst_row_stride < (size_t)Wout * dst_dpitch)
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "stride smaller than the extent it spans\n");
+    const long Ml = (long)Hout * Wout, Kl = (long)kh * kw * dpitch;
+    if (Ml > 0x7fffffffL || Kl > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large\n");
+    const int M = (int)Ml, K = (int)Kl;
+    // the loaders address both tensors with 32-bit byte offsets through buffer resources
+    const size_t src_bytes = ((size_t)(H - 1) * src_row_stride + (size_t)W * dpitch) * sizeof(float);
+    const size_t filt_bytes = ((size_t)(N - 1) * filt_stride + (size_t)(kh - 1) * filt_row_stride + (size_t)kw * dpitch) * sizeof(float);
+    if (src_bytes >= 0x80000000ull || filt_bytes >= 0x80000000ull)
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "source tensor and filter bank must each stay below 2 GiB\n");
+    TensorOut out{Wout, dst_dpitch, dst_row_stride, dst_row_stride == (size_t)Wout * dst_dpitch, relu};
+    Batch one;
+    one.stream = g_rt.stream;
+    const int variant = pick_sgemm_variant(M, N, K, 1);
+    const int oy = flag ? kh / 2 : 0, ox = flag ? kw / 2 : 0;
+    // a bias is the "+ C" operand with row stride 0: every output pixel adds the same N values
+    // small images: too few tiles for the chip, the one-wave-per-block kernel takes them (conv_chain16.hpp)
+    if (const int chain = pick_chain_shape(M, N, K, 1)) {
+        Im2colA<false> a{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
+        FilterB<false> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
+        if (chain == 11) return launch_conv_chain16<Chain16<2, 1, 4, 4>>(a, b, bias, dst, out, M, N, K);
+        if (chain == 12) return launch_conv_chain16<Chain16<1, 1, 8, 2>>(a, b, bias, dst, out, M, N, K);
+        return launch_conv_chain16<Chain16<4, 2, 2, 3>>(a, b, bias, dst, out, M, N, K);
+    }
+    if (dpitch % 16 == 0) {      // a whole K step inside one tap: the tap walk runs on the scalar unit
+        Im2colAUniform a{{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes}};
+        FilterBUniform b{{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes}};
+        return dispatch_sgemm(variant, a, b, bias, 0, dst, out, M, N, K, one);
+    }
+    if (dpitch % 8 == 0) {       // the 8 consecutive k of a staging task never straddle a tap
+        Im2colA<true> a{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
+        FilterB<true> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
+        return dispatch_sgemm(variant, a, b, bias, 0, dst, out, M, N, K, one);
+    }
+    Im2colA<false> a{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
+    FilterB<false> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
+    return dispatch_sgemm(variant, a, b, bias, 0, dst, out, M, N, K, one);
+}
+
+}  // namespace decx_hip

@@ -1,0 +1,136 @@
+// fp32 tile launchers, the table of tile shapes and the shape choosers, shared by the dense GEMM and the convolution
+// translation units (each instantiates the kernels for its own operand sources).
+#pragma once
+#include "runtime.hpp"
+#include "sgemm_tile.hpp"
+
+namespace decx_hip {
+
+template <class S, class ASrc, class BSrc, class Out, bool HAS_C>
+int launch_sgemm_tile_c(const ASrc& a, const BSrc& b, const float* Cin, int ldc, float* D, const Out& out, int M, int N,
+                        int K, const Batch& batch) {
+    auto kern = sgemm_tile_kernel<S, ASrc, BSrc, Out, HAS_C>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)S::template lds_bytes<BSrc>()));
+        attr_done = true;
+    }
+    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    const long total = (long)tiles_m * tiles_n;
+    if (total > 0x7fffffffL || batch.count > 65535) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
+    const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
+    hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::template lds_bytes<BSrc>(), batch.stream, a, b, Cin,
+                       ldc, D, out, M, N, K, tiles_m, tiles_n, group_m, batch.stride_c, batch.stride_d, 0);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+template <class S, class ASrc, class BSrc, class Out>
+int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, float* D, const Out& out, int M, int N,
+                      int K, const Batch& batch) {
+    if (Cin != nullptr) return launch_sgemm_tile_c<S, ASrc, BSrc, Out, true>(a, b, Cin, ldc, D, out, M, N, K, batch);
+    return launch_sgemm_tile_c<S, ASrc, BSrc, Out, false>(a, b, Cin, ldc, D, out, M, N, K, batch);
+}
+
+// Tile shapes (variant numbers of decx_hip_set_sgemm_variant; results are identical for all of them):
+//   1: 256x256x16, 2x2 waves of 128x128   -- one wave per SIMD, highest reuse per LDS byte
+//   2: 128x128x16, 2x2 waves of  64x64    -- mid-size problems, several workgroups per CU
+//   3: 256x128x16, 2x2 waves of 128x64    -- narrow N
+//   4: 224x128x16, 1x4 waves of 224x32    -- 7/8 of shape 3 per tile: fills more CUs when M/256 tiles leave many idle
+//   5, 6: shapes 3 and 4 compiled for one wave per SIMD (512 registers, two staging sets) -- for long K walks and for
+//         launches that put at most one workgroup on a CU anyway
+//   7: 256x256x16, 4x2 waves of  64x128   -- two waves per SIMD: the matrix pipe takes the next MFMA from the other wave
+//         while one wave issues its loads and LDS traffic (a lone wave leaves ~3.5 idle cycles between 64-cycle MFMAs);
+//         the default for large problems, 1-2 % ahead of shape 1
+//   8:  64x64x16,  2x2 waves of  32x32    -- small problems: 1024^3 has only 64 tiles of 128x128 for 256 CUs
+//   9: 128x64x16,  2x2 waves of  64x32
+//  10: 224x256x16, 1x8 waves of 224x32    -- two waves per SIMD like 7; 7/8 of its tile, for tile counts that 7 rounds badly
+//  14: 192x192x16, 2x2 waves of  96x96    -- dense GEMM only: sizes that 256 and 128 divide into a bad number of tiles
+//         (3072^2 is 144 tiles of 256^2, 576 of 128^2, and exactly 256 of these)
+//  15: 224x128x16, 2x4 waves of 128x32 (upper row) and 96x32 (lower row) -- shape 6 on two waves per SIMD: each SIMD
+//         carries a 4-block and a 3-block wave
+// and, for dense GEMM only, the one-wave-per-16x16-block kernel of sgemm_chain16.hpp:
+//  11:  32x32x64,  2x2 computing + 4 moving waves, two workgroups per CU -- results too small to fill the chip with tiles
+//  12:  16x16x64,  1 computing + 2 moving waves -- at most one 16x16 block per CU: the fastest a single chain can walk K
+//  13:  64x64x64,  8 computing waves of two blocks each + 4 moving waves -- results of about one such tile per CU (1024^2)
+typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
+typedef SgemmShape<128, 128, 16, 2, 2, 2> SShapeSmall;
+typedef SgemmShape<256, 128, 16, 2, 2, 2> SShapeTall;
+typedef SgemmShape<224, 128, 16, 1, 4, 2> SShape224;
+typedef SgemmShape<256, 128, 16, 2, 2, 1> SShapeTallSolo;
+typedef SgemmShape<224, 128, 16, 1, 4, 1> SShape224Solo;
+typedef SgemmShape<256, 256, 16, 4, 2, 2, 2> SShapeBig8;
+typedef SgemmShape<224, 256, 16, 1, 8, 2, 2> SShape224Wide;   // 8 waves of 224x32, two per SIMD
+typedef SgemmShape<192, 192, 16, 2, 2, 1> SShape192;
+typedef SgemmShape<224, 128, 16, 2, 4, 2, 2, true> SShape224Split;   // 8 waves, 4 + 3 row blocks per SIMD
+typedef SgemmShape<64, 64, 16, 2, 2, 4> SShapeTiny;      // 2x2 waves of 32x32
+typedef SgemmShape<128, 64, 16, 2, 2, 4> SShapeTiny2;    // 2x2 waves of 64x32
+
+// Tile shape by a small cost model: a CU works through ceil(tiles / CUs) tiles one after another (tiles that share a CU
+// share its matrix pipe, so residency does not change this), a tile costs its area divided by how well that shape keeps
+// the pipe busy (measured on large squares, relative to shape 7).  The 256x128 and 224x128 shapes come in a
+// two-workgroups-per-CU build, better on short K walks where one tile's prologue and epilogue overlap the other's loop,
+// and a one-workgroup-per-CU build with deeper prefetch, better on long ones (224x128: shape 15, which measured 5-6 %
+// ahead of shape 6 on the 224x224x64 convolution under 128 filters; the same split of the 224x256 tile, and 256x128 on
+// 8 waves of 128x32, measured no better than shapes 10 and 5 and are not built).
+inline int pick_sgemm_variant(int M, int N, int K, int batch, bool dense = false) {
+    if ((g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) || g_rt.sgemm_variant == 15) return g_rt.sgemm_variant;
+    if (g_rt.sgemm_variant == 14) return dense ? 14 : 2;
+    const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+    struct Cand { int variant, bm, bn; double eff; };
+    const Cand cands[] = {{7, 256, 256, 1.00}, {10, 224, 256, 0.96}, {3, 256, 128, 0.95}, {4, 224, 128, 0.94}, {2, 128, 128, 0.89},
+                          {9, 128, 64, 0.83}, {8, 64, 64, 0.78}, {14, 192, 192, 0.93}};
+    int best = 7;
+    double best_cost = 0.0;
+    for (const Cand& c : cands) {
+        if (c.variant == 14 && !dense) continue;
+        const long tiles = (long)cdiv(M, c.bm) * cdiv(N, c.bn) * batch;
+        const double cost = (double)((tiles + cus - 1) / cus) * c.bm * c.bn / c.eff;
+        if (best_cost == 0.0 || cost < best_cost) {
+            best_cost = cost;
+            const bool one_per_cu = tiles <= cus || K >= 1024;
+            best = one_per_cu && c.variant == 3 ? 5 : one_per_cu && c.variant == 4 ? 15 : c.variant;
+        }
+    }
+    return best;
+}
+
+template <class ASrc, class BSrc, class Out>
+int dispatch_sgemm(int variant, const ASrc& a, const BSrc& b, const float* Cin, int ldc, float* D, const Out& out, int M,
+                   int N, int K, const Batch& batch) {
+    switch (variant) {
+        case 1: return launch_sgemm_tile<SShapeBig>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 3: return launch_sgemm_tile<SShapeTall>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 4: return launch_sgemm_tile<SShape224>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 5: return launch_sgemm_tile<SShapeTallSolo>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 6: return launch_sgemm_tile<SShape224Solo>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 7: return launch_sgemm_tile<SShapeBig8>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 8: return launch_sgemm_tile<SShapeTiny>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 9: return launch_sgemm_tile<SShapeTiny2>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 10: return launch_sgemm_tile<SShape224Wide>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 15: return launch_sgemm_tile<SShape224Split>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        default: return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K, batch);
+    }
+}
+
+// Which shape of the one-wave-per-block kernel (sgemm_chain16.hpp) a result of M x N takes, or 0 for the tiles.
+// Measured: ahead of the tiles up to about ten 32x32 tiles per CU -- 1536x1536 on 256 CUs -- 1.7x at 1024x8192x1024, 9x at
+// 64x65536x1024.  All paths give the same bits, so this is a choice of speed only.
+inline int pick_chain_shape(int M, int N, int K, int batch) {
+    if (g_rt.sgemm_variant >= 11 && g_rt.sgemm_variant <= 13) return g_rt.sgemm_variant;
+    if ((g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) || g_rt.sgemm_variant >= 14) return 0;
+    const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+    const long blocks16 = (long)cdiv(M, 16) * cdiv(N, 16) * batch, tiles32 = (long)cdiv(M, 32) * cdiv(N, 32) * batch;
+    // In units of one round of 32x32 tiles (two per CU, 512 on 256 CUs): a round of 64x64 tiles (one per CU) costs
+    // 1.55, further rounds of 32x32 tiles overlap with the first and cost 0.9 each once there is more than
+    // one (measured on squares of 640 .. 2560 at K = 512 and 2048).  Beyond 10 (K < 1024: 4) 32x32 tiles per CU
+    // the 32x32x2 tiles are ahead -- the block-chain kernels have the longer prologue.
+    const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch;
+    const double cost64 = 1.55 * (double)((tiles64 + cus - 1) / cus), pairs = (double)tiles32 / (2.0 * cus);
+    const double cost32 = pairs <= 1.0 ? 1.0 : 0.9 * (pairs + 0.5);
+    const long tile_limit = (K >= 1024 ? 10 : 4) * cus;
+    return blocks16 <= cus ? 12 : tiles32 > tile_limit ? 0 : cost64 < cost32 ? 13 : 11;
+}
+
+}  // namespace decx_hip

@@ -277,12 +277,6 @@ struct Im2colAUniform : Im2colA<true> {
     }
 };
 
-// ReLU exactly as the reference's element-wise kernel computes it (nn/operators/ReLU.h:57-82): the value times
-// float(sign bit clear).  Hence a negative input gives -0.0f, -inf gives NaN, NaN stays NaN.
-__device__ __forceinline__ float relu_by_sign(float v) {
-    return (float)((~__float_as_uint(v)) >> 31) * v;
-}
-
 // Result addressing: dense matrices (row m at m*ld) or the convolution's output tensor (pixel (y,x) at
 // y*row_stride + x*dpitch).  relu: apply relu_by_sign to every result element before it is stored.
 struct DenseOut {

@@ -17,6 +17,12 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kWave = 64;      // CDNA wavefront width
 constexpr int kXcds = 8;       // MI355X: 8 accelerator complex dies, 32 CUs and one 4 MiB L2 each
 
+// ReLU exactly as the reference's element-wise kernel computes it (nn/operators/ReLU.h:57-82): the value times
+// float(sign bit clear).  Hence a negative input gives -0.0f, -inf gives NaN, NaN stays NaN.
+__device__ __forceinline__ float relu_by_sign(float v) {
+    return (float)((~__float_as_uint(v)) >> 31) * v;
+}
+
 struct TileCoord {
     int tm, tn;
 };

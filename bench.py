@@ -34,11 +34,33 @@ def log(msg):
     print("[bench] " + msg, file=sys.stderr, flush=True)
 
 
+# Side workloads only (the headline runs exactly --warmup + --steps launches): lower bounds on the warm-up and on the
+# timed region, in milliseconds of back-to-back launches.  A sub-millisecond kernel launched after a host-side pause
+# starts on a chip that has clocked down and speeds up over the first tens of milliseconds (config 4 of the convolution:
+# 0.079 ms per launch at first, 0.069 ms from about 250 launches on), so a few dozen launches measure the ramp.
+SIDE_MIN_WARM_MS = 0.0
+SIDE_MIN_TIMED_MS = 0.0
+
+
 def time_launches(capi, launch, steps, warmup):
-    """Returns (wall ms per step, HIP-event ms per step) for `steps` back-to-back launches on the library's stream."""
+    """Returns (wall ms per step, HIP-event ms per step) for back-to-back launches on the library's stream: `warmup`
+    untimed and `steps` timed ones, both extended to the SIDE_MIN_* durations when those are set."""
+    t0 = time.perf_counter()
     for _ in range(warmup):
         launch()
     capi.sync()
+    if SIDE_MIN_WARM_MS > 0:
+        while (time.perf_counter() - t0) * 1e3 < SIDE_MIN_WARM_MS:
+            for _ in range(max(warmup, 1)):
+                launch()
+            capi.sync()
+    if SIDE_MIN_TIMED_MS > 0 and warmup > 0:
+        t1 = time.perf_counter()
+        for _ in range(warmup):
+            launch()
+        capi.sync()
+        pilot_ms = (time.perf_counter() - t1) * 1e3 / warmup
+        steps = max(steps, min(int(SIDE_MIN_TIMED_MS / max(pilot_ms, 1e-3)) + 1, 5000))
     t0 = time.perf_counter()
     capi.timer_start()
     for _ in range(steps):
@@ -287,6 +309,10 @@ def main():
     # the chip clocks down: give them more launches, and a longer warm-up, than the headline needs
     side_steps = max(20, min(args.steps * 3, 60))
     side_warmup = max(args.warmup, 10)
+    global SIDE_MIN_WARM_MS, SIDE_MIN_TIMED_MS
+    SIDE_MIN_WARM_MS, SIDE_MIN_TIMED_MS = 60.0, 30.0
+    also["side_timing"] = {"min_warmup_ms": SIDE_MIN_WARM_MS, "min_timed_ms": SIDE_MIN_TIMED_MS,
+                           "what": "every workload under `also` is warmed up and timed over at least this many ms of back-to-back launches"}
     if want("fp16"):
         r = bench_hgemm(capi, workloads, 8192, side_steps, side_warmup, 5)
         also["fp16_8192_f32acc"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),

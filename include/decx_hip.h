@@ -232,8 +232,8 @@ int decx_hip_timer_stop(float* milliseconds);
 const char* decx_hip_last_error(void);
 
 /* Tile-shape override for experiments: 0 = automatic choice by problem shape; other values select a fixed
- * kernel variant (see the table in backup_1_amd/csrc/decx_hip.hip).  Returns the previous value.  fp32 results never depend on
- * it (every shape walks k in the same order); fp16 results can differ in the last bit of the fp32 sum. */
+ * kernel variant (tables in backup_1_amd/csrc/sgemm_launch.hpp and hgemm.hip).  Returns the previous value.  fp32 results
+ * never depend on it (every shape walks k in the same order); fp16 results can differ in the last bit of the fp32 sum. */
 int decx_hip_set_sgemm_variant(int variant);
 int decx_hip_set_hgemm_variant(int variant);
 

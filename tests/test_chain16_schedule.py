@@ -71,5 +71,5 @@ def test_kernel_source_has_the_modelled_constants_and_bounds():
     src = open(os.path.join(csrc, "sgemm_chain16.hpp")).read()
     assert "BK = 64" in src and "LDS_BUFFERS = 3" in src
     assert "fetch_chunk + 1 < full_chunks" in src and "c0 + DEPTH <= full_chunks" in src
-    launches = open(os.path.join(csrc, "decx_hip.hip")).read()
+    launches = open(os.path.join(csrc, "sgemm_dense.hip")).read()
     assert "Chain16<2, 1, 4, 4>" in launches and "Chain16<1, 1, 8, 2>" in launches and "Chain16<4, 2, 2, 3>" in launches
