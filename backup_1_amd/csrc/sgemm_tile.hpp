@@ -285,6 +285,8 @@ struct DenseOut {
     bool relu = false;
     bool vec = false;      // every row of the result starts 16-byte aligned: runs of consecutive columns go out as one store
     __device__ __forceinline__ size_t offset(int m) const { return (size_t)m * ld; }
+    __device__ __forceinline__ bool rows_at_pitch() const { return true; }      // row m starts at pitched_offset(m)
+    __device__ __forceinline__ size_t pitched_offset(int m) const { return (size_t)m * ld; }
     __device__ __forceinline__ float finish(float v) const { return relu ? relu_by_sign(v) : v; }
 };
 struct TensorOut {
@@ -295,6 +297,8 @@ struct TensorOut {
     static constexpr bool vec = false;
     static constexpr bool PRELOAD_C = false;     // the "+ C" operand is a bias row, added to the finished sum
     __device__ __forceinline__ float finish(float v) const { return relu ? relu_by_sign(v) : v; }
+    __device__ __forceinline__ bool rows_at_pitch() const { return dense; }
+    __device__ __forceinline__ size_t pitched_offset(int m) const { return (size_t)m * dpitch; }
     __device__ __forceinline__ size_t offset(int m) const {
         if (dense) return (size_t)m * dpitch;
         const int y = m / Wout, x = m - y * Wout;
@@ -842,37 +846,44 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         // ---- epilogue.  Lane li holds, per row, the columns strip_col(ni, li) of its wave's strip: NI consecutive ones when B
         // came from a row-major matrix (one vector store per row where alignment and the edge allow), 32 apart otherwise.
         // dst = A*B + C adds C here (C may alias dst: every element is read and written by the same lane).
+        // FULL: the whole tile lies inside the result and row m starts at m times the pitch -- no bounds checks (each
+        // one is a branch around its store) and no division per row; the choice is one scalar branch per workgroup.
+        auto store_rows = [&](auto full_tag) {
+            constexpr bool FULL = decltype(full_tag)::value;
 #pragma unroll
-        for (int mi = 0; mi < MI; ++mi)
+            for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-                if (m < M) {
-                    float* drow = D + out.offset(m);
-                    const float* crow = HAS_C ? Cin + (size_t)m * ldc : nullptr;
-                    const bool add_c = HAS_C && !PRELOAD_C && (!SPLIT_K || blockIdx.z == 0);
-                    if (BSrc::ROW_MAJOR_LDS && !SPLIT_K && NI > 1 && NI != 3) {      // runs of 3 floats are not aligned for one store
-                        const int n0 = bn0 + wn0 + NI * li;
-                        if (out.vec && n0 + NI <= N) {
-                            typedef float vec_t __attribute__((ext_vector_type(NI)));
-                            vec_t v;
+                for (int r = 0; r < 16; ++r) {
+                    const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                    if (FULL || m < M) {
+                        float* drow = D + (FULL ? out.pitched_offset(m) : out.offset(m));
+                        const float* crow = HAS_C ? Cin + (size_t)m * ldc : nullptr;
+                        const bool add_c = HAS_C && !PRELOAD_C && (!SPLIT_K || blockIdx.z == 0);
+                        if (BSrc::ROW_MAJOR_LDS && !SPLIT_K && NI > 1 && NI != 3) {      // runs of 3 floats are not aligned for one store
+                            const int n0 = bn0 + wn0 + NI * li;
+                            if (out.vec && (FULL || n0 + NI <= N)) {
+                                typedef float vec_t __attribute__((ext_vector_type(NI)));
+                                vec_t v;
 #pragma unroll
-                            for (int ni = 0; ni < NI; ++ni) v[ni] = out.finish(add_c ? acc[mi][ni][r] + crow[n0 + ni] : acc[mi][ni][r]);
-                            *reinterpret_cast<vec_t*>(drow + n0) = v;
-                            continue;
+                                for (int ni = 0; ni < NI; ++ni) v[ni] = out.finish(add_c ? acc[mi][ni][r] + crow[n0 + ni] : acc[mi][ni][r]);
+                                *reinterpret_cast<vec_t*>(drow + n0) = v;
+                                continue;
+                            }
                         }
-                    }
 #pragma unroll
-                    for (int ni = 0; ni < NI; ++ni) {
-                        const int n = bn0 + wn0 + BSrc::template strip_col<S>(ni, li);
-                        if (n < N) {
-                            const float v = add_c ? acc[mi][ni][r] + crow[n] : acc[mi][ni][r];
-                            if (SPLIT_K) unsafeAtomicAdd(drow + n, v);      // hardware fp32 add in L2
-                            else drow[n] = out.finish(v);
+                        for (int ni = 0; ni < NI; ++ni) {
+                            const int n = bn0 + wn0 + BSrc::template strip_col<S>(ni, li);
+                            if (FULL || n < N) {
+                                const float v = add_c ? acc[mi][ni][r] + crow[n] : acc[mi][ni][r];
+                                if (SPLIT_K) unsafeAtomicAdd(drow + n, v);      // hardware fp32 add in L2
+                                else drow[n] = out.finish(v);
+                            }
                         }
                     }
                 }
-            }
+        };
+        if (!SPLIT_K && out.rows_at_pitch() && bm0 + BM <= M && bn0 + BN <= N) store_rows(std::true_type{});
+        else store_rows(std::false_type{});
     };
     if constexpr (S::UNEVEN_M) {
         // a branch on the scalar unit: the two wave rows run different instances, with the same sequence of barriers
