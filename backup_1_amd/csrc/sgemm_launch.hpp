@@ -48,6 +48,8 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //  10: 224x256x16, 1x8 waves of 224x32    -- two waves per SIMD like 7; 7/8 of its tile, for tile counts that 7 rounds badly
 //  14: 192x192x16, 2x2 waves of  96x96    -- dense GEMM only: sizes that 256 and 128 divide into a bad number of tiles
 //         (3072^2 is 144 tiles of 256^2, 576 of 128^2, and exactly 256 of these)
+//  16: shape 2 compiled for one wave per SIMD (two staging sets, one workgroup per CU): ahead of shape 2 wherever the
+//         cost model picks 128x128 tiles (2048^3: 0.140 -> 0.126 ms; 2048x2048x4096, two rounds: 0.259 -> 0.247 ms)
 //  15: 224x128x16, 2x4 waves of 128x32 (upper row) and 96x32 (lower row) -- shape 6 on two waves per SIMD: each SIMD
 //         carries a 4-block and a 3-block wave
 // and, for dense GEMM only, the one-wave-per-16x16-block kernel of sgemm_chain16.hpp:
@@ -64,6 +66,7 @@ typedef SgemmShape<256, 256, 16, 4, 2, 2, 2> SShapeBig8;
 typedef SgemmShape<224, 256, 16, 1, 8, 2, 2> SShape224Wide;   // 8 waves of 224x32, two per SIMD
 typedef SgemmShape<192, 192, 16, 2, 2, 1> SShape192;
 typedef SgemmShape<224, 128, 16, 2, 4, 2, 2, true> SShape224Split;   // 8 waves, 4 + 3 row blocks per SIMD
+typedef SgemmShape<128, 128, 16, 2, 2, 1> SShapeSmallSolo;
 typedef SgemmShape<64, 64, 16, 2, 2, 4> SShapeTiny;      // 2x2 waves of 32x32
 typedef SgemmShape<128, 64, 16, 2, 2, 4> SShapeTiny2;    // 2x2 waves of 64x32
 
@@ -75,11 +78,11 @@ typedef SgemmShape<128, 64, 16, 2, 2, 4> SShapeTiny2;    // 2x2 waves of 64x32
 // ahead of shape 6 on the 224x224x64 convolution under 128 filters; the same split of the 224x256 tile, and 256x128 on
 // 8 waves of 128x32, measured no better than shapes 10 and 5 and are not built).
 inline int pick_sgemm_variant(int M, int N, int K, int batch, bool dense = false) {
-    if ((g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) || g_rt.sgemm_variant == 15) return g_rt.sgemm_variant;
+    if ((g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) || g_rt.sgemm_variant == 15 || g_rt.sgemm_variant == 16) return g_rt.sgemm_variant;
     if (g_rt.sgemm_variant == 14) return dense ? 14 : 2;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     struct Cand { int variant, bm, bn; double eff; };
-    const Cand cands[] = {{7, 256, 256, 1.00}, {10, 224, 256, 0.96}, {3, 256, 128, 0.95}, {4, 224, 128, 0.94}, {2, 128, 128, 0.89},
+    const Cand cands[] = {{7, 256, 256, 1.00}, {10, 224, 256, 0.96}, {3, 256, 128, 0.95}, {4, 224, 128, 0.94}, {2, 128, 128, 0.92},
                           {9, 128, 64, 0.83}, {8, 64, 64, 0.78}, {14, 192, 192, 0.93}};
     int best = 7;
     double best_cost = 0.0;
@@ -90,7 +93,7 @@ inline int pick_sgemm_variant(int M, int N, int K, int batch, bool dense = false
         if (best_cost == 0.0 || cost < best_cost) {
             best_cost = cost;
             const bool one_per_cu = tiles <= cus || K >= 1024;
-            best = one_per_cu && c.variant == 3 ? 5 : one_per_cu && c.variant == 4 ? 15 : c.variant;
+            best = one_per_cu && c.variant == 3 ? 5 : one_per_cu && c.variant == 4 ? 15 : c.variant == 2 ? 16 : c.variant;
         }
     }
     return best;
@@ -110,6 +113,7 @@ int dispatch_sgemm(int variant, const ASrc& a, const BSrc& b, const float* Cin, 
         case 9: return launch_sgemm_tile<SShapeTiny2>(a, b, Cin, ldc, D, out, M, N, K, batch);
         case 10: return launch_sgemm_tile<SShape224Wide>(a, b, Cin, ldc, D, out, M, N, K, batch);
         case 15: return launch_sgemm_tile<SShape224Split>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 16: return launch_sgemm_tile<SShapeSmallSolo>(a, b, Cin, ldc, D, out, M, N, K, batch);
         default: return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K, batch);
     }
 }

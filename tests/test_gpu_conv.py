@@ -15,7 +15,7 @@ CASES = [  # H, W, C, N, kh, kw, flag
 ]
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 15])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 15, 16])
 @pytest.mark.parametrize("case", CASES)
 def test_integer_exact(gpu, oracle, case, variant):
     H, W, C, N, kh, kw, flag = case
@@ -24,7 +24,7 @@ def test_integer_exact(gpu, oracle, case, variant):
     assert np.array_equal(gpu_conv(src, filt, flag, variant=variant), oracle.conv2_chain(src, filt, flag))
 
 
-@pytest.mark.parametrize("variant", [0, 2, 6, 7, 8, 11, 12, 13, 15])
+@pytest.mark.parametrize("variant", [0, 2, 6, 7, 8, 11, 12, 13, 15, 16])
 @pytest.mark.parametrize("case", CASES)
 def test_real_valued_data_bit_exact_with_the_chain(gpu, oracle, case, variant):
     # channel counts 3, 4, 6, 8, 12-ish exercise both loader builds (channel pitch a multiple of 8 or only of 4)
