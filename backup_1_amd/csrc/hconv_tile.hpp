@@ -115,6 +115,18 @@ __device__ __forceinline__ void hconv_store_tile(const f32x16 (&acc)[S::MI][S::N
     constexpr int UNITS_PER_ROW = BN / 8, OUT_PASSES = BM * UNITS_PER_ROW / NT;
     // whole 16-byte units when dst allows it (pixel pitch a multiple of 8 halves, 16-byte aligned base), else half by half
     const bool vec = out.dpitch % 8 == 0 && out.row_stride % 8 == 0 && (reinterpret_cast<size_t>(out.dst) & 15) == 0;
+    // a whole tile of a tensor whose pixels lie back to back: pixel m starts at m * dpitch -- no bounds branches, no
+    // division per piece (one scalar test per workgroup)
+    if (vec && out.row_stride == (size_t)out.Wout * out.dpitch && bm0 + BM <= M && bn0 + BN <= N) {
+#pragma unroll
+        for (int p = 0; p < OUT_PASSES; ++p) {
+            const int id = tid + p * NT, row = id / UNITS_PER_ROW, u = id % UNITS_PER_ROW;
+            const _Float16* t8 = tile + row * S::OUT_ROW + 8 * u;
+            const u32x2 lo = *reinterpret_cast<const u32x2*>(t8), hi = *reinterpret_cast<const u32x2*>(t8 + 4);
+            *reinterpret_cast<u32x4*>(out.dst + (size_t)(bm0 + row) * out.dpitch + bn0 + 8 * u) = u32x4{lo[0], lo[1], hi[0], hi[1]};
+        }
+        return;
+    }
 #pragma unroll
     for (int p = 0; p < OUT_PASSES; ++p) {
         const int id = tid + p * NT, row = id / UNITS_PER_ROW, u = id % UNITS_PER_ROW;
