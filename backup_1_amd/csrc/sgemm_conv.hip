@@ -5,6 +5,15 @@
 
 namespace decx_hip {
 
+// One translation unit per loader build instantiates the tile kernels for it (sgemm_conv_uniform.hip,
+// sgemm_conv_paired.hip, sgemm_conv_plain.hip): they compile side by side.
+int conv_dispatch_uniform(int variant, const Im2colAUniform& a, const FilterBUniform& b, const float* bias, float* dst,
+                          const TensorOut& out, int M, int N, int K, const Batch& batch);
+int conv_dispatch_paired(int variant, const Im2colA<true>& a, const FilterB<true>& b, const float* bias, float* dst,
+                         const TensorOut& out, int M, int N, int K, const Batch& batch);
+int conv_dispatch_plain(int variant, const Im2colA<false>& a, const FilterB<false>& b, const float* bias, float* dst,
+                        const TensorOut& out, int M, int N, int K, const Batch& batch);
+
 template <class S>
 int launch_conv_chain16(const Im2colA<false>& img, const FilterB<false>& fb, const float* bias, float* dst, const TensorOut& out,
                         int M, int N, int K) {
@@ -66,16 +75,16 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
     if (dpitch % 16 == 0) {      // a whole K step inside one tap: the tap walk runs on the scalar unit
         Im2colAUniform a{{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes}};
         FilterBUniform b{{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes}};
-        return dispatch_sgemm(variant, a, b, bias, 0, dst, out, M, N, K, one);
+        return conv_dispatch_uniform(variant, a, b, bias, dst, out, M, N, K, one);
     }
     if (dpitch % 8 == 0) {       // the 8 consecutive k of a staging task never straddle a tap
         Im2colA<true> a{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
         FilterB<true> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
-        return dispatch_sgemm(variant, a, b, bias, 0, dst, out, M, N, K, one);
+        return conv_dispatch_paired(variant, a, b, bias, dst, out, M, N, K, one);
     }
     Im2colA<false> a{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
     FilterB<false> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
-    return dispatch_sgemm(variant, a, b, bias, 0, dst, out, M, N, K, one);
+    return conv_dispatch_plain(variant, a, b, bias, dst, out, M, N, K, one);
 }
 
 }  // namespace decx_hip

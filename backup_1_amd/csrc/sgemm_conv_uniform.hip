@@ -1,0 +1,13 @@
+// fp32 fused im2col convolution: the tile kernels (sgemm_tile.hpp) for the loaders of
+// a channel pitch that is a multiple of the K step (the tap walk runs on the scalar unit).
+#include "sgemm_launch.hpp"
+
+namespace decx_hip {
+
+int conv_dispatch_uniform(int variant, const Im2colAUniform& a, const FilterBUniform& b, const float* bias, float* dst,
+                     const TensorOut& out, int M, int N, int K, const Batch& batch) {
+    // a bias is the "+ C" operand with row stride 0: every output pixel adds the same N values
+    return dispatch_sgemm(variant, a, b, bias, 0, dst, out, M, N, K, batch);
+}
+
+}  // namespace decx_hip
