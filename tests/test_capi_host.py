@@ -42,3 +42,19 @@ def test_init_without_device_fails_cleanly():
     rc = capi.lib().decx_hip_init(ctypes.byref(dev))
     assert rc != 0 and not capi.lib().decx_hip_is_init()
     assert capi.last_error().strip() != ""
+
+
+def test_every_hip_source_is_in_the_makefile():
+    # the library is one translation unit per kernel family: a source missing from SRCS would silently drop its entry points
+    csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "backup_1_amd", "csrc")
+    mk = open(os.path.join(csrc, "Makefile")).read().replace("\\\n", " ")
+    srcs = next(l for l in mk.splitlines() if l.startswith("SRCS")).split(":=")[1].split()
+    assert sorted(srcs) == sorted(f for f in os.listdir(csrc) if f.endswith(".hip"))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in r.stderr
