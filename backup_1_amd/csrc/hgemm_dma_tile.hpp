@@ -343,22 +343,28 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
             }
         return;
     }
-    // ---- epilogue: round once to binary16; dst = A*B + C adds C (as fp32) first ---------------------------------------
+    // ---- epilogue: round once to binary16; dst = A*B + C adds C (as fp32) first.  A tile that lies wholly inside the
+    // result stores without bounds checks (each one is a branch around its store; one scalar test per workgroup).
+    auto store_tile = [&](auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;
 #pragma unroll
-    for (int mi = 0; mi < MI; ++mi)
+        for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
-            if (m < M) {
-                _Float16* drow = D + (size_t)m * ldd;
-                const _Float16* crow = HAS_C ? Cin + (size_t)m * ldc : nullptr;
+            for (int r = 0; r < 16; ++r) {
+                const int m = bm0 + wm0 + mi * 32 + (r >> 2) * 8 + lh * 4 + (r & 3);
+                if (FULL || m < M) {
+                    _Float16* drow = D + (size_t)m * ldd;
+                    const _Float16* crow = HAS_C ? Cin + (size_t)m * ldc : nullptr;
 #pragma unroll
-                for (int ni = 0; ni < NI; ++ni) {
-                    const int n = bn0 + wn0 + ni * 32 + li;
-                    if (n < N) drow[n] = (_Float16)(HAS_C ? acc[mi][ni][r] + (float)crow[n] : acc[mi][ni][r]);
+                    for (int ni = 0; ni < NI; ++ni) {
+                        const int n = bn0 + wn0 + ni * 32 + li;
+                        if (FULL || n < N) drow[n] = (_Float16)(HAS_C ? acc[mi][ni][r] + (float)crow[n] : acc[mi][ni][r]);
+                    }
                 }
             }
-        }
+    };
+    if (bm0 + BM <= M && bn0 + BN <= N) store_tile(std::true_type{});
+    else store_tile(std::false_type{});
 }
 
 }  // namespace decx_hip
