@@ -111,7 +111,11 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
                              (long)H * W < (1L << 22);
     const bool narrow = N <= 64;
     const bool many_tiles = narrow ? (long)cdiv(M, 256) >= 3 * cus / 4 : tall;
-    if (taprow_fits && ((many_tiles && (g_rt.hgemm_variant < 12 || g_rt.hgemm_variant > 13)) || g_rt.hgemm_variant == 14)) {
+    // measured in steady state against the other kernels' best: ahead from a quarter of the CUs holding a tile (64 tiles:
+    // 128x128x128 under 128 5x5 filters 36.3 -> 34.1 us; 98 tiles: 112x112x128 under 256 3x3 filters 17.4 -> 16.8 us),
+    // behind at 26 tiles (56x56x256 under 256 filters, where the split over K wins)
+    const bool taprow_tiles = (long)cdiv(M, 256) * (narrow ? 1 : cdiv(N, 128)) >= cus / 4;
+    if (taprow_fits && ((taprow_tiles && (g_rt.hgemm_variant < 12 || g_rt.hgemm_variant > 13)) || g_rt.hgemm_variant == 14)) {
         auto launch_taprow = [&](auto shape) -> int {
             typedef decltype(shape) S;
             static_assert(S::PATCH_ROWS == 320, "the fit test above is written for this patch");
