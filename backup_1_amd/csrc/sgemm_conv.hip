@@ -65,7 +65,13 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
     const int oy = flag ? kh / 2 : 0, ox = flag ? kw / 2 : 0;
     // a bias is the "+ C" operand with row stride 0: every output pixel adds the same N values
     // small images: too few tiles for the chip, the one-wave-per-block kernel takes them (conv_chain16.hpp)
-    if (const int chain = pick_chain_shape(M, N, K, 1)) {
+    // (its 64x64 shape walks a convolution 14 % slower than a dense product of the same size -- the moving waves do the
+    // im2col addressing -- so once 128x64 tiles cover three quarters of the CUs the tiles are ahead: 112x112x128 under 128
+    // filters 57.1 -> 50.6 us)
+    int chain = pick_chain_shape(M, N, K, 1);
+    if (chain == 13 && g_rt.sgemm_variant == 0 && (long)cdiv(M, 128) * cdiv(N, 64) >= 3 * (g_rt.compute_units > 0 ? g_rt.compute_units : 256) / 4)
+        chain = 0;
+    if (chain) {
         Im2colA<false> a{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
         FilterB<false> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
         if (chain == 11) return launch_conv_chain16<Chain16<2, 1, 4, 4>>(a, b, bias, dst, out, M, N, K);
