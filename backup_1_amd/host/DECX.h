@@ -61,7 +61,9 @@ struct alignas(2) Half {
 Half Float2Half(const float& x);
 float Half2Float(const Half& x);
 
-// classes/Matrix.h:34-64
+// classes/Matrix.h:34-64.  TotalBytes() is width * height * sizeof(T) (Matrix.h:104, :262-263), not the pitched size.
+// operator= of every container shares src's payload instead of copying it, as in the reference (Matrix.h:510-530):
+// both objects then address the same memory, and it is freed when the last holder releases it.
 template <typename T>
 class Matrix {
 public:
@@ -215,8 +217,9 @@ DH GEMM(GPU_Matrix<float>& A, GPU_Matrix<float>& B, GPU_Matrix<float>& dst);
 DH GEMM(GPU_Matrix<float>& A, GPU_Matrix<float>& B, GPU_Matrix<float>& C, GPU_Matrix<float>& dst);
 DH GEMM(GPU_Matrix<Half>& A, GPU_Matrix<Half>& B, GPU_Matrix<Half>& dst);
 DH GEMM(GPU_Matrix<Half>& A, GPU_Matrix<Half>& B, GPU_Matrix<Half>& C, GPU_Matrix<Half>& dst);
-// GEMM/CUDA/extreme_shapes/GEMM_long_Lr.h:22.  dst = A * B for short-M / long-K shapes (split-K underneath).  Unlike
-// the reference it checks initialisation and dimensions, sizes dst, handles any shape and reports its status.
+// GEMM/CUDA/extreme_shapes/GEMM_long_Lr.h:22.  dst = A * B for short-M / long-K shapes: one fused chain per output over
+// ascending k like the reference's kernel (no split over K), so the result is bit-identical to GEMM's.  Unlike the
+// reference it checks initialisation and dimensions, sizes dst, handles any shape and reports its status.
 DH GEMM_Long_Lr(GPU_Matrix<float>& A, GPU_Matrix<float>& B, GPU_Matrix<float>& dst);
 // GEMM/CUDA/large_squares/GEMM3.h:27-36.  dst[i] = A[i] * B[i] (+ C[i]) for every matrix of the arrays, uploads and
 // downloads overlapped with the kernels.

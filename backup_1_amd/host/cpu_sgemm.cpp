@@ -65,8 +65,19 @@ DH sgemm(Matrix<float>& A_, Matrix<float>& B_, Matrix<float>& dst_) {
     if (!A || !B || !dst) return DH{decx::DECX_FAIL_ErrorParams, factory_msg};
     if (A->width != B->height) return DH{decx::DECX_FAIL_DimsNotMatching, dims_msg};       // sgemm.h:35-38
     const int M = (int)A->height, K = (int)A->width, N = (int)B->width;
-    if (!dst->re_construct((uint)N, (uint)M, decx::Page_Default)) return DH{decx::DECX_FAIL_ALLOCATION, alloc_msg};
-    if (M == 0 || N == 0) return DH{decx::DECX_SUCCESS, ok_msg};
+    // a dst that is (or shares its payload with) an operand is computed into a fresh matrix whose payload it then takes
+    decx::_Matrix<float> fresh;
+    decx::_Matrix<float>* user_dst = dst;
+    if (dst == A || dst == B || dst->shares_block_with(*A) || dst->shares_block_with(*B)) {
+        if (!fresh.construct((uint)N, (uint)M, decx::Page_Default)) return DH{decx::DECX_FAIL_ALLOCATION, alloc_msg};
+        dst = &fresh;
+    } else if (!dst->re_construct((uint)N, (uint)M, decx::Page_Default)) {
+        return DH{decx::DECX_FAIL_ALLOCATION, alloc_msg};
+    }
+    if (M == 0 || N == 0) {
+        if (dst != user_dst) user_dst->share_from(fresh);
+        return DH{decx::DECX_SUCCESS, ok_msg};
+    }
 
     const int n8 = (N + 7) / 8 * 8;                      // columns are produced in units of 8, inside the pitch
     const int panels = (n8 + kPanel - 1) / kPanel;
@@ -111,6 +122,7 @@ DH sgemm(Matrix<float>& A_, Matrix<float>& B_, Matrix<float>& dst_) {
         }
     });
     std::free(packed);
+    if (dst != user_dst) user_dst->share_from(fresh);
     return DH{decx::DECX_SUCCESS, ok_msg};
 }
 

@@ -75,11 +75,28 @@ de::DH gemm_host(de::Matrix<T>& A_, de::Matrix<T>& B_, de::Matrix<T>* C_, de::Ma
     if (C && (C->width != B->width || C->height != A->height))                            // GEMM.h:154-157
         return de::DH{decx::DECX_FAIL_DimsNotMatching, kMDims};
     const int M = (int)A->height, K = (int)A->width, N = (int)B->width;
-    // dst takes its size from the operands (GEMM.h:73); when C is the same object it already has it and keeps its data
-    if (!dst->re_construct((uint)N, (uint)M, decx::Page_Locked)) return alloc_fail();
+    // dst takes its size from the operands (GEMM.h:73).  The pipeline below downloads finished regions of dst while
+    // later panels of A and B are still being uploaded, so a dst that is (or shares its payload with) A or B is
+    // computed into a fresh matrix whose payload dst then takes over; a dst that shares C's payload is used in
+    // place whatever its store type (C is read and dst written region by region, in that order), since
+    // re_construct with another store type would free C's data before it is uploaded.
+    const bool over_operand = dst == A || dst == B || dst->shares_block_with(*A) || dst->shares_block_with(*B);
+    const bool over_c = C && (dst == C || dst->shares_block_with(*C));
+    decx::_Matrix<T> fresh;
+    decx::_Matrix<T>* out = dst;
+    if (over_operand) {
+        if (!fresh.construct((uint)N, (uint)M, decx::Page_Locked)) return alloc_fail();
+        out = &fresh;
+    } else if (over_c) {
+        if (dst->width != (uint)N || dst->height != (uint)M || !dst->Mat.ptr) return de::DH{decx::DECX_FAIL_DimsNotMatching, kMDims};
+    } else if (!dst->re_construct((uint)N, (uint)M, decx::Page_Locked)) {
+        return alloc_fail();
+    }
     // allocation, uploads, kernel and download, pipelined over row panels, all below the C ABI
-    return from_status(HostGemmCall<T>::run(A->Mat.ptr, (int)A->pitch, B->Mat.ptr, (int)B->pitch, C ? C->Mat.ptr : nullptr,
-                                            C ? (int)C->pitch : 0, dst->Mat.ptr, (int)dst->pitch, M, N, K));
+    const int rc = HostGemmCall<T>::run(A->Mat.ptr, (int)A->pitch, B->Mat.ptr, (int)B->pitch, C ? C->Mat.ptr : nullptr,
+                                        C ? (int)C->pitch : 0, out->Mat.ptr, (int)out->pitch, M, N, K);
+    if (rc == 0 && out != dst) dst->share_from(fresh);   // dst now shares the fresh payload; the operand it stood for keeps its own
+    return from_status(rc);
 }
 
 template <typename T>
@@ -339,13 +356,16 @@ DH conv_host(Tensor<T>& src_, TensorArray<T>& kernel_, Tensor<T>& dst_, const in
     int Hout = 0, Wout = 0;
     DH pre = conv_precheck(src->depth, ker->depth, H, W, kh, kw, flag, Hout, Wout);
     if (pre.error_type != decx::DECX_SUCCESS) return pre;
-    if (!dst->re_construct((uint)Wout, (uint)Hout, ker->tensor_num, decx::Page_Locked)) return alloc_fail();   // :178
+    decx::_Tensor<T> out_shape;
+    out_shape.attribute_assign((uint)Wout, (uint)Hout, ker->tensor_num, decx::Page_Locked);
     DeviceTemp dS, dK, dD;
-    if (dS.alloc(src->total_bytes) || dK.alloc(ker->total_bytes) || dD.alloc(dst->total_bytes)) return alloc_fail();
+    if (dS.alloc(src->total_bytes) || dK.alloc(ker->total_bytes) || dD.alloc(out_shape.total_bytes)) return alloc_fail();
     int rc = decx_hip_memcpy(dS.ptr, src->Tens.ptr, src->total_bytes, DECX_HIP_H2D);
     if (rc) return from_status(rc);
     rc = decx_hip_memcpy(dK.ptr, ker->TensArr.ptr, ker->total_bytes, DECX_HIP_H2D);
     if (rc) return from_status(rc);
+    // sized (and zero-filled) only now that the operands are on the device: dst may be src or share its payload
+    if (!dst->re_construct((uint)Wout, (uint)Hout, ker->tensor_num, decx::Page_Locked)) return alloc_fail();   // :178
     rc = decx_hip_memset(dD.ptr, 0, dst->total_bytes);   // the width / channel padding of dst stays zero
     if (rc) return from_status(rc);
     rc = ConvCall<T>::run(static_cast<const T*>(dS.ptr), H, W, (int)src->dpitch, src->dp_x_wp, static_cast<const T*>(dK.ptr),
@@ -423,7 +443,7 @@ DH ReLU_f_Rec(GPU_Matrix<float>& src, GPU_Matrix<float>& dst, GPU_Matrix<uchar>&
     if (!a.ok) return a.status;
     auto* map = dynamic_cast<decx::_GPU_Matrix<uchar>*>(&rec_map);
     if (!map) return DH{decx::DECX_FAIL_ErrorParams, kNotFactory};
-    if ((!map->Mat.ptr || map->total_bytes < a.len / 8) && !map->re_construct(a.src->pitch / 8, a.src->height))
+    if ((!map->Mat.ptr || map->_total_bytes < a.len / 8) && !map->re_construct(a.src->pitch / 8, a.src->height))
         return map->last_status == DECX_HIP_FAIL_ALLOCATION ? alloc_fail() : from_status(map->last_status);
     return from_status(decx_hip_relu_f32_rec(a.src->Mat.ptr, a.dst->Mat.ptr, map->Mat.ptr, a.len));
 }
@@ -434,7 +454,7 @@ DH ReLU_f_Backward(GPU_Matrix<float>& src, GPU_Matrix<float>& dst, GPU_Matrix<uc
     auto* map = dynamic_cast<decx::_GPU_Matrix<uchar>*>(&rec_map);
     if (!map) return DH{decx::DECX_FAIL_ErrorParams, kNotFactory};
     static char dims_msg[] = "Matrix Dims don't match each other";
-    if (!map->Mat.ptr || map->total_bytes < a.len / 8) return DH{decx::DECX_FAIL_DimsNotMatching, dims_msg};
+    if (!map->Mat.ptr || map->_total_bytes < a.len / 8) return DH{decx::DECX_FAIL_DimsNotMatching, dims_msg};
     return from_status(decx_hip_relu_f32_backward(a.src->Mat.ptr, a.dst->Mat.ptr, map->Mat.ptr, a.len));
 }
 }  // namespace nn

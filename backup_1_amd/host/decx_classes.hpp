@@ -5,10 +5,19 @@
 //                         zero-filled on allocation (classes/Tensor.h:162-184, :312, :389-394)
 //   TensorArray         : tensor_num tensors back to back, stride _gap = dp_x_wp * height
 //                         (classes/TensorArray.h:174-198, :349-352, :521-525)
-// Field names follow the reference so that code reading them ports directly.
+// Field names and their meaning follow the reference, so that code reading them ports directly:
+//   Matrix / GPU_Matrix : element_num = width*height, total_bytes = element_num*sizeof(T)          (the true extent)
+//                         _element_num = pitch*height, _total_bytes = _element_num*sizeof(T)        (the allocation)
+//                         (Matrix.h:253-267, :308-322; GPU_Matrix.h:211-223, :259-271); TotalBytes() = total_bytes
+//   Tensor(Array), MatrixArray : element_num = true count, _element_num = padded count, total_bytes = padded bytes
+//                         (Tensor.h:162-184, TensorArray.h:174-198, MatrixArray.h:222-239)
+// operator= shares the payload like the reference (Matrix.h:510-530, GPU_Matrix.h:441-451, Tensor.h:501-526,
+// MatrixArray.h:473-498: the block pointer is copied and its reference count raised): both objects then read and write
+// the same memory, release() of one leaves the other valid, the last release frees it.
 #pragma once
 #include <cstdlib>
 #include <cstring>
+#include <memory>
 
 #include "../../include/decx_hip.h"
 #include "DECX.h"
@@ -46,6 +55,29 @@ struct HostBlock {
         else std::free(ptr);
         ptr = nullptr;
     }
+    HostBlock() = default;
+    HostBlock(const HostBlock&) = delete;
+    HostBlock& operator=(const HostBlock&) = delete;
+    ~HostBlock() { free(); }
+};
+
+// Device storage through the C ABI; zero-filled over its whole (padded) size.
+struct DeviceBlock {
+    void* ptr = nullptr;
+    int alloc(size_t bytes) {
+        free();
+        int rc = decx_hip_malloc(&ptr, bytes ? bytes : 64);
+        if (rc != 0) { ptr = nullptr; return rc; }
+        return decx_hip_memset(ptr, 0, bytes);
+    }
+    void free() {
+        if (ptr) decx_hip_free(ptr);
+        ptr = nullptr;
+    }
+    DeviceBlock() = default;
+    DeviceBlock(const DeviceBlock&) = delete;
+    DeviceBlock& operator=(const DeviceBlock&) = delete;
+    ~DeviceBlock() { free(); }
 };
 
 template <typename T>
@@ -55,15 +87,15 @@ struct PtrInfo {   // the reference's decx::PtrInfo<T> exposes .ptr (core/memory
 
 template <typename T>
 class _Matrix : public de::Matrix<T> {
-    HostBlock block_;
+    std::shared_ptr<HostBlock> block_;
 
 public:
     uint width = 0, height = 0;
     unsigned short Store_Type = Page_Default;
-    size_t element_num = 0, total_bytes = 0;     // padded (pitch * height)
+    size_t element_num = 0, total_bytes = 0;     // true extent: width * height            (Matrix.h:262-263)
     uint pitch = 0;
     PtrInfo<T> Mat;
-    size_t _element_num = 0, _total_bytes = 0;   // true (width * height)
+    size_t _element_num = 0, _total_bytes = 0;   // the allocation: pitch * height         (Matrix.h:265-266)
 
     _Matrix() {}
     _Matrix(uint w, uint h, int store_type) { construct(w, h, store_type); }
@@ -72,48 +104,56 @@ public:
         height = h;
         Store_Type = (unsigned short)store_type;
         pitch = ceil_to(w, matrix_align<T>());
-        _element_num = (size_t)w * h;
-        _total_bytes = _element_num * sizeof(T);
-        element_num = (size_t)pitch * h;
+        element_num = (size_t)w * h;
         total_bytes = element_num * sizeof(T);
+        _element_num = (size_t)pitch * h;
+        _total_bytes = _element_num * sizeof(T);
     }
     bool construct(uint w, uint h, int store_type) {
         attribute_assign(w, h, store_type);
-        bool ok = block_.alloc(total_bytes, store_type);
-        Mat.ptr = static_cast<T*>(block_.ptr);
+        block_ = std::make_shared<HostBlock>();
+        bool ok = block_->alloc(_total_bytes, store_type);
+        Mat.ptr = static_cast<T*>(block_->ptr);
         return ok;
     }
-    bool re_construct(uint w, uint h, int store_type) {
+    bool re_construct(uint w, uint h, int store_type) {   // Matrix.h:238-248: a no-op only when nothing changes
         if (Mat.ptr && w == width && h == height && store_type == Store_Type) return true;
         return construct(w, h, store_type);
     }
+    bool shares_block_with(const _Matrix<T>& o) const { return block_ && block_ == o.block_; }
     uint Width() override { return width; }
     uint Height() override { return height; }
     size_t TotalBytes() override { return total_bytes; }
     T& index(const int row, const int col) override { return Mat.ptr[(size_t)pitch * row + col]; }
     void release() override {
-        block_.free();
+        block_.reset();
         Mat.ptr = nullptr;
     }
-    de::Matrix<T>& operator=(de::Matrix<T>& src) override {   // shallow alias in the reference; deep copy is the safe reading
-        _Matrix<T>& s = dynamic_cast<_Matrix<T>&>(src);
-        if (&s != this) {
-            construct(s.width, s.height, s.Store_Type);
-            std::memcpy(Mat.ptr, s.Mat.ptr, total_bytes);
-        }
+    void share_from(_Matrix<T>& s) {
+        if (&s == this) return;
+        block_ = s.block_;
+        attribute_assign(s.width, s.height, s.Store_Type);
+        Mat.ptr = s.Mat.ptr;
+    }
+    de::Matrix<T>& operator=(de::Matrix<T>& src) override {   // shares src's block (Matrix.h:510-530)
+        share_from(dynamic_cast<_Matrix<T>&>(src));
         return *this;
     }
+    _Matrix(const _Matrix&) = delete;
+    _Matrix& operator=(const _Matrix&) = delete;
     ~_Matrix() override { release(); }
 };
 
 template <typename T>
 class _GPU_Matrix : public de::GPU_Matrix<T> {
+    std::shared_ptr<DeviceBlock> block_;
+
 public:
     uint width = 0, height = 0;
-    size_t element_num = 0, total_bytes = 0;     // padded
+    size_t element_num = 0, total_bytes = 0;     // true extent: width * height            (GPU_Matrix.h:218-219)
     uint pitch = 0;
     PtrInfo<T> Mat;                              // DEVICE pointer
-    size_t _element_num = 0, _total_bytes = 0;
+    size_t _element_num = 0, _total_bytes = 0;   // the allocation: pitch * height         (GPU_Matrix.h:221-222)
     int last_status = 0;                         // status of the most recent allocation / copy
 
     _GPU_Matrix() {}
@@ -122,19 +162,18 @@ public:
         width = w;
         height = h;
         pitch = ceil_to(w, matrix_align<T>());
-        _element_num = (size_t)w * h;
-        _total_bytes = _element_num * sizeof(T);
-        element_num = (size_t)pitch * h;
+        element_num = (size_t)w * h;
         total_bytes = element_num * sizeof(T);
+        _element_num = (size_t)pitch * h;
+        _total_bytes = _element_num * sizeof(T);
     }
     bool construct(uint w, uint h) {
         release();
         attribute_assign(w, h);
-        void* p = nullptr;
-        last_status = decx_hip_malloc(&p, total_bytes);
-        if (last_status != 0) return false;
-        Mat.ptr = static_cast<T*>(p);
-        last_status = decx_hip_memset(p, 0, total_bytes);   // the whole pitched buffer (the reference clears only width*height bytes)
+        block_ = std::make_shared<DeviceBlock>();
+        // zero the whole pitched buffer (the reference clears only total_bytes of it, GPU_Matrix.h:152, :167)
+        last_status = block_->alloc(_total_bytes);
+        Mat.ptr = static_cast<T*>(block_->ptr);
         return last_status == 0;
     }
     bool re_construct(uint w, uint h) {
@@ -157,13 +196,16 @@ public:
                                         (size_t)width * sizeof(T), height, DECX_HIP_D2H);
     }
     void release() override {
-        if (Mat.ptr) decx_hip_free(Mat.ptr);
+        block_.reset();
         Mat.ptr = nullptr;
     }
-    de::GPU_Matrix<T>& operator=(de::GPU_Matrix<T>& src) override {
+    de::GPU_Matrix<T>& operator=(de::GPU_Matrix<T>& src) override {   // shares src's block (GPU_Matrix.h:441-451)
         _GPU_Matrix<T>& s = dynamic_cast<_GPU_Matrix<T>&>(src);
-        if (&s != this && construct(s.width, s.height))
-            last_status = decx_hip_memcpy(Mat.ptr, s.Mat.ptr, total_bytes, DECX_HIP_D2D);
+        if (&s != this) {
+            block_ = s.block_;
+            attribute_assign(s.width, s.height);
+            Mat.ptr = s.Mat.ptr;
+        }
         return *this;
     }
     ~_GPU_Matrix() override { release(); }
@@ -171,7 +213,7 @@ public:
 
 template <typename T>
 class _Tensor : public de::Tensor<T> {
-    HostBlock block_;
+    std::shared_ptr<HostBlock> block_;
 
 public:
     uint width = 0, height = 0, depth = 0;
@@ -197,8 +239,9 @@ public:
     }
     bool construct(uint w, uint h, uint d, int store_type) {
         attribute_assign(w, h, d, store_type);
-        bool ok = block_.alloc(total_bytes, store_type);
-        Tens.ptr = static_cast<T*>(block_.ptr);
+        block_ = std::make_shared<HostBlock>();
+        bool ok = block_->alloc(total_bytes, store_type);
+        Tens.ptr = static_cast<T*>(block_->ptr);
         if (ok) std::memset(Tens.ptr, 0, total_bytes);
         return ok;
     }
@@ -213,16 +256,17 @@ public:
     uint Height() override { return height; }
     uint Depth() override { return depth; }
     T& index(const int x, const int y, const int z) override { return Tens.ptr[(size_t)x * dp_x_wp + (size_t)y * dpitch + z]; }
-    de::Tensor<T>& operator=(de::Tensor<T>& src) override {
+    de::Tensor<T>& operator=(de::Tensor<T>& src) override {   // shares src's block (Tensor.h:501-526)
         _Tensor<T>& s = dynamic_cast<_Tensor<T>&>(src);
         if (&s != this) {
-            construct(s.width, s.height, s.depth, s._store_type);
-            std::memcpy(Tens.ptr, s.Tens.ptr, total_bytes);
+            block_ = s.block_;
+            attribute_assign(s.width, s.height, s.depth, s._store_type);
+            Tens.ptr = s.Tens.ptr;
         }
         return *this;
     }
     void release() override {
-        block_.free();
+        block_.reset();
         Tens.ptr = nullptr;
     }
     ~_Tensor() override { release(); }
@@ -230,7 +274,7 @@ public:
 
 template <typename T>
 class _TensorArray : public de::TensorArray<T> {
-    HostBlock block_;
+    std::shared_ptr<HostBlock> block_;
 
 public:
     uint width = 0, height = 0, depth = 0, tensor_num = 0;
@@ -258,8 +302,9 @@ public:
     }
     bool construct(uint w, uint h, uint d, uint n, int store_type) {
         attribute_assign(w, h, d, n, store_type);
-        bool ok = block_.alloc(total_bytes, store_type);
-        TensArr.ptr = static_cast<T*>(block_.ptr);
+        block_ = std::make_shared<HostBlock>();
+        bool ok = block_->alloc(total_bytes, store_type);
+        TensArr.ptr = static_cast<T*>(block_->ptr);
         if (ok) std::memset(TensArr.ptr, 0, total_bytes);
         return ok;
     }
@@ -270,16 +315,17 @@ public:
     T& index(const int x, const int y, const int z, const int tensor_id) override {
         return TensArr.ptr[(size_t)tensor_id * _gap + (size_t)x * dp_x_wp + (size_t)y * dpitch + z];
     }
-    de::TensorArray<T>& operator=(de::TensorArray<T>& src) override {
+    de::TensorArray<T>& operator=(de::TensorArray<T>& src) override {   // shares src's block (TensorArray.h:529-554)
         _TensorArray<T>& s = dynamic_cast<_TensorArray<T>&>(src);
         if (&s != this) {
-            construct(s.width, s.height, s.depth, s.tensor_num, s._store_type);
-            std::memcpy(TensArr.ptr, s.TensArr.ptr, total_bytes);
+            block_ = s.block_;
+            attribute_assign(s.width, s.height, s.depth, s.tensor_num, s._store_type);
+            TensArr.ptr = s.TensArr.ptr;
         }
         return *this;
     }
     void release() override {
-        block_.free();
+        block_.reset();
         TensArr.ptr = nullptr;
     }
     ~_TensorArray() override { release(); }
@@ -288,7 +334,7 @@ public:
 // classes/MatrixArray.h:222-239 (attributes), :367-370 (index)
 template <typename T>
 class _MatrixArray : public de::MatrixArray<T> {
-    HostBlock block_;
+    std::shared_ptr<HostBlock> block_;
 
 public:
     int _store_type = Page_Default;
@@ -313,8 +359,9 @@ public:
     }
     bool construct(uint w, uint h, uint n, int flag) {
         attribute_assign(w, h, n, flag);
-        bool ok = block_.alloc(total_bytes, flag);
-        MatArr.ptr = static_cast<T*>(block_.ptr);
+        block_ = std::make_shared<HostBlock>();
+        bool ok = block_->alloc(total_bytes, flag);
+        MatArr.ptr = static_cast<T*>(block_->ptr);
         return ok;
     }
     bool re_construct(uint w, uint h, uint n, int flag) {
@@ -324,17 +371,19 @@ public:
     uint Width() override { return width; }
     uint Height() override { return height; }
     uint MatrixNumber() override { return (uint)ArrayNumber; }
+    bool shares_block_with(const _MatrixArray<T>& o) const { return block_ && block_ == o.block_; }
     T& index(uint row, uint col, size_t seq) override { return MatArr.ptr[seq * _plane + (size_t)row * pitch + col]; }
-    de::MatrixArray<T>& operator=(de::MatrixArray<T>& src) override {
+    de::MatrixArray<T>& operator=(de::MatrixArray<T>& src) override {   // shares src's block (MatrixArray.h:473-498)
         _MatrixArray<T>& s = dynamic_cast<_MatrixArray<T>&>(src);
         if (&s != this) {
-            construct(s.width, s.height, (uint)s.ArrayNumber, s._store_type);
-            std::memcpy(MatArr.ptr, s.MatArr.ptr, total_bytes);
+            block_ = s.block_;
+            attribute_assign(s.width, s.height, (uint)s.ArrayNumber, s._store_type);
+            MatArr.ptr = s.MatArr.ptr;
         }
         return *this;
     }
     void release() override {
-        block_.free();
+        block_.reset();
         MatArr.ptr = nullptr;
     }
     ~_MatrixArray() override { release(); }
@@ -342,6 +391,8 @@ public:
 
 template <typename T>
 class _GPU_Tensor : public de::GPU_Tensor<T> {
+    std::shared_ptr<DeviceBlock> block_;
+
 public:
     uint width = 0, height = 0, depth = 0;
     uint dpitch = 0, wpitch = 0;
@@ -366,11 +417,9 @@ public:
     bool construct(uint w, uint h, uint d) {
         release();
         attribute_assign(w, h, d);
-        void* p = nullptr;
-        last_status = decx_hip_malloc(&p, total_bytes);
-        if (last_status != 0) return false;
-        Tens.ptr = static_cast<T*>(p);
-        last_status = decx_hip_memset(p, 0, total_bytes);
+        block_ = std::make_shared<DeviceBlock>();
+        last_status = block_->alloc(total_bytes);
+        Tens.ptr = static_cast<T*>(block_->ptr);
         return last_status == 0;
     }
     bool re_construct(uint w, uint h, uint d) {
@@ -380,10 +429,13 @@ public:
     uint Width() override { return width; }
     uint Height() override { return height; }
     uint Depth() override { return depth; }
-    de::GPU_Tensor<T>& operator=(de::GPU_Tensor<T>& src) override {
+    de::GPU_Tensor<T>& operator=(de::GPU_Tensor<T>& src) override {   // shares src's block (GPU_Tensor.h)
         _GPU_Tensor<T>& s = dynamic_cast<_GPU_Tensor<T>&>(src);
-        if (&s != this && construct(s.width, s.height, s.depth))
-            last_status = decx_hip_memcpy(Tens.ptr, s.Tens.ptr, total_bytes, DECX_HIP_D2D);
+        if (&s != this) {
+            block_ = s.block_;
+            attribute_assign(s.width, s.height, s.depth);
+            Tens.ptr = s.Tens.ptr;
+        }
         return *this;
     }
     void Load_from_host(de::Tensor<T>& src) override {
@@ -397,7 +449,7 @@ public:
         last_status = decx_hip_memcpy(d.Tens.ptr, Tens.ptr, total_bytes, DECX_HIP_D2H);
     }
     void release() override {
-        if (Tens.ptr) decx_hip_free(Tens.ptr);
+        block_.reset();
         Tens.ptr = nullptr;
     }
     ~_GPU_Tensor() override { release(); }
@@ -405,6 +457,8 @@ public:
 
 template <typename T>
 class _GPU_TensorArray : public de::GPU_TensorArray<T> {
+    std::shared_ptr<DeviceBlock> block_;
+
 public:
     uint width = 0, height = 0, depth = 0, tensor_num = 0;
     uint dpitch = 0, wpitch = 0;
@@ -431,11 +485,9 @@ public:
     bool construct(uint w, uint h, uint d, uint n) {
         release();
         attribute_assign(w, h, d, n);
-        void* p = nullptr;
-        last_status = decx_hip_malloc(&p, total_bytes);
-        if (last_status != 0) return false;
-        TensArr.ptr = static_cast<T*>(p);
-        last_status = decx_hip_memset(p, 0, total_bytes);
+        block_ = std::make_shared<DeviceBlock>();
+        last_status = block_->alloc(total_bytes);
+        TensArr.ptr = static_cast<T*>(block_->ptr);
         return last_status == 0;
     }
     uint Width() override { return width; }
@@ -452,14 +504,17 @@ public:
         if (d.width != width || d.height != height || d.depth != depth || d.tensor_num != tensor_num) { last_status = DECX_HIP_FAIL_DIMS; return; }
         last_status = decx_hip_memcpy(d.TensArr.ptr, TensArr.ptr, total_bytes, DECX_HIP_D2H);
     }
-    de::GPU_TensorArray<T>& operator=(de::GPU_TensorArray<T>& src) override {
+    de::GPU_TensorArray<T>& operator=(de::GPU_TensorArray<T>& src) override {   // shares src's block
         _GPU_TensorArray<T>& s = dynamic_cast<_GPU_TensorArray<T>&>(src);
-        if (&s != this && construct(s.width, s.height, s.depth, s.tensor_num))
-            last_status = decx_hip_memcpy(TensArr.ptr, s.TensArr.ptr, total_bytes, DECX_HIP_D2D);
+        if (&s != this) {
+            block_ = s.block_;
+            attribute_assign(s.width, s.height, s.depth, s.tensor_num);
+            TensArr.ptr = s.TensArr.ptr;
+        }
         return *this;
     }
     void release() override {
-        if (TensArr.ptr) decx_hip_free(TensArr.ptr);
+        block_.reset();
         TensArr.ptr = nullptr;
     }
     ~_GPU_TensorArray() override { release(); }

@@ -63,11 +63,12 @@ static std::vector<float> chain(de::Matrix<float>& A, de::Matrix<float>& B, de::
 // ------------------------------------------------------------------ CPU-only checks ----------------------------
 static void containers_follow_reference_pitch_rules() {
     de::Matrix<float>& m = de::CreateMatrixRef<float>(13, 7, decx::Page_Default);
-    CHECK(m.Width() == 13 && m.Height() == 7 && m.TotalBytes() == 16u * 7 * 4);     // pitch = ceil8(13) = 16
+    CHECK(m.Width() == 13 && m.Height() == 7 && m.TotalBytes() == 13u * 7 * 4);     // width*height*sizeof (Matrix.h:262-263), not the pitched size
     m.index(6, 12) = 3.5f;
     CHECK((&m.index(6, 12)) - (&m.index(0, 0)) == 6 * 16 + 12);
     de::Matrix<de::Half>& h = de::CreateMatrixRef<de::Half>(17, 3, decx::Page_Default);
-    CHECK(h.TotalBytes() == 32u * 3 * 2);                                             // pitch = ceil16(17) = 32
+    CHECK(h.TotalBytes() == 17u * 3 * 2);                                             // Matrix.h:317-318
+    CHECK((&h.index(1, 0)) - (&h.index(0, 0)) == 32);                                 // pitch = ceil16(17) = 32
     de::Tensor<float>& t = de::CreateTensorRef<float>(5, 6, 3, decx::Page_Default);  // width 5, height 6, depth 3
     CHECK(t.Width() == 5 && t.Height() == 6 && t.Depth() == 3);
     CHECK((&t.index(1, 0, 0)) - (&t.index(0, 0, 0)) == 8 * 4);                        // wpitch 8, dpitch 4
@@ -79,6 +80,49 @@ static void containers_follow_reference_pitch_rules() {
     CHECK(ta.TensorNum() == 5 && (&ta.index(0, 0, 0, 1)) - (&ta.index(0, 0, 0, 0)) == 3 * 4 * 64);   // _gap
     CHECK((&ta.index(1, 2, 7, 0)) - (&ta.index(0, 0, 0, 0)) == 1 * 4 * 64 + 2 * 64 + 7);
     m.release(); h.release(); t.release(); ta.release();
+}
+
+static void assignment_shares_the_payload() {   // Matrix.h:510-530, Tensor.h:501-526: the block is shared and counted
+    de::Matrix<float>& a = de::CreateMatrixRef<float>(13, 7, decx::Page_Default);
+    de::Matrix<float>& b = de::CreateMatrixRef<float>();
+    fill(a, small_int);
+    b = a;
+    CHECK(b.Width() == 13 && b.Height() == 7 && b.TotalBytes() == a.TotalBytes());
+    CHECK(&b.index(3, 5) == &a.index(3, 5));                       // same memory, not a copy
+    a.index(3, 5) = 42.f;
+    CHECK(b.index(3, 5) == 42.f);
+    a.release();                                                    // the other holder keeps the block alive
+    CHECK(b.index(3, 5) == 42.f);
+    b.index(6, 12) = 1.f;
+    b.release();
+    de::Tensor<float>& t = de::CreateTensorRef<float>(5, 6, 3, decx::Page_Default);
+    de::Tensor<float>& u = de::CreateTensorRef<float>();
+    u = t;
+    CHECK(&u.index(2, 1, 1) == &t.index(2, 1, 1) && u.Depth() == 3);
+    t.release();
+    u.index(5, 4, 2) = 2.f;
+    u.release();
+    de::MatrixArray<float>& ma = de::CreateMatrixArrayRef<float>(9, 4, 3, decx::Page_Default);
+    de::MatrixArray<float>& mb = de::CreateMatrixArrayRef<float>();
+    mb = ma;
+    CHECK(&mb.index(3, 8, 2) == &ma.index(3, 8, 2) && mb.MatrixNumber() == 3);
+    ma.release(); mb.release();
+}
+
+static void cpu_sgemm_into_an_operand() {        // dst is A (square): computed aside, then dst takes the new payload
+    const int S = 40;
+    de::Matrix<float>& A = de::CreateMatrixRef<float>(S, S, decx::Page_Default);
+    de::Matrix<float>& B = de::CreateMatrixRef<float>(S, S, decx::Page_Default);
+    de::Matrix<float>& A2 = de::CreateMatrixRef<float>();
+    fill(A, unif); fill(B, unif);
+    std::vector<float> want = chain(A, B);
+    A2 = A;                                                          // a second holder of A's payload
+    std::vector<float> a_before = dense(A);
+    CHECK(de::cpu::sgemm(A, B, A).error_type == decx::DECX_SUCCESS);
+    std::vector<float> got = dense(A);
+    CHECK(std::memcmp(got.data(), want.data(), got.size() * 4) == 0);
+    CHECK(dense(A2) == a_before);                                    // the old payload is untouched
+    A.release(); B.release(); A2.release();
 }
 
 static void half_conversion() {
@@ -188,11 +232,40 @@ static void gemm_fp32_all_flavours() {
     std::vector<float> want = chain(A, B, &C);
     CHECK(de::cuda::GEMM(A, B, C, C).error_type == 0);                     // dst aliasing C
     CHECK(dense(C) == want);
+    {   // a pageable C used in place keeps its data (re-constructing it as pinned would drop C before the upload)
+        de::Matrix<float>& Cp = de::CreateMatrixRef<float>(N, M, decx::Page_Default);
+        fill(Cp, small_int);
+        std::vector<float> want_p = chain(A, B, &Cp);
+        CHECK(de::cuda::GEMM(A, B, Cp, Cp).error_type == 0);
+        CHECK(dense(Cp) == want_p);
+        Cp.release();
+        // dst is A itself (square): computed aside, dst then holds the product
+        de::Matrix<float>& S1 = de::CreateMatrixRef<float>(96, 96, decx::Page_Default);
+        de::Matrix<float>& S2 = de::CreateMatrixRef<float>(96, 96, decx::Page_Locked);
+        fill(S1, small_int); fill(S2, small_int);
+        std::vector<float> want_s = chain(S1, S2);
+        CHECK(de::cuda::GEMM(S1, S2, S1).error_type == 0);
+        CHECK(dense(S1) == want_s);
+        std::vector<float> want_t = chain(S1, S2);
+        CHECK(de::cuda::GEMM(S1, S2, S2).error_type == 0);
+        CHECK(dense(S2) == want_t);
+        S1.release(); S2.release();
+    }
     // device-resident flavours
     de::GPU_Matrix<float>& dA = de::CreateGPUMatrixRef<float>(K, M);
     de::GPU_Matrix<float>& dB = de::CreateGPUMatrixRef<float>(N, K);
     de::GPU_Matrix<float>& dC = de::CreateGPUMatrixRef<float>(N, M);
     de::GPU_Matrix<float>& dD = de::CreateGPUMatrixRef<float>();          // empty: GEMM sizes it (GEMM.h:414)
+    CHECK(dA.TotalBytes() == (size_t)K * M * 4 && dB.TotalBytes() == (size_t)N * K * 4);   // width*height*sizeof (GPU_Matrix.h:218-219)
+    {
+        de::GPU_Matrix<de::Half>& dh = de::CreateGPUMatrixRef<de::Half>(17, 3);
+        CHECK(dh.TotalBytes() == 17u * 3 * 2);                             // GPU_Matrix.h:266-267
+        de::GPU_Matrix<de::Half>& dh2 = de::CreateGPUMatrixRef<de::Half>();
+        dh2 = dh;                                                          // shares the device block (GPU_Matrix.h:441-451)
+        dh.release();
+        CHECK(dh2.Width() == 17 && dh2.TotalBytes() == 17u * 3 * 2);
+        dh2.release();
+    }
     fill(A, unif); fill(B, unif); fill(C, unif);
     dA.Load_from_host(A); dB.Load_from_host(B); dC.Load_from_host(C);
     CHECK(de::cuda::GEMM(dA, dB, dD).error_type == 0 && dD.Width() == (uint)N && dD.Height() == (uint)M);
@@ -467,6 +540,8 @@ int main(int argc, char** argv) {
     std::string mode = argc > 1 ? argv[1] : "cpu";
     if (mode == "cpu") {
         RUN(containers_follow_reference_pitch_rules);
+        RUN(assignment_shares_the_payload);
+        RUN(cpu_sgemm_into_an_operand);
         RUN(half_conversion);
         RUN(gemm_refuses_before_init);
         RUN(cpu_sgemm_matches_chain_bit_for_bit);
