@@ -619,4 +619,15 @@ int decx_hip_set_hgemm_variant(int variant) {
     return prev;
 }
 
+int decx_hip_b_read_extent(int N, int tile_n, int unit) {
+    if (N <= 0 || tile_n <= 0 || unit <= 0 || tile_n % unit) return -1;
+    int last = -1;
+    for (int bn0 = 0; bn0 < N; bn0 += tile_n)                    // every tile column of the launch
+        for (int g = 0; g < tile_n; g += unit) {                 // every column group a tile stages
+            const int col = clamp_group_col(bn0 + g, N, unit) + unit - 1;
+            if (col > last) last = col;
+        }
+    return last;
+}
+
 }  // extern "C"

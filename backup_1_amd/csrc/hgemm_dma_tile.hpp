@@ -108,7 +108,7 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
         const int kr = chunk * (64 / UB) + lane / UB;
         const int u = (lane % UB) ^ ((kr & 3) << 2);
         int col = bn0 + 8 * u;
-        if (col > ldb - 8) col = ldb - 8;                      // stay inside the pitch; such columns are never stored
+        col = clamp_group_col(col, N, 8);                      // stay inside the operand; such columns are never stored
         b_off[j] = (uint32_t)(((size_t)kr * ldb + col) * sizeof(_Float16));
     }
     const size_t b_step = (size_t)BK * ldb;
@@ -298,7 +298,7 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
             u32x4 v = {0u, 0u, 0u, 0u};
             if (k0 + kr < K) {
                 int col = bn0 + 8 * u;
-                if (col > ldb - 8) col = ldb - 8;
+                col = clamp_group_col(col, N, 8);
                 v = *reinterpret_cast<const u32x4*>(B + (size_t)(k0 + kr) * ldb + col);
             }
             b_stage[p] = v;

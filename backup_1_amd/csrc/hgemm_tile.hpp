@@ -107,7 +107,7 @@ __global__ __launch_bounds__(S::NT) void hgemm_tile_kernel(const _Float16* __res
             if (!tail || k < K) {
                 const int col = bn0 + 8 * u;
                 if (VEC) {
-                    const int cc = col <= ldb - 8 ? col : ldb - 8;    // stay inside the pitch; such columns are never stored
+                    const int cc = clamp_group_col(col, N, 8);    // stay inside the operand; such columns are never stored
                     v = *reinterpret_cast<const u32x4*>(B + (size_t)k * ldb + cc);
                 } else {
                     v = load_unit(B + (size_t)k * ldb, col, N, true);

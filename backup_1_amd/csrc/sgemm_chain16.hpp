@@ -177,7 +177,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_chain16_kernel
             const int q = pt + p * S::MOVE_THREADS, rest = q / 32;
             const int k = 16 * (rest % 4) + q % 16, cq = 2 * (rest / 4) + (q / 16) % 2;
             int col = bn0 + 4 * cq;
-            if (col > ldb - 4) col = ldb - 4;     // stay inside the pitch; such columns are never stored
+            col = clamp_group_col(col, N, 4);     // stay inside the operand; such columns are never stored
             quad_k[PA + p] = k;
             src[PA + p] = B + (size_t)k * ldb + col;
             dst[PA + p] = lds_byte_address(Bs) + 4u * (unsigned)((k % 4) * S::B_PLANE + (4 * cq) * S::LINE + k / 4);   // element e: line 4cq + e

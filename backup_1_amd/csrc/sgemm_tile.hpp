@@ -365,7 +365,7 @@ struct DenseB {
             f32x4 v = {0.f, 0.f, 0.f, 0.f};
             if (!TAIL || k < K) {
                 if (VEC) {
-                    const int cc = col <= ldb - 4 ? col : ldb - 4;   // stay inside the pitch; such columns are never stored
+                    const int cc = clamp_group_col(col, N, 4);   // stay inside the operand; such columns are never stored
                     v = *reinterpret_cast<const f32x4*>(B + (size_t)k * ldb + cc);
                 } else {
 #pragma unroll

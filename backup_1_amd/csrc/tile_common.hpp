@@ -23,6 +23,17 @@ __device__ __forceinline__ float relu_by_sign(float v) {
     return (float)((~__float_as_uint(v)) >> 31) * v;
 }
 
+// Where a loader fetches the `unit`-wide column group that starts at column `col` (a multiple of `unit`) of a
+// row-major B with N valid columns: groups that start at or beyond N rounded up to `unit` are moved back onto the last
+// group that holds a valid column.  Such columns are computed and never stored.  The bound is the extent of the
+// operand the caller described, not its pitch: B may be a column range of a wider matrix (pointer moved right, parent
+// pitch), and then B + ldb of the last row lies beyond the parent's allocation.  With B 16-byte aligned and ldb a
+// multiple of `unit`, N rounded up to `unit` never exceeds the parent's pitch.
+__host__ __device__ __forceinline__ constexpr int clamp_group_col(int col, int N, int unit) {
+    const int last = (N + unit - 1) / unit * unit - unit;
+    return col < last ? col : last;
+}
+
 struct TileCoord {
     int tm, tn;
 };

@@ -237,6 +237,14 @@ const char* decx_hip_last_error(void);
 int decx_hip_set_sgemm_variant(int variant);
 int decx_hip_set_hgemm_variant(int variant);
 
+/* Host-only arithmetic check (no device call, no counterpart in the reference): the largest column index, relative to
+ * the B pointer passed to a GEMM entry point, that the vector loaders of a kernel with tile_n-wide tiles fetch when B
+ * has N valid columns and is read in groups of `unit` columns (4 for fp32, 8 for fp16) -- computed with the very
+ * function the kernels use to place those fetches.  It is N rounded up to `unit`, minus 1, whatever the tile width:
+ * B may therefore be a column range of a wider matrix (B = parent + c0, ldb = the parent's pitch, c0 a multiple of
+ * `unit`) without any row being read beyond the parent's pitch.  Returns -1 on bad arguments. */
+int decx_hip_b_read_extent(int N, int tile_n, int unit);
+
 #ifdef __cplusplus
 }
 #endif

@@ -58,3 +58,28 @@ def test_bench_refuses_more_than_one_gpu():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU" in r.stderr
+
+
+# widths of the tiles the GEMM kernels are built with (sgemm_launch.hpp, sgemm_chain16.hpp, hgemm.hip) and the width
+# of their vector fetches: 4 floats, 8 halves
+B_TILE_WIDTHS = {4: (16, 32, 64, 128, 192, 256), 8: (64, 128, 256)}
+
+
+@pytest.mark.parametrize("unit", (4, 8))
+def test_b_loaders_stay_inside_a_column_range_of_a_wider_matrix(unit):
+    """B may be columns [c0, c0 + N) of a parent matrix (pointer moved right, parent pitch): the last row of that view
+    ends with the parent's allocation, so no fetch may go beyond column roundup(N, unit) - 1 of the view, whatever the
+    tile width.  A bound taken from the pitch instead (fetch up to ldb - unit) would leave the parent's last row by up
+    to c0 columns."""
+    L = capi.lib()
+    for tile_n in B_TILE_WIDTHS[unit]:
+        for N in list(range(1, 3 * tile_n + 2)) + [952, 3000, 4500, 8191, 8192]:
+            extent = L.decx_hip_b_read_extent(N, tile_n, unit)
+            assert extent == (N + unit - 1) // unit * unit - 1, (N, tile_n, unit, extent)
+    # the case that showed the defect: K = 1024 rows of a parent with pitch 3000 = exactly 3000 pages of 4 KiB, last
+    # column panel c0 = 2048 with 952 columns, 64-wide tiles: the fetch must end inside the parent's last row
+    K, ldb_parent, c0, cols = 1024, 3000, 2048, 952
+    extent = L.decx_hip_b_read_extent(cols, 64, 4)
+    last_element = (K - 1) * ldb_parent + c0 + extent
+    assert last_element < K * ldb_parent
+    assert L.decx_hip_b_read_extent(0, 64, 4) == -1 and L.decx_hip_b_read_extent(8, 60, 8) == -1
