@@ -619,6 +619,12 @@ int decx_hip_set_hgemm_variant(int variant) {
     return prev;
 }
 
+int decx_hip_set_splitk_mode(int mode) {
+    int prev = g_rt.splitk_atomic;
+    g_rt.splitk_atomic = mode ? 1 : 0;
+    return prev;
+}
+
 int decx_hip_b_read_extent(int N, int tile_n, int unit) {
     if (N <= 0 || tile_n <= 0 || unit <= 0 || tile_n % unit) return -1;
     int last = -1;

@@ -80,7 +80,8 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
     if (splits > 1) {
         const int steps_per_split = cdiv(all_steps, splits);
         splits = cdiv(all_steps, steps_per_split);                     // no empty range
-        if (int rc = ensure_partial((size_t)M * N * sizeof(float))) return rc;
+        const bool ordered = !g_rt.splitk_atomic;             // one workspace plane per range, added in range order
+        if (int rc = ensure_partial((size_t)M * N * sizeof(float) * (ordered ? splits : 1))) return rc;
         static bool split_attr_done = false;
         if (!split_attr_done) {
             HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hconv_tile_kernel<HconvSquare, true, true>),
@@ -91,15 +92,17 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
         }
         const size_t count = (size_t)M * N;
         const unsigned fill_blocks = (unsigned)((count + 255) / 256 < 4096 ? (count + 255) / 256 : 4096);
-        enqueue_zero_region(g_rt.partial, N, M, N, g_rt.stream);
+        if (!ordered) enqueue_zero_region(g_rt.partial, N, M, N, g_rt.stream);
+        const size_t plane = ordered ? count : (size_t)0;
         const dim3 grid((unsigned)total, (unsigned)splits);
         if (tap_uniform)
             hipLaunchKernelGGL((hconv_tile_kernel<HconvSquare, true, true>), grid, dim3(HconvSquare::NT), HconvSquare::LDS_BYTES,
-                               g_rt.stream, img, fb, out, M, N, Kw, tiles_n, g_rt.partial, steps_per_split);
+                               g_rt.stream, img, fb, out, M, N, Kw, tiles_n, g_rt.partial, steps_per_split, plane);
         else
             hipLaunchKernelGGL((hconv_tile_kernel<HconvSquare, false, true>), grid, dim3(HconvSquare::NT), HconvSquare::LDS_BYTES,
-                               g_rt.stream, img, fb, out, M, N, Kw, tiles_n, g_rt.partial, steps_per_split);
-        hipLaunchKernelGGL(hconv_split_finish_kernel, dim3(fill_blocks), dim3(256), 0, g_rt.stream, g_rt.partial, out, M, N);
+                               g_rt.stream, img, fb, out, M, N, Kw, tiles_n, g_rt.partial, steps_per_split, plane);
+        hipLaunchKernelGGL(hconv_split_finish_kernel, dim3(fill_blocks), dim3(256), 0, g_rt.stream, g_rt.partial, ordered ? splits : 1, count,
+                           out, M, N);
         HIP_TRY(hipGetLastError());
         return 0;
     }
@@ -154,7 +157,7 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
             }
             const long tiles = cdiv(M, S::BM);
             hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, out, M, N, Kw, 1,
-                               static_cast<float*>(nullptr), 0);
+                               static_cast<float*>(nullptr), 0, (size_t)0);
             HIP_TRY(hipGetLastError());
             return 0;
         };
@@ -180,7 +183,7 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
     auto launch = [&](auto kern, auto shape) {
         typedef decltype(shape) S;
         hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, out, M, N, Kw, tiles_n,
-                           static_cast<float*>(nullptr), 0);
+                           static_cast<float*>(nullptr), 0, (size_t)0);
     };
     if (tall && tap_uniform) launch(hconv_tile_kernel<HconvTall, true>, HconvTall{});
     else if (tall) launch(hconv_tile_kernel<HconvTall, false>, HconvTall{});

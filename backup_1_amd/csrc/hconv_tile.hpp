@@ -150,12 +150,13 @@ __device__ __forceinline__ void hconv_store_tile(const f32x16 (&acc)[S::MI][S::N
 // (tap row, tap column, channel) is the same for every lane up to a constant and runs on the scalar unit; a load then
 // costs the vector unit one add (plus the column check of an image load), and a filter load nothing at all.
 // SPLIT_K (small images: few tiles, many K steps): blockIdx.y selects a range of steps_per_split K steps; the tile's fp32
-// partial sums are added with atomics to a dense M x N fp32 workspace `partial` (zeroed beforehand), and
-// hconv_split_finish_kernel applies bias and ReLU and writes the binary16 tensor.
+// partial sums go to a workspace of dense M x N fp32 planes: range y stores into plane y (partial_plane floats apart;
+// nothing to zero), or, with partial_plane == 0, all ranges add into one zeroed plane with atomics.
+// hconv_split_finish_kernel adds the planes in range order, applies bias and ReLU and writes the binary16 tensor.
 template <class S, bool TAP_UNIFORM, bool SPLIT_K = false>
 __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, HalfFilters fb, HalfTensorOut out, int M, int N,
                                                            int Kw /* K in words */, int tiles_n, float* partial,
-                                                           int steps_per_split) {
+                                                           int steps_per_split, size_t partial_plane) {
     constexpr int BM = S::BM, BN = S::BN, NT = S::NT, U = S::U, MI = S::MI, NI = S::NI;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     constexpr int A_BYTES = S::A_UNITS * 16, B_BYTES = S::B_UNITS * 16;     // one buffer of either operand
@@ -320,6 +321,8 @@ __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, Hal
         });
 
     if (SPLIT_K) {
+        const bool ordered = partial_plane != 0;                 // uniform over the launch
+        float* plane = partial + (size_t)blockIdx.y * partial_plane;
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
@@ -329,7 +332,10 @@ __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, Hal
 #pragma unroll
                     for (int ni = 0; ni < NI; ++ni) {
                         const int n = bn0 + wn0 + ni * 32 + li;
-                        if (n < N) unsafeAtomicAdd(partial + (size_t)m * N + n, acc[mi][ni][r]);
+                        if (n < N) {
+                            if (ordered) plane[(size_t)m * N + n] = acc[mi][ni][r];
+                            else unsafeAtomicAdd(plane + (size_t)m * N + n, acc[mi][ni][r]);
+                        }
                     }
                 }
             }
@@ -339,12 +345,15 @@ __global__ __launch_bounds__(S::NT, 2) void hconv_tile_kernel(HalfImage img, Hal
     hconv_store_tile<S>(acc, lds_raw, out, M, N, bm0, bn0, wm0, wn0, tid, pixel_of);
 }
 
-// dst(pixel m, filter n) = half(relu(partial[m][n] + bias[n])): the end of a split-K convolution.
-static __global__ __launch_bounds__(256) void hconv_split_finish_kernel(const float* __restrict__ partial, HalfTensorOut out, int M, int N) {
+// dst(pixel m, filter n) = half(relu(plane 0 + plane 1 + ... + bias[n])), added in that order: the end of a split-K
+// convolution.  partial holds `planes` dense M x N fp32 planes, `plane` floats apart.
+static __global__ __launch_bounds__(256) void hconv_split_finish_kernel(const float* __restrict__ partial, int planes, size_t plane,
+                                                                 HalfTensorOut out, int M, int N) {
     const size_t total = (size_t)M * N;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const int m = (int)(i / N), n = (int)(i - (size_t)m * N);
         float v = partial[i];
+        for (int s = 1; s < planes; ++s) v += partial[(size_t)s * plane + i];
         if (out.bias != nullptr) v += (float)out.bias[n];
         if (out.relu) v = relu_by_sign(v);
         out.dst[(size_t)(m / out.Wout) * out.row_stride + (size_t)(m % out.Wout) * out.dpitch + n] = (_Float16)v;

@@ -76,66 +76,106 @@ int launch_hgemm_dma_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb
                        reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
                        reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N, K,
                        tiles_m, tiles_n, group_m, batch.stride_a, batch.stride_b, batch.stride_c, batch.stride_d,
-                       static_cast<float*>(nullptr), 0);
+                       static_cast<float*>(nullptr), 0, (size_t)0);
     HIP_TRY(hipGetLastError());
     return 0;
 }
 
 // fp16 GEMM whose result has too few tiles to fill the chip while K is long: K is cut into ranges that run as separate
-// workgroups (blockIdx.z) and add their fp32 partial sums to a workspace with atomics; a second kernel adds C and
-// rounds to binary16 once.  fp32 sums in no fixed order: the result can differ in its last bit from run to run, inside
-// the 2e-3 rule of the fp16 path.  (fp32 GEMM never does this: its results are bit-exact chains.)
-int hgemm_splitk_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
-                         int ldd, int M, int N, int K, int splits, hipStream_t stream) {
+// workgroups (blockIdx.z).  Each range stores its fp32 partial sums into a plane of its own in a workspace, and a second
+// kernel adds the planes in range order, adds C and rounds to binary16 once: the same bits on every run.  In the atomic
+// mode (decx_hip_set_splitk_mode(1)) all ranges add into one zeroed plane in whatever order they arrive, so the last
+// bit can differ between runs.  (fp32 GEMM never splits K by itself: its results are bit-exact chains.)
+struct SplitPlan {
+    int splits, k_split_len;
+};
+static SplitPlan plan_hgemm_split(int K, int splits) {
+    typedef HShapeDmaSmall S;
+    const int k_split_len = cdiv(cdiv(K, splits), S::BK) * S::BK;
+    return SplitPlan{cdiv(K, k_split_len), k_split_len};                 // no empty range
+}
+
+// the automatic number of K ranges for an M x N x K product (0: do not split) -- the choice of hgemm_enqueue.
+// Measured, in us: a tile walks K at 6.7 ns per k (1.6 times that when two workgroups share a CU); a launch costs about
+// 4, the finishing kernel and its launch 5.5, a partial sum stored and read back (or an atomic add) about 3 ps.
+static int auto_hgemm_splits(int M, int N, int K) {
+    const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+    const long tiles = (long)cdiv(M, 128) * cdiv(N, 128);
+    long splits = (2 * cus + tiles - 1) / tiles;
+    if (splits > K / 512) splits = K / 512;                        // at least 8 K steps per range
+    if (splits < 2 || (size_t)M * N > ((size_t)1 << 26)) return 0;
+    const double t_whole = 4.0 + 0.0067 * K * (double)((tiles + cus - 1) / cus);
+    const double share = tiles * splits > cus ? 1.6 : 1.0;
+    const double t_split = (g_rt.splitk_atomic ? 9.0 : 5.5) + 3.1e-6 * M * N * splits +
+                           0.0067 * ((double)K / splits) * share * (double)((tiles * splits + 2 * cus - 1) / (2 * cus));
+    return t_split < 0.85 * t_whole ? (int)splits : 0;
+}
+
+static int hgemm_splitk_launch(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
+                               int ldd, int M, int N, int K, const SplitPlan& plan, float* workspace, bool ordered,
+                               hipStream_t stream) {
     typedef HShapeDmaSmall S;                      // 128x128x64, LDS-DMA staged, two workgroups per CU
-    if (int rc = ensure_partial((size_t)M * N * sizeof(float))) return rc;
     auto kern = hgemm_dma_kernel<S, false, true>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
-        attr_done = true;
-    }
     const size_t total = (size_t)M * N;
     const unsigned fill_blocks = (unsigned)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
-    enqueue_zero_region(g_rt.partial, N, M, N, stream);
-    const int k_split_len = cdiv(cdiv(K, splits), S::BK) * S::BK;
-    splits = cdiv(K, k_split_len);                                                        // no empty range
+    if (!ordered) enqueue_zero_region(workspace, N, M, N, stream);
     const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
     const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)splits), dim3(S::NT), S::LDS_BYTES, stream,
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n), 1, (unsigned)plan.splits), dim3(S::NT), S::LDS_BYTES, stream,
                        reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
                        static_cast<const _Float16*>(nullptr), 0, reinterpret_cast<_Float16*>(D), ldd, M, N, K, tiles_m, tiles_n,
-                       group_m, (size_t)0, (size_t)0, (size_t)0, (size_t)0, g_rt.partial, k_split_len);
-    hipLaunchKernelGGL(hgemm_split_finish_kernel, dim3(fill_blocks), dim3(256), 0, stream, g_rt.partial,
-                       reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N);
+                       group_m, (size_t)0, (size_t)0, (size_t)0, (size_t)0, workspace, plan.k_split_len, ordered ? total : (size_t)0);
+    hipLaunchKernelGGL(hgemm_split_finish_kernel, dim3(fill_blocks), dim3(256), 0, stream, workspace, ordered ? plan.splits : 1,
+                       total, reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N);
     HIP_TRY(hipGetLastError());
     return 0;
+}
+
+static int allow_split_kernel_lds() {
+    typedef HShapeDmaSmall S;
+    static bool attr_done = false;
+    if (!attr_done) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hgemm_dma_kernel<S, false, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+        attr_done = true;
+    }
+    return 0;
+}
+
+int hgemm_splitk_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
+                         int ldd, int M, int N, int K, int splits, hipStream_t stream) {
+    const SplitPlan plan = plan_hgemm_split(K, splits);
+    const bool ordered = !g_rt.splitk_atomic;
+    if (int rc = ensure_partial((size_t)M * N * sizeof(float) * (ordered ? plan.splits : 1))) return rc;
+    if (int rc = allow_split_kernel_lds()) return rc;
+    return hgemm_splitk_launch(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, plan, g_rt.partial, ordered, stream);
+}
+
+static bool hgemm_vector_path(const uint16_t* A, int lda, const uint16_t* B, int ldb, const Batch& batch) {
+    // the LDS-DMA tiles address a tile's rows with 32-bit byte offsets from the tile's first row: 256 rows of A, 64 of B
+    const bool narrow = (size_t)lda * 256 * sizeof(uint16_t) < ((size_t)1 << 32) && (size_t)ldb * 64 * sizeof(uint16_t) < ((size_t)1 << 32);
+    return aligned16(A) && aligned16(B) && lda % 8 == 0 && ldb % 8 == 0 && ldb >= 8 && batch.stride_a % 8 == 0 &&
+           batch.stride_b % 8 == 0 && narrow;
 }
 
 int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                   int ldd, int M, int N, int K, const Batch& batch) {
     if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
-    // the LDS-DMA tiles address a tile's rows with 32-bit byte offsets from the tile's first row: 256 rows of A, 64 of B
-    const bool narrow = (size_t)lda * 256 * sizeof(uint16_t) < ((size_t)1 << 32) && (size_t)ldb * 64 * sizeof(uint16_t) < ((size_t)1 << 32);
-    const bool vec = aligned16(A) && aligned16(B) && lda % 8 == 0 && ldb % 8 == 0 && ldb >= 8 && batch.stride_a % 8 == 0 &&
-                     batch.stride_b % 8 == 0 && narrow;
+    const bool vec = hgemm_vector_path(A, lda, B, ldb, batch);
     if (!vec) return launch_hgemm_tile<HShapeSmall, false>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     int variant = g_rt.hgemm_variant;
     {
-        // few 128x128 tiles and a long K: split K (variant 11 forces it, any other fixed variant switches it off).
-        // Measured, in us: a tile walks K at 6.7 ns per k (1.6 times that when two workgroups share a CU); a launch costs
-        // about 4, the zero fill and the finishing kernel 9 together, an atomic add to the workspace 3.1 ps.
-        const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
-        const long tiles = (long)cdiv(M, 128) * cdiv(N, 128);
-        long splits = (2 * cus + tiles - 1) / tiles;
-        if (splits > K / 512) splits = K / 512;                        // at least 8 K steps per range
-        if (splits >= 2 && batch.count == 1 && (size_t)M * N <= ((size_t)1 << 26)) {
-            const double t_whole = 4.0 + 0.0067 * K * (double)((tiles + cus - 1) / cus);
-            const double share = tiles * splits > cus ? 1.6 : 1.0;
-            const double t_split = 9.0 + 3.1e-6 * M * N * splits +
-                                   0.0067 * ((double)K / splits) * share * (double)((tiles * splits + 2 * cus - 1) / (2 * cus));
-            if (variant == 11 || ((variant < 1 || variant > 11) && t_split < 0.85 * t_whole))
-                return hgemm_splitk_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, (int)splits, batch.stream);
+        // few 128x128 tiles and a long K: split K (variant 11 forces it, any other fixed variant switches it off)
+        if (batch.count == 1 && (variant < 1 || variant > 10)) {
+            int splits = auto_hgemm_splits(M, N, K);
+            if (variant == 11 && splits == 0 && K >= 1024 && (size_t)M * N <= ((size_t)1 << 26)) {
+                const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+                const long tiles = (long)cdiv(M, 128) * cdiv(N, 128);
+                long s = (2 * cus + tiles - 1) / tiles;
+                if (s > K / 512) s = K / 512;
+                splits = s >= 2 ? (int)s : 0;
+            }
+            if (splits >= 2) return hgemm_splitk_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, splits, batch.stream);
         }
         if (variant == 11) variant = 0;
     }

@@ -50,15 +50,19 @@ __device__ __forceinline__ void wait_dma_then_barrier() {
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" : : "n"(N) : "memory");
 }
 
-// SPLIT_K: blockIdx.z selects a range of K (k_split_len long, a multiple of BK); the tile's fp32 partial sums are added
-// with atomics to a dense M x N fp32 workspace `partial` (zeroed beforehand) instead of being rounded and stored.
+// SPLIT_K: blockIdx.z selects a range of K (k_split_len long, a multiple of BK); the tile's fp32 partial sums go to a
+// workspace of dense M x N fp32 planes instead of being rounded and stored.  partial_plane != 0: range z stores its
+// sums into plane z (partial + z * partial_plane) with plain stores -- every element of a plane inside the result is
+// written by exactly one workgroup, so nothing has to be zeroed, and the finishing kernel adds the planes in range
+// order: a result that is the same on every run.  partial_plane == 0: all ranges add into one plane (zeroed
+// beforehand) with atomics, in whatever order they arrive.
 template <class S, bool HAS_C, bool SPLIT_K = false>
 __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __restrict__ A, int lda,
                                                           const _Float16* __restrict__ B, int ldb, const _Float16* Cin,
                                                           int ldc, _Float16* D, int ldd, int M, int N, int K, int tiles_m,
                                                           int tiles_n, int group_m, size_t a_batch_stride,
                                                           size_t b_batch_stride, size_t c_batch_stride, size_t d_batch_stride,
-                                                          float* partial, int k_split_len) {
+                                                          float* partial, int k_split_len, size_t partial_plane) {
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, NT = S::NT, UA = S::UA, UB = S::UB, MI = S::MI, NI = S::NI;
     constexpr int STAGES = S::STAGES;
     static_assert(!(SPLIT_K && HAS_C), "C joins a split product in the finishing kernel");
@@ -328,6 +332,8 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
 #undef DECX_PIN
 
     if (SPLIT_K) {
+        const bool ordered = partial_plane != 0;                 // uniform over the launch
+        float* plane = partial + (size_t)blockIdx.z * partial_plane;
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
@@ -337,7 +343,10 @@ __global__ __launch_bounds__(S::NT) void hgemm_dma_kernel(const _Float16* __rest
 #pragma unroll
                     for (int ni = 0; ni < NI; ++ni) {
                         const int n = bn0 + wn0 + ni * 32 + li;
-                        if (n < N) unsafeAtomicAdd(partial + (size_t)m * N + n, acc[mi][ni][r]);
+                        if (n < N) {
+                            if (ordered) plane[(size_t)m * N + n] = acc[mi][ni][r];
+                            else unsafeAtomicAdd(plane + (size_t)m * N + n, acc[mi][ni][r]);
+                        }
                     }
                 }
             }

@@ -223,13 +223,15 @@ __global__ __launch_bounds__(S::NT) void hgemm_tile_kernel(const _Float16* __res
         }
 }
 
-// D = half(partial + C): the end of a split-K product (hgemm_dma_kernel with SPLIT_K).  partial is dense M x N fp32.
-static __global__ __launch_bounds__(256) void hgemm_split_finish_kernel(const float* __restrict__ partial, const _Float16* Cin, int ldc,
-                                                                 _Float16* D, int ldd, int M, int N) {
+// D = half(plane 0 + plane 1 + ... + C), added in that order: the end of a split-K product (hgemm_dma_kernel with
+// SPLIT_K).  partial holds `planes` dense M x N fp32 planes, `plane` floats apart (one plane in the atomic mode).
+static __global__ __launch_bounds__(256) void hgemm_split_finish_kernel(const float* __restrict__ partial, int planes, size_t plane,
+                                                                 const _Float16* Cin, int ldc, _Float16* D, int ldd, int M, int N) {
     const size_t total = (size_t)M * N;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const size_t m = i / N, n = i - m * N;
         float v = partial[i];
+        for (int s = 1; s < planes; ++s) v += partial[(size_t)s * plane + i];
         if (Cin != nullptr) v += (float)Cin[m * ldc + n];
         D[m * ldd + n] = (_Float16)v;
     }

@@ -22,6 +22,8 @@ struct Runtime {
     int hgemm_variant = 0;
     float* partial = nullptr;      // fp32 workspace of the fp16 split-K path, grown on demand, kept until the process ends
     size_t partial_bytes = 0;
+    int splitk_atomic = 0;         // fp16 split-K: 0 = one workspace plane per K range, added in range order (the same
+                                   // result on every run); 1 = all ranges add into one plane with atomics
     int group_m = 8;   // tile-rows per raster group of the XCD-aware tile walk (env DECX_HIP_GROUP_M overrides, for tuning)
 };
 extern Runtime g_rt;

@@ -92,14 +92,23 @@ int decx_hip_sgemm_async(const float* A, int lda, const float* B, int ldb, const
  * Products are accumulated in fp32 and rounded to binary16 (nearest even) once, on store; the reference accumulates
  * in binary16 (GEMM_kernel_def.cuh:100-121), which this library deliberately does not reproduce.
  * Fast path needs A, B 16-byte aligned with lda, ldb multiples of 8 (DECX pitch is a multiple of 16 halves).
- * Results with very few 128x128 tiles and a long K (say 64 x 65536 x 1024) are computed by K ranges in parallel, whose
- * fp32 partial sums meet in a workspace the library allocates on first use (M*N floats, kept for later calls; growing
- * it synchronises the device) and are rounded to binary16 once: the order of the additions is not fixed, so such a
- * result can differ in its last bit from run to run (never on integer-valued data), within the tolerance above. */
+ * Results with very few 128x128 tiles and a long K (say 64 x 65536 x 1024) are computed by K ranges in parallel: each
+ * range writes its fp32 partial sums into a plane of its own in a workspace the library allocates on first use (M*N
+ * floats per range, kept for later calls; growing it synchronises the device -- so the _async entry points must not be
+ * called from two host threads at once), the planes are added in range order and the sum is rounded to binary16
+ * once.  Like every reference path the result is therefore the same on every run; decx_hip_set_splitk_mode selects
+ * the older scheme in which all ranges add into one plane with atomics, in no fixed order. */
 int decx_hip_hgemm_f32acc(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                           int ldd, int M, int N, int K);
 int decx_hip_hgemm_f32acc_async(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
                                 uint16_t* D, int ldd, int M, int N, int K);
+
+/* How the fp16 entry points (decx_hip_hgemm_f32acc*, decx_hip_conv2_im2col_f16*) combine the K ranges of a product they
+ * split over K: 0 (default) = one workspace plane per range, added in range order -- run-to-run reproducible, as every
+ * path of the reference is (its long-K kernel is a single chain, GEMM_long_linear_region.cuh:35-55); 1 = atomic adds
+ * into one plane, whose order is not fixed (last-bit differences between runs on real-valued data; needs M*N floats
+ * of workspace instead of M*N per range).  Returns the previous mode. */
+int decx_hip_set_splitk_mode(int mode);
 
 /* A faster, NOT bit-exact alternative for the shape class of de::cuda::GEMM_Long_Lr(GPU_Matrix<float>& A, B, dst)
  * (GEMM/CUDA/extreme_shapes/GEMM_long_Lr.h:22-50; kernel GEMM_long_linear_region.cuh:73-131): short M, long K, whose

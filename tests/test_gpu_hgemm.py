@@ -7,7 +7,7 @@ exact product rounded once to binary16.
 import numpy as np
 import pytest
 
-from backup_1_amd import workloads
+from backup_1_amd import capi, workloads
 from gpu_helpers import gpu_hgemm, rel_err_vs_abs_scale
 
 pytestmark = pytest.mark.gpu
@@ -77,6 +77,29 @@ def test_split_k_for_few_tiles_and_long_k(gpu, oracle, shape):
     for variant in (0, 11, 2):
         got = from_bits(gpu_hgemm(Ar, Br, variant=variant))[rows]
         assert np.max((np.abs(got - ref) - np.abs(ref) / 2048.0) / scale) < TOL, variant
+
+
+def test_split_k_is_the_same_on_every_run(gpu, oracle):
+    # one workspace plane per K range, added in range order: real-valued data give the same bits on every run, as every
+    # path of the reference does (its long-K kernel is one chain, GEMM_long_linear_region.cuh:35-55).  The atomic mode
+    # keeps the tolerance only.
+    M, K, N = 64, 65536, 1024
+    A, B = to_bits(workloads.uniform_pm1((M, K), 36)), to_bits(workloads.uniform_pm1((K, N), 37))
+    first = gpu_hgemm(A, B)
+    for _ in range(3):
+        assert np.array_equal(gpu_hgemm(A, B), first)
+    rows = np.arange(0, M, 5, dtype=np.int32)
+    ref, scale = oracle.gemm_f64_rows_f16(A, B, rows)
+    assert np.max((np.abs(from_bits(first)[rows] - ref) - np.abs(ref) / 2048.0) / scale) < TOL
+    prev = capi.lib().decx_hip_set_splitk_mode(1)
+    try:
+        assert prev == 0
+        atomic = from_bits(gpu_hgemm(A, B))[rows]
+    finally:
+        assert capi.lib().decx_hip_set_splitk_mode(prev) == 1
+    assert np.max((np.abs(atomic - ref) - np.abs(ref) / 2048.0) / scale) < TOL
+    # a product that is not split must not care about the mode
+    assert np.array_equal(gpu_hgemm(A[:, :512], B[:512], variant=8), gpu_hgemm(A[:, :512], B[:512], variant=8))
 
 
 def test_rounding_to_half_is_nearest_even(gpu):
