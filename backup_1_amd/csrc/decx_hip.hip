@@ -373,6 +373,7 @@ int decx_hip_init(int* device) {
         HIP_TRY(hipEventCreate(&g_rt.ev_start));
         HIP_TRY(hipEventCreate(&g_rt.ev_stop));
         if (const char* gm = getenv("DECX_HIP_GROUP_M")) { int v = atoi(gm); if (v > 0) g_rt.group_m = v; }
+        if (int rc = hgemm_static_scratch_init(dev)) return rc;
         g_rt.is_init = true;
     }
     if (device) *device = g_rt.device;
@@ -496,6 +497,10 @@ int decx_hip_hgemm_f32acc_async(const uint16_t* A, int lda, const uint16_t* B, i
 int decx_hip_hgemm_f32acc(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                           int ldd, int M, int N, int K) {
     return finish(hgemm_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, single_on_library_stream()));
+}
+int decx_hip_hgemm_f32acc_noalloc(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
+                                  uint16_t* D, int ldd, int M, int N, int K, int splits) {
+    return finish(hgemm_splitk_static_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, splits));
 }
 int decx_hip_hgemm_f32acc_batched(const uint16_t* A, int lda, size_t stride_a, const uint16_t* B, int ldb, size_t stride_b,
                                   const uint16_t* Cin, int ldc, size_t stride_c, uint16_t* D, int ldd, size_t stride_d, int M,

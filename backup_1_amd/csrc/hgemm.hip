@@ -200,4 +200,48 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
     return launch_hgemm_tile<HShapeSmall, true>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The K-range route on a workspace that is part of the library's code object instead of an allocation: for callers
+// that must not allocate device memory (code under graph capture, serving loops, harnesses that forbid it).  Every GPU
+// the library is loaded on holds its own copy of the array until the process ends; host code reaches it only through
+// the address hipGetSymbolAddress returns for the current device.
+// ---------------------------------------------------------------------------------------------------------------
+constexpr size_t kScratchBytes = DECX_HIP_STATIC_WORKSPACE_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kMaxDevices = 64;
+static float* g_scratch_ptr[kMaxDevices] = {};
+
+int hgemm_static_scratch_init(int device) {
+    if (device < 0 || device >= kMaxDevices) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "device ordinal out of range\n");
+    if (g_scratch_ptr[device]) return 0;
+    void* ptr = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));     // the current device's copy
+    if (!ptr) return fail(DECX_HIP_FAIL_ALLOCATION, "the static workspace has no device address\n");
+    if (int rc = allow_split_kernel_lds()) return rc;            // done here so that the entry point only launches
+    g_scratch_ptr[device] = static_cast<float*>(ptr);
+    return 0;
+}
+
+int hgemm_splitk_static_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
+                                uint16_t* D, int ldd, int M, int N, int K, int splits) {
+    Batch one;
+    one.stream = g_rt.stream;
+    if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, one)) return rc;
+    float* workspace = g_rt.device >= 0 && g_rt.device < kMaxDevices ? g_scratch_ptr[g_rt.device] : nullptr;
+    if (!workspace) return fail(DECX_HIP_FAIL_NOT_INIT, "CUDA should be initialized first\n");
+    if (!hgemm_vector_path(A, lda, B, ldb, one))
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "the allocation-free entry point needs 16-byte aligned A, B with lda, ldb multiples of 8\n");
+    if (splits <= 0) splits = auto_hgemm_splits(M, N, K);
+    if (splits < 1) splits = 1;                                  // one range: still through the workspace, no allocation
+    if (splits > (K + 63) / 64) splits = (K + 63) / 64;
+    const SplitPlan plan = plan_hgemm_split(K, splits);
+    const size_t need = (size_t)M * N * sizeof(float) * plan.splits;
+    if (need > kScratchBytes)
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS,
+                    "M*N*4 bytes times %d K ranges = %zu bytes exceed the static workspace of %zu bytes; use decx_hip_hgemm_f32acc\n",
+                    plan.splits, need, kScratchBytes);
+    // always one plane per range, added in range order: nothing in the workspace has to start at zero
+    return hgemm_splitk_launch(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, plan, workspace, true, g_rt.stream);
+}
+
 }  // namespace decx_hip

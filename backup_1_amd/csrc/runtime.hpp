@@ -72,6 +72,11 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
                  int flag, const float* bias = nullptr, bool relu = false);
 int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                   int ldd, int M, int N, int K, const Batch& batch);
+// the K-range route of hgemm_enqueue on the library's static device workspace (no allocation); splits <= 0: automatic
+int hgemm_splitk_static_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
+                                uint16_t* D, int ldd, int M, int N, int K, int splits);
+// looks up the device address of the static workspace for the current device and prepares the kernels that use it
+int hgemm_static_scratch_init(int device);
 int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_stride, const uint16_t* filt, int N, int kh,
                   int kw, size_t filt_stride, size_t filt_row_stride, uint16_t* dst, int dst_dpitch, size_t dst_row_stride,
                   int flag, const uint16_t* bias, bool relu);

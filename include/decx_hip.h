@@ -110,6 +110,20 @@ int decx_hip_hgemm_f32acc_async(const uint16_t* A, int lda, const uint16_t* B, i
  * of workspace instead of M*N per range).  Returns the previous mode. */
 int decx_hip_set_splitk_mode(int mode);
 
+/* decx_hip_hgemm_f32acc for callers that cannot allocate device memory.  It has no counterpart in the reference: it is
+ * for code under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  Same arguments, arithmetic
+ * and result as decx_hip_hgemm_f32acc on its K-range route (`splits` ranges of K; <= 0: the count decx_hip_hgemm_f32acc
+ * would choose, 1 if it would not split), but the fp32 planes of the ranges live in a fixed array inside the library's
+ * code object, DECX_HIP_STATIC_WORKSPACE_BYTES per GPU, held until the process ends.  It calls no allocating routine.
+ * Needs A, B 16-byte aligned with lda, ldb multiples of 8, and M*N*4 bytes times the number of ranges within the
+ * workspace: larger problems are refused with DECX_HIP_FAIL_ERROR_PARAMS and a message that says so (they fill the
+ * chip without splitting K: decx_hip_hgemm_f32acc does not allocate for them either).  Every call on a GPU uses that
+ * GPU's one array: calls that overlap on one GPU (two host threads, two processes' worth of streams) race; nothing in
+ * the array has to be zero beforehand, each range overwrites the plane it owns.  Blocks until complete. */
+#define DECX_HIP_STATIC_WORKSPACE_BYTES ((size_t)32 << 20)
+int decx_hip_hgemm_f32acc_noalloc(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
+                                  uint16_t* D, int ldd, int M, int N, int K, int splits);
+
 /* A faster, NOT bit-exact alternative for the shape class of de::cuda::GEMM_Long_Lr(GPU_Matrix<float>& A, B, dst)
  * (GEMM/CUDA/extreme_shapes/GEMM_long_Lr.h:22-50; kernel GEMM_long_linear_region.cuh:73-131): short M, long K, whose
  * M x N tiles alone leave most of the chip idle.  The reference's kernel there is one fused chain per output like all
