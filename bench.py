@@ -24,10 +24,46 @@ sys.path.insert(0, ROOT)
 PEAK_FP32_MATRIX_TFLOPS = 157.3     # MI355X dense fp32 MFMA
 PEAK_FP16_MATRIX_TFLOPS = 2516.6    # MI355X dense fp16 MFMA (2.5 PFLOP/s)
 PEAK_HBM_GBPS = 8000.0              # MI355X HBM3E
-# HBM-side bytes per launch of the headline kernel (fp32 8192^3), from the FETCH_SIZE / WRITE_SIZE counter runs
-# summarised in profiles/hbm_traffic_fetch_write_size.txt (read factor 2.0, write factor 1.0 against a copy kernel).
-# Counters cannot be read from inside this script; the figure is only reported for the workload it was measured on.
-MEASURED_TRAFFIC_BYTES_FP32_8192 = 3.773e9
+# HBM-side bytes per launch of the headline kernel come from the FETCH_SIZE / WRITE_SIZE counter runs recorded in
+# profiles/traffic.json (kernel, bytes, the commit they were measured at).  Counters cannot be read from inside this
+# script; the figure is only reported for the workload and tile shape it was measured on, with its source beside it.
+TRAFFIC_FILE = os.path.join("profiles", "traffic.json")
+
+
+def measured_traffic(size, sgemm_variant):
+    """(bytes per launch, where the figure comes from) of the headline kernel, or (None, reason)."""
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_FILE)) as f:
+            table = json.load(f)["kernels"]
+    except (OSError, ValueError, KeyError) as e:
+        return None, "%s unreadable: %s" % (TRAFFIC_FILE, e)
+    for name, rec in table.items():
+        if rec.get("size") == size and sgemm_variant in rec.get("sgemm_variants", []):
+            return rec["traffic_bytes"], "%s: %s, measured at commit %s" % (TRAFFIC_FILE, name, rec.get("measured_at_commit"))
+    return None, "no counter run recorded for this size and tile shape"
+
+
+def verify_sgemm_rows(capi, dD, ldd, A, B, nrows, seed):
+    """Bit-compare `nrows` sampled rows of the device result with the oracle's fused chain (outside any timed region;
+    the oracle is only the checker)."""
+    import oracle
+    M, N = A.shape[0], B.shape[1]
+    rows = np.sort(np.random.Generator(np.random.PCG64(seed)).choice(M, size=min(nrows, M), replace=False)).astype(np.int32)
+    got = dD.download((M, ldd), np.float32)[rows, :N]
+    want = oracle.sgemm_chain_rows(A, B, rows)
+    return bool(np.array_equal(got.view(np.uint32), want.view(np.uint32))), int(rows.size)
+
+
+def verify_hgemm_rows(capi, dD, ldd, Abits, Bbits, nrows, seed):
+    """Sampled rows of the binary16 result against fp64 on the same binary16 inputs: max |x - r| / sum |a||b| (less
+    the half-ulp of the final rounding) must stay below 2e-3."""
+    import oracle
+    M, N = Abits.shape[0], Bbits.shape[1]
+    rows = np.sort(np.random.Generator(np.random.PCG64(seed)).choice(M, size=min(nrows, M), replace=False)).astype(np.int32)
+    got = dD.download((M, ldd), np.uint16)[rows, :N].view(np.float16).astype(np.float64)
+    ref, scale = oracle.gemm_f64_rows_f16(Abits, Bbits, rows)
+    err = float(np.max((np.abs(got - ref) - np.abs(ref) / 2048.0) / scale))
+    return err < 2e-3, max(err, 0.0), int(rows.size)
 
 
 def log(msg):
@@ -71,7 +107,7 @@ def time_launches(capi, launch, steps, warmup):
     return wall_ms / steps, ev_ms / steps
 
 
-def bench_sgemm(capi, workloads, M, K, N, steps, warmup, seed, dist="uniform"):
+def bench_sgemm(capi, workloads, M, K, N, steps, warmup, seed, dist="uniform", verify_rows=0):
     if dist == "uniform":
         A, B = workloads.uniform_pm1((M, K), seed), workloads.uniform_pm1((K, N), seed + 1)
     else:
@@ -86,11 +122,15 @@ def bench_sgemm(capi, workloads, M, K, N, steps, warmup, seed, dist="uniform"):
     wall, ev = time_launches(capi, launch, steps, warmup)
     flops = 2.0 * M * N * K
     med, mn = per_launch_stats(capi, launch, 10)
-    return {"ms_wall": wall, "ms_kernel": ev, "tflops": flops / (wall * 1e-3) / 1e12, "tflops_kernel": flops / (ev * 1e-3) / 1e12,
-            "flops": flops, "A": A, "B": B, "ms_median": med, "ms_min": mn}
+    out = {"ms_wall": wall, "ms_kernel": ev, "tflops": flops / (wall * 1e-3) / 1e12, "tflops_kernel": flops / (ev * 1e-3) / 1e12,
+           "flops": flops, "A": A, "B": B, "ms_median": med, "ms_min": mn}
+    if verify_rows:
+        # the result of the launches just timed, checked after the timed region
+        out["verified"], out["verified_rows"] = verify_sgemm_rows(capi, dD, ldd, A, B, verify_rows, seed + 2)
+    return out
 
 
-def bench_hgemm(capi, workloads, n, steps, warmup, seed, shape=None):
+def bench_hgemm(capi, workloads, n, steps, warmup, seed, shape=None, verify_rows=0):
     M, K, N = shape if shape else (n, n, n)
     A = workloads.uniform_pm1((M, K), seed).astype(np.float16).view(np.uint16)
     B = workloads.uniform_pm1((K, N), seed + 1).astype(np.float16).view(np.uint16)
@@ -99,7 +139,10 @@ def bench_hgemm(capi, workloads, n, steps, warmup, seed, shape=None):
     launch = lambda: capi.hgemm(dA.ptr, K, dB.ptr, N, dD.ptr, N, M, N, K, blocking=False)
     wall, ev = time_launches(capi, launch, steps, warmup)
     flops = 2.0 * M * N * K
-    return {"ms_wall": wall, "ms_kernel": ev, "tflops": flops / (wall * 1e-3) / 1e12, "tflops_kernel": flops / (ev * 1e-3) / 1e12}
+    out = {"ms_wall": wall, "ms_kernel": ev, "tflops": flops / (wall * 1e-3) / 1e12, "tflops_kernel": flops / (ev * 1e-3) / 1e12}
+    if verify_rows:
+        out["verified"], out["max_rel_err"], out["verified_rows"] = verify_hgemm_rows(capi, dD, N, A, B, verify_rows, seed + 2)
+    return out
 
 
 def bench_conv(capi, workloads, steps, warmup, H=224, W=224, C=64, N=128):
@@ -255,7 +298,7 @@ def bench_conv_fused(capi, workloads, steps, warmup):
     return {"ms_wall": best, "tflops": flops / (best * 1e-3) / 1e12}
 
 
-def cpu_baseline(A, B, rows):
+def cpu_baseline(workloads, A, B, rows):
     """The restated DECX_cpu thread-pool SGEMM (oracle/, kind "port") on the first `rows` rows of the headline A times
     the full B: B re-pack included, 12 tasks on a pool of min(hardware threads, 16) workers, as the reference sizes it."""
     import oracle
@@ -269,10 +312,22 @@ def cpu_baseline(A, B, rows):
         dt = time.perf_counter() - t0
         best = dt if best is None else min(best, dt)
     flops = 2.0 * rows * N * A.shape[1]
+    # configuration 1 of the baseline file: the same routine on the fp32 1024^3 problem (de::cpu::sgemm, sgemm.h:28-60)
+    A1, B1 = workloads.uniform_pm1((1024, 1024), 1), workloads.uniform_pm1((1024, 1024), 2)
+    out1 = np.zeros((1024, 1024), np.float32)
+    best1 = None
+    for _ in range(5):
+        t0 = time.perf_counter()
+        oracle.decx_cpu_sgemm(A1, B1, out=out1)
+        dt = time.perf_counter() - t0
+        best1 = dt if best1 is None else min(best1, dt)
     return {"value": flops / best / 1e12, "unit": "TFLOP/s", "cores": min(workers, 12), "kind": "port",
-            "sample": "restated DECX_cpu thread-pool SGEMM (B re-pack + 32x16x64 AVX2 FMA blocks, 3x4 task grid, pool of %d "
-                      "workers, g++ -O2) on rows 0..%d of the 8192^3 fp32 workload x full B, best of 2, %.2f s" %
-                      (workers, rows - 1, best)}
+            "host_cores": os.cpu_count(), "pool_workers": workers, "tasks": 12,
+            "fp32_1024_cube": {"gflops": round(2.0 * 1024 ** 3 / best1 / 1e9, 1), "ms": round(best1 * 1e3, 3),
+                               "what": "config 1 (M=N=K=1024, uniform[-1,1]) through the same routine, best of 5"},
+            "sample": "restated DECX_cpu thread-pool SGEMM (B re-pack + 32x16x64 AVX2 FMA blocks, 12 tasks = 3x4 grid on a pool "
+                      "of %d workers, so at most 12 cores work at once; host reports %d logical CPUs; AVX2+FMA, g++ -O2) on rows "
+                      "0..%d of the 8192^3 fp32 workload x full B, best of 2, %.2f s" % (workers, os.cpu_count() or 0, rows - 1, best)}
 
 
 def main():
@@ -283,6 +338,7 @@ def main():
     ap.add_argument("--size", type=int, default=8192, help="square size of the headline fp32 GEMM")
     ap.add_argument("--sgemm-variant", type=int, default=0, help="force a fp32 tile shape (0 = automatic)")
     ap.add_argument("--hgemm-variant", type=int, default=0, help="force a fp16 tile shape (0 = automatic)")
+    ap.add_argument("--no-verify", action="store_true", help="skip the post-run comparison of sampled rows with the oracle")
     ap.add_argument("--only", default="", help="comma list of: headline,fp16,sq4096,small,ragged,conv,relu,host,cpu (default all)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -301,8 +357,10 @@ def main():
 
     n = args.size
     log("headline: fp32 GEMM %d^3" % n)
-    head = bench_sgemm(capi, workloads, n, n, n, args.steps, args.warmup, 1234)
+    head = bench_sgemm(capi, workloads, n, n, n, args.steps, args.warmup, 1234, verify_rows=0 if args.no_verify else 16)
     log("  %.3f ms/step wall, %.3f ms/launch by HIP events -> %.1f TFLOP/s" % (head["ms_wall"], head["ms_kernel"], head["tflops"]))
+    if "verified" in head:
+        log("  %d sampled rows of the timed result bit-equal to the oracle's chain: %s" % (head["verified_rows"], head["verified"]))
 
     also = {}
     # the side workloads are sub-millisecond kernels launched after a host-side pause (data generation, uploads) in which
@@ -314,9 +372,12 @@ def main():
     also["side_timing"] = {"min_warmup_ms": SIDE_MIN_WARM_MS, "min_timed_ms": SIDE_MIN_TIMED_MS,
                            "what": "every workload under `also` is warmed up and timed over at least this many ms of back-to-back launches"}
     if want("fp16"):
-        r = bench_hgemm(capi, workloads, 8192, side_steps, side_warmup, 5)
+        r = bench_hgemm(capi, workloads, 8192, side_steps, side_warmup, 5, verify_rows=0 if args.no_verify else 16)
         also["fp16_8192_f32acc"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
                                     "frac_of_fp16_dense_peak": round(r["tflops_kernel"] / PEAK_FP16_MATRIX_TFLOPS, 4)}
+        if "verified" in r:
+            also["fp16_8192_f32acc"].update({"verified": r["verified"], "verified_rows": r["verified_rows"],
+                                             "max_rel_err_vs_fp64": float("%.3e" % r["max_rel_err"]), "tolerance": 2e-3})
         log("fp16 8192^3: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
     if want("sq4096"):
         r = bench_sgemm(capi, workloads, 4096, 4096, 4096, side_steps, side_warmup, 1234)
@@ -403,10 +464,11 @@ def main():
         also["cpu_conv_baseline"] = cpu_conv_baseline(workloads)
         log("cpu conv baseline: %.1f ms" % also["cpu_conv_baseline"]["ms"])
         log("cpu baseline (oracle port of the DECX_cpu thread-pool SGEMM) ...")
-        cpu = cpu_baseline(head["A"], head["B"], rows=min(n, 3072))
+        cpu = cpu_baseline(workloads, head["A"], head["B"], rows=min(n, 3072))
         log("  %.4f TFLOP/s on %d cores" % (cpu["value"], cpu["cores"]))
 
     achieved = head["tflops_kernel"]
+    traffic, traffic_source = measured_traffic(n, args.sgemm_variant)
     line = {
         # the metric's name as the baseline file spells it; `value` is its first component (fp32 8192^3), the fraction of
         # peak is roofline.frac, and the fp16 and conv components are under `also`
@@ -419,10 +481,13 @@ def main():
                                "operands (GPU_Matrix path)" % n},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_MATRIX_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK_FP32_MATRIX_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES_FP32_8192 if (n == 8192 and args.sgemm_variant in (0, 7)) else None,
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": "sgemm_tile_kernel", "flop_per_launch": head["flops"],
                      "avg_launch_ms_hip_events": round(head["ms_kernel"], 4),
                      "single_launch_ms_median": round(head["ms_median"], 4), "single_launch_ms_min": round(head["ms_min"], 4)},
+        "verified": head.get("verified"),
+        "verified_how": ("%d sampled rows of the result of the timed launches, bit-compared with the CPU oracle's fused chain "
+                         "after the timed region" % head["verified_rows"]) if "verified" in head else "skipped (--no-verify)",
         "cpu_baseline": cpu,
         "also": also,
     }

@@ -10,6 +10,7 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+    config.addinivalue_line("markers", "sanitizer: builds and runs the host-side C++ under -fsanitize=thread / address (CPU only)")
 
 
 @pytest.fixture(scope="session")

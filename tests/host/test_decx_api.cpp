@@ -1,6 +1,7 @@
 // Exercises the DECX-named C++ API (backup_1_amd/host/DECX.h) the way the reference's demo programs do
 // (test/test/CUDA_GEMM/CUDA_GEMM.cpp, test/test/"generating classes"/*.h), but with assertions, and checks results
-// against the CPU oracle (liboracle.so).  Usage: test_decx_api cpu | gpu
+// against the CPU oracle (liboracle.so).  Usage: test_decx_api cpu | cpu-small | gpu   (cpu-small: what the sanitizer
+// builds of backup_1_amd/host/Makefile run)
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -20,6 +21,8 @@ int oracle_conv2_chain(const float* src, int H, int W, int dpitch, long src_row_
 int oracle_conv2_f64_f16(const uint16_t* src, int H, int W, int dpitch, long src_row_stride, const uint16_t* filt, int N,
                          int kh, int kw, long filt_stride, long filt_row_stride, double* out, double* scale, int flag,
                          int nthreads);
+int oracle_decx_cpu_sgemm(const float* A, long lda, const float* B, long ldb, float* D, long ldd, int M, int N, int K,
+                          int nthreads);
 void oracle_gemm_f64_rows_f16(const uint16_t* A, long lda, const uint16_t* B, long ldb, const int* rows, int nrows,
                               double* out, double* abs_out, int N, int K, int nthreads);
 }
@@ -160,8 +163,29 @@ static void cpu_sgemm_case(int M, int K, int N, bool ints) {
     CHECK(std::memcmp(got.data(), want.data(), got.size() * 4) == 0);                // bit-identical to the fused chain
     A.release(); B.release(); C.release();
 }
+// the restated thread-pool SGEMM of the oracle (12 tasks on a pool of workers, packaged tasks and futures) against its own
+// scalar chain: the data-race and memory checks of the sanitizer builds run over this
+static void oracle_pool_sgemm_case(int M, int K, int N) {
+    const int n8 = (N + 7) / 8 * 8;
+    std::vector<float> a((size_t)M * K), b((size_t)K * n8, 0.f), d((size_t)M * n8, 0.f), bd((size_t)K * N), want((size_t)M * N);
+    for (auto& v : a) v = unif();
+    for (int k = 0; k < K; ++k) for (int j = 0; j < N; ++j) bd[(size_t)k * N + j] = b[(size_t)k * n8 + j] = unif();
+    CHECK(oracle_decx_cpu_sgemm(a.data(), K, b.data(), n8, d.data(), n8, M, N, K, 0) == 0);
+    oracle_sgemm_chain_fast(a.data(), K, bd.data(), N, nullptr, 0, want.data(), N, M, N, K, 0);
+    bool same = true;
+    for (int i = 0; i < M; ++i) same = same && std::memcmp(&d[(size_t)i * n8], &want[(size_t)i * N], (size_t)N * 4) == 0;
+    CHECK(same);
+}
+static void oracle_thread_pool_sgemm() {
+    oracle_pool_sgemm_case(200, 136, 72);
+    oracle_pool_sgemm_case(97, 64, 40);
+    oracle_pool_sgemm_case(33, 24, 9);
+    for (int rep = 0; rep < 3; ++rep) oracle_pool_sgemm_case(64, 128, 128);      // the pool is reused between calls
+}
+
+static bool g_small = false;     // "cpu-small": the sanitizer builds skip the one large case
 static void cpu_sgemm_matches_chain_bit_for_bit() {
-    cpu_sgemm_case(1024, 1024, 1024, false);      // config 1
+    if (!g_small) cpu_sgemm_case(1024, 1024, 1024, false);      // config 1
     cpu_sgemm_case(100, 136, 72, false);
     cpu_sgemm_case(33, 7, 9, false);
     cpu_sgemm_case(1, 1, 1, false);
@@ -538,7 +562,9 @@ static void conv_flavours_and_flags() {
 
 int main(int argc, char** argv) {
     std::string mode = argc > 1 ? argv[1] : "cpu";
-    if (mode == "cpu") {
+    if (mode == "cpu" || mode == "cpu-small") {
+        g_small = mode == "cpu-small";
+        RUN(oracle_thread_pool_sgemm);
         RUN(containers_follow_reference_pitch_rules);
         RUN(assignment_shares_the_payload);
         RUN(cpu_sgemm_into_an_operand);
