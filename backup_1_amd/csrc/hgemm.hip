@@ -2,6 +2,7 @@
 #include "runtime.hpp"
 #include "hgemm_dma_tile.hpp"
 #include "hgemm_tile.hpp"
+#include "hgemm_mfma16_tile.hpp"
 
 namespace decx_hip {
 
@@ -18,8 +19,11 @@ namespace decx_hip {
 //   9: as 8 with 3 stages (one workgroup per CU) -- small problems
 //  10: 256x128x64, 2x2 waves of 128x64, 2-stage LDS-DMA pipeline
 //   6: as 4 with 4x2 waves of 64x128 (two waves per SIMD)
-//   7: as 4 with 2x4 waves of 128x64 (two waves per SIMD) -- the default for large problems: the chip is power-capped on
-//      this kernel (MFMA busy x clock stays ~1.27 GHz-equivalents whatever the schedule), and this one is 1 % ahead
+//   7: as 4 with 2x4 waves of 128x64 (two waves per SIMD) -- the best of the 32x32x16 shapes: the chip is power-capped on
+//      them (MFMA busy x clock stays ~1.27 GHz-equivalents whatever the schedule), and this one is 1 % ahead
+//  15: 256x256x64, 2x4 waves of 128x64 on v_mfma_f32_16x16x32_f16, 2-stage LDS-DMA pipeline, result written through LDS in
+//      16-byte pieces (hgemm_mfma16_tile.hpp) -- the default for large problems: 8 % faster than 7 at 8192^3, because
+//      this instruction draws less power per flop on real-valued data
 //  11: split-K on shape 8 through an fp32 workspace (hgemm_splitk_enqueue) -- few tiles and a long K
 // and, for the fp16 convolution only: 12 keeps its register-staged kernels, 13 takes its LDS-DMA kernel for any image
 // whose channel pitch allows it, 14 its tap-row kernel; each switches its split over K off (experiments and tests)
@@ -33,6 +37,32 @@ typedef HgemmDmaShape<256, 256, 64, 2, 4, 2> HShapeDma64W8b;     // 8 waves, 128
 typedef HgemmDmaShape<128, 128, 64, 2, 2, 2> HShapeDmaSmall;     // 4 waves, 64x64 each, 64 KB of LDS: two workgroups per CU
 typedef HgemmDmaShape<128, 128, 64, 2, 2, 3> HShapeDmaSmall3;
 typedef HgemmDmaShape<256, 128, 64, 2, 2, 2> HShapeDmaTall;      // 4 waves, 128x64 each
+
+typedef Hgemm16Shape<256, 256, 2, 4> HShape16;                   // 8 waves, 128x64 each, 16x16x32 MFMAs
+
+int launch_hgemm_mfma16(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
+                        int ldd, int M, int N, int K, const Batch& batch) {
+    typedef HShape16 S;
+    auto kern = Cin ? hgemm_mfma16_kernel<S, true> : hgemm_mfma16_kernel<S, false>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hgemm_mfma16_kernel<S, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hgemm_mfma16_kernel<S, false>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+        attr_done = true;
+    }
+    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    const long total = (long)tiles_m * tiles_n;
+    if (total > 0x7fffffffL || batch.count > 65535) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
+    const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
+    hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::LDS_BYTES, batch.stream,
+                       reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
+                       reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N, K,
+                       tiles_m, tiles_n, group_m, batch.stride_a, batch.stride_b, batch.stride_c, batch.stride_d);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
 
 template <class S, bool VEC>
 int launch_hgemm_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
@@ -166,7 +196,7 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
     int variant = g_rt.hgemm_variant;
     {
         // few 128x128 tiles and a long K: split K (variant 11 forces it, any other fixed variant switches it off)
-        if (batch.count == 1 && (variant < 1 || variant > 10)) {
+        if (batch.count == 1 && (variant < 1 || variant > 10) && variant != 15) {
             int splits = auto_hgemm_splits(M, N, K);
             if (variant == 11 && splits == 0 && K >= 1024 && (size_t)M * N <= ((size_t)1 << 26)) {
                 const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
@@ -179,15 +209,16 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
         }
         if (variant == 11) variant = 0;
     }
-    if (variant < 1 || variant > 10) {
+    if (variant < 1 || (variant > 10 && variant != 15)) {
         // same cost model as the fp32 picker: rounds of tiles per CU x tile area / measured shape efficiency
         const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
         const long big = (long)cdiv(M, 256) * cdiv(N, 256) * batch.count, small = (long)cdiv(M, 128) * cdiv(N, 128) * batch.count;
         const double cost_big = (double)((big + cus - 1) / cus) * 65536.0;
         const double cost_small = (double)((small + cus - 1) / cus) * 16384.0 / 0.75;
         // the small tile with three LDS stages holds one workgroup per CU: only worth it when there is at most one to hold
-        variant = cost_big <= cost_small ? 7 : (small <= cus ? 9 : 8);
+        variant = cost_big <= cost_small ? 15 : (small <= cus ? 9 : 8);
     }
+    if (variant == 15) return launch_hgemm_mfma16(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     if (variant == 3) return launch_hgemm_dma_tile<HShapeDma>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     if (variant == 4) return launch_hgemm_dma_tile<HShapeDma64>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     if (variant == 5) return launch_hgemm_dma_tile<HShapeDma5>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);

@@ -1,0 +1,366 @@
+// fp16-in / fp32-accumulate tile on v_mfma_f32_16x16x32_f16, fed by the LDS-DMA pipeline of hgemm_dma_tile.hpp.
+//
+// Why another MFMA shape: on real-valued operands the chip runs the fp16 matrix pipe against its power limit, not its
+// issue rate (an MFMA-only loop reaches 2.45 PFLOP/s on all-zero registers and 1.67 on uniform[-1,1] ones with
+// v_mfma_f32_32x32x16_f16 -- and 1.90-1.93 with v_mfma_f32_16x16x32_f16, which sums 32 products per accumulator access
+// instead of 16).  Everything around the instruction is kept: 256 x 256 x 64 tile, 8 waves of 128 x 64 (two per SIMD),
+// two LDS stages filled by global_load_lds_dwordx4, 16-byte units XOR-swizzled on the global side.
+//
+// What is new besides the instruction:
+//   * LDS keeps the stages of one operand next to each other ([A0][A1][B0][B1]) and the K walk is unrolled over the two
+//     stages, so that stage, k-block and row block of a fragment read are compile-time constants that fold into the
+//     instruction's offset field: no address arithmetic between the MFMAs.
+//   * The B swizzle also moves rows 8 apart (the four 16-lane groups of a transposing read fetch rows 8g .. 8g+3 of
+//     the same columns) onto different banks.
+//   * The matrix B fragment is the MFMA's first operand and the matrix A fragment its second: the accumulators then hold
+//     the tile transposed, i.e. a lane owns 4 CONSECUTIVE COLUMNS of one row.  The epilogue rounds them to binary16,
+//     parks the wave's 128 x 64 piece in LDS (the operand buffers are free by then) and writes it out as 16-byte
+//     pieces, 128 contiguous bytes per row.
+//   * A K step is cut into four units of 16 MFMAs (k-block x half of the wave's rows); a unit's fragments are fetched
+//     during the unit before it, which keeps 2 x (4 A + 4 B) fragments in registers instead of 2 x (8 + 4).
+// Needs 16-byte aligned A, B with lda, ldb multiples of 8, like the other LDS-DMA tiles.
+#pragma once
+#include "hgemm_dma_tile.hpp"
+
+namespace decx_hip {
+
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+// B unit (k, u) of a stage: as b_unit_slot, plus bit 1 of the unit index flipped for odd k / 8
+__device__ __forceinline__ int b16_unit_slot(int k, int u, int UB) {
+    return k * UB + (u ^ (((k & 3) << 2) | (((k >> 3) & 1) << 1)));
+}
+
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_>
+struct Hgemm16Shape {
+    static constexpr int BM = BM_, BN = BN_, BK = 64, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+    static constexpr int NWAVES = WAVES_M * WAVES_N, NT = NWAVES * kWave;
+    static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+    static constexpr int MI = WM / 16, NI = WN / 16;            // 16 x 16 accumulator blocks of a wave
+    static constexpr int MH = 2, UM = MI / MH;                  // a unit = one k-block x UM row blocks
+    static constexpr int KS = BK / 32, UNITS = KS * MH;
+    static constexpr int UA = BK / 8, UB = BN / 8;              // 16-byte units per LDS row
+    static constexpr int A_UNITS = BM * UA, B_UNITS = BK * UB;
+    static constexpr int A_BYTES = A_UNITS * 16, B_BYTES = B_UNITS * 16;
+    static constexpr int STAGES = 2;
+    static constexpr size_t LDS_BYTES = (size_t)STAGES * (A_BYTES + B_BYTES);
+    static constexpr int A_LOADS = A_UNITS / 64 / NWAVES, B_LOADS = B_UNITS / 64 / NWAVES, LOADS = A_LOADS + B_LOADS;
+    static constexpr int A_PASSES = A_UNITS / NT, B_PASSES = B_UNITS / NT;
+    static_assert(MI % MH == 0 && UNITS % 2 == 0 && KS % 2 == 0, "fragment sets must line up across units and K steps");
+    static_assert(UA == 8 && UB >= 16 && (UB & (UB - 1)) == 0, "swizzles assume 8 units per A row and >= 16 per B row");
+    static_assert(A_UNITS % (64 * NWAVES) == 0 && B_UNITS % (64 * NWAVES) == 0, "DMA chunks must divide over the waves");
+    static_assert((size_t)NWAVES * WM * WN * 2 <= LDS_BYTES, "the epilogue parks every wave's piece in LDS");
+    static_assert((STAGES - 1) * A_BYTES + (MI - 1) * 16 * UA * 16 < 65536 && (STAGES - 1) * B_BYTES + (32 * (KS - 1) + 4) * UB * 16 < 65536,
+                  "fragment reads address stage, k-block and row block through the 16-bit offset field");
+};
+
+template <class S, bool HAS_C>
+__global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __restrict__ A, int lda,
+                                                             const _Float16* __restrict__ B, int ldb, const _Float16* Cin,
+                                                             int ldc, _Float16* D, int ldd, int M, int N, int K, int tiles_m,
+                                                             int tiles_n, int group_m, size_t a_batch_stride,
+                                                             size_t b_batch_stride, size_t c_batch_stride, size_t d_batch_stride) {
+    constexpr int BM = S::BM, BN = S::BN, BK = S::BK, NT = S::NT, UA = S::UA, UB = S::UB, MI = S::MI, NI = S::NI;
+    constexpr int UM = S::UM, MH = S::MH, KS = S::KS, UNITS = S::UNITS;
+    constexpr int A_BYTES = S::A_BYTES, B_BYTES = S::B_BYTES;
+    constexpr int BLK = UM * NI;                                // MFMAs per unit
+    A += (size_t)blockIdx.y * a_batch_stride;
+    B += (size_t)blockIdx.y * b_batch_stride;
+    if (HAS_C) Cin += (size_t)blockIdx.y * c_batch_stride;
+    D += (size_t)blockIdx.y * d_batch_stride;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];   // [A stage 0][A stage 1][B stage 0][B stage 1]
+    const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds_raw;
+
+    const TileCoord tc = xcd_grouped_tile(blockIdx.x, tiles_m, tiles_n, group_m);
+    const int bm0 = tc.tm * BM, bn0 = tc.tn * BN;
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
+    const int wm0 = (wave / S::WAVES_N) * S::WM, wn0 = (wave % S::WAVES_N) * S::WN;
+    const int lg = lane >> 4, li = lane & 15;                   // 16-lane group = k sub-block, lane in group = row / column
+
+    // ---- DMA sources: wave-uniform bases that advance by one K step per fetched step + loop-invariant lane offsets
+    const int m_first = bm0 < M ? bm0 : M - 1;
+    const _Float16* a_base = A + (size_t)m_first * lda;
+    const _Float16* b_base = B;
+    uint32_t a_off[S::A_LOADS], b_off[S::B_LOADS];
+#pragma unroll
+    for (int j = 0; j < S::A_LOADS; ++j) {
+        const int chunk = wave * S::A_LOADS + j;                // 64 units = 8 rows
+        const int r = chunk * (64 / UA) + lane / UA;
+        const int q = (lane % UA) ^ ((r / (16 / UA)) % UA);     // the unit whose swizzled slot is this lane
+        int m = bm0 + r;
+        if (m >= M) m = M - 1;                                  // rows past the end are computed and never stored
+        a_off[j] = (uint32_t)(((size_t)(m - m_first) * lda + 8 * q) * sizeof(_Float16));
+    }
+#pragma unroll
+    for (int j = 0; j < S::B_LOADS; ++j) {
+        const int chunk = wave * S::B_LOADS + j;                // 64 units = 64 / UB k-rows
+        const int kr = chunk * (64 / UB) + lane / UB;
+        const int u = (lane % UB) ^ (((kr & 3) << 2) | (((kr >> 3) & 1) << 1));
+        const int col = clamp_group_col(bn0 + 8 * u, N, 8);     // stay inside the operand; such columns are never stored
+        b_off[j] = (uint32_t)(((size_t)kr * ldb + col) * sizeof(_Float16));
+    }
+    // Every K step fetches the step two ahead of it into the stage it leaves, also the last two, which have nothing left
+    // to fetch: their loads repeat the last whole step (the bases stop there) into a stage nobody reads again.  All
+    // steps are then the same code with the same wait counts, at the price of two redundant step loads per tile.
+    const int full_steps = K / BK;
+    int steps_fetched = 0;
+    const size_t b_step = (size_t)BK * ldb;
+    auto issue_one = [&](auto stage_tag, auto j_tag) {
+        constexpr int STG = decltype(stage_tag)::value, J = decltype(j_tag)::value;
+        if constexpr (J < S::A_LOADS) {
+            dma_load16(a_base, a_off[J], lds_base + (uint32_t)(STG * A_BYTES) + (uint32_t)(wave * S::A_LOADS + J) * 1024u);
+        } else {
+            constexpr int JB = J - S::A_LOADS;
+            dma_load16(b_base, b_off[JB], lds_base + (uint32_t)(2 * A_BYTES + STG * B_BYTES) + (uint32_t)(wave * S::B_LOADS + JB) * 1024u);
+        }
+        if constexpr (J == S::LOADS - 1) {
+            ++steps_fetched;
+            const bool more = steps_fetched < full_steps;        // scalar: the next fetch is a new step
+            a_base += more ? BK : 0;
+            b_base += more ? b_step : (size_t)0;
+        }
+    };
+
+    f32x4v acc[MI][NI];
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = f32x4v{0.f, 0.f, 0.f, 0.f};
+
+    // ---- fragment reads: per-lane byte offsets inside stage 0; stage, k-block, row block and the low / high half of a
+    // transposing read are constants added in the instruction
+    //   A fragment of row block rb, k-block kb : lane (lg, li) reads the 8 halves k = 32 kb + 8 lg .. + 7 of row 16 rb + li
+    //   B fragment of column block ni, k-block kb: two transposing reads of 4 rows each; lane (lg, li) supplies the address
+    //     of row 32 kb + 8 lg + li / 4 (+ 4), columns 16 ni + 4 (li % 4) .. + 3, and receives column 16 ni + li of 4 rows
+    uint32_t a_rd[KS], b_rd[NI];
+#pragma unroll
+    for (int kb = 0; kb < KS; ++kb) a_rd[kb] = (uint32_t)a_unit_slot(wm0 + li, 4 * kb + lg, UA) * 16u;
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni) {
+        const int col = wn0 + 16 * ni + 4 * (li & 3);
+        b_rd[ni] = (uint32_t)(2 * A_BYTES) + (uint32_t)b16_unit_slot(8 * lg + (li >> 2), col >> 3, UB) * 16u + (uint32_t)(col & 7) * 2u;
+    }
+    static_assert(16 % (16 / UA) == 0 && (16 / (16 / UA)) % UA == 0, "row blocks of 16 must not change the A swizzle");
+    typedef short i16x8 __attribute__((ext_vector_type(8)));
+    f16x8 af[2][UM];                                            // by unit parity
+    i16x4 blo[2][NI], bhi[2][NI];                               // by k-block parity
+    auto read_a = [&](auto set_tag, auto slot_tag, auto stage_tag, auto kb_tag, auto rb_tag) {
+        constexpr int OFF = decltype(stage_tag)::value * A_BYTES + decltype(rb_tag)::value * (16 * UA * 16);
+        af[decltype(set_tag)::value][decltype(slot_tag)::value] =
+            __builtin_bit_cast(f16x8, *reinterpret_cast<const u32x4*>(lds_raw + a_rd[decltype(kb_tag)::value] + OFF));
+    };
+    auto read_b = [&](auto set_tag, auto stage_tag, auto kb_tag, auto ni_tag, auto hi_tag) {
+        constexpr int SET = decltype(set_tag)::value, NIX = decltype(ni_tag)::value, HI = decltype(hi_tag)::value;
+        constexpr int OFF = decltype(stage_tag)::value * B_BYTES + (32 * decltype(kb_tag)::value + 4 * HI) * (UB * 16);
+        const i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) i16x4*)(lds_raw + b_rd[NIX] + OFF));
+        if constexpr (HI) bhi[SET][NIX] = v;
+        else blo[SET][NIX] = v;
+    };
+    // read number R of the fragments a K step starts with (unit 0: row blocks 0 .. UM-1, k-block 0), in the order its
+    // first MFMAs need them: A block 0, all of B, the other A blocks
+    constexpr int FIRST_READS = UM + 2 * NI;
+    auto read_first = [&](auto stage_tag, auto r_tag) {
+        constexpr int R = decltype(r_tag)::value;
+        typedef std::integral_constant<int, 0> I0;
+        if constexpr (R == 0) read_a(I0{}, I0{}, stage_tag, I0{}, I0{});
+        else if constexpr (R <= 2 * NI)
+            read_b(I0{}, stage_tag, I0{}, std::integral_constant<int, (R - 1) / 2>{}, std::integral_constant<int, (R - 1) % 2>{});
+        else read_a(I0{}, std::integral_constant<int, R - 2 * NI>{}, stage_tag, I0{}, std::integral_constant<int, R - 2 * NI>{});
+    };
+    // MFMA number I of unit U: row block (U % MH) * UM + I / NI, column block I % NI
+    auto mfma_one = [&](auto u_tag, auto i_tag) {
+        constexpr int U = decltype(u_tag)::value, I = decltype(i_tag)::value;
+        constexpr int KB = U / MH, MIX = (U % MH) * UM + I / NI, NIX = I % NI;
+        const i16x4 lo = blo[KB & 1][NIX], hi = bhi[KB & 1][NIX];
+        const i16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        acc[MIX][NIX] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, both), af[U & 1][I / NI], acc[MIX][NIX], 0, 0, 0);
+    };
+#define DECX_PIN() __builtin_amdgcn_sched_barrier(0)
+
+    // One K step from stage STG.  On entry af[0] / b*[0] hold the fragments of unit 0; on exit those of the next step's.
+    // Units 0 .. UNITS-2: the first MFMAs each carry one LDS read of the next unit's A fragments and of this unit's share
+    // of the next k-block's B fragments.  Last unit: a few MFMAs, then wait for the next step's data + barrier -- nobody
+    // reads this stage any more -- and between the remaining MFMAs the DMA refill of this stage and the first fragments
+    // of the next step from the other stage.
+    auto k_step = [&](auto stg_tag) {
+        constexpr int STG = decltype(stg_tag)::value;
+        typedef std::integral_constant<int, STG> Stg;
+        typedef std::integral_constant<int, STG ^ 1> Next;
+        static_for<0, UNITS - 1>([&](auto u_tag) {
+            constexpr int U = decltype(u_tag)::value, KB = U / MH, H = U % MH;
+            constexpr int NU = U + 1, NKB = NU / MH, NH = NU % MH;
+            constexpr int NB = (KB + 1 < KS) ? 2 * NI / MH : 0;          // B reads of the next k-block in this unit
+            constexpr int NR = UM + NB;
+            static_assert(NR <= BLK, "one read per MFMA slot");
+            static_for<0, BLK>([&](auto i_tag) {
+                constexpr int I = decltype(i_tag)::value;
+                if constexpr (I < UM) {
+                    read_a(std::integral_constant<int, NU & 1>{}, i_tag, Stg{}, std::integral_constant<int, NKB>{},
+                           std::integral_constant<int, NH * UM + I>{});
+                } else if constexpr (I < NR) {
+                    constexpr int RB = H * NB + (I - UM);
+                    read_b(std::integral_constant<int, (KB + 1) & 1>{}, Stg{}, std::integral_constant<int, KB + 1>{},
+                           std::integral_constant<int, RB / 2>{}, std::integral_constant<int, RB % 2>{});
+                }
+                mfma_one(u_tag, i_tag);
+                DECX_PIN();
+            });
+        });
+        typedef std::integral_constant<int, UNITS - 1> Last;
+        constexpr int PRE = BLK / 4, SLOTS = BLK - PRE;
+        static_for<0, PRE>([&](auto i_tag) {
+            mfma_one(Last{}, i_tag);
+            DECX_PIN();
+        });
+        wait_dma_then_barrier<0>();
+        DECX_PIN();
+        static_for<0, SLOTS>([&](auto i_tag) {
+            constexpr int I = decltype(i_tag)::value;
+            static_for<(I * S::LOADS) / SLOTS, ((I + 1) * S::LOADS) / SLOTS>([&](auto j_tag) { issue_one(Stg{}, j_tag); });
+            // two reads per slot until they are all out: the next step's first MFMAs follow closely
+            constexpr int R0 = 2 * I < FIRST_READS ? 2 * I : FIRST_READS, R1 = 2 * I + 2 < FIRST_READS ? 2 * I + 2 : FIRST_READS;
+            static_for<R0, R1>([&](auto r_tag) { read_first(Next{}, r_tag); });
+            mfma_one(Last{}, std::integral_constant<int, PRE + I>{});
+            DECX_PIN();
+        });
+    };
+
+    typedef std::integral_constant<int, 0> I0;
+    typedef std::integral_constant<int, 1> I1;
+    if (full_steps > 0) {
+        // an odd number of steps starts in stage 1, so that the walk below always ends with the pair (stage 0, stage 1)
+        const bool odd = full_steps & 1;
+        if (odd) {
+            static_for<0, S::LOADS>([&](auto j) { issue_one(I1{}, j); });
+            static_for<0, S::LOADS>([&](auto j) { issue_one(I0{}, j); });
+            wait_dma_then_barrier<0>();
+            static_for<0, FIRST_READS>([&](auto r) { read_first(I1{}, r); });
+            DECX_PIN();
+            k_step(I1{});
+        } else {
+            static_for<0, S::LOADS>([&](auto j) { issue_one(I0{}, j); });
+            static_for<0, S::LOADS>([&](auto j) { issue_one(I1{}, j); });
+            wait_dma_then_barrier<0>();
+            static_for<0, FIRST_READS>([&](auto r) { read_first(I0{}, r); });
+            DECX_PIN();
+        }
+        for (int t = odd ? 1 : 0; t < full_steps; t += 2) {
+            k_step(I0{});
+            k_step(I1{});
+        }
+    }
+
+    // ---- partial last K step: through registers into stage 0 (zero-filled beyond K), then all of its units
+    if (full_steps * BK < K) {
+        const int k0 = full_steps * BK;
+        u32x4 a_stage[S::A_PASSES], b_stage[S::B_PASSES];
+#pragma unroll
+        for (int p = 0; p < S::A_PASSES; ++p) {
+            const int id = tid + p * NT;
+            const int r = id / UA, q = id % UA;
+            int m = bm0 + r;
+            if (m >= M) m = M - 1;
+            const int k = k0 + 8 * q;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (k < K) {
+                v = *reinterpret_cast<const u32x4*>(A + (size_t)m * lda + k);
+                const int keep = K - k;
+                if (keep < 8) {
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) v[w] &= (2 * w + 1 < keep) ? 0xffffffffu : (2 * w < keep ? 0x0000ffffu : 0u);
+                }
+            }
+            a_stage[p] = v;
+        }
+#pragma unroll
+        for (int p = 0; p < S::B_PASSES; ++p) {
+            const int id = tid + p * NT;
+            const int kr = id / UB, u = id % UB;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (k0 + kr < K) v = *reinterpret_cast<const u32x4*>(B + (size_t)(k0 + kr) * ldb + clamp_group_col(bn0 + 8 * u, N, 8));
+            b_stage[p] = v;
+        }
+        wait_dma_then_barrier<0>();                             // everybody is done with every buffer
+        u32x4* Ab = reinterpret_cast<u32x4*>(lds_raw);
+        u32x4* Bb = reinterpret_cast<u32x4*>(lds_raw + 2 * A_BYTES);
+#pragma unroll
+        for (int p = 0; p < S::A_PASSES; ++p) {
+            const int id = tid + p * NT;
+            Ab[a_unit_slot(id / UA, id % UA, UA)] = a_stage[p];
+        }
+#pragma unroll
+        for (int p = 0; p < S::B_PASSES; ++p) {
+            const int id = tid + p * NT;
+            Bb[b16_unit_slot(id / UB, id % UB, UB)] = b_stage[p];
+        }
+        __syncthreads();
+        static_for<0, UNITS>([&](auto u_tag) {
+            constexpr int U = decltype(u_tag)::value, KB = U / MH, H = U % MH;
+            static_for<0, UM>([&](auto r) {
+                read_a(std::integral_constant<int, U & 1>{}, r, I0{}, std::integral_constant<int, KB>{},
+                       std::integral_constant<int, H * UM + decltype(r)::value>{});
+            });
+            if constexpr (H == 0)
+                static_for<0, 2 * NI>([&](auto r) {
+                    read_b(std::integral_constant<int, KB & 1>{}, I0{}, std::integral_constant<int, KB>{},
+                           std::integral_constant<int, decltype(r)::value / 2>{}, std::integral_constant<int, decltype(r)::value % 2>{});
+                });
+            static_for<0, BLK>([&](auto i_tag) { mfma_one(u_tag, i_tag); });
+        });
+    }
+#undef DECX_PIN
+
+    // ---- epilogue.  acc[mi][ni][e] is element (row 16 mi + li, column 16 ni + 4 lg + e) of the wave's piece.  dst = A*B + C
+    // adds C in fp32; one rounding to binary16; the piece goes to LDS (rows of WN halves, 16-byte pieces XOR-swizzled by
+    // the row) and leaves as 16-byte stores.
+    wait_dma_then_barrier<0>();                                 // nobody reads operands any more, and the last (redundant) stage loads have landed
+    constexpr int ROW_BYTES = S::WN * 2, PIECES = S::WN / 8, ROWS_PER_PASS = kWave / PIECES, PASSES = S::WM / ROWS_PER_PASS;
+    static_assert(PIECES >= 8 && (PIECES & (PIECES - 1)) == 0 && kWave % PIECES == 0, "piece swizzle");
+    unsigned char* park = lds_raw + (size_t)wave * (S::WM * ROW_BYTES);
+    const int m_wave = bm0 + wm0, n_wave = bn0 + wn0;
+#pragma unroll
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) {
+            const int row = 16 * mi + li, col = 16 * ni + 4 * lg;
+            f32x4v v = acc[mi][ni];
+            if (HAS_C) {
+                const int m = m_wave + row, n = n_wave + col;
+                if (m < M) {
+                    const _Float16* crow = Cin + (size_t)m * ldc + n;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (n + e < N) v[e] += (float)crow[e];
+                }
+            }
+            const f16x4 h = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+            const int piece = col >> 3;
+            *reinterpret_cast<u32x2*>(park + row * ROW_BYTES + ((piece ^ (row & 7)) << 4) + ((lg & 1) << 3)) = __builtin_bit_cast(u32x2, h);
+        }
+    // the wave reads back what it wrote itself: LDS operations of a wave complete in order, no barrier needed
+    const bool vec_d = ((reinterpret_cast<uintptr_t>(D) | (uintptr_t)(ldd * 2)) & 15) == 0;
+    const bool whole = bm0 + BM <= M && bn0 + BN <= N && vec_d;     // one scalar test instead of checks around every store
+#pragma unroll
+    for (int pass = 0; pass < PASSES; ++pass) {
+        const int row = pass * ROWS_PER_PASS + lane / PIECES, piece = lane % PIECES;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(park + row * ROW_BYTES + ((piece ^ (row & 7)) << 4));
+        const int m = m_wave + row, n = n_wave + 8 * piece;
+        _Float16* dp = D + (size_t)m * ldd + n;
+        if (whole) {
+            *reinterpret_cast<u32x4*>(dp) = v;
+        } else if (m < M) {
+            if (vec_d && n + 8 <= N) {
+                *reinterpret_cast<u32x4*>(dp) = v;
+            } else {
+                const f16x8 h = __builtin_bit_cast(f16x8, v);
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (n + e < N) dp[e] = h[e];
+            }
+        }
+    }
+}
+
+}  // namespace decx_hip

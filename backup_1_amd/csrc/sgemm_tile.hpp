@@ -87,13 +87,6 @@ __device__ __forceinline__ unsigned lds_byte_address(const void* p) {
 // Workgroup barrier that first waits for this wave's own LDS traffic, stated explicitly because the compiler's wait
 // counting does not see the inline-asm stores above.
 __device__ __forceinline__ void lds_sync() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-template <int I, int N, class F>
-__device__ __forceinline__ void static_for(F&& f) {
-    if constexpr (I < N) {
-        f(std::integral_constant<int, I>{});
-        static_for<I + 1, N>(f);
-    }
-}
 
 // A K step of dk as an increment of the im2col position (c, kj, ki): dk = (dki*kw + dkj)*dpitch + dc, and of the byte
 // offset of that position inside a tensor whose rows are row_stride floats apart.  Worked out once per kernel so that

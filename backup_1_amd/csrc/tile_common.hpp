@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 namespace decx_hip {
 
@@ -32,6 +33,15 @@ __device__ __forceinline__ float relu_by_sign(float v) {
 __host__ __device__ __forceinline__ constexpr int clamp_group_col(int col, int N, int unit) {
     const int last = (N + unit - 1) / unit * unit - unit;
     return col < last ? col : last;
+}
+
+// f(integral_constant<int, I>) for I = I0 .. N-1, unrolled at compile time
+template <int I, int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
 }
 
 struct TileCoord {
