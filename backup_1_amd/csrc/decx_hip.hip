@@ -624,6 +624,10 @@ int decx_hip_set_hgemm_variant(int variant) {
     return prev;
 }
 
+int decx_hip_hgemm_probe(int ablate, const uint16_t* A, int lda, const uint16_t* B, int ldb, uint16_t* D, int ldd, int M, int N, int K) {
+    return hgemm_probe_enqueue(ablate, A, lda, B, ldb, D, ldd, M, N, K);
+}
+
 int decx_hip_set_splitk_mode(int mode) {
     int prev = g_rt.splitk_atomic;
     g_rt.splitk_atomic = mode ? 1 : 0;

@@ -64,6 +64,36 @@ int launch_hgemm_mfma16(const uint16_t* A, int lda, const uint16_t* B, int ldb, 
     return 0;
 }
 
+// Measurement variants of the kernel above (decx_hip_hgemm_probe): same launch, parts of the K walk left out.
+int hgemm_probe_enqueue(int ablate, const uint16_t* A, int lda, const uint16_t* B, int ldb, uint16_t* D, int ldd, int M, int N, int K) {
+    typedef HShape16 S;
+    Batch batch;
+    batch.stream = g_rt.stream;
+    if (int rc = check_gemm_args(A, lda, B, ldb, nullptr, 0, D, ldd, M, N, K, batch)) return rc;
+    if (!aligned16(A) || !aligned16(B) || lda % 8 || ldb % 8 || (size_t)lda * 512 >= ((size_t)1 << 32) || (size_t)ldb * 128 >= ((size_t)1 << 32))
+        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "the probe needs 16-byte aligned A, B with lda, ldb multiples of 8\n");
+    void (*kern)(const _Float16*, int, const _Float16*, int, const _Float16*, int, _Float16*, int, int, int, int, int, int, int, size_t,
+                 size_t, size_t, size_t) = nullptr;
+    switch (ablate) {
+        case 0: kern = hgemm_mfma16_kernel<S, false, 0>; break;
+        case 1: kern = hgemm_mfma16_kernel<S, false, 1>; break;
+        case 3: kern = hgemm_mfma16_kernel<S, false, 3>; break;
+        case 4: kern = hgemm_mfma16_kernel<S, false, 4>; break;
+        case 5: kern = hgemm_mfma16_kernel<S, false, 5>; break;
+        case 7: kern = hgemm_mfma16_kernel<S, false, 7>; break;
+        default: return fail(DECX_HIP_FAIL_ERROR_PARAMS, "probe variants: 0, 1, 3, 4, 5, 7\n");
+    }
+    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(S::NT), S::LDS_BYTES, batch.stream,
+                       reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
+                       static_cast<const _Float16*>(nullptr), 0, reinterpret_cast<_Float16*>(D), ldd, M, N, K, tiles_m, tiles_n, group_m,
+                       (size_t)0, (size_t)0, (size_t)0, (size_t)0);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 template <class S, bool VEC>
 int launch_hgemm_tile(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                       int ldd, int M, int N, int K, const Batch& batch) {

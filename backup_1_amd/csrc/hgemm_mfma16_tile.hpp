@@ -54,7 +54,11 @@ struct Hgemm16Shape {
                   "fragment reads address stage, k-block and row block through the 16-bit offset field");
 };
 
-template <class S, bool HAS_C>
+// ABLATE != 0 builds measurement variants that leave work out of the K walk and produce no meaningful result (the cost of
+// each part of the kernel is the difference between two of them): bit 0 = the K walk issues no DMA loads (LDS keeps
+// the first two K steps), bit 1 = it issues no LDS reads (the registers keep the first fragments), bit 2 = the result
+// is not stored.  Only decx_hip_hgemm_probe launches them.
+template <class S, bool HAS_C, int ABLATE = 0>
 __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __restrict__ A, int lda,
                                                              const _Float16* __restrict__ B, int ldb, const _Float16* Cin,
                                                              int ldc, _Float16* D, int ldd, int M, int N, int K, int tiles_m,
@@ -106,8 +110,9 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
     const int full_steps = K / BK;
     int steps_fetched = 0;
     const size_t b_step = (size_t)BK * ldb;
-    auto issue_one = [&](auto stage_tag, auto j_tag) {
+    auto issue_one = [&](auto stage_tag, auto j_tag, auto in_walk_tag) {
         constexpr int STG = decltype(stage_tag)::value, J = decltype(j_tag)::value;
+        if constexpr ((ABLATE & 1) && decltype(in_walk_tag)::value) return;
         if constexpr (J < S::A_LOADS) {
             dma_load16(a_base, a_off[J], lds_base + (uint32_t)(STG * A_BYTES) + (uint32_t)(wave * S::A_LOADS + J) * 1024u);
         } else {
@@ -196,7 +201,8 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
             static_assert(NR <= BLK, "one read per MFMA slot");
             static_for<0, BLK>([&](auto i_tag) {
                 constexpr int I = decltype(i_tag)::value;
-                if constexpr (I < UM) {
+                if constexpr (ABLATE & 2) {
+                } else if constexpr (I < UM) {
                     read_a(std::integral_constant<int, NU & 1>{}, i_tag, Stg{}, std::integral_constant<int, NKB>{},
                            std::integral_constant<int, NH * UM + I>{});
                 } else if constexpr (I < NR) {
@@ -218,10 +224,10 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
         DECX_PIN();
         static_for<0, SLOTS>([&](auto i_tag) {
             constexpr int I = decltype(i_tag)::value;
-            static_for<(I * S::LOADS) / SLOTS, ((I + 1) * S::LOADS) / SLOTS>([&](auto j_tag) { issue_one(Stg{}, j_tag); });
+            static_for<(I * S::LOADS) / SLOTS, ((I + 1) * S::LOADS) / SLOTS>([&](auto j_tag) { issue_one(Stg{}, j_tag, std::true_type{}); });
             // two reads per slot until they are all out: the next step's first MFMAs follow closely
             constexpr int R0 = 2 * I < FIRST_READS ? 2 * I : FIRST_READS, R1 = 2 * I + 2 < FIRST_READS ? 2 * I + 2 : FIRST_READS;
-            static_for<R0, R1>([&](auto r_tag) { read_first(Next{}, r_tag); });
+            if constexpr (!(ABLATE & 2)) static_for<R0, R1>([&](auto r_tag) { read_first(Next{}, r_tag); });
             mfma_one(Last{}, std::integral_constant<int, PRE + I>{});
             DECX_PIN();
         });
@@ -233,18 +239,24 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
         // an odd number of steps starts in stage 1, so that the walk below always ends with the pair (stage 0, stage 1)
         const bool odd = full_steps & 1;
         if (odd) {
-            static_for<0, S::LOADS>([&](auto j) { issue_one(I1{}, j); });
-            static_for<0, S::LOADS>([&](auto j) { issue_one(I0{}, j); });
+            static_for<0, S::LOADS>([&](auto j) { issue_one(I1{}, j, std::false_type{}); });
+            static_for<0, S::LOADS>([&](auto j) { issue_one(I0{}, j, std::false_type{}); });
             wait_dma_then_barrier<0>();
             static_for<0, FIRST_READS>([&](auto r) { read_first(I1{}, r); });
             DECX_PIN();
             k_step(I1{});
         } else {
-            static_for<0, S::LOADS>([&](auto j) { issue_one(I0{}, j); });
-            static_for<0, S::LOADS>([&](auto j) { issue_one(I1{}, j); });
+            static_for<0, S::LOADS>([&](auto j) { issue_one(I0{}, j, std::false_type{}); });
+            static_for<0, S::LOADS>([&](auto j) { issue_one(I1{}, j, std::false_type{}); });
             wait_dma_then_barrier<0>();
             static_for<0, FIRST_READS>([&](auto r) { read_first(I0{}, r); });
             DECX_PIN();
+        }
+        if constexpr (ABLATE & 2) {                              // the sets the walk would have filled
+#pragma unroll
+            for (int x = 0; x < UM; ++x) af[1][x] = af[0][x];
+#pragma unroll
+            for (int x = 0; x < NI; ++x) blo[1][x] = bhi[0][x], bhi[1][x] = blo[0][x];
         }
         for (int t = odd ? 1 : 0; t < full_steps; t += 2) {
             k_step(I0{});
@@ -348,6 +360,7 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
         const u32x4 v = *reinterpret_cast<const u32x4*>(park + row * ROW_BYTES + ((piece ^ (row & 7)) << 4));
         const int m = m_wave + row, n = n_wave + 8 * piece;
         _Float16* dp = D + (size_t)m * ldd + n;
+        if ((ABLATE & 4) && K >= 0) continue;                    // (a condition the compiler cannot fold, so the sums stay live)
         if (whole) {
             *reinterpret_cast<u32x4*>(dp) = v;
         } else if (m < M) {

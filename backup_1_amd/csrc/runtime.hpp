@@ -72,6 +72,8 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
                  int flag, const float* bias = nullptr, bool relu = false);
 int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                   int ldd, int M, int N, int K, const Batch& batch);
+// measurement variants of the large fp16 tile with parts of its K walk left out (no meaningful result)
+int hgemm_probe_enqueue(int ablate, const uint16_t* A, int lda, const uint16_t* B, int ldb, uint16_t* D, int ldd, int M, int N, int K);
 // the K-range route of hgemm_enqueue on the library's static device workspace (no allocation); splits <= 0: automatic
 int hgemm_splitk_static_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
                                 uint16_t* D, int ldd, int M, int N, int K, int splits);

@@ -145,6 +145,30 @@ def bench_hgemm(capi, workloads, n, steps, warmup, seed, shape=None, verify_rows
     return out
 
 
+def bench_fp16_ladder(capi, workloads, steps, warmup, n=8192):
+    """The large fp16 tile kernel with parts of its K walk left out (decx_hip_hgemm_probe), on uniform[-1,1] operands
+    and on all-zero ones: what each part costs, and what the operand values cost (the same instructions on zeros draw
+    less power, so the chip clocks higher).  Every rung issues the same matrix instructions: 2 n^3 flop."""
+    A = workloads.uniform_pm1((n, n), 5).astype(np.float16).view(np.uint16)
+    B = workloads.uniform_pm1((n, n), 6).astype(np.float16).view(np.uint16)
+    dA, dB = capi.DeviceBuffer.from_numpy(A), capi.DeviceBuffer.from_numpy(B)
+    dZ = capi.DeviceBuffer(n * n * 2)
+    dZ.fill(0)
+    dD = capi.DeviceBuffer(n * n * 2)
+    rungs = [(7, "matrix instructions only"), (5, "+ LDS fragment reads"), (4, "+ global->LDS loads (whole K walk, no stores)"),
+             (0, "whole kernel")]
+    out = []
+    for ablate, what in rungs:
+        row = {"ablate": ablate, "what": what}
+        for tag, a, b in (("uniform", dA, dB), ("zeros", dZ, dZ)):
+            launch = lambda: capi.check(capi.lib().decx_hip_hgemm_probe(ablate, a.ptr, n, b.ptr, n, dD.ptr, n, n, n, n))
+            wall, ev = time_launches(capi, launch, steps, warmup)
+            row["tflops_" + tag] = round(2.0 * n ** 3 / (ev * 1e-3) / 1e12, 1)
+            row["ms_" + tag] = round(ev, 4)
+        out.append(row)
+    return out
+
+
 def bench_conv(capi, workloads, steps, warmup, H=224, W=224, C=64, N=128):
     kh = kw = 3
     src, filt = workloads.conv_case(H=H, W=W, C=C, N=N)
@@ -339,7 +363,7 @@ def main():
     ap.add_argument("--sgemm-variant", type=int, default=0, help="force a fp32 tile shape (0 = automatic)")
     ap.add_argument("--hgemm-variant", type=int, default=0, help="force a fp16 tile shape (0 = automatic)")
     ap.add_argument("--no-verify", action="store_true", help="skip the post-run comparison of sampled rows with the oracle")
-    ap.add_argument("--only", default="", help="comma list of: headline,fp16,sq4096,small,ragged,conv,relu,host,cpu (default all)")
+    ap.add_argument("--only", default="", help="comma list of: headline,fp16,sq4096,small,ragged,conv,relu,host,cpu (default all); extra: ladder, copy")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); --gpus %d is not supported. "
@@ -379,6 +403,10 @@ def main():
             also["fp16_8192_f32acc"].update({"verified": r["verified"], "verified_rows": r["verified_rows"],
                                              "max_rel_err_vs_fp64": float("%.3e" % r["max_rel_err"]), "tolerance": 2e-3})
         log("fp16 8192^3: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+    if "ladder" in only:
+        also["fp16_8192_ladder"] = bench_fp16_ladder(capi, workloads, side_steps, side_warmup)
+        for row in also["fp16_8192_ladder"]:
+            log("fp16 ladder, %-48s %7.1f TFLOP/s on uniform[-1,1], %7.1f on zeros" % (row["what"], row["tflops_uniform"], row["tflops_zeros"]))
     if want("sq4096"):
         r = bench_sgemm(capi, workloads, 4096, 4096, 4096, side_steps, side_warmup, 1234)
         also["fp32_4096"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
