@@ -352,8 +352,7 @@ static __global__ __launch_bounds__(256) void hconv_split_finish_kernel(const fl
     const size_t total = (size_t)M * N;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const int m = (int)(i / N), n = (int)(i - (size_t)m * N);
-        float v = partial[i];
-        for (int s = 1; s < planes; ++s) v += partial[(size_t)s * plane + i];
+        float v = ordered_plane_sum(partial, planes, plane, i);
         if (out.bias != nullptr) v += (float)out.bias[n];
         if (out.relu) v = relu_by_sign(v);
         out.dst[(size_t)(m / out.Wout) * out.row_stride + (size_t)(m % out.Wout) * out.dpitch + n] = (_Float16)v;

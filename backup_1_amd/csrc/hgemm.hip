@@ -24,6 +24,9 @@ namespace decx_hip {
 //  15: 256x256x64, 2x4 waves of 128x64 on v_mfma_f32_16x16x32_f16, 2-stage LDS-DMA pipeline, result written through LDS in
 //      16-byte pieces (hgemm_mfma16_tile.hpp) -- the default for large problems: 8 % faster than 7 at 8192^3, because
 //      this instruction draws less power per flop on real-valued data
+//  16: as 15 with 4 LDS stages of 32 k instead of 2 of 64 (three K steps in flight instead of one): measured equal to 15 at
+//      8192^3 (1381 vs 1396 TFLOP/s), and so were 5 stages and a refill spread over the following step -- the wait for the
+//      loads is not what the kernel loses time to; kept as the second instantiation of the kernel's stage arithmetic
 //  11: split-K on shape 8 through an fp32 workspace (hgemm_splitk_enqueue) -- few tiles and a long K
 // and, for the fp16 convolution only: 12 keeps its register-staged kernels, 13 takes its LDS-DMA kernel for any image
 // whose channel pitch allows it, 14 its tap-row kernel; each switches its split over K off (experiments and tests)
@@ -38,11 +41,12 @@ typedef HgemmDmaShape<128, 128, 64, 2, 2, 2> HShapeDmaSmall;     // 4 waves, 64x
 typedef HgemmDmaShape<128, 128, 64, 2, 2, 3> HShapeDmaSmall3;
 typedef HgemmDmaShape<256, 128, 64, 2, 2, 2> HShapeDmaTall;      // 4 waves, 128x64 each
 
-typedef Hgemm16Shape<256, 256, 2, 4> HShape16;                   // 8 waves, 128x64 each, 16x16x32 MFMAs
+typedef Hgemm16Shape<256, 256, 64, 2, 4, 2> HShape16;            // 8 waves, 128x64 each, 16x16x32 MFMAs, 2 stages of 64 k
+typedef Hgemm16Shape<256, 256, 32, 2, 4, 4> HShape16K32S4;       // 4 stages of 32 k
 
+template <class S>
 int launch_hgemm_mfma16(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                         int ldd, int M, int N, int K, const Batch& batch) {
-    typedef HShape16 S;
     auto kern = Cin ? hgemm_mfma16_kernel<S, true> : hgemm_mfma16_kernel<S, false>;
     static bool attr_done = false;
     if (!attr_done) {
@@ -161,7 +165,9 @@ static SplitPlan plan_hgemm_split(int K, int splits) {
 static int auto_hgemm_splits(int M, int N, int K) {
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     const long tiles = (long)cdiv(M, 128) * cdiv(N, 128);
-    long splits = (2 * cus + tiles - 1) / tiles;
+    // ranges for two workgroups per CU with atomics; one per CU when every range writes and the finishing kernel reads a
+    // plane of its own (measured: 64x65536x1024 49 us with 32 ranges, 52 with 64; 128x16384x2048 38 with 16, 42 with 32)
+    long splits = ((g_rt.splitk_atomic ? 2 : 1) * cus + tiles - 1) / tiles;
     if (splits > K / 512) splits = K / 512;                        // at least 8 K steps per range
     if (splits < 2 || (size_t)M * N > ((size_t)1 << 26)) return 0;
     const double t_whole = 4.0 + 0.0067 * K * (double)((tiles + cus - 1) / cus);
@@ -226,7 +232,7 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
     int variant = g_rt.hgemm_variant;
     {
         // few 128x128 tiles and a long K: split K (variant 11 forces it, any other fixed variant switches it off)
-        if (batch.count == 1 && (variant < 1 || variant > 10) && variant != 15) {
+        if (batch.count == 1 && (variant < 1 || variant > 10) && (variant < 15 || variant > 16)) {
             int splits = auto_hgemm_splits(M, N, K);
             if (variant == 11 && splits == 0 && K >= 1024 && (size_t)M * N <= ((size_t)1 << 26)) {
                 const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
@@ -239,7 +245,7 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
         }
         if (variant == 11) variant = 0;
     }
-    if (variant < 1 || (variant > 10 && variant != 15)) {
+    if (variant < 1 || (variant > 10 && (variant < 15 || variant > 16))) {
         // same cost model as the fp32 picker: rounds of tiles per CU x tile area / measured shape efficiency
         const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
         const long big = (long)cdiv(M, 256) * cdiv(N, 256) * batch.count, small = (long)cdiv(M, 128) * cdiv(N, 128) * batch.count;
@@ -248,7 +254,8 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
         // the small tile with three LDS stages holds one workgroup per CU: only worth it when there is at most one to hold
         variant = cost_big <= cost_small ? 15 : (small <= cus ? 9 : 8);
     }
-    if (variant == 15) return launch_hgemm_mfma16(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 15) return launch_hgemm_mfma16<HShape16>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 16) return launch_hgemm_mfma16<HShape16K32S4>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     if (variant == 3) return launch_hgemm_dma_tile<HShapeDma>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     if (variant == 4) return launch_hgemm_dma_tile<HShapeDma64>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     if (variant == 5) return launch_hgemm_dma_tile<HShapeDma5>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);

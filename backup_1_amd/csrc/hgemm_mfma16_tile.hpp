@@ -31,9 +31,29 @@ __device__ __forceinline__ int b16_unit_slot(int k, int u, int UB) {
     return k * UB + (u ^ (((k & 3) << 2) | (((k >> 3) & 1) << 1)));
 }
 
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_>
+// A unit (m, q) of a stage with 4 units per row (BK = 32): the unit index rotated by 2 (m / 4), which keeps the fragment
+// reads of 16-row blocks (lane group lg takes unit lg of rows m .. m + 15) on distinct banks in every service phase of a
+// 16-byte LDS read.  With 8 units per row (BK = 64) the XOR swizzle of hgemm_tile.hpp already does.
+__device__ __forceinline__ int a16_unit_slot(int m, int q, int UA) {
+    return UA == 4 ? m * 4 + ((q + 2 * (m >> 2)) & 3) : a_unit_slot(m, q, UA);
+}
+// the unit that lands in slot s of row m (inverse of the above, for the global side of the DMA)
+__device__ __forceinline__ int a16_unit_in_slot(int m, int s, int UA) {
+    return UA == 4 ? ((s - 2 * (m >> 2)) & 3) : (s ^ ((m / (16 / UA)) % UA));
+}
+
+// dma_load16 with a tag in the instruction text.  Two branches of a dispatch that issue the same loads into different
+// stages are otherwise merged by the compiler into one sequence whose operands are selected per branch -- in vector
+// registers, which the scalar operands of this instruction do not accept.
+template <int TAG>
+__device__ __forceinline__ void dma_load16_tagged(const void* sbase, uint32_t lane_off, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 ; load %3"
+                 : : "v"(lane_off), "s"(sbase), "s"(lds_base), "n"(TAG) : "memory", "m0");
+}
+
+template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_>
 struct Hgemm16Shape {
-    static constexpr int BM = BM_, BN = BN_, BK = 64, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;
     static constexpr int NWAVES = WAVES_M * WAVES_N, NT = NWAVES * kWave;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
     static constexpr int MI = WM / 16, NI = WN / 16;            // 16 x 16 accumulator blocks of a wave
@@ -42,16 +62,24 @@ struct Hgemm16Shape {
     static constexpr int UA = BK / 8, UB = BN / 8;              // 16-byte units per LDS row
     static constexpr int A_UNITS = BM * UA, B_UNITS = BK * UB;
     static constexpr int A_BYTES = A_UNITS * 16, B_BYTES = B_UNITS * 16;
-    static constexpr int STAGES = 2;
     static constexpr size_t LDS_BYTES = (size_t)STAGES * (A_BYTES + B_BYTES);
     static constexpr int A_LOADS = A_UNITS / 64 / NWAVES, B_LOADS = B_UNITS / 64 / NWAVES, LOADS = A_LOADS + B_LOADS;
     static constexpr int A_PASSES = A_UNITS / NT, B_PASSES = B_UNITS / NT;
-    static_assert(MI % MH == 0 && UNITS % 2 == 0 && KS % 2 == 0, "fragment sets must line up across units and K steps");
-    static_assert(UA == 8 && UB >= 16 && (UB & (UB - 1)) == 0, "swizzles assume 8 units per A row and >= 16 per B row");
+    static_assert(BK == 32 || BK == 64, "one or two k-blocks of 32 per K step");
+    static_assert(MI % MH == 0 && UNITS % 2 == 0, "fragment sets of A alternate by unit");
+    // fragment sets of B alternate by k-block, so the unrolled walk covers the stages once or (odd count of k-blocks) twice
+    static constexpr int WALK = (STAGES * KS) % 2 == 0 ? STAGES : 2 * STAGES;
+    static_assert(STAGES >= 2, "need at least double buffering");
+    static_assert(UB >= 16 && (UB & (UB - 1)) == 0, "the B swizzle needs >= 16 units per row");
     static_assert(A_UNITS % (64 * NWAVES) == 0 && B_UNITS % (64 * NWAVES) == 0, "DMA chunks must divide over the waves");
     static_assert((size_t)NWAVES * WM * WN * 2 <= LDS_BYTES, "the epilogue parks every wave's piece in LDS");
-    static_assert((STAGES - 1) * A_BYTES + (MI - 1) * 16 * UA * 16 < 65536 && (STAGES - 1) * B_BYTES + (32 * (KS - 1) + 4) * UB * 16 < 65536,
-                  "fragment reads address stage, k-block and row block through the 16-bit offset field");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS of a CU");
+    // fragment reads address stage, k-block and row block through the 16-bit offset field, from one of two per-lane bases
+    // (the second one HI_STAGE stages further on) when the stages of an operand span more than 64 KB
+    static constexpr int HI_STAGE = (STAGES + 1) / 2;
+    static_assert((HI_STAGE - 1) * A_BYTES + (MI - 1) * 16 * UA * 16 < 65536 && (HI_STAGE - 1) * B_BYTES + (32 * (KS - 1) + 4) * UB * 16 < 65536,
+                  "offsets from a base must fit 16 bits");
+    static_assert(LOADS * (STAGES - 2) <= 63, "vmcnt is a 6-bit counter");
 };
 
 // ABLATE != 0 builds measurement variants that leave work out of the K walk and produce no meaningful result (the cost of
@@ -65,14 +93,14 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
                                                              int tiles_n, int group_m, size_t a_batch_stride,
                                                              size_t b_batch_stride, size_t c_batch_stride, size_t d_batch_stride) {
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, NT = S::NT, UA = S::UA, UB = S::UB, MI = S::MI, NI = S::NI;
-    constexpr int UM = S::UM, MH = S::MH, KS = S::KS, UNITS = S::UNITS;
+    constexpr int UM = S::UM, MH = S::MH, KS = S::KS, UNITS = S::UNITS, STAGES = S::STAGES, WALK = S::WALK;
     constexpr int A_BYTES = S::A_BYTES, B_BYTES = S::B_BYTES;
     constexpr int BLK = UM * NI;                                // MFMAs per unit
     A += (size_t)blockIdx.y * a_batch_stride;
     B += (size_t)blockIdx.y * b_batch_stride;
     if (HAS_C) Cin += (size_t)blockIdx.y * c_batch_stride;
     D += (size_t)blockIdx.y * d_batch_stride;
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];   // [A stage 0][A stage 1][B stage 0][B stage 1]
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];   // [A stages][B stages]
     const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds_raw;
 
     const TileCoord tc = xcd_grouped_tile(blockIdx.x, tiles_m, tiles_n, group_m);
@@ -89,9 +117,9 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
     uint32_t a_off[S::A_LOADS], b_off[S::B_LOADS];
 #pragma unroll
     for (int j = 0; j < S::A_LOADS; ++j) {
-        const int chunk = wave * S::A_LOADS + j;                // 64 units = 8 rows
+        const int chunk = wave * S::A_LOADS + j;                // 64 units = 64 / UA rows
         const int r = chunk * (64 / UA) + lane / UA;
-        const int q = (lane % UA) ^ ((r / (16 / UA)) % UA);     // the unit whose swizzled slot is this lane
+        const int q = a16_unit_in_slot(r, lane % UA, UA);       // the unit whose swizzled slot is this lane
         int m = bm0 + r;
         if (m >= M) m = M - 1;                                  // rows past the end are computed and never stored
         a_off[j] = (uint32_t)(((size_t)(m - m_first) * lda + 8 * q) * sizeof(_Float16));
@@ -104,9 +132,9 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
         const int col = clamp_group_col(bn0 + 8 * u, N, 8);     // stay inside the operand; such columns are never stored
         b_off[j] = (uint32_t)(((size_t)kr * ldb + col) * sizeof(_Float16));
     }
-    // Every K step fetches the step two ahead of it into the stage it leaves, also the last two, which have nothing left
-    // to fetch: their loads repeat the last whole step (the bases stop there) into a stage nobody reads again.  All
-    // steps are then the same code with the same wait counts, at the price of two redundant step loads per tile.
+    // Every K step fetches the step STAGES ahead of it into the stage it leaves, also the last STAGES, which have nothing
+    // left to fetch: their loads repeat the last whole step (the bases stop there) into stages nobody reads again.  All
+    // steps are then the same code with the same wait counts, at the price of STAGES redundant step loads per tile.
     const int full_steps = K / BK;
     int steps_fetched = 0;
     const size_t b_step = (size_t)BK * ldb;
@@ -114,10 +142,10 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
         constexpr int STG = decltype(stage_tag)::value, J = decltype(j_tag)::value;
         if constexpr ((ABLATE & 1) && decltype(in_walk_tag)::value) return;
         if constexpr (J < S::A_LOADS) {
-            dma_load16(a_base, a_off[J], lds_base + (uint32_t)(STG * A_BYTES) + (uint32_t)(wave * S::A_LOADS + J) * 1024u);
+            dma_load16_tagged<STG * 64 + J>(a_base, a_off[J], lds_base + (uint32_t)(STG * A_BYTES) + (uint32_t)(wave * S::A_LOADS + J) * 1024u);
         } else {
             constexpr int JB = J - S::A_LOADS;
-            dma_load16(b_base, b_off[JB], lds_base + (uint32_t)(2 * A_BYTES + STG * B_BYTES) + (uint32_t)(wave * S::B_LOADS + JB) * 1024u);
+            dma_load16_tagged<STG * 64 + J>(b_base, b_off[JB], lds_base + (uint32_t)(STAGES * A_BYTES + STG * B_BYTES) + (uint32_t)(wave * S::B_LOADS + JB) * 1024u);
         }
         if constexpr (J == S::LOADS - 1) {
             ++steps_fetched;
@@ -138,61 +166,80 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
     //   A fragment of row block rb, k-block kb : lane (lg, li) reads the 8 halves k = 32 kb + 8 lg .. + 7 of row 16 rb + li
     //   B fragment of column block ni, k-block kb: two transposing reads of 4 rows each; lane (lg, li) supplies the address
     //     of row 32 kb + 8 lg + li / 4 (+ 4), columns 16 ni + 4 (li % 4) .. + 3, and receives column 16 ni + li of 4 rows
-    uint32_t a_rd[KS], b_rd[NI];
+    constexpr int HI = S::HI_STAGE;
+    constexpr bool TWO_BASES = (STAGES - 1) * A_BYTES + (MI - 1) * 16 * UA * 16 >= 65536 || (STAGES - 1) * B_BYTES + (32 * (KS - 1) + 4) * UB * 16 >= 65536;
+    uint32_t a_rd[KS], b_rd[NI], a_rd_hi[KS], b_rd_hi[NI];
 #pragma unroll
-    for (int kb = 0; kb < KS; ++kb) a_rd[kb] = (uint32_t)a_unit_slot(wm0 + li, 4 * kb + lg, UA) * 16u;
+    for (int kb = 0; kb < KS; ++kb) {
+        a_rd[kb] = (uint32_t)a16_unit_slot(wm0 + li, 4 * kb + lg, UA) * 16u;
+        a_rd_hi[kb] = a_rd[kb] + (uint32_t)(HI * A_BYTES);
+    }
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni) {
         const int col = wn0 + 16 * ni + 4 * (li & 3);
-        b_rd[ni] = (uint32_t)(2 * A_BYTES) + (uint32_t)b16_unit_slot(8 * lg + (li >> 2), col >> 3, UB) * 16u + (uint32_t)(col & 7) * 2u;
+        b_rd[ni] = (uint32_t)(STAGES * A_BYTES) + (uint32_t)b16_unit_slot(8 * lg + (li >> 2), col >> 3, UB) * 16u + (uint32_t)(col & 7) * 2u;
+        b_rd_hi[ni] = b_rd[ni] + (uint32_t)(HI * B_BYTES);
     }
-    static_assert(16 % (16 / UA) == 0 && (16 / (16 / UA)) % UA == 0, "row blocks of 16 must not change the A swizzle");
+    static_assert(UA == 4 || (16 % (16 / UA) == 0 && (16 / (16 / UA)) % UA == 0), "row blocks of 16 must not change the A swizzle");
     typedef short i16x8 __attribute__((ext_vector_type(8)));
     f16x8 af[2][UM];                                            // by unit parity
-    i16x4 blo[2][NI], bhi[2][NI];                               // by k-block parity
+    i16x4 blo[2][NI], bhi[2][NI];                               // by the parity of the k-block counted over the whole walk
+    if constexpr (ABLATE & 2) {
+#pragma unroll
+        for (int x = 0; x < NI; ++x) blo[0][x] = blo[1][x] = bhi[0][x] = bhi[1][x] = i16x4{0, 0, 0, 0};
+    }
     auto read_a = [&](auto set_tag, auto slot_tag, auto stage_tag, auto kb_tag, auto rb_tag) {
-        constexpr int OFF = decltype(stage_tag)::value * A_BYTES + decltype(rb_tag)::value * (16 * UA * 16);
-        af[decltype(set_tag)::value][decltype(slot_tag)::value] =
-            __builtin_bit_cast(f16x8, *reinterpret_cast<const u32x4*>(lds_raw + a_rd[decltype(kb_tag)::value] + OFF));
+        constexpr int STG = decltype(stage_tag)::value;
+        constexpr bool HIGH = TWO_BASES && STG >= HI;
+        constexpr int OFF = (HIGH ? STG - HI : STG) * A_BYTES + decltype(rb_tag)::value * (16 * UA * 16);
+        const uint32_t base = HIGH ? a_rd_hi[decltype(kb_tag)::value] : a_rd[decltype(kb_tag)::value];
+        af[decltype(set_tag)::value][decltype(slot_tag)::value] = __builtin_bit_cast(f16x8, *reinterpret_cast<const u32x4*>(lds_raw + base + OFF));
     };
     auto read_b = [&](auto set_tag, auto stage_tag, auto kb_tag, auto ni_tag, auto hi_tag) {
-        constexpr int SET = decltype(set_tag)::value, NIX = decltype(ni_tag)::value, HI = decltype(hi_tag)::value;
-        constexpr int OFF = decltype(stage_tag)::value * B_BYTES + (32 * decltype(kb_tag)::value + 4 * HI) * (UB * 16);
-        const i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (__attribute__((address_space(3))) i16x4*)(lds_raw + b_rd[NIX] + OFF));
-        if constexpr (HI) bhi[SET][NIX] = v;
+        constexpr int SET = decltype(set_tag)::value, NIX = decltype(ni_tag)::value, HALF = decltype(hi_tag)::value;
+        constexpr int STG = decltype(stage_tag)::value;
+        constexpr bool HIGH = TWO_BASES && STG >= HI;
+        constexpr int OFF = (HIGH ? STG - HI : STG) * B_BYTES + (32 * decltype(kb_tag)::value + 4 * HALF) * (UB * 16);
+        const uint32_t base = HIGH ? b_rd_hi[NIX] : b_rd[NIX];
+        const i16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4*)(lds_raw + base + OFF));
+        if constexpr (HALF) bhi[SET][NIX] = v;
         else blo[SET][NIX] = v;
     };
-    // read number R of the fragments a K step starts with (unit 0: row blocks 0 .. UM-1, k-block 0), in the order its
-    // first MFMAs need them: A block 0, all of B, the other A blocks
+    // The walk is unrolled over WALK steps; step V of it works in stage V % STAGES, and k-block KB of it uses B fragment set
+#define DECX_BSET(V, KB) (((V) * KS + (KB)) & 1)
+    // read number R of the fragments a K step in stage STG starts with (unit 0: row blocks 0 .. UM-1, k-block 0), in the
+    // order its first MFMAs need them: A block 0, all of B, the other A blocks
     constexpr int FIRST_READS = UM + 2 * NI;
-    auto read_first = [&](auto stage_tag, auto r_tag) {
-        constexpr int R = decltype(r_tag)::value;
+    auto read_first = [&](auto v_tag, auto r_tag) {
+        constexpr int R = decltype(r_tag)::value, V = decltype(v_tag)::value;
         typedef std::integral_constant<int, 0> I0;
-        if constexpr (R == 0) read_a(I0{}, I0{}, stage_tag, I0{}, I0{});
+        typedef std::integral_constant<int, V % STAGES> Stg;
+        typedef std::integral_constant<int, DECX_BSET(V, 0)> BSet;
+        if constexpr (R == 0) read_a(I0{}, I0{}, Stg{}, I0{}, I0{});
         else if constexpr (R <= 2 * NI)
-            read_b(I0{}, stage_tag, I0{}, std::integral_constant<int, (R - 1) / 2>{}, std::integral_constant<int, (R - 1) % 2>{});
-        else read_a(I0{}, std::integral_constant<int, R - 2 * NI>{}, stage_tag, I0{}, std::integral_constant<int, R - 2 * NI>{});
+            read_b(BSet{}, Stg{}, I0{}, std::integral_constant<int, (R - 1) / 2>{}, std::integral_constant<int, (R - 1) % 2>{});
+        else read_a(I0{}, std::integral_constant<int, R - 2 * NI>{}, Stg{}, I0{}, std::integral_constant<int, R - 2 * NI>{});
     };
-    // MFMA number I of unit U: row block (U % MH) * UM + I / NI, column block I % NI
-    auto mfma_one = [&](auto u_tag, auto i_tag) {
+    // MFMA number I of unit U of walk step V: row block (U % MH) * UM + I / NI, column block I % NI
+    auto mfma_one = [&](auto v_tag, auto u_tag, auto i_tag) {
         constexpr int U = decltype(u_tag)::value, I = decltype(i_tag)::value;
-        constexpr int KB = U / MH, MIX = (U % MH) * UM + I / NI, NIX = I % NI;
-        const i16x4 lo = blo[KB & 1][NIX], hi = bhi[KB & 1][NIX];
+        constexpr int KB = U / MH, MIX = (U % MH) * UM + I / NI, NIX = I % NI, BS = DECX_BSET(decltype(v_tag)::value, KB);
+        const i16x4 lo = blo[BS][NIX], hi = bhi[BS][NIX];
         const i16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         acc[MIX][NIX] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, both), af[U & 1][I / NI], acc[MIX][NIX], 0, 0, 0);
     };
 #define DECX_PIN() __builtin_amdgcn_sched_barrier(0)
 
-    // One K step from stage STG.  On entry af[0] / b*[0] hold the fragments of unit 0; on exit those of the next step's.
-    // Units 0 .. UNITS-2: the first MFMAs each carry one LDS read of the next unit's A fragments and of this unit's share
-    // of the next k-block's B fragments.  Last unit: a few MFMAs, then wait for the next step's data + barrier -- nobody
-    // reads this stage any more -- and between the remaining MFMAs the DMA refill of this stage and the first fragments
-    // of the next step from the other stage.
-    auto k_step = [&](auto stg_tag) {
-        constexpr int STG = decltype(stg_tag)::value;
+    // One K step from stage STG.  On entry af[0] and the B set of its first k-block hold the fragments of unit 0; on exit
+    // those of the next step.  Units 0 .. UNITS-2: the first MFMAs each carry one LDS read of the next unit's A fragments
+    // and of this unit's share of the next k-block's B fragments.  Last unit: a few MFMAs, then wait for the next step's
+    // data + barrier -- nobody reads this stage any more -- and between the remaining MFMAs the DMA refill of this stage
+    // (the loads of the STAGES - 2 steps in between may still be in flight at the wait) and the first fragments of the
+    // next step from the next stage.
+    auto k_step = [&](auto v_tag) {
+        constexpr int V = decltype(v_tag)::value, STG = V % STAGES;
         typedef std::integral_constant<int, STG> Stg;
-        typedef std::integral_constant<int, STG ^ 1> Next;
+        typedef std::integral_constant<int, (V + 1) % WALK> Next;
         static_for<0, UNITS - 1>([&](auto u_tag) {
             constexpr int U = decltype(u_tag)::value, KB = U / MH, H = U % MH;
             constexpr int NU = U + 1, NKB = NU / MH, NH = NU % MH;
@@ -207,20 +254,22 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
                            std::integral_constant<int, NH * UM + I>{});
                 } else if constexpr (I < NR) {
                     constexpr int RB = H * NB + (I - UM);
-                    read_b(std::integral_constant<int, (KB + 1) & 1>{}, Stg{}, std::integral_constant<int, KB + 1>{},
+                    read_b(std::integral_constant<int, DECX_BSET(V, KB + 1)>{}, Stg{}, std::integral_constant<int, KB + 1>{},
                            std::integral_constant<int, RB / 2>{}, std::integral_constant<int, RB % 2>{});
                 }
-                mfma_one(u_tag, i_tag);
+                mfma_one(v_tag, u_tag, i_tag);
                 DECX_PIN();
             });
         });
         typedef std::integral_constant<int, UNITS - 1> Last;
         constexpr int PRE = BLK / 4, SLOTS = BLK - PRE;
         static_for<0, PRE>([&](auto i_tag) {
-            mfma_one(Last{}, i_tag);
+            mfma_one(v_tag, Last{}, i_tag);
             DECX_PIN();
         });
-        wait_dma_then_barrier<0>();
+        // loads of this wave that may still be in flight when it meets the others: those of the STAGES - 2 steps after the next
+        constexpr int WAITN = (ABLATE & 1) ? 0 : S::LOADS * (STAGES - 2);
+        wait_dma_then_barrier<WAITN>();
         DECX_PIN();
         static_for<0, SLOTS>([&](auto i_tag) {
             constexpr int I = decltype(i_tag)::value;
@@ -228,39 +277,44 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
             // two reads per slot until they are all out: the next step's first MFMAs follow closely
             constexpr int R0 = 2 * I < FIRST_READS ? 2 * I : FIRST_READS, R1 = 2 * I + 2 < FIRST_READS ? 2 * I + 2 : FIRST_READS;
             if constexpr (!(ABLATE & 2)) static_for<R0, R1>([&](auto r_tag) { read_first(Next{}, r_tag); });
-            mfma_one(Last{}, std::integral_constant<int, PRE + I>{});
+            mfma_one(v_tag, Last{}, std::integral_constant<int, PRE + I>{});
             DECX_PIN();
         });
     };
 
     typedef std::integral_constant<int, 0> I0;
-    typedef std::integral_constant<int, 1> I1;
     if (full_steps > 0) {
-        // an odd number of steps starts in stage 1, so that the walk below always ends with the pair (stage 0, stage 1)
-        const bool odd = full_steps & 1;
-        if (odd) {
-            static_for<0, S::LOADS>([&](auto j) { issue_one(I1{}, j, std::false_type{}); });
-            static_for<0, S::LOADS>([&](auto j) { issue_one(I0{}, j, std::false_type{}); });
-            wait_dma_then_barrier<0>();
-            static_for<0, FIRST_READS>([&](auto r) { read_first(I1{}, r); });
-            DECX_PIN();
-            k_step(I1{});
-        } else {
-            static_for<0, S::LOADS>([&](auto j) { issue_one(I0{}, j, std::false_type{}); });
-            static_for<0, S::LOADS>([&](auto j) { issue_one(I1{}, j, std::false_type{}); });
-            wait_dma_then_barrier<0>();
-            static_for<0, FIRST_READS>([&](auto r) { read_first(I0{}, r); });
-            DECX_PIN();
-        }
+        // The walk starts at walk step `first` such that it ends with step WALK - 1: a first pass that begins at `first`,
+        // then whole passes.  The prologue fills all stages, K step j into stage (first + j) % STAGES.
+        const int first = (WALK - full_steps % WALK) % WALK;
+        static_for<0, WALK>([&](auto v0) {
+            if (first == decltype(v0)::value) {
+                static_for<0, STAGES>([&](auto j) {
+                    typedef std::integral_constant<int, (decltype(v0)::value + decltype(j)::value) % STAGES> Stg;
+                    static_for<0, S::LOADS>([&](auto l) { issue_one(Stg{}, l, std::false_type{}); });
+                });
+                wait_dma_then_barrier<S::LOADS*(STAGES - 1)>();          // step 0 has landed
+                static_for<0, FIRST_READS>([&](auto r) { read_first(v0, r); });
+            }
+        });
+        DECX_PIN();
         if constexpr (ABLATE & 2) {                              // the sets the walk would have filled
 #pragma unroll
             for (int x = 0; x < UM; ++x) af[1][x] = af[0][x];
 #pragma unroll
-            for (int x = 0; x < NI; ++x) blo[1][x] = bhi[0][x], bhi[1][x] = blo[0][x];
+            for (int x = 0; x < NI; ++x) {
+                const i16x4 lo = blo[0][x] | blo[1][x], hi = bhi[0][x] | bhi[1][x];      // whichever set was read
+                blo[0][x] = blo[1][x] = lo;
+                bhi[0][x] = bhi[1][x] = hi;
+            }
         }
-        for (int t = odd ? 1 : 0; t < full_steps; t += 2) {
-            k_step(I0{});
-            k_step(I1{});
+        // the first pass skips the walk steps before `first` (a scalar branch around each step)
+        int skip = first;
+        for (int t = -first; t < full_steps; t += WALK) {
+            static_for<0, WALK>([&](auto v) {
+                if (decltype(v)::value >= skip) k_step(v);
+            });
+            skip = 0;
         }
     }
 
@@ -296,11 +350,11 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
         }
         wait_dma_then_barrier<0>();                             // everybody is done with every buffer
         u32x4* Ab = reinterpret_cast<u32x4*>(lds_raw);
-        u32x4* Bb = reinterpret_cast<u32x4*>(lds_raw + 2 * A_BYTES);
+        u32x4* Bb = reinterpret_cast<u32x4*>(lds_raw + STAGES * A_BYTES);
 #pragma unroll
         for (int p = 0; p < S::A_PASSES; ++p) {
             const int id = tid + p * NT;
-            Ab[a_unit_slot(id / UA, id % UA, UA)] = a_stage[p];
+            Ab[a16_unit_slot(id / UA, id % UA, UA)] = a_stage[p];
         }
 #pragma unroll
         for (int p = 0; p < S::B_PASSES; ++p) {
@@ -316,12 +370,13 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
             });
             if constexpr (H == 0)
                 static_for<0, 2 * NI>([&](auto r) {
-                    read_b(std::integral_constant<int, KB & 1>{}, I0{}, std::integral_constant<int, KB>{},
+                    read_b(std::integral_constant<int, DECX_BSET(0, KB)>{}, I0{}, std::integral_constant<int, KB>{},
                            std::integral_constant<int, decltype(r)::value / 2>{}, std::integral_constant<int, decltype(r)::value % 2>{});
                 });
-            static_for<0, BLK>([&](auto i_tag) { mfma_one(u_tag, i_tag); });
+            static_for<0, BLK>([&](auto i_tag) { mfma_one(I0{}, u_tag, i_tag); });
         });
     }
+#undef DECX_BSET
 #undef DECX_PIN
 
     // ---- epilogue.  acc[mi][ni][e] is element (row 16 mi + li, column 16 ni + 4 lg + e) of the wave's piece.  dst = A*B + C

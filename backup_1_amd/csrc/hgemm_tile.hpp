@@ -230,8 +230,7 @@ static __global__ __launch_bounds__(256) void hgemm_split_finish_kernel(const fl
     const size_t total = (size_t)M * N;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const size_t m = i / N, n = i - m * N;
-        float v = partial[i];
-        for (int s = 1; s < planes; ++s) v += partial[(size_t)s * plane + i];
+        float v = ordered_plane_sum(partial, planes, plane, i);
         if (Cin != nullptr) v += (float)Cin[m * ldc + n];
         D[m * ldd + n] = (_Float16)v;
     }

@@ -44,6 +44,23 @@ __device__ __forceinline__ void static_for(F&& f) {
     }
 }
 
+// plane 0 + plane 1 + ... of element i of `planes` fp32 planes `plane` floats apart, added in that order (the fixed
+// order is what makes a split-K result the same on every run); the loads of 8 planes are issued together, the
+// additions stay sequential
+__device__ __forceinline__ float ordered_plane_sum(const float* __restrict__ partial, int planes, size_t plane, size_t i) {
+    float v = partial[i];
+    int s = 1;
+    for (; s + 8 <= planes; s += 8) {
+        float p[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) p[j] = __builtin_nontemporal_load(partial + (size_t)(s + j) * plane + i);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v += p[j];
+    }
+    for (; s < planes; ++s) v += partial[(size_t)s * plane + i];
+    return v;
+}
+
 struct TileCoord {
     int tm, tn;
 };

@@ -27,7 +27,7 @@ SHAPES = [(1, 1, 1), (3, 5, 7), (31, 17, 33), (32, 32, 32), (128, 32, 128), (129
           (300, 70, 500), (257, 1500, 255), (64, 8, 1000), (1000, 3, 64), (513, 129, 259)]
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 15])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 15, 16])
 @pytest.mark.parametrize("shape", SHAPES)
 def test_integer_exact_all_tiles(gpu, shape, variant):
     M, K, N = shape
@@ -53,7 +53,7 @@ def test_a_times_b_plus_c(gpu):
     A, B = workloads.small_ints((M, K), 21, -3, 3), workloads.small_ints((K, N), 22, -3, 3)
     C = workloads.small_ints((M, N), 23, -50, 50)
     want = (A.astype(np.float64) @ B.astype(np.float64) + C).astype(np.float16).view(np.uint16)
-    for variant in (1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 15):
+    for variant in (1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 15, 16):
         assert np.array_equal(gpu_hgemm(to_bits(A), to_bits(B), to_bits(C), variant=variant), want)
 
 
@@ -119,7 +119,7 @@ def test_random_vs_fp64(gpu, oracle, case):
     Ab, Bb = oracle.float_to_half(A), oracle.float_to_half(B)
     rows = np.arange(0, M, max(1, M // 50), dtype=np.int32)
     ref, scale = oracle.gemm_f64_rows_f16(Ab, Bb, rows)
-    for variant in (1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 15):
+    for variant in (1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 15, 16):
         got = from_bits(gpu_hgemm(Ab, Bb, variant=variant))[rows]
         err = rel_err_vs_abs_scale(got, ref, scale)
         print("%s variant %d: max |x-r|/sum|a||b| = %.3e (bound %.1e)" % (case, variant, err, TOL))
@@ -151,7 +151,7 @@ def test_config5_8192_cube_sampled_rows(gpu, oracle):
     assert np.array_equal(goti.sum(axis=0), Ai.astype(np.float64).sum(axis=0) @ Bi.astype(np.float64))
 
 
-@pytest.mark.parametrize("variant", [0, 2, 4, 7, 15])
+@pytest.mark.parametrize("variant", [0, 2, 4, 7, 15, 16])
 def test_batched_hgemm_one_launch(gpu, variant):
     batch, M, K, N = 3, 256, 128, 512
     A = workloads.small_ints((batch, M, K), 91, -3, 3)

@@ -39,7 +39,7 @@ def test_fp32_b_is_a_column_range(gpu, oracle, variant, shape):
     assert np.all(out[:, N:] == -5.0)
 
 
-@pytest.mark.parametrize("variant", [0, 2, 7, 8, 15])
+@pytest.mark.parametrize("variant", [0, 2, 7, 8, 15, 16])
 @pytest.mark.parametrize("shape", [(96, 64, 40, 24, 64), (256, 128, 952, 2048, 3000), (256, 256, 1000, 1024, 2024)])
 def test_fp16_b_is_a_column_range(gpu, variant, shape):
     M, K, N, c0, pb = shape
