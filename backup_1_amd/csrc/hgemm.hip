@@ -26,7 +26,9 @@ namespace decx_hip {
 //      this instruction draws less power per flop on real-valued data
 //  16: as 15 with 4 LDS stages of 32 k instead of 2 of 64 (three K steps in flight instead of one): measured equal to 15 at
 //      8192^3 (1381 vs 1396 TFLOP/s), and so were 5 stages and a refill spread over the following step -- the wait for the
-//      loads is not what the kernel loses time to; kept as the second instantiation of the kernel's stage arithmetic
+//      loads is not what the kernel loses time to (4 waves of 128x128, a quarter fewer LDS reads, measured 1387 too: on
+//      uniform[-1,1] data every arrangement ends at the same power-limited rate); kept as the second instantiation of
+//      the kernel's stage arithmetic
 //  11: split-K on shape 8 through an fp32 workspace (hgemm_splitk_enqueue) -- few tiles and a long K
 // and, for the fp16 convolution only: 12 keeps its register-staged kernels, 13 takes its LDS-DMA kernel for any image
 // whose channel pitch allows it, 14 its tap-row kernel; each switches its split over K off (experiments and tests)
