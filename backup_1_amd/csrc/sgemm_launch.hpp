@@ -52,6 +52,8 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //         cost model picks 128x128 tiles (2048^3: 0.140 -> 0.126 ms; 2048x2048x4096, two rounds: 0.259 -> 0.247 ms)
 //  15: 224x128x16, 2x4 waves of 128x32 (upper row) and 96x32 (lower row) -- shape 6 on two waves per SIMD: each SIMD
 //         carries a 4-block and a 3-block wave
+//  17: 208x128x16, 2x4 waves of 112x32 (three 32-row blocks and one of 16 rows on v_mfma_f32_16x16x4_f32) and 96x32:
+//         convolution only (filter-bank B); 6 1/2 blocks per SIMD for results whose rows fill the CUs badly in steps of 32
 // and, for dense GEMM only, the one-wave-per-16x16-block kernel of sgemm_chain16.hpp:
 //  11:  32x32x64,  2x2 computing + 4 moving waves, two workgroups per CU -- results too small to fill the chip with tiles
 //  12:  16x16x64,  1 computing + 2 moving waves -- at most one 16x16 block per CU: the fastest a single chain can walk K
@@ -66,6 +68,7 @@ typedef SgemmShape<256, 256, 16, 4, 2, 2, 2> SShapeBig8;
 typedef SgemmShape<224, 256, 16, 1, 8, 2, 2> SShape224Wide;   // 8 waves of 224x32, two per SIMD
 typedef SgemmShape<192, 192, 16, 2, 2, 1> SShape192;
 typedef SgemmShape<224, 128, 16, 2, 4, 2, 2, true> SShape224Split;   // 8 waves, 4 + 3 row blocks per SIMD
+typedef SgemmShape<208, 128, 16, 2, 4, 2, 2, true, true> SShape208Split;   // 8 waves, 3 1/2 + 3 row blocks per SIMD (filter-bank B only)
 typedef SgemmShape<128, 128, 16, 2, 2, 1> SShapeSmallSolo;
 typedef SgemmShape<64, 64, 16, 2, 2, 4> SShapeTiny;      // 2x2 waves of 32x32
 typedef SgemmShape<128, 64, 16, 2, 2, 4> SShapeTiny2;    // 2x2 waves of 64x32
@@ -78,7 +81,7 @@ typedef SgemmShape<128, 64, 16, 2, 2, 4> SShapeTiny2;    // 2x2 waves of 64x32
 // ahead of shape 6 on the 224x224x64 convolution under 128 filters; the same split of the 224x256 tile, and 256x128 on
 // 8 waves of 128x32, measured no better than shapes 10 and 5 and are not built).
 inline int pick_sgemm_variant(int M, int N, int K, int batch, bool dense = false) {
-    if ((g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) || g_rt.sgemm_variant == 15 || g_rt.sgemm_variant == 16) return g_rt.sgemm_variant;
+    if ((g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) || (g_rt.sgemm_variant >= 15 && g_rt.sgemm_variant <= 17)) return g_rt.sgemm_variant;
     if (g_rt.sgemm_variant == 14) return dense ? 14 : 2;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     // At most 8 K steps and several rounds of tiles: the launch is bound by writing the result, and two small workgroups
@@ -87,11 +90,14 @@ inline int pick_sgemm_variant(int M, int N, int K, int batch, bool dense = false
     if (K <= 128 && (long)cdiv(M, 128) * cdiv(N, 128) * batch >= 2 * cus) return 2;
     struct Cand { int variant, bm, bn; double eff; };
     const Cand cands[] = {{7, 256, 256, 1.00}, {10, 224, 256, 0.96}, {3, 256, 128, 0.95}, {4, 224, 128, 0.94}, {2, 128, 128, 0.92},
-                          {9, 128, 64, 0.83}, {8, 64, 64, 0.78}, {14, 192, 192, 0.93}};
+                          {9, 128, 64, 0.83}, {8, 64, 64, 0.78}, {14, 192, 192, 0.93}, {17, 208, 128, 0.90}};
     int best = 7;
     double best_cost = 0.0;
     for (const Cand& c : cands) {
         if (c.variant == 14 && !dense) continue;
+        // 208 rows (a block of 16 among them): filter-bank B only, and only as the single round of a launch that 224-row
+        // tiles would leave an eighth of the chip idle in (224x224x64 under 128 filters: 242 tiles, 65.0 -> 63.0 us)
+        if (c.variant == 17 && (dense || (long)cdiv(M, c.bm) * cdiv(N, c.bn) * batch > cus)) continue;
         const long tiles = (long)cdiv(M, c.bm) * cdiv(N, c.bn) * batch;
         const double cost = (double)((tiles + cus - 1) / cus) * c.bm * c.bn / c.eff;
         if (best_cost == 0.0 || cost < best_cost) {
@@ -118,6 +124,9 @@ int dispatch_sgemm(int variant, const ASrc& a, const BSrc& b, const float* Cin, 
         case 10: return launch_sgemm_tile<SShape224Wide>(a, b, Cin, ldc, D, out, M, N, K, batch);
         case 15: return launch_sgemm_tile<SShape224Split>(a, b, Cin, ldc, D, out, M, N, K, batch);
         case 16: return launch_sgemm_tile<SShapeSmallSolo>(a, b, Cin, ldc, D, out, M, N, K, batch);
+        case 17:
+            if constexpr (!BSrc::ROW_MAJOR_LDS) return launch_sgemm_tile<SShape208Split>(a, b, Cin, ldc, D, out, M, N, K, batch);
+            else return launch_sgemm_tile<SShape224Split>(a, b, Cin, ldc, D, out, M, N, K, batch);
         default: return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K, batch);
     }
 }

@@ -399,6 +399,9 @@ struct DenseB {
     // column (relative to the wave's strip) held by lane li in block ni
     template <class S>
     __device__ __forceinline__ static int strip_col(int ni, int li) { return S::NI * li + ni; }
+    // (half blocks of 16 rows exist for the filter-bank layout only; never called)
+    template <class S>
+    __device__ __forceinline__ void read_half_frags(const float*, int, int, int, float (*)[2]) const {}
 };
 
 // B as a bank of N filters, filter n holding its taps channel-innermost: column n of the lowered GEMM is filter n and
@@ -497,6 +500,19 @@ struct FilterB {
             for (int e = 0; e < 4; ++e) frag[e][ni] = v[e];
         }
     }
+    // operands of k-group s for a 16-row half block (v_mfma_f32_16x16x4_f32, lane = 16 * slot + i): bh[c][j] =
+    // B[8s + 4j + slot][wn0 + 16c + i] -- plane 2s + slot % 2, elements slot / 2 and 2 + slot / 2 of the column's quad
+    template <class S>
+    __device__ __forceinline__ void read_half_frags(const float* buf, int s, int lane, int wn0, float (*bh)[2]) const {
+        const int slot = lane >> 4, i = lane & 15;
+        const f32x4* plane = reinterpret_cast<const f32x4*>(buf) + (2 * s + (slot & 1)) * S::B_ROW;
+#pragma unroll
+        for (int c = 0; c < 2 * S::NI; ++c) {
+            const float* q = reinterpret_cast<const float*>(plane + b_slot(wn0 + 16 * c + i)) + (slot >> 1);
+            bh[c][0] = q[0];
+            bh[c][1] = q[2];
+        }
+    }
     template <class S>
     __device__ __forceinline__ static int strip_col(int ni, int li) { return 32 * ni + li; }
 };
@@ -527,7 +543,7 @@ struct FilterBUniform : FilterB<true> {
 };
 
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int WAVES_PER_SIMD_ = 1,
-          int STAGE_SETS_ = (WAVES_PER_SIMD_ == 1 ? 2 : 1), bool UNEVEN_M_ = false>
+          int STAGE_SETS_ = (WAVES_PER_SIMD_ == 1 ? 2 : 1), bool UNEVEN_M_ = false, bool HALF_BLOCK_ = false>
 struct SgemmShape {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_;
     static constexpr int WAVES_PER_SIMD = WAVES_PER_SIMD_;   // occupancy the register budget is held to
@@ -541,9 +557,13 @@ struct SgemmShape {
     // (224 rows = 4 + 3 blocks).  Waves w and w + WAVES_N land on the same SIMD, so every SIMD carries one wave of
     // each kind and the same number of MFMAs per K step.
     static constexpr bool UNEVEN_M = UNEVEN_M_;
-    static constexpr int MI = UNEVEN_M ? (BM / 32 + 1) / 2 : BM / WAVES_M / 32;      // blocks of the upper wave row
-    static constexpr int MI_LOW = UNEVEN_M ? BM / 32 - MI : MI;                      // blocks of the other wave rows
-    static constexpr int WM = MI * 32, WN = BN / WAVES_N;
+    // HALF_BLOCK (with UNEVEN_M, filter-bank B only): BM is an odd multiple of 16 and what the upper wave row has more
+    // than the lower one is a block of 16 rows, computed with v_mfma_f32_16x16x4_f32 (208 rows = 3 1/2 + 3 blocks): tiles
+    // a sixteenth finer, for results whose rows divide badly over the CUs in steps of 32.
+    static constexpr bool HALF_BLOCK = HALF_BLOCK_;
+    static constexpr int MI = HALF_BLOCK ? BM / 64 : UNEVEN_M ? (BM / 32 + 1) / 2 : BM / WAVES_M / 32;      // 32-row blocks of the upper wave row
+    static constexpr int MI_LOW = HALF_BLOCK ? MI : UNEVEN_M ? BM / 32 - MI : MI;    // blocks of the other wave rows
+    static constexpr int WM = MI * 32 + (HALF_BLOCK ? 16 : 0), WN = BN / WAVES_N;
     static constexpr int NI = WN / 32;
     static constexpr int KQ = BK / 4;                         // k-quads per step
     static constexpr int KGROUPS = KQ / 2;                    // groups of 8 consecutive k per step
@@ -561,8 +581,9 @@ struct SgemmShape {
     static constexpr size_t lds_bytes() {
         return 2 * ((size_t)KQ * A_ROW * sizeof(f32x4) + (size_t)BSrc::template lds_floats<SgemmShape>() * sizeof(float));
     }
-    static_assert(UNEVEN_M ? (WAVES_M == 2 && BM % 32 == 0 && MI_LOW >= 1 && WAVES_N % 4 == 0) : BM % (WAVES_M * 32) == 0,
-                  "wave tile must be whole 32x32 blocks");
+    static_assert(HALF_BLOCK ? (UNEVEN_M && WAVES_M == 2 && BM % 32 == 16 && MI >= 1 && WAVES_N % 4 == 0)
+                  : UNEVEN_M ? (WAVES_M == 2 && BM % 32 == 0 && MI_LOW >= 1 && WAVES_N % 4 == 0) : BM % (WAVES_M * 32) == 0,
+                  "wave tile must be whole 32x32 blocks (plus one block of 16 rows with HALF_BLOCK)");
     static_assert(BN % (WAVES_N * 32) == 0, "wave tile must be whole 32x32 blocks");
     static_assert(BK % 8 == 0, "a K step is whole quad pairs");
     static_assert(NT % KGROUPS == 0, "A staging: KGROUPS lanes per row");
@@ -571,6 +592,9 @@ struct SgemmShape {
 // SPLIT_K: blockIdx.z selects a K range of k_split_len (a multiple of BK); every range adds its partial products to dst
 // with fp32 atomics, so dst must hold zeros beforehand and the summation order over ranges is not fixed.  C, if any, is
 // added by range 0.
+template <bool HAS_C, class Out>
+struct HAS_C_PRELOAD_GUARD { static constexpr bool value = HAS_C && Out::PRELOAD_C; };
+
 template <class S, class ASrc, class BSrc, class Out, bool HAS_C, bool SPLIT_K = false>
 __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(ASrc a_src, BSrc b_src, const float* Cin, int ldc, float* D,
                                                            Out out, int M, int N, int K, int tiles_m, int tiles_n,
@@ -663,8 +687,16 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
 
     // Everything from here on depends on how many 32-row blocks the wave owns, a compile-time count: one instance of the
     // K walk and the epilogue per count, chosen per wave below.
-    auto run = [&](auto mi_tag) {
+    auto run = [&](auto mi_tag, auto half_tag) {
         constexpr int MI = decltype(mi_tag)::value;
+        // HALF: this wave also owns the 16 rows below its MI blocks, as 2 NI blocks of 16 x 16 (v_mfma_f32_16x16x4_f32:
+        // lane 16 slot + i feeds row i / column i at k-slot slot, per element fma over slots 0..3 in ascending order, and
+        // holds rows 4 slot .. 4 slot + 3 of column i) -- two of them per k-group and column block, k ascending
+        constexpr bool HALF = decltype(half_tag)::value;
+        constexpr int HC = HALF ? 2 * NI : 0;
+        static_assert(!HALF || (!BSrc::ROW_MAJOR_LDS && !HAS_C_PRELOAD_GUARD<HAS_C, Out>::value), "half blocks: filter-bank B, C added at the end");
+        const int hs = lane >> 4, hi = lane & 15;                 // k-slot and row / column inside a 16 x 16 block
+        const int hm0 = wm0 + MI * 32;                            // first row of the half block inside the tile
         // Accumulators start at zero, or at C for dst = A*B + C on dense matrices: the reference's chain starts from C
         // (GEMM.cuh:223), and starting anywhere else would round differently.  A convolution's bias is added at the end.
         constexpr bool PRELOAD_C = HAS_C && Out::PRELOAD_C;
@@ -675,6 +707,9 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
             for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[mi][ni][r] = 0.f;
+        f32x4 acc_h[HC > 0 ? HC : 1];
+#pragma unroll
+        for (int c = 0; c < HC; ++c) acc_h[c] = f32x4{0.f, 0.f, 0.f, 0.f};
         if (PRELOAD_C && (!SPLIT_K || blockIdx.z == 0)) {
 #pragma unroll
             for (int mi = 0; mi < MI; ++mi)
@@ -691,31 +726,51 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
 
         // Fragments of one quad pair s: A, per 32-row block one float4 = four consecutive k of this lane's k-slot; B, per
         // k of the pair (e) and block (ni) one float, fetched as the B source's LDS layout dictates.
-        typedef float BFrag[4][NI];
-        auto read_frags = [&](int buf, int s, f32x4* af, BFrag& bf) {
+        // The half block's operands of a quad pair: ah[j] = A[hm0 + hi][8s + 4j + hs], bh[c][j] = B[8s + 4j + hs][16c + hi],
+        // j = 0, 1 -- elements hs / 2 and 2 + hs / 2 of the quad in plane 2s + hs % 2.
+        struct Frags {
+            f32x4 af[MI];
+            float bf[4][NI];
+            float ah[2];
+            float bh[HC > 0 ? HC : 1][2];
+        };
+        auto read_frags = [&](int buf, int s, Frags& f) {
             const f32x4* Ab = As + buf * KQ * S::A_ROW;
             const int q = 2 * s + lh;
 #pragma unroll
-            for (int mi = 0; mi < MI; ++mi) af[mi] = Ab[q * S::A_ROW + wm0 + mi * 32 + li];
-            b_src.template read_frags<S>(Bs + buf * B_BUF, s, lh, li, wn0, bf);
+            for (int mi = 0; mi < MI; ++mi) f.af[mi] = Ab[q * S::A_ROW + wm0 + mi * 32 + li];
+            b_src.template read_frags<S>(Bs + buf * B_BUF, s, lh, li, wn0, f.bf);
+            if constexpr (HALF) {
+                const float* aq = reinterpret_cast<const float*>(Ab + (2 * s + (hs & 1)) * S::A_ROW + hm0 + hi) + (hs >> 1);
+                f.ah[0] = aq[0];
+                f.ah[1] = aq[2];
+                b_src.template read_half_frags<S>(Bs + buf * B_BUF, s, lane, wn0, f.bh);
+            }
         };
-        // MFMAs number lo .. hi-1 of a quad pair, in the order (e, mi, ni); a full pair is 4*MI*NI of them.
-        constexpr int PAIR_MFMAS = 4 * MI * NI;
-        auto mfma_range = [&](const f32x4* af, const BFrag& bf, auto lo_tag, auto hi_tag) {
+        // MFMAs number lo .. hi-1 of a quad pair: the 4*MI*NI of the 32-row blocks in the order (e, mi, ni), with the HC
+        // of the half block for k = 8s .. 8s+3 (j = 0) after those of e = 1 and the HC for k = 8s+4 .. 8s+7 after e = 3.
+        constexpr int FULL_MFMAS = 4 * MI * NI, PAIR_MFMAS = FULL_MFMAS + 2 * HC, HALF_PAIR = FULL_MFMAS / 2 + HC;
+        auto mfma_range = [&](const Frags& f, auto lo_tag, auto hi_tag) {
             constexpr int LO = decltype(lo_tag)::value, HI = decltype(hi_tag)::value;
 #pragma unroll
             for (int i = LO; i < HI; ++i) {
-                const int e = i / (MI * NI), mi = (i / NI) % MI, ni = i % NI;
-                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[mi][e], bf[e][ni], acc[mi][ni], 0, 0, 0);
+                const int j = i / HALF_PAIR, within = i % HALF_PAIR;      // which half of the pair's k, position inside it
+                if (within < FULL_MFMAS / 2) {
+                    const int x = j * (FULL_MFMAS / 2) + within;
+                    const int e = x / (MI * NI), mi = (x / NI) % MI, ni = x % NI;
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.af[mi][e], f.bf[e][ni], acc[mi][ni], 0, 0, 0);
+                } else if constexpr (HALF) {
+                    const int c = within - FULL_MFMAS / 2;
+                    acc_h[c] = __builtin_amdgcn_mfma_f32_16x16x4f32(f.ah[j], f.bh[c][j], acc_h[c], 0, 0, 0);
+                }
             }
         };
         auto compute_stage = [&](int buf) {      // unpipelined: used for the peeled steps only
 #pragma unroll
             for (int s = 0; s < KQ / 2; ++s) {
-                f32x4 af[MI];
-                BFrag bf;
-                read_frags(buf, s, af, bf);
-                mfma_range(af, bf, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
+                Frags f;
+                read_frags(buf, s, f);
+                mfma_range(f, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
             }
         };
 
@@ -744,9 +799,8 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
 
         static_assert(KQ == 4, "the pipelined loop is written for two quad pairs per K step");
         constexpr int VMEM_OPS = S::A_PASSES + B_QUADS;     // global loads per thread and step
-        constexpr int FRAG_OPS = MI + BSrc::template frag_reads<S>();   // LDS reads per quad pair
-        f32x4 af0[MI], af1[MI];
-        BFrag bf0, bf1;
+        constexpr int FRAG_OPS = MI + BSrc::template frag_reads<S>() + (HALF ? 1 + HC : 0);   // LDS reads per quad pair
+        Frags f0, f1;
 
         // Steady state of one K step t (fragments of its first quad pair are in af0/bf0):
         //   pair 0 MFMAs   interleaved with: global loads of step t+SETS, LDS reads of pair 1
@@ -756,8 +810,8 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         auto pipelined_step = [&](auto set_tag, int buf) {
             constexpr int SET = decltype(set_tag)::value;
             load_stage(set_tag, std::false_type{});
-            read_frags(buf, 1, af1, bf1);
-            mfma_range(af0, bf0, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
+            read_frags(buf, 1, f1);
+            mfma_range(f0, std::integral_constant<int, 0>{}, std::integral_constant<int, PAIR_MFMAS>{});
             // scheduling-group masks: 0x002 VALU, 0x008 MFMA, 0x020 VMEM read, 0x100 DS read, 0x200 DS write
             constexpr int G0 = PAIR_MFMAS / (VMEM_OPS + FRAG_OPS) > 0 ? PAIR_MFMAS / (VMEM_OPS + FRAG_OPS) : 1;
 #pragma unroll
@@ -781,13 +835,13 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
             static_for<0, WRITE_OPS>([&](auto w_tag) {
                 constexpr int W = decltype(w_tag)::value;
                 write_one(StoreSet{}, buf ^ 1, w_tag);
-                mfma_range(af1, bf1, std::integral_constant<int, W * EARLY / WRITE_OPS>{}, std::integral_constant<int, (W + 1) * EARLY / WRITE_OPS>{});
+                mfma_range(f1, std::integral_constant<int, W * EARLY / WRITE_OPS>{}, std::integral_constant<int, (W + 1) * EARLY / WRITE_OPS>{});
                 __builtin_amdgcn_sched_barrier(0);
             });
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
             __builtin_amdgcn_sched_barrier(0);
-            read_frags(buf ^ 1, 0, af0, bf0);
-            mfma_range(af1, bf1, std::integral_constant<int, EARLY>{}, std::integral_constant<int, PAIR_MFMAS>{});
+            read_frags(buf ^ 1, 0, f0);
+            mfma_range(f1, std::integral_constant<int, EARLY>{}, std::integral_constant<int, PAIR_MFMAS>{});
             __builtin_amdgcn_sched_group_barrier(0x100, FRAG_OPS, 2);
             __builtin_amdgcn_sched_group_barrier(0x008, LATE, 2);
             __builtin_amdgcn_sched_barrier(0);
@@ -796,7 +850,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         int t = 0;
         if constexpr (SETS == 2) {
             if (full_steps > 2) {
-                read_frags(0, 0, af0, bf0);
+                read_frags(0, 0, f0);
                 for (; t + 3 < full_steps; t += 2) {      // steps t and t+1 both fetch a full step (t+2, t+3 < full_steps)
                     pipelined_step(Set0{}, 0);
                     pipelined_step(Set1{}, 1);
@@ -822,7 +876,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
             }
         } else {
             if (full_steps > 1) {
-                read_frags(0, 0, af0, bf0);
+                read_frags(0, 0, f0);
                 for (; t + 1 < full_steps; ++t) pipelined_step(Set0{}, t & 1);   // fetches step t+1, a full one
             }
             for (; t < T; ++t) {
@@ -877,13 +931,30 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
         };
         if (!SPLIT_K && out.rows_at_pitch() && bm0 + BM <= M && bn0 + BN <= N) store_rows(std::true_type{});
         else store_rows(std::false_type{});
+        if constexpr (HALF) {
+            // the half block: lane (hs, hi) holds rows 4 hs .. 4 hs + 3 of column 16 c + hi
+            const bool full = out.rows_at_pitch() && bm0 + BM <= M && bn0 + BN <= N;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int m = bm0 + hm0 + 4 * hs + r;
+                if (full || m < M) {
+                    float* drow = D + (full ? out.pitched_offset(m) : out.offset(m));
+                    const float* crow = HAS_C ? Cin + (size_t)m * ldc : nullptr;
+#pragma unroll
+                    for (int c = 0; c < HC; ++c) {
+                        const int n = bn0 + wn0 + 16 * c + hi;
+                        if (full || n < N) drow[n] = out.finish(HAS_C ? acc_h[c][r] + crow[n] : acc_h[c][r]);
+                    }
+                }
+            }
+        }
     };
     if constexpr (S::UNEVEN_M) {
         // a branch on the scalar unit: the two wave rows run different instances, with the same sequence of barriers
-        if (__builtin_amdgcn_readfirstlane(wave) < S::WAVES_N) run(std::integral_constant<int, S::MI>{});
-        else run(std::integral_constant<int, S::MI_LOW>{});
+        if (__builtin_amdgcn_readfirstlane(wave) < S::WAVES_N) run(std::integral_constant<int, S::MI>{}, std::integral_constant<bool, S::HALF_BLOCK>{});
+        else run(std::integral_constant<int, S::MI_LOW>{}, std::false_type{});
     } else {
-        run(std::integral_constant<int, S::MI>{});
+        run(std::integral_constant<int, S::MI>{}, std::false_type{});
     }
 }
 

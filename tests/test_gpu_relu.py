@@ -78,7 +78,7 @@ def test_argument_errors(gpu):
     assert L.decx_hip_relu_f32(d.ptr, d.ptr, 0) == 0
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 11, 12, 13])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 11, 12, 13, 15, 17])
 def test_fused_conv_bias_relu_equals_separate_passes(gpu, oracle, variant):
     H, W, C, N = 29, 31, 12, 70
     src, filt = workloads.normal((H, W, C), 5), workloads.normal((N, 3, 3, C), 6)
