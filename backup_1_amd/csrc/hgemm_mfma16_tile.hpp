@@ -417,7 +417,7 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
         _Float16* dp = D + (size_t)m * ldd + n;
         if ((ABLATE & 4) && K >= 0) continue;                    // (a condition the compiler cannot fold, so the sums stay live)
         if (whole) {
-            *reinterpret_cast<u32x4*>(dp) = v;
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dp));      // written once, not read by this launch
         } else if (m < M) {
             if (vec_d && n + 8 <= N) {
                 *reinterpret_cast<u32x4*>(dp) = v;

@@ -274,6 +274,7 @@ struct Im2colAUniform : Im2colA<true> {
 // y*row_stride + x*dpitch).  relu: apply relu_by_sign to every result element before it is stored.
 struct DenseOut {
     static constexpr bool PRELOAD_C = true;      // "+ C" enters the accumulators before the K walk
+    static constexpr bool STREAM_OUT = false;    // (non-temporal stores lose 1.5 % on the ragged 3000x1500x4500 product)
     int ld;
     bool relu = false;
     bool vec = false;      // every row of the result starts 16-byte aligned: runs of consecutive columns go out as one store
@@ -289,6 +290,7 @@ struct TensorOut {
     bool relu = false;
     static constexpr bool vec = false;
     static constexpr bool PRELOAD_C = false;     // the "+ C" operand is a bias row, added to the finished sum
+    static constexpr bool STREAM_OUT = true;     // the result is written once and not read by this launch: non-temporal stores
     __device__ __forceinline__ float finish(float v) const { return relu ? relu_by_sign(v) : v; }
     __device__ __forceinline__ bool rows_at_pitch() const { return dense; }
     __device__ __forceinline__ size_t pitched_offset(int m) const { return (size_t)m * dpitch; }
@@ -923,6 +925,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
                             if (FULL || n < N) {
                                 const float v = add_c ? acc[mi][ni][r] + crow[n] : acc[mi][ni][r];
                                 if (SPLIT_K) unsafeAtomicAdd(drow + n, v);      // hardware fp32 add in L2
+                                else if constexpr (Out::STREAM_OUT) __builtin_nontemporal_store(out.finish(v), drow + n);
                                 else drow[n] = out.finish(v);
                             }
                         }
@@ -943,7 +946,7 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_tile_kernel(AS
 #pragma unroll
                     for (int c = 0; c < HC; ++c) {
                         const int n = bn0 + wn0 + 16 * c + hi;
-                        if (full || n < N) drow[n] = out.finish(HAS_C ? acc_h[c][r] + crow[n] : acc_h[c][r]);
+                        if (full || n < N) __builtin_nontemporal_store(out.finish(HAS_C ? acc_h[c][r] + crow[n] : acc_h[c][r]), drow + n);
                     }
                 }
             }
