@@ -86,8 +86,9 @@ int hgemm_probe_enqueue(int ablate, const uint16_t* A, int lda, const uint16_t* 
         case 3: kern = hgemm_mfma16_kernel<S, false, 3>; break;
         case 4: kern = hgemm_mfma16_kernel<S, false, 4>; break;
         case 5: kern = hgemm_mfma16_kernel<S, false, 5>; break;
+        case 6: kern = hgemm_mfma16_kernel<S, false, 6>; break;
         case 7: kern = hgemm_mfma16_kernel<S, false, 7>; break;
-        default: return fail(DECX_HIP_FAIL_ERROR_PARAMS, "probe variants: 0, 1, 3, 4, 5, 7\n");
+        default: return fail(DECX_HIP_FAIL_ERROR_PARAMS, "probe variants: 0, 1, 3, 4, 5, 6, 7\n");
     }
     HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
     const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);

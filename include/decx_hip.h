@@ -249,7 +249,7 @@ int decx_hip_copy_kernel(void* dst, const void* src, size_t bytes);
  * the large fp16 GEMM tile kernel of decx_hip_hgemm_f32acc with parts of its K walk left out, so that the cost of each
  * part can be read off as the difference between two variants.  `ablate` is a sum of: 1 = no global -> LDS loads inside
  * the K walk, 2 = no LDS -> register reads inside it (the matrix instructions keep running on the first fragments),
- * 4 = the result is not stored; allowed values 0 (the whole kernel), 1, 3, 4, 5, 7.  Every variant issues the same
+ * 4 = the result is not stored; allowed values 0 (the whole kernel), 1, 3, 4, 5, 6, 7.  Every variant issues the same
  * matrix instructions; all but 0 leave D meaningless or untouched.  Arguments as decx_hip_hgemm_f32acc without C; A, B
  * 16-byte aligned with lda, ldb multiples of 8. */
 int decx_hip_hgemm_probe(int ablate, const uint16_t* A, int lda, const uint16_t* B, int ldb, uint16_t* D, int ldd, int M, int N, int K);
