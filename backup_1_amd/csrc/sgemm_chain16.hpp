@@ -174,8 +174,8 @@ __global__ __launch_bounds__(S::NT, S::WAVES_PER_SIMD) void sgemm_chain16_kernel
         }
 #pragma unroll
         for (int p = 0; p < PB; ++p) {
-            const int q = pt + p * S::MOVE_THREADS, rest = q / 32;
-            const int k = 16 * (rest % 4) + q % 16, cq = 2 * (rest / 4) + (q / 16) % 2;
+            const int q = pt + p * S::MOVE_THREADS;
+            const int k = (q / 4) % 64, cq = 4 * (q / 256) + q % 4;
             int col = bn0 + 4 * cq;
             col = clamp_group_col(col, N, 4);     // stay inside the operand; such columns are never stored
             quad_k[PA + p] = k;
