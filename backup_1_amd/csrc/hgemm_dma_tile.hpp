@@ -37,19 +37,6 @@ struct HgemmDmaShape : HgemmShape<BM_, BN_, BK_, WAVES_M_, WAVES_N_> {
     static_assert(STAGES >= 2, "need at least double buffering");
 };
 
-// One 16-byte-per-lane load from global memory (wave-uniform base + per-lane byte offset) straight into LDS at
-// lds_base + 16*lane (lds_base wave-uniform).
-__device__ __forceinline__ void dma_load16(const void* sbase, uint32_t lane_off, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 : : "v"(lane_off), "s"(sbase), "s"(lds_base) : "memory", "m0");
-}
-
-template <int N>
-__device__ __forceinline__ void wait_dma_then_barrier() {
-    // my loads older than the N most recent have landed; my LDS reads are done; then everybody meets
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" : : "n"(N) : "memory");
-}
-
 // SPLIT_K: blockIdx.z selects a range of K (k_split_len long, a multiple of BK); the tile's fp32 partial sums go to a
 // workspace of dense M x N fp32 planes instead of being rounded and stored.  partial_plane != 0: range z stores its
 // sums into plane z (partial + z * partial_plane) with plain stores -- every element of a plane inside the result is

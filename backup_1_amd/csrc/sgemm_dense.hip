@@ -1,6 +1,7 @@
 // fp32 dense GEMM: argument checks, kernel choice and launch (sgemm_tile.hpp, sgemm_chain16.hpp), split-K.
 #include "sgemm_launch.hpp"
 #include "sgemm_chain16.hpp"
+#include "sgemm_dma64.hpp"
 
 namespace decx_hip {
 
@@ -57,6 +58,30 @@ int launch_sgemm_chain16(const float* A, int lda, const float* B, int ldb, const
     return 0;
 }
 
+// 64x64 tiles fed by LDS-DMA loads (sgemm_dma64.hpp): for results of about one such tile per CU.
+template <class S>
+int launch_sgemm_dma64(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
+                       int N, int K, const Batch& batch, bool relu) {
+    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    const long total = (long)tiles_m * tiles_n;
+    if (total > 0x7fffffffL || batch.count > 65535) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
+    auto kern = Cin ? sgemm_dma64_kernel<S, true> : sgemm_dma64_kernel<S, false>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(sgemm_dma64_kernel<S, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(sgemm_dma64_kernel<S, false>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
+        attr_done = true;
+    }
+    const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
+    hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::LDS_BYTES, batch.stream, A, lda, B, ldb,
+                       Cin, ldc, D, ldd, M, N, K, tiles_m, tiles_n, group_m, relu, batch.stride_a, batch.stride_b, batch.stride_c,
+                       batch.stride_d);
+    HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
                   int N, int K, const Batch& batch, bool relu) {
     if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
@@ -64,6 +89,11 @@ int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float*
     const bool vec_a = aligned16(A) && lda % 4 == 0 && batch.stride_a % 4 == 0;
     const bool vec_b = aligned16(B) && ldb % 4 == 0 && ldb >= 4 && batch.stride_b % 4 == 0;
     DenseOut out{ldd, relu, aligned16(D) && ldd % 4 == 0 && batch.stride_d % 4 == 0};
+    if (vec_a && vec_b && lda < kDmaMaxPitch && ldb < kDmaMaxPitch) {
+        const int dma = pick_dma64_shape(M, N, K, batch.count);
+        if (dma == 18) return launch_sgemm_dma64<Dma64<32, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+        if (dma == 19) return launch_sgemm_dma64<Dma64<64, 3>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+    }
     if (vec_a && vec_b) {
         const int chain = pick_chain_shape(M, N, K, batch.count);
         if (chain == 11) return launch_sgemm_chain16<Chain16<2, 1, 4, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);

@@ -1,0 +1,249 @@
+// fp32 GEMM for results of about one 64x64 tile per CU (1024^3: 256 tiles on 256 CUs): operands go from global memory
+// straight into LDS, and nothing but matrix instructions and their operand reads runs on the computing waves.
+//
+// With one tile per CU a workgroup is four waves, one per SIMD, and each wave's 32x32 block is ONE dependent chain of
+// v_mfma_f32_32x32x2_f32 (64 cycles each): every other instruction the SIMD has to issue delays that chain.  The
+// register-staged kernels spend a global load, two LDS stores and their address arithmetic per 16 bytes of operand;
+// measured on the block-chain kernel at this size, the staging costs a quarter of the matrix pipe's time.  Here a
+// global_load_lds_dwordx4 moves 16 bytes per lane into LDS with no register, no LDS store and no wait on the wave's
+// side: 4 such loads per wave and K step of 32, against 16 MFMAs.
+//
+// The price is that LDS holds the operands as they lie in memory, and a lane of the 32x32x2 instruction wants ONE
+// float per operand and instruction: lane (i, s), i = 0..31, s = 0..1, feeds A[i][2j + s] and B[2j + s][i] to MFMA j.
+//   B [k][64 columns]: 32 lanes read 32 consecutive floats of row 2j + s -- conflict-free; rows 2j+s and 2j+2+s of
+//     two successive MFMAs come with one ds_read2st64_b32.
+//   A [row][k]: a 16-byte unit holds k = 4q .. 4q+3 of a row, i.e. the operands of MFMAs 2q and 2q+1 for both s: lane
+//     (i, s) reads floats s and s + 2 of it with one ds_read2_b32.  Unit q of row r sits in slot q ^ (r % 8) of the
+//     row, so that the 32 rows of a read spread over all banks (each bank four times -- one float per lane and unit
+//     allows no less).  The swizzle is applied on the global side: the lane whose LDS place is slot t of row r fetches
+//     unit t ^ (r % 8).
+// One LDS read per MFMA in all, issued right behind it.
+//
+// Pipeline: STAGES LDS buffers, one barrier per K step.  The step is computed in two halves from two fragment sets:
+// during the first half the second half's fragments are read; the second half starts with the barrier (before it the
+// wave waits for its own loads of step t+1, after it nobody reads step t's buffer any more), then issues the loads of
+// step t+STAGES into that buffer and reads the first half of step t+1, all between its MFMAs.  Loads never run past
+// the last whole step: the source pointers stop there (later refills fetch that step again and are never read), which
+// keeps every step the same code with the same wait counts.  A ragged last step (K % BK) is staged through registers
+// with zeros past K and only the MFMAs that hold a k < K are issued.
+//
+// Arithmetic: per output one fused multiply-add chain over ascending k -- slot 0 then slot 1 inside an instruction,
+// instructions in order -- exactly the chain of sgemm_tile_kernel and of the reference.
+// Requires 16-byte aligned A and B with lda, ldb multiples of 4 (and below 2^23 so that a tile's byte offsets fit 32 bits).
+#pragma once
+#include "sgemm_tile.hpp"
+
+namespace decx_hip {
+
+template <int BK_, int STAGES_>
+struct Dma64 {
+    static constexpr int BM = 64, BN = 64, BK = BK_, STAGES = STAGES_, NWAVES = 4, NT = 64 * NWAVES;
+    static constexpr int UA = BK / 4;                                   // 16-byte units per row of A and step
+    static constexpr int UB = BN / 4;                                   // 16-byte units per row of B
+    static constexpr int A_UNITS = BM * UA, B_UNITS = BK * UB;
+    static constexpr int A_LOADS = A_UNITS / 64 / NWAVES, B_LOADS = B_UNITS / 64 / NWAVES;   // per wave and step, 1 KiB each
+    static constexpr int LOADS = A_LOADS + B_LOADS;
+    static constexpr int STAGE_FLOATS = (A_UNITS + B_UNITS) * 4;
+    static constexpr size_t LDS_BYTES = (size_t)STAGES * STAGE_FLOATS * sizeof(float);
+    static constexpr int HALF = BK / 4;                                 // MFMAs per half step
+    static_assert(BK % 16 == 0 && UA >= 8 && 64 % UA == 0, "whole units per half step; the swizzle needs 8 slots a row");
+    static_assert(A_UNITS % (64 * NWAVES) == 0 && B_UNITS % (64 * NWAVES) == 0, "loads divide over the waves");
+    static_assert(STAGES >= 2 && LOADS * (STAGES - 1) <= 63, "vmcnt is a 6-bit counter");
+};
+
+template <class S, bool HAS_C>
+__global__ __launch_bounds__(S::NT) void sgemm_dma64_kernel(const float* __restrict__ A, int lda, const float* __restrict__ B,
+                                                            int ldb, const float* Cin, int ldc, float* D, int ldd, int M, int N,
+                                                            int K, int tiles_m, int tiles_n, int group_m, bool relu,
+                                                            size_t a_batch_stride, size_t b_batch_stride, size_t c_batch_stride,
+                                                            size_t d_batch_stride) {
+    constexpr int BK = S::BK, UA = S::UA, UB = S::UB, STAGES = S::STAGES, HALF = S::HALF;
+    A += (size_t)blockIdx.y * a_batch_stride;
+    B += (size_t)blockIdx.y * b_batch_stride;
+    if (HAS_C) Cin += (size_t)blockIdx.y * c_batch_stride;
+    D += (size_t)blockIdx.y * d_batch_stride;
+    extern __shared__ __attribute__((aligned(16))) float lds[];      // [STAGES][A: 64 rows x UA units | B: BK rows x 16 units]
+    const uint32_t lds_base = lds_byte_address(lds);
+
+    const TileCoord tc = xcd_grouped_tile(blockIdx.x, tiles_m, tiles_n, group_m);
+    const int bm0 = tc.tm * S::BM, bn0 = tc.tn * S::BN;
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
+    const int wm0 = (wave / 2) * 32, wn0 = (wave % 2) * 32;
+    const int li = lane % 32, ls = lane / 32;          // row (of A) or column (of B) inside the wave's block, and k-slot
+    const int full_steps = K / BK, rem = K - full_steps * BK;
+
+    // ---- sources of this wave's loads: a wave-uniform base per operand that moves one K step per fetched step, plus
+    // loop-invariant byte offsets per lane (rows of this tile only)
+    const float* a_base = A + (size_t)bm0 * lda;
+    const float* b_base = B;
+    const size_t b_step = (size_t)BK * ldb;
+    uint32_t a_off[S::A_LOADS], b_off[S::B_LOADS];
+#pragma unroll
+    for (int j = 0; j < S::A_LOADS; ++j) {
+        const int row = (wave * S::A_LOADS + j) * (64 / UA) + lane / UA;     // 64 units = 64 / UA rows
+        const int q = (lane % UA) ^ (row & 7);                                // the unit whose swizzled slot is this lane
+        int m = bm0 + row;
+        if (m >= M) m = M - 1;                                                // rows past the end are computed and never stored
+        a_off[j] = (uint32_t)(((size_t)(m - bm0) * lda + 4 * q) * sizeof(float));
+    }
+#pragma unroll
+    for (int j = 0; j < S::B_LOADS; ++j) {
+        const int kr = (wave * S::B_LOADS + j) * (64 / UB) + lane / UB;      // 64 units = 64 / UB rows of k
+        const int col = clamp_group_col(bn0 + 4 * (lane % UB), N, 4);        // stay inside the operand; such columns are never stored
+        b_off[j] = (uint32_t)(((size_t)kr * ldb + col) * sizeof(float));
+    }
+    int fetch_step = 0;                                // steps whose loads have gone out
+    auto issue_one = [&](int stage, auto j_tag) {
+        constexpr int J = decltype(j_tag)::value;
+        const uint32_t base = lds_base + (uint32_t)stage * (S::STAGE_FLOATS * 4u);
+        if constexpr (J < S::A_LOADS) {
+            dma_load16(a_base, a_off[J], base + (uint32_t)(wave * S::A_LOADS + J) * 1024u);
+        } else {
+            dma_load16(b_base, b_off[J - S::A_LOADS], base + (uint32_t)(S::A_UNITS * 16) + (uint32_t)(wave * S::B_LOADS + J - S::A_LOADS) * 1024u);
+        }
+        if constexpr (J == S::LOADS - 1) {
+            ++fetch_step;
+            const bool more = fetch_step < full_steps;                        // scalar: the pointers stop on the last whole step
+            a_base += more ? BK : 0;
+            b_base += more ? b_step : (size_t)0;
+        }
+    };
+
+    // ---- where this lane's operands lie: unit q of its row of A in every buffer, its column of B in rows s, s+2, ...
+    const float* pa[STAGES][UA];
+    const float* pb[STAGES];
+    {
+        const int row = wm0 + li;
+#pragma unroll
+        for (int st = 0; st < STAGES; ++st) {
+#pragma unroll
+            for (int q = 0; q < UA; ++q) pa[st][q] = lds + st * S::STAGE_FLOATS + (row * UA + (q ^ (row & 7))) * 4 + ls;
+            pb[st] = lds + st * S::STAGE_FLOATS + S::A_UNITS * 4 + ls * S::BN + wn0 + li;
+        }
+    }
+
+    // accumulators: lane holds D[8 (r / 4) + 4 ls + r % 4][li] of its block; the chains start at C when there is one
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        acc[r] = 0.f;
+        if (HAS_C) {
+            const int m = bm0 + wm0 + (r >> 2) * 8 + ls * 4 + (r & 3), n = bn0 + wn0 + li;
+            if (m < M && n < N) acc[r] = Cin[(size_t)m * ldc + n];
+        }
+    }
+
+    // fragment sets: set 0 feeds the first half of a step, set 1 the second
+    float af[2][HALF], bf[2][HALF];
+    // read number n (0 .. HALF-1) of half `h` of the step in buffer `st`: even n an A unit, odd n two rows of B; each
+    // serves MFMAs 2 (n / 2) and 2 (n / 2) + 1 of the half
+    auto read_one = [&](auto st_tag, auto h_tag, auto n_tag) {
+        constexpr int ST = decltype(st_tag)::value, H = decltype(h_tag)::value, NR = decltype(n_tag)::value, U = NR / 2;
+        if constexpr (NR % 2 == 0) {
+            const float* p = pa[ST][H * (HALF / 2) + U];
+            af[H][2 * U] = p[0];
+            af[H][2 * U + 1] = p[2];
+        } else {
+            const float* p = pb[ST] + 2 * (H * HALF + 2 * U) * S::BN;
+            bf[H][2 * U] = p[0];
+            bf[H][2 * U + 1] = p[2 * S::BN];
+        }
+    };
+
+    if (full_steps > 0) {
+        // The walk below is ONE unrolled pass over the STAGES buffers, entered part-way the first time, so that the last
+        // step always ends a pass: step 0 lies in buffer `first`.
+        const int first = (STAGES - full_steps % STAGES) % STAGES;
+        static_for<0, STAGES>([&](auto s_tag) {
+            int stage = first + decltype(s_tag)::value;
+            stage -= stage >= STAGES ? STAGES : 0;
+            static_for<0, S::LOADS>([&](auto j) { issue_one(stage, j); });
+        });
+        wait_dma_then_barrier<S::LOADS*(STAGES - 1)>();                      // step 0 has landed
+        static_for<0, HALF>([&](auto n_tag) {          // first half of step 0, from buffer `first`
+            constexpr int NR = decltype(n_tag)::value, U = NR / 2;
+            const float* p = (NR % 2 == 0 ? pa[0][U] : pb[0] + 4 * U * S::BN) + first * S::STAGE_FLOATS;
+            (NR % 2 == 0 ? af : bf)[0][2 * U] = p[0];
+            (NR % 2 == 0 ? af : bf)[0][2 * U + 1] = p[NR % 2 == 0 ? 2 : 2 * S::BN];
+        });
+
+        auto k_step = [&](auto st_tag) {
+            constexpr int ST = decltype(st_tag)::value;
+            typedef std::integral_constant<int, (ST + 1) % STAGES> NextStage;
+            typedef std::integral_constant<int, 0> H0;
+            typedef std::integral_constant<int, 1> H1;
+            static_for<0, HALF>([&](auto i_tag) {
+                constexpr int I = decltype(i_tag)::value;
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[0][I], bf[0][I], acc, 0, 0, 0);
+                read_one(st_tag, H1{}, i_tag);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            static_for<0, HALF>([&](auto i_tag) {
+                constexpr int I = decltype(i_tag)::value;
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[1][I], bf[1][I], acc, 0, 0, 0);
+                if constexpr (I == 0) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    wait_dma_then_barrier<S::LOADS*(STAGES - 2)>();          // step t+1 has landed; step t's buffer is free
+                } else {
+                    if constexpr (I - 1 < S::LOADS) issue_one(ST, std::integral_constant<int, I - 1>{});
+                    if constexpr (I == 1) read_one(NextStage{}, H0{}, std::integral_constant<int, 0>{});
+                    read_one(NextStage{}, H0{}, i_tag);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        };
+        static_assert(S::LOADS <= HALF - 1, "the loads of a step go out behind MFMAs 1 .. HALF-1 of its second half");
+        int skip = first;
+        for (int t = -first; t < full_steps; t += STAGES) {
+            static_for<0, STAGES>([&](auto st) {
+                if (decltype(st)::value >= skip) k_step(st);
+            });
+            skip = 0;
+        }
+        wait_dma_then_barrier<0>();                                          // nothing is in flight into LDS any more
+    }
+
+    if (rem > 0) {
+        // the ragged last step, through registers into buffer 0: zeros from K on
+        const int k0 = full_steps * BK;
+#pragma unroll
+        for (int p = 0; p < S::A_UNITS / S::NT; ++p) {
+            const int id = tid + p * S::NT, row = id / UA, q = id % UA, k = k0 + 4 * q;
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            if (k < K) {
+                int m = bm0 + row;
+                if (m >= M) m = M - 1;
+                v = *reinterpret_cast<const f32x4*>(A + (size_t)m * lda + k);      // lda % 4 == 0 keeps the quad inside the pitch
+                if (k + 1 >= K) v[1] = 0.f;
+                if (k + 2 >= K) v[2] = 0.f;
+                if (k + 3 >= K) v[3] = 0.f;
+            }
+            *reinterpret_cast<f32x4*>(lds + (row * UA + (q ^ (row & 7))) * 4) = v;
+        }
+#pragma unroll
+        for (int p = 0; p < S::B_UNITS / S::NT; ++p) {
+            const int id = tid + p * S::NT, kr = id / UB, u = id % UB, k = k0 + kr;
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            if (k < K) v = *reinterpret_cast<const f32x4*>(B + (size_t)k * ldb + clamp_group_col(bn0 + 4 * u, N, 4));
+            *reinterpret_cast<f32x4*>(lds + S::A_UNITS * 4 + (kr * UB + u) * 4) = v;
+        }
+        lds_sync();
+        static_for<0, 2>([&](auto h_tag) {
+            constexpr int H = decltype(h_tag)::value;
+            static_for<0, HALF>([&](auto n) { read_one(std::integral_constant<int, 0>{}, h_tag, n); });
+            static_for<0, HALF>([&](auto i_tag) {
+                constexpr int I = decltype(i_tag)::value;
+                if (2 * (H * HALF + I) < rem) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[H][I], bf[H][I], acc, 0, 0, 0);
+            });
+        });
+    }
+
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int m = bm0 + wm0 + (r >> 2) * 8 + ls * 4 + (r & 3), n = bn0 + wn0 + li;
+        if (m < M && n < N) D[(size_t)m * ldd + n] = relu ? relu_by_sign(acc[r]) : acc[r];
+    }
+}
+
+}  // namespace decx_hip

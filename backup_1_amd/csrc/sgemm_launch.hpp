@@ -150,4 +150,23 @@ inline int pick_chain_shape(int M, int N, int K, int batch) {
     return blocks16 <= cus ? 12 : tiles32 > tile_limit ? 0 : cost64 < cost32 ? 13 : 11;
 }
 
+// The 64x64 tiles fed by LDS-DMA loads (sgemm_dma64.hpp) address a tile's rows with 32-bit byte offsets from the
+// tile's first row: 63 rows of a pitch below 2^23 floats stay below 2^31.
+constexpr int kDmaMaxPitch = 1 << 23;
+
+// Which shape of the LDS-DMA kernel a result of M x N takes, or 0 for the other kernels.  Measured on 256 CUs against
+// the automatic choice among the others: ahead from about half a 64x64 tile per CU (768^2: 16.1 -> 14.5 us) to about six
+// (2560^2: 270 -> 266 us), by most around one per CU (1024^3: 23.3 -> 18.3 us, 1024x8192x1024: 158 -> 122 us); below, the
+// block-chain kernels fill more of the chip, above, the big tiles re-use their operands better.  Steps of 64 k in three
+// buffers (96 KiB: one workgroup per CU) are ahead on a long K with at most one tile per CU, steps of 32 k in four
+// buffers (64 KiB: two workgroups share a CU) everywhere else.  All paths give the same bits.
+inline int pick_dma64_shape(int M, int N, int K, int batch) {
+    if (g_rt.sgemm_variant == 18 || g_rt.sgemm_variant == 19) return g_rt.sgemm_variant;
+    if (g_rt.sgemm_variant != 0) return 0;
+    const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+    const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch;
+    if (2 * tiles64 < cus || 4 * tiles64 > 25 * cus) return 0;
+    return tiles64 <= cus && K >= 1024 ? 19 : 18;
+}
+
 }  // namespace decx_hip

@@ -61,6 +61,19 @@ __device__ __forceinline__ float ordered_plane_sum(const float* __restrict__ par
     return v;
 }
 
+// One 16-byte-per-lane load from global memory (wave-uniform base + per-lane byte offset) straight into LDS at
+// lds_base + 16*lane (lds_base wave-uniform).
+__device__ __forceinline__ void dma_load16(const void* sbase, uint32_t lane_off, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 : : "v"(lane_off), "s"(sbase), "s"(lds_base) : "memory", "m0");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_dma_then_barrier() {
+    // my loads older than the N most recent have landed; my LDS reads are done; then everybody meets
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_waitcnt lgkmcnt(0)\n\ts_barrier" : : "n"(N) : "memory");
+}
+
 struct TileCoord {
     int tm, tn;
 };
