@@ -1,12 +1,13 @@
-// fp32 GEMM for results of about one 64x64 tile per CU (1024^3: 256 tiles on 256 CUs): operands go from global memory
+// fp32 GEMM for results of a few tiles per CU (1024^3: 256 tiles of 64x64 on 256 CUs): operands go from global memory
 // straight into LDS, and nothing but matrix instructions and their operand reads runs on the computing waves.
 //
-// With one tile per CU a workgroup is four waves, one per SIMD, and each wave's 32x32 block is ONE dependent chain of
-// v_mfma_f32_32x32x2_f32 (64 cycles each): every other instruction the SIMD has to issue delays that chain.  The
+// A workgroup is four waves, one per SIMD, each owning MI x NI blocks of 32x32.  With one 64x64 tile per CU that is ONE
+// block per wave = one dependent chain of v_mfma_f32_32x32x2_f32 (64 cycles each), and every other instruction the SIMD
+// has to issue delays that chain.  The
 // register-staged kernels spend a global load, two LDS stores and their address arithmetic per 16 bytes of operand;
 // measured on the block-chain kernel at this size, the staging costs a quarter of the matrix pipe's time.  Here a
 // global_load_lds_dwordx4 moves 16 bytes per lane into LDS with no register, no LDS store and no wait on the wave's
-// side: 4 such loads per wave and K step of 32, against 16 MFMAs.
+// side: 4 such loads per wave and K step of 32 on the 64x64 tile, against 16 MFMAs.
 //
 // The price is that LDS holds the operands as they lie in memory, and a lane of the 32x32x2 instruction wants ONE
 // float per operand and instruction: lane (i, s), i = 0..31, s = 0..1, feeds A[i][2j + s] and B[2j + s][i] to MFMA j.
@@ -17,7 +18,8 @@
 //     row, so that the 32 rows of a read spread over all banks (each bank four times -- one float per lane and unit
 //     allows no less).  The swizzle is applied on the global side: the lane whose LDS place is slot t of row r fetches
 //     unit t ^ (r % 8).
-// One LDS read per MFMA in all, issued right behind it.
+// One LDS read per MFMA in all on the 64x64 tile (wave blocks of 2x2 re-use each operand twice: one read per two MFMAs,
+// and four interleaved chains), issued right behind it.
 //
 // Pipeline: STAGES LDS buffers, one barrier per K step.  The step is computed in two halves from two fragment sets:
 // during the first half the second half's fragments are read; the second half starts with the barrier (before it the
@@ -35,9 +37,10 @@
 
 namespace decx_hip {
 
-template <int BK_, int STAGES_>
-struct Dma64 {
-    static constexpr int BM = 64, BN = 64, BK = BK_, STAGES = STAGES_, NWAVES = 4, NT = 64 * NWAVES;
+template <int BM_, int BN_, int BK_, int STAGES_>
+struct DmaTile {
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, STAGES = STAGES_, NWAVES = 4, NT = 64 * NWAVES;
+    static constexpr int WM = BM / 2, WN = BN / 2, MI = WM / 32, NI = WN / 32;      // 2 x 2 waves of MI x NI blocks
     static constexpr int UA = BK / 4;                                   // 16-byte units per row of A and step
     static constexpr int UB = BN / 4;                                   // 16-byte units per row of B
     static constexpr int A_UNITS = BM * UA, B_UNITS = BK * UB;
@@ -45,32 +48,36 @@ struct Dma64 {
     static constexpr int LOADS = A_LOADS + B_LOADS;
     static constexpr int STAGE_FLOATS = (A_UNITS + B_UNITS) * 4;
     static constexpr size_t LDS_BYTES = (size_t)STAGES * STAGE_FLOATS * sizeof(float);
-    static constexpr int HALF = BK / 4;                                 // MFMAs per half step
+    static constexpr int HALF = BK / 4;                                 // k pairs (one MFMA per block each) per half step
+    static constexpr int READS = (MI + NI) * HALF / 2, MFMAS = HALF * MI * NI;       // per half step and wave
+    static_assert(BM % 64 == 0 && BN % 64 == 0 && BN <= 256, "whole blocks per wave; a load covers whole rows of B");
     static_assert(BK % 16 == 0 && UA >= 8 && 64 % UA == 0, "whole units per half step; the swizzle needs 8 slots a row");
     static_assert(A_UNITS % (64 * NWAVES) == 0 && B_UNITS % (64 * NWAVES) == 0, "loads divide over the waves");
     static_assert(STAGES >= 2 && LOADS * (STAGES - 1) <= 63, "vmcnt is a 6-bit counter");
+    static_assert(LOADS <= MFMAS - 1 && READS <= MFMAS, "loads and reads go out behind the MFMAs of a half step");
 };
 
 template <class S, bool HAS_C>
-__global__ __launch_bounds__(S::NT) void sgemm_dma64_kernel(const float* __restrict__ A, int lda, const float* __restrict__ B,
-                                                            int ldb, const float* Cin, int ldc, float* D, int ldd, int M, int N,
-                                                            int K, int tiles_m, int tiles_n, int group_m, bool relu,
-                                                            size_t a_batch_stride, size_t b_batch_stride, size_t c_batch_stride,
-                                                            size_t d_batch_stride) {
-    constexpr int BK = S::BK, UA = S::UA, UB = S::UB, STAGES = S::STAGES, HALF = S::HALF;
+__global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restrict__ A, int lda, const float* __restrict__ B,
+                                                          int ldb, const float* Cin, int ldc, float* D, int ldd, int M, int N,
+                                                          int K, int tiles_m, int tiles_n, int group_m, bool relu,
+                                                          size_t a_batch_stride, size_t b_batch_stride, size_t c_batch_stride,
+                                                          size_t d_batch_stride) {
+    constexpr int BK = S::BK, UA = S::UA, UB = S::UB, STAGES = S::STAGES, HALF = S::HALF, MI = S::MI, NI = S::NI;
+    constexpr int READS = S::READS, MFMAS = S::MFMAS;
     A += (size_t)blockIdx.y * a_batch_stride;
     B += (size_t)blockIdx.y * b_batch_stride;
     if (HAS_C) Cin += (size_t)blockIdx.y * c_batch_stride;
     D += (size_t)blockIdx.y * d_batch_stride;
-    extern __shared__ __attribute__((aligned(16))) float lds[];      // [STAGES][A: 64 rows x UA units | B: BK rows x 16 units]
+    extern __shared__ __attribute__((aligned(16))) float lds[];      // [STAGES][A: BM rows x UA units | B: BK rows x UB units]
     const uint32_t lds_base = lds_byte_address(lds);
 
     const TileCoord tc = xcd_grouped_tile(blockIdx.x, tiles_m, tiles_n, group_m);
     const int bm0 = tc.tm * S::BM, bn0 = tc.tn * S::BN;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
-    const int wm0 = (wave / 2) * 32, wn0 = (wave % 2) * 32;
-    const int li = lane % 32, ls = lane / 32;          // row (of A) or column (of B) inside the wave's block, and k-slot
+    const int wm0 = (wave / 2) * S::WM, wn0 = (wave % 2) * S::WN;
+    const int li = lane % 32, ls = lane / 32;          // row (of A) or column (of B) inside a block, and k-slot
     const int full_steps = K / BK, rem = K - full_steps * BK;
 
     // ---- sources of this wave's loads: a wave-uniform base per operand that moves one K step per fetched step, plus
@@ -110,46 +117,63 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma64_kernel(const float* __restr
         }
     };
 
-    // ---- where this lane's operands lie: unit q of its row of A in every buffer, its column of B in rows s, s+2, ...
-    const float* pa[STAGES][UA];
-    const float* pb[STAGES];
-    {
-        const int row = wm0 + li;
+    // ---- where this lane's operands lie: unit q of its row of every row block of A in every buffer, its column of every
+    // column block of B in rows s, s+2, ...
+    const float* pa[STAGES][MI][UA];
+    const float* pb[STAGES][NI];
 #pragma unroll
-        for (int st = 0; st < STAGES; ++st) {
+    for (int st = 0; st < STAGES; ++st) {
 #pragma unroll
-            for (int q = 0; q < UA; ++q) pa[st][q] = lds + st * S::STAGE_FLOATS + (row * UA + (q ^ (row & 7))) * 4 + ls;
-            pb[st] = lds + st * S::STAGE_FLOATS + S::A_UNITS * 4 + ls * S::BN + wn0 + li;
+        for (int mi = 0; mi < MI; ++mi) {
+            const int row = wm0 + 32 * mi + li;
+#pragma unroll
+            for (int q = 0; q < UA; ++q) pa[st][mi][q] = lds + st * S::STAGE_FLOATS + (row * UA + (q ^ (row & 7))) * 4 + ls;
         }
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) pb[st][ni] = lds + st * S::STAGE_FLOATS + S::A_UNITS * 4 + ls * S::BN + wn0 + 32 * ni + li;
     }
 
-    // accumulators: lane holds D[8 (r / 4) + 4 ls + r % 4][li] of its block; the chains start at C when there is one
-    f32x16 acc;
+    // accumulators: lane holds D[8 (r / 4) + 4 ls + r % 4][li] of each of its blocks; the chains start at C when there is one
+    f32x16 acc[MI][NI];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        acc[r] = 0.f;
-        if (HAS_C) {
-            const int m = bm0 + wm0 + (r >> 2) * 8 + ls * 4 + (r & 3), n = bn0 + wn0 + li;
-            if (m < M && n < N) acc[r] = Cin[(size_t)m * ldc + n];
-        }
-    }
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                acc[mi][ni][r] = 0.f;
+                if (HAS_C) {
+                    const int m = bm0 + wm0 + 32 * mi + (r >> 2) * 8 + ls * 4 + (r & 3), n = bn0 + wn0 + 32 * ni + li;
+                    if (m < M && n < N) acc[mi][ni][r] = Cin[(size_t)m * ldc + n];
+                }
+            }
 
     // fragment sets: set 0 feeds the first half of a step, set 1 the second
-    float af[2][HALF], bf[2][HALF];
-    // read number n (0 .. HALF-1) of half `h` of the step in buffer `st`: even n an A unit, odd n two rows of B; each
-    // serves MFMAs 2 (n / 2) and 2 (n / 2) + 1 of the half
-    auto read_one = [&](auto st_tag, auto h_tag, auto n_tag) {
-        constexpr int ST = decltype(st_tag)::value, H = decltype(h_tag)::value, NR = decltype(n_tag)::value, U = NR / 2;
-        if constexpr (NR % 2 == 0) {
-            const float* p = pa[ST][H * (HALF / 2) + U];
-            af[H][2 * U] = p[0];
-            af[H][2 * U + 1] = p[2];
+    float af[2][HALF][MI], bf[2][HALF][NI];
+    // Read number n (0 .. READS-1) of half `h` of the step that lies `stage_floats` past the pointers of buffer ST: reads
+    // (MI + NI) u .. (MI + NI) u + MI + NI - 1 fetch the operands of k pairs 2u and 2u + 1 of the half -- an A unit per
+    // row block, then two rows of B per column block.
+    auto read_one = [&](auto st_tag, auto h_tag, auto n_tag, int stage_floats) {
+        constexpr int ST = decltype(st_tag)::value, H = decltype(h_tag)::value, NR = decltype(n_tag)::value;
+        constexpr int U = NR / (MI + NI), W = NR % (MI + NI);
+        if constexpr (W < MI) {
+            const float* p = pa[ST][W][H * (HALF / 2) + U] + stage_floats;
+            af[H][2 * U][W] = p[0];
+            af[H][2 * U + 1][W] = p[2];
         } else {
-            const float* p = pb[ST] + 2 * (H * HALF + 2 * U) * S::BN;
-            bf[H][2 * U] = p[0];
-            bf[H][2 * U + 1] = p[2 * S::BN];
+            const float* p = pb[ST][W - MI] + 2 * (H * HALF + 2 * U) * S::BN + stage_floats;
+            bf[H][2 * U][W - MI] = p[0];
+            bf[H][2 * U + 1][W - MI] = p[2 * S::BN];
         }
     };
+    // MFMA number m (0 .. MFMAS-1) of half `h`: k pair m / (MI NI) of the half, blocks in turn
+    auto mfma_one = [&](auto h_tag, auto m_tag) {
+        constexpr int H = decltype(h_tag)::value, MM = decltype(m_tag)::value;
+        constexpr int I = MM / (MI * NI), BMI = (MM / NI) % MI, BNI = MM % NI;
+        acc[BMI][BNI] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[H][I][BMI], bf[H][I][BNI], acc[BMI][BNI], 0, 0, 0);
+    };
+    typedef std::integral_constant<int, 0> I0;
+    typedef std::integral_constant<int, 1> I1;
 
     if (full_steps > 0) {
         // The walk below is ONE unrolled pass over the STAGES buffers, entered part-way the first time, so that the last
@@ -161,39 +185,37 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma64_kernel(const float* __restr
             static_for<0, S::LOADS>([&](auto j) { issue_one(stage, j); });
         });
         wait_dma_then_barrier<S::LOADS*(STAGES - 1)>();                      // step 0 has landed
-        static_for<0, HALF>([&](auto n_tag) {          // first half of step 0, from buffer `first`
-            constexpr int NR = decltype(n_tag)::value, U = NR / 2;
-            const float* p = (NR % 2 == 0 ? pa[0][U] : pb[0] + 4 * U * S::BN) + first * S::STAGE_FLOATS;
-            (NR % 2 == 0 ? af : bf)[0][2 * U] = p[0];
-            (NR % 2 == 0 ? af : bf)[0][2 * U + 1] = p[NR % 2 == 0 ? 2 : 2 * S::BN];
-        });
+        static_for<0, READS>([&](auto n) { read_one(I0{}, I0{}, n, first * S::STAGE_FLOATS); });      // its first half
 
         auto k_step = [&](auto st_tag) {
             constexpr int ST = decltype(st_tag)::value;
             typedef std::integral_constant<int, (ST + 1) % STAGES> NextStage;
-            typedef std::integral_constant<int, 0> H0;
-            typedef std::integral_constant<int, 1> H1;
-            static_for<0, HALF>([&](auto i_tag) {
-                constexpr int I = decltype(i_tag)::value;
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[0][I], bf[0][I], acc, 0, 0, 0);
-                read_one(st_tag, H1{}, i_tag);
+            // first half: read n goes out behind MFMA n MFMAS / READS
+            static_for<0, MFMAS>([&](auto m_tag) {
+                constexpr int MM = decltype(m_tag)::value;
+                mfma_one(I0{}, m_tag);
+                static_for<0, READS>([&](auto n_tag) {
+                    if constexpr (decltype(n_tag)::value * MFMAS / READS == MM) read_one(st_tag, I1{}, n_tag, 0);
+                });
                 __builtin_amdgcn_sched_barrier(0);
             });
-            static_for<0, HALF>([&](auto i_tag) {
-                constexpr int I = decltype(i_tag)::value;
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[1][I], bf[1][I], acc, 0, 0, 0);
-                if constexpr (I == 0) {
+            // second half: the barrier behind its first MFMA, then the loads of step t+STAGES behind MFMAs 1, 2, ... and
+            // read n of the next step's first half behind MFMA 1 + n (MFMAS - 1) / READS
+            static_for<0, MFMAS>([&](auto m_tag) {
+                constexpr int MM = decltype(m_tag)::value;
+                mfma_one(I1{}, m_tag);
+                if constexpr (MM == 0) {
                     __builtin_amdgcn_sched_barrier(0);
                     wait_dma_then_barrier<S::LOADS*(STAGES - 2)>();          // step t+1 has landed; step t's buffer is free
                 } else {
-                    if constexpr (I - 1 < S::LOADS) issue_one(ST, std::integral_constant<int, I - 1>{});
-                    if constexpr (I == 1) read_one(NextStage{}, H0{}, std::integral_constant<int, 0>{});
-                    read_one(NextStage{}, H0{}, i_tag);
+                    if constexpr (MM - 1 < S::LOADS) issue_one(ST, std::integral_constant<int, MM - 1>{});
+                    static_for<0, READS>([&](auto n_tag) {
+                        if constexpr (1 + decltype(n_tag)::value * (MFMAS - 1) / READS == MM) read_one(NextStage{}, I0{}, n_tag, 0);
+                    });
                 }
                 __builtin_amdgcn_sched_barrier(0);
             });
         };
-        static_assert(S::LOADS <= HALF - 1, "the loads of a step go out behind MFMAs 1 .. HALF-1 of its second half");
         int skip = first;
         for (int t = -first; t < full_steps; t += STAGES) {
             static_for<0, STAGES>([&](auto st) {
@@ -231,19 +253,26 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma64_kernel(const float* __restr
         lds_sync();
         static_for<0, 2>([&](auto h_tag) {
             constexpr int H = decltype(h_tag)::value;
-            static_for<0, HALF>([&](auto n) { read_one(std::integral_constant<int, 0>{}, h_tag, n); });
-            static_for<0, HALF>([&](auto i_tag) {
-                constexpr int I = decltype(i_tag)::value;
-                if (2 * (H * HALF + I) < rem) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[H][I], bf[H][I], acc, 0, 0, 0);
+            static_for<0, READS>([&](auto n) { read_one(I0{}, h_tag, n, 0); });
+            static_for<0, MFMAS>([&](auto m_tag) {
+                if (2 * (H * HALF + decltype(m_tag)::value / (MI * NI)) < rem) mfma_one(h_tag, m_tag);
             });
         });
     }
 
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int m = bm0 + wm0 + (r >> 2) * 8 + ls * 4 + (r & 3), n = bn0 + wn0 + li;
-        if (m < M && n < N) D[(size_t)m * ldd + n] = relu ? relu_by_sign(acc[r]) : acc[r];
-    }
+    for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = bm0 + wm0 + 32 * mi + (r >> 2) * 8 + ls * 4 + (r & 3);
+            if (m < M) {
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni) {
+                    const int n = bn0 + wn0 + 32 * ni + li;
+                    if (n < N) D[(size_t)m * ldd + n] = relu ? relu_by_sign(acc[mi][ni][r]) : acc[mi][ni][r];
+                }
+            }
+        }
 }
 
 }  // namespace decx_hip

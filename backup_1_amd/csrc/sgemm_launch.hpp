@@ -150,7 +150,7 @@ inline int pick_chain_shape(int M, int N, int K, int batch) {
     return blocks16 <= cus ? 12 : tiles32 > tile_limit ? 0 : cost64 < cost32 ? 13 : 11;
 }
 
-// The 64x64 tiles fed by LDS-DMA loads (sgemm_dma64.hpp) address a tile's rows with 32-bit byte offsets from the
+// The 64x64 tiles fed by LDS-DMA loads (sgemm_dma_tile.hpp) address a tile's rows with 32-bit byte offsets from the
 // tile's first row: 63 rows of a pitch below 2^23 floats stay below 2^31.
 constexpr int kDmaMaxPitch = 1 << 23;
 
@@ -159,12 +159,16 @@ constexpr int kDmaMaxPitch = 1 << 23;
 // (2560^2: 270 -> 266 us), by most around one per CU (1024^3: 23.3 -> 18.3 us, 1024x8192x1024: 158 -> 122 us); below, the
 // block-chain kernels fill more of the chip, above, the big tiles re-use their operands better.  Steps of 64 k in three
 // buffers (96 KiB: one workgroup per CU) are ahead on a long K with at most one tile per CU, steps of 32 k in four
-// buffers (64 KiB: two workgroups share a CU) everywhere else.  All paths give the same bits.
-inline int pick_dma64_shape(int M, int N, int K, int batch) {
-    if (g_rt.sgemm_variant == 18 || g_rt.sgemm_variant == 19) return g_rt.sgemm_variant;
+// buffers (64 KiB: two workgroups share a CU) everywhere else.  Shapes 20 - 22 are 128x128, 64x128 and 128x64 tiles of
+// the same kernel; only the first is chosen automatically.  All paths give the same bits.
+inline int pick_dma_shape(int M, int N, int K, int batch) {
+    if (g_rt.sgemm_variant >= 18 && g_rt.sgemm_variant <= 22) return g_rt.sgemm_variant;
     if (g_rt.sgemm_variant != 0) return 0;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
-    const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch;
+    const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch, tiles128 = (long)cdiv(M, 128) * cdiv(N, 128) * batch;
+    // one 128x128 tile (2 x 2 blocks a wave, each operand read once for two blocks) on nearly every CU:
+    // 2048^3 128.5 -> 124.4 us, 2048x8192x2048 501 -> 476 us (144 TFLOP/s)
+    if (tiles128 <= cus && 10 * tiles128 >= 9 * cus) return 20;
     if (2 * tiles64 < cus || 4 * tiles64 > 25 * cus) return 0;
     return tiles64 <= cus && K >= 1024 ? 19 : 18;
 }
