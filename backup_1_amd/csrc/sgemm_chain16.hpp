@@ -20,6 +20,9 @@
 //   T = 1: a 16x16 tile, one computing wave and two moving waves -- three waves on three different SIMDs of a CU, so
 //          the chain runs undisturbed: for results of at most one block per CU (241 ns per chunk, against 218 for bare
 //          MFMAs);
+//   1 x 2: a 16x32 tile, two computing and two moving waves -- four waves on the four SIMDs of a CU, the chains as
+//          undisturbed as in the 16x16 shape, A staged once for both blocks and B in whole 128-byte lines: for results
+//          of more than one 16x16 block per CU but at most one such tile (14x14x512 under 512 filters: 208 tiles);
 //   T = 2: a 32x32 tile, 2x2 computing waves and four moving waves, one of each per SIMD: half the staging work per
 //          block (A and B tiles are shared) but it runs on the computing waves' SIMDs: for more blocks than CUs.  Built
 //          with 4 register sets for 128 registers, so that two workgroups share a CU and one's MFMAs fill the gaps
@@ -44,14 +47,14 @@
 
 namespace decx_hip {
 
-// T x T blocks of 16x16 per workgroup tile; a computing wave owns NB blocks that lie side by side (NB independent chains,
+// TM x TN blocks of 16x16 per workgroup tile; a computing wave owns NB blocks that lie side by side (NB independent chains,
 // interleaved, sharing the A operands); DEPTH_ register sets; WAVES_PER_SIMD_ is what the register budget is cut for.
-template <int T, int NB_, int DEPTH_, int WAVES_PER_SIMD_>
-struct Chain16 {
-    static_assert((T == 1 || T == 2 || T == 4) && T % NB_ == 0, "tiles of 1x1, 2x2 or 4x4 blocks");
+template <int TM, int TN, int NB_, int DEPTH_, int WAVES_PER_SIMD_>
+struct Chain16Rect {
+    static_assert((TM == 1 || TM == 2 || TM == 4) && (TN == 1 || TN == 2 || TN == 4) && TN % NB_ == 0, "tiles of 1, 2 or 4 blocks a side");
     static constexpr int WAVES_PER_SIMD = WAVES_PER_SIMD_;
-    static constexpr int BM = 16 * T, BN = 16 * T, BK = 64, NB = NB_;
-    static constexpr int COMPUTE_WAVES = T * T / NB, MOVE_THREADS = T == 1 ? 128 : 256;
+    static constexpr int BM = 16 * TM, BN = 16 * TN, BK = 64, NB = NB_;
+    static constexpr int COMPUTE_WAVES = TM * TN / NB, MOVE_THREADS = TM * TN <= 2 ? 128 : 256;
     static constexpr int NT = 64 * COMPUTE_WAVES + MOVE_THREADS;     // computing waves first, then the moving waves
     static constexpr int PA = 16 * BM / MOVE_THREADS, PB = 16 * BN / MOVE_THREADS;   // quads of A and of B per moving thread and chunk
     static constexpr int DEPTH = DEPTH_;                             // register sets: chunks of K in flight from global memory (even)
@@ -60,8 +63,10 @@ struct Chain16 {
     static constexpr int A_FLOATS = 4 * A_PLANE, B_FLOATS = 4 * B_PLANE;
     static constexpr int LDS_BUFFERS = 3;
     static constexpr size_t LDS_BYTES = LDS_BUFFERS * (size_t)(A_FLOATS + B_FLOATS) * sizeof(float);
-    static_assert(16 * BM % MOVE_THREADS == 0 && NT <= 1024, "staging divides evenly");
+    static_assert(16 * BM % MOVE_THREADS == 0 && 16 * BN % MOVE_THREADS == 0 && NT <= 1024, "staging divides evenly");
 };
+template <int T, int NB_, int DEPTH_, int WAVES_PER_SIMD_>
+using Chain16 = Chain16Rect<T, T, NB_, DEPTH_, WAVES_PER_SIMD_>;
 
 // two floats to LDS, OFF0 and OFF1 dwords past byte_addr (each below 256)
 template <int OFF0, int OFF1>

@@ -76,6 +76,7 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
         FilterB<false> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
         if (chain == 11) return launch_conv_chain16<Chain16<2, 1, 4, 4>>(a, b, bias, dst, out, M, N, K);
         if (chain == 12) return launch_conv_chain16<Chain16<1, 1, 8, 2>>(a, b, bias, dst, out, M, N, K);
+        if (chain == 23) return launch_conv_chain16<Chain16Rect<1, 2, 1, 6, 2>>(a, b, bias, dst, out, M, N, K);
         return launch_conv_chain16<Chain16<4, 2, 2, 3>>(a, b, bias, dst, out, M, N, K);
     }
     if (dpitch % 16 == 0) {      // a whole K step inside one tap: the tap walk runs on the scalar unit

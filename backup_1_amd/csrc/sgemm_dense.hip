@@ -102,6 +102,7 @@ int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float*
         if (chain == 11) return launch_sgemm_chain16<Chain16<2, 1, 4, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
         if (chain == 12) return launch_sgemm_chain16<Chain16<1, 1, 8, 2>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
         if (chain == 13) return launch_sgemm_chain16<Chain16<4, 2, 2, 3>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+        if (chain == 23) return launch_sgemm_chain16<Chain16Rect<1, 2, 1, 6, 2>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
     }
     if (vec_a && vec_b) {
         DenseA<true> a{A, lda, M, K, batch.stride_a};

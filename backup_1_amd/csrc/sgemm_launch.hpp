@@ -135,7 +135,7 @@ int dispatch_sgemm(int variant, const ASrc& a, const BSrc& b, const float* Cin, 
 // Measured: ahead of the tiles up to about ten 32x32 tiles per CU -- 1536x1536 on 256 CUs -- 1.7x at 1024x8192x1024, 9x at
 // 64x65536x1024.  All paths give the same bits, so this is a choice of speed only.
 inline int pick_chain_shape(int M, int N, int K, int batch) {
-    if (g_rt.sgemm_variant >= 11 && g_rt.sgemm_variant <= 13) return g_rt.sgemm_variant;
+    if ((g_rt.sgemm_variant >= 11 && g_rt.sgemm_variant <= 13) || g_rt.sgemm_variant == 23) return g_rt.sgemm_variant;
     if ((g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) || g_rt.sgemm_variant >= 14) return 0;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     const long blocks16 = (long)cdiv(M, 16) * cdiv(N, 16) * batch, tiles32 = (long)cdiv(M, 32) * cdiv(N, 32) * batch;
@@ -147,7 +147,11 @@ inline int pick_chain_shape(int M, int N, int K, int batch) {
     const double cost64 = 1.55 * (double)((tiles64 + cus - 1) / cus), pairs = (double)tiles32 / (2.0 * cus);
     const double cost32 = pairs <= 1.0 ? 1.0 : 0.9 * (pairs + 0.5);
     const long tile_limit = (K >= 1024 ? 10 : 4) * cus;
-    return blocks16 <= cus ? 12 : tiles32 > tile_limit ? 0 : cost64 < cost32 ? 13 : 11;
+    // At most one 16x16 block per CU: shape 12.  More, but at most one 16x32 tile per CU: shape 23, whose chains run as
+    // undisturbed (128x16384x1024: 98.6 -> 59.5 us, 196x4608x512: 29.9 -> 18.9 us, 64x65536x2048: 389 -> 319 us).
+    if (blocks16 <= cus) return 12;
+    if ((long)cdiv(M, 16) * cdiv(N, 32) * batch <= cus) return 23;
+    return tiles32 > tile_limit ? 0 : cost64 < cost32 ? 13 : 11;
 }
 
 // The 64x64 tiles fed by LDS-DMA loads (sgemm_dma_tile.hpp) address a tile's rows with 32-bit byte offsets from the

@@ -15,7 +15,7 @@ CASES = [  # H, W, C, N, kh, kw, flag
 ]
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 15, 16, 17])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 15, 16, 17, 23])
 @pytest.mark.parametrize("case", CASES)
 def test_integer_exact(gpu, oracle, case, variant):
     H, W, C, N, kh, kw, flag = case
@@ -24,7 +24,7 @@ def test_integer_exact(gpu, oracle, case, variant):
     assert np.array_equal(gpu_conv(src, filt, flag, variant=variant), oracle.conv2_chain(src, filt, flag))
 
 
-@pytest.mark.parametrize("variant", [0, 2, 6, 7, 8, 11, 12, 13, 15, 16, 17])
+@pytest.mark.parametrize("variant", [0, 2, 6, 7, 8, 11, 12, 13, 15, 16, 17, 23])
 @pytest.mark.parametrize("case", CASES)
 def test_real_valued_data_bit_exact_with_the_chain(gpu, oracle, case, variant):
     # channel counts 3, 4, 6, 8, 12-ish exercise both loader builds (channel pitch a multiple of 8 or only of 4)
@@ -56,7 +56,7 @@ def test_config4_224x224x64_128_filters(gpu, oracle):
     src, filt = workloads.conv_case()
     ref = oracle.conv2_chain(src, filt, 1)
     # same arithmetic as the reference's lowered GEMM (single fused chain over k = (ki*kw + kj)*dpitch + c): same bits
-    for variant in (0, 1, 2, 3, 4, 7, 11, 13, 15, 17):
+    for variant in (0, 1, 2, 3, 4, 7, 11, 13, 15, 17, 23):
         assert np.array_equal(gpu_conv(src, filt, 1, variant=variant).view(np.uint32), ref.view(np.uint32)), variant
     si, fi = workloads.small_ints((224, 224, 64), 71, -4, 4), workloads.small_ints((128, 3, 3, 64), 72, -4, 4)
     assert np.array_equal(gpu_conv(si, fi, 1), oracle.conv2_chain(si, fi, 1))

@@ -20,7 +20,7 @@ def test_random_gemms_bit_exact(gpu, oracle, seed):
     for case in range(10):
         M, N = int(rng.integers(1, 420)), int(rng.integers(1, 420))
         K = int(rng.choice([int(rng.integers(1, 70)), int(rng.integers(1, 700))]))
-        variant = int(rng.integers(0, 23))
+        variant = int(rng.integers(0, 24))
         align = int(rng.choice([8, 8, 4, 1]))          # DECX pitch, a 16-byte pitch, an unaligned pitch
         with_c, relu = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
         A, B = workloads.normal((M, K), 100 * seed + case), workloads.normal((K, N), 100 * seed + case + 50)
@@ -39,7 +39,7 @@ def test_random_convolutions_bit_exact(gpu, oracle, seed):
         kh, kw = int(rng.choice([1, 3, 5, 7])), int(rng.choice([1, 3, 5, 7]))
         H, W = int(rng.integers(kh, 40)), int(rng.integers(kw, 40))
         C, N = int(rng.integers(1, 40)), int(rng.integers(1, 150))
-        flag, variant = int(rng.integers(0, 2)), int(rng.choice(list(range(14)) + [15, 16, 17]))
+        flag, variant = int(rng.integers(0, 2)), int(rng.choice(list(range(14)) + [15, 16, 17, 23]))
         src = workloads.normal((H, W, C), 300 * seed + case)
         filt = workloads.normal((N, kh, kw, C), 300 * seed + case + 150)
         ref = oracle.conv2_chain(src, filt, flag)
