@@ -413,11 +413,16 @@ def main():
                              "frac_of_fp32_matrix_peak": round(r["tflops_kernel"] / PEAK_FP32_MATRIX_TFLOPS, 4)}
         log("fp32 4096^3: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
     if want("small"):
-        # results too small to fill the chip with 256x256 tiles: the one-wave-per-16x16-block kernel takes them
+        # results too small to fill the chip with 256x256 tiles: 64x64 tiles fed by LDS-DMA loads (one per CU at
+        # 1024 x 1024), the one-wave-per-16x16-block kernel for the thin long-K product below
         r = bench_sgemm(capi, workloads, 1024, 1024, 1024, side_steps, side_warmup, 77)
         also["fp32_1024"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
                              "frac_of_fp32_matrix_peak": round(r["tflops_kernel"] / PEAK_FP32_MATRIX_TFLOPS, 4)}
         log("fp32 1024^3: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+        r = bench_sgemm(capi, workloads, 1024, 8192, 1024, side_steps, side_warmup, 76)
+        also["fp32_1024x8192x1024"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
+                                       "frac_of_fp32_matrix_peak": round(r["tflops_kernel"] / PEAK_FP32_MATRIX_TFLOPS, 4)}
+        log("fp32 1024x8192x1024: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
         r = bench_sgemm(capi, workloads, 64, 65536, 1024, side_steps, side_warmup, 78)
         # one fused chain per output cannot be split over K: the bound is 8 cycles per k of a single MFMA chain
         chain_ms = 65536 / 4 * 32 / (info["clock_khz"] * 1e3) * 1e3
