@@ -54,10 +54,14 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //         carries a 4-block and a 3-block wave
 //  17: 208x128x16, 2x4 waves of 112x32 (three 32-row blocks and one of 16 rows on v_mfma_f32_16x16x4_f32) and 96x32:
 //         convolution only (filter-bank B); 6 1/2 blocks per SIMD for results whose rows fill the CUs badly in steps of 32
-// and, for dense GEMM only, the one-wave-per-16x16-block kernel of sgemm_chain16.hpp:
+// the one-wave-per-16x16-block kernel of sgemm_chain16.hpp (dense GEMM and small-image convolutions):
 //  11:  32x32x64,  2x2 computing + 4 moving waves, two workgroups per CU -- results too small to fill the chip with tiles
 //  12:  16x16x64,  1 computing + 2 moving waves -- at most one 16x16 block per CU: the fastest a single chain can walk K
 //  13:  64x64x64,  8 computing waves of two blocks each + 4 moving waves -- results of about one such tile per CU (1024^2)
+//  23:  16x32x64,  2 computing + 2 moving waves, one per SIMD -- at most one such tile per CU
+// and, for dense GEMM only, the tiles fed by LDS-DMA loads of sgemm_dma_tile.hpp (2x2 waves, one per SIMD):
+//  18:  64x64, K steps of 32 in 4 LDS buffers     19:  64x64, K steps of 64 in 3 buffers
+//  20: 128x128 (2x2 blocks per wave), 21: 64x128, 22: 128x64, K steps of 32 in 4 buffers
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
 typedef SgemmShape<128, 128, 16, 2, 2, 2> SShapeSmall;
 typedef SgemmShape<256, 128, 16, 2, 2, 2> SShapeTall;
