@@ -96,6 +96,8 @@ int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float*
         if (dma == 20) return launch_sgemm_dma<DmaTile<128, 128, 32, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
         if (dma == 21) return launch_sgemm_dma<DmaTile<64, 128, 32, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
         if (dma == 22) return launch_sgemm_dma<DmaTile<128, 64, 32, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+        if (dma == 24) return launch_sgemm_dma<DmaTile<32, 32, 64, 3, 16>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+        if (dma == 25) return launch_sgemm_dma<DmaTile<64, 32, 64, 3, 16>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
     }
     if (vec_a && vec_b) {
         const int chain = pick_chain_shape(M, N, K, batch.count);

@@ -21,6 +21,15 @@
 // One LDS read per MFMA in all on the 64x64 tile (wave blocks of 2x2 re-use each operand twice: one read per two MFMAs,
 // and four interleaved chains), issued right behind it.
 //
+// The same kernel on 16x16 blocks (v_mfma_f32_16x16x4_f32: four k per instruction, 32 cycles, so a chain walks K twice
+// as fast) serves results with fewer than four 32x32 blocks per CU, and results whose 64x64 tiles fill the last round of
+// CUs badly.  Lane (i, s), i = 0..15, s = 0..3, feeds A[i][4j + s] and B[4j + s][i] to MFMA j: float s of unit j of its row
+// of A -- ONE ds_read_b32 per MFMA, the 16 rows of a read in 8 different slots, so every bank serves two lanes, which is
+// all 64 lanes on 32 banks can have; reading two units with one ds_read2_b32 ties the slots of a row to pairs, leaves
+// four lanes on a bank, and with four waves reading made the LDS the bound (384x8192x384: 41.4 us against 32.9) -- and
+// 16 consecutive floats of row 4j + s of B, where the units of odd rows swap halves of 32 columns so that the four rows
+// of a read cover all banks twice; rows 4j + s and 4j + 4 + s again come with one read.
+//
 // Pipeline: STAGES LDS buffers, one barrier per K step.  The step is computed in two halves from two fragment sets:
 // during the first half the second half's fragments are read; the second half starts with the barrier (before it the
 // wave waits for its own loads of step t+1, after it nobody reads step t's buffer any more), then issues the loads of
@@ -37,10 +46,15 @@
 
 namespace decx_hip {
 
-template <int BM_, int BN_, int BK_, int STAGES_>
+// BLK_ = 32: blocks of 32x32 on v_mfma_f32_32x32x2_f32 (two k per instruction, 64 cycles); BLK_ = 16: blocks of 16x16 on
+// v_mfma_f32_16x16x4_f32 (four k per instruction, 32 cycles: a chain walks K twice as fast), for results with fewer
+// than four 32x32 blocks per CU.
+template <int BM_, int BN_, int BK_, int STAGES_, int BLK_ = 32>
 struct DmaTile {
-    static constexpr int BM = BM_, BN = BN_, BK = BK_, STAGES = STAGES_, NWAVES = 4, NT = 64 * NWAVES;
-    static constexpr int WM = BM / 2, WN = BN / 2, MI = WM / 32, NI = WN / 32;      // 2 x 2 waves of MI x NI blocks
+    static constexpr bool APAIR = BLK_ == 32;                         // one read of A serves two MFMAs of a block
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, STAGES = STAGES_, BLK = BLK_, NWAVES = 4, NT = 64 * NWAVES;
+    static constexpr int WM = BM / 2, WN = BN / 2, MI = WM / BLK, NI = WN / BLK;    // 2 x 2 waves of MI x NI blocks
+    static constexpr int KI = BLK == 32 ? 2 : 4;                        // k per instruction
     static constexpr int UA = BK / 4;                                   // 16-byte units per row of A and step
     static constexpr int UB = BN / 4;                                   // 16-byte units per row of B
     static constexpr int A_UNITS = BM * UA, B_UNITS = BK * UB;
@@ -48,13 +62,17 @@ struct DmaTile {
     static constexpr int LOADS = A_LOADS + B_LOADS;
     static constexpr int STAGE_FLOATS = (A_UNITS + B_UNITS) * 4;
     static constexpr size_t LDS_BYTES = (size_t)STAGES * STAGE_FLOATS * sizeof(float);
-    static constexpr int HALF = BK / 4;                                 // k pairs (one MFMA per block each) per half step
-    static constexpr int READS = (MI + NI) * HALF / 2, MFMAS = HALF * MI * NI;       // per half step and wave
-    static_assert(BM % 64 == 0 && BN % 64 == 0 && BN <= 256, "whole blocks per wave; a load covers whole rows of B");
+    // slot of unit q of row `row` of A inside its row, and of unit u of row k of B (see the header)
+    __device__ static constexpr int a_slot(int row, int q) { return q ^ (row & 7); }
+    __device__ static constexpr int b_slot(int k, int u) { return BLK == 32 ? u : u ^ (4 * (k & 1)); }
+    static constexpr int HALF = BK / KI / 2;                            // MFMAs per block and half step
+    static constexpr int READS = ((APAIR ? MI : 2 * MI) + NI) * HALF / 2, MFMAS = HALF * MI * NI;       // per half step and wave
+    static_assert((BLK == 32 || BLK == 16) && BM % (2 * BLK) == 0 && BN % (2 * BLK) == 0 && BN <= 256 && UB >= 8 && 64 % UB == 0,
+                  "whole blocks per wave; a load covers whole rows of B");
     static_assert(BK % 16 == 0 && UA >= 8 && 64 % UA == 0, "whole units per half step; the swizzle needs 8 slots a row");
     static_assert(A_UNITS % (64 * NWAVES) == 0 && B_UNITS % (64 * NWAVES) == 0, "loads divide over the waves");
     static_assert(STAGES >= 2 && LOADS * (STAGES - 1) <= 63, "vmcnt is a 6-bit counter");
-    static_assert(LOADS <= MFMAS - 1 && READS <= MFMAS, "loads and reads go out behind the MFMAs of a half step");
+    static_assert(LOADS <= MFMAS - 1, "the loads go out behind the MFMAs of a half step");
 };
 
 template <class S, bool HAS_C>
@@ -77,7 +95,7 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restric
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
     const int wm0 = (wave / 2) * S::WM, wn0 = (wave % 2) * S::WN;
-    const int li = lane % 32, ls = lane / 32;          // row (of A) or column (of B) inside a block, and k-slot
+    const int li = lane % S::BLK, ls = lane / S::BLK;  // row (of A) or column (of B) inside a block, and k-slot
     const int full_steps = K / BK, rem = K - full_steps * BK;
 
     // ---- sources of this wave's loads: a wave-uniform base per operand that moves one K step per fetched step, plus
@@ -89,7 +107,7 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restric
 #pragma unroll
     for (int j = 0; j < S::A_LOADS; ++j) {
         const int row = (wave * S::A_LOADS + j) * (64 / UA) + lane / UA;     // 64 units = 64 / UA rows
-        const int q = (lane % UA) ^ (row & 7);                                // the unit whose swizzled slot is this lane
+        const int q = S::a_slot(row, lane % UA);                              // the unit whose swizzled slot is this lane (the swizzles are involutions)
         int m = bm0 + row;
         if (m >= M) m = M - 1;                                                // rows past the end are computed and never stored
         a_off[j] = (uint32_t)(((size_t)(m - bm0) * lda + 4 * q) * sizeof(float));
@@ -97,7 +115,7 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restric
 #pragma unroll
     for (int j = 0; j < S::B_LOADS; ++j) {
         const int kr = (wave * S::B_LOADS + j) * (64 / UB) + lane / UB;      // 64 units = 64 / UB rows of k
-        const int col = clamp_group_col(bn0 + 4 * (lane % UB), N, 4);        // stay inside the operand; such columns are never stored
+        const int col = clamp_group_col(bn0 + 4 * S::b_slot(kr, lane % UB), N, 4);    // stay inside the operand; such columns are never stored
         b_off[j] = (uint32_t)(((size_t)kr * ldb + col) * sizeof(float));
     }
     int fetch_step = 0;                                // steps whose loads have gone out
@@ -119,58 +137,71 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restric
 
     // ---- where this lane's operands lie: unit q of its row of every row block of A in every buffer, its column of every
     // column block of B in rows s, s+2, ...
+    constexpr int BLK = S::BLK;
     const float* pa[STAGES][MI][UA];
     const float* pb[STAGES][NI];
 #pragma unroll
     for (int st = 0; st < STAGES; ++st) {
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) {
-            const int row = wm0 + 32 * mi + li;
+            const int row = wm0 + BLK * mi + li;
 #pragma unroll
-            for (int q = 0; q < UA; ++q) pa[st][mi][q] = lds + st * S::STAGE_FLOATS + (row * UA + (q ^ (row & 7))) * 4 + ls;
+            for (int q = 0; q < UA; ++q) pa[st][mi][q] = lds + st * S::STAGE_FLOATS + (row * UA + S::a_slot(row, q)) * 4 + ls;
         }
 #pragma unroll
-        for (int ni = 0; ni < NI; ++ni) pb[st][ni] = lds + st * S::STAGE_FLOATS + S::A_UNITS * 4 + ls * S::BN + wn0 + 32 * ni + li;
+        for (int ni = 0; ni < NI; ++ni) {
+            const int col = wn0 + BLK * ni + li;                  // rows ls, ls + KI, ... of B: their parity is that of ls
+            pb[st][ni] = lds + st * S::STAGE_FLOATS + S::A_UNITS * 4 + ls * S::BN + S::b_slot(ls, col / 4) * 4 + col % 4;
+        }
     }
 
-    // accumulators: lane holds D[8 (r / 4) + 4 ls + r % 4][li] of each of its blocks; the chains start at C when there is one
-    f32x16 acc[MI][NI];
+    // accumulators: lane holds, of each of its blocks, D[8 (r / 4) + 4 ls + r % 4][li], r = 0 .. 15 (32x32), or
+    // D[4 ls + r][li], r = 0 .. 3 (16x16); the chains start at C when there is one
+    constexpr int ACC = BLK == 32 ? 16 : 4;
+    typedef float acc_t __attribute__((ext_vector_type(ACC)));
+    auto acc_row = [&](int mi, int r) { return wm0 + BLK * mi + (BLK == 32 ? (r >> 2) * 8 + ls * 4 + (r & 3) : 4 * ls + r); };
+    acc_t acc[MI][NI];
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
         for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
+            for (int r = 0; r < ACC; ++r) {
                 acc[mi][ni][r] = 0.f;
                 if (HAS_C) {
-                    const int m = bm0 + wm0 + 32 * mi + (r >> 2) * 8 + ls * 4 + (r & 3), n = bn0 + wn0 + 32 * ni + li;
+                    const int m = bm0 + acc_row(mi, r), n = bn0 + wn0 + BLK * ni + li;
                     if (m < M && n < N) acc[mi][ni][r] = Cin[(size_t)m * ldc + n];
                 }
             }
 
     // fragment sets: set 0 feeds the first half of a step, set 1 the second
     float af[2][HALF][MI], bf[2][HALF][NI];
-    // Read number n (0 .. READS-1) of half `h` of the step that lies `stage_floats` past the pointers of buffer ST: reads
-    // (MI + NI) u .. (MI + NI) u + MI + NI - 1 fetch the operands of k pairs 2u and 2u + 1 of the half -- an A unit per
-    // row block, then two rows of B per column block.
+    // Read number n (0 .. READS-1) of half `h` of the step that lies `stage_floats` past the pointers of buffer ST.  The
+    // reads come in groups that fetch the operands of MFMAs 2u and 2u + 1 (of every block) of the half: per row block one
+    // read of A (32x32: both floats of a unit) or two (16x16: a float of each of two units), then two rows of B per
+    // column block.
     auto read_one = [&](auto st_tag, auto h_tag, auto n_tag, int stage_floats) {
         constexpr int ST = decltype(st_tag)::value, H = decltype(h_tag)::value, NR = decltype(n_tag)::value;
-        constexpr int U = NR / (MI + NI), W = NR % (MI + NI);
-        if constexpr (W < MI) {
-            const float* p = pa[ST][W][H * (HALF / 2) + U] + stage_floats;
+        constexpr int AR = S::APAIR ? MI : 2 * MI;      // reads of A per two k steps
+        constexpr int U = NR / (AR + NI), W = NR % (AR + NI);
+        if constexpr (W < AR && S::APAIR) {
+            const float* p = pa[ST][W][H * (HALF / 2) + U] + stage_floats;        // floats s and s + 2 of a unit
             af[H][2 * U][W] = p[0];
             af[H][2 * U + 1][W] = p[2];
+        } else if constexpr (W < AR) {                                           // float s of one unit
+            af[H][2 * U + W / MI][W % MI] = pa[ST][W % MI][H * HALF + 2 * U + W / MI][stage_floats];
         } else {
-            const float* p = pb[ST][W - MI] + 2 * (H * HALF + 2 * U) * S::BN + stage_floats;
-            bf[H][2 * U][W - MI] = p[0];
-            bf[H][2 * U + 1][W - MI] = p[2 * S::BN];
+            const float* p = pb[ST][W - AR] + S::KI * (H * HALF + 2 * U) * S::BN + stage_floats;
+            bf[H][2 * U][W - AR] = p[0];
+            bf[H][2 * U + 1][W - AR] = p[S::KI * S::BN];
         }
     };
     // MFMA number m (0 .. MFMAS-1) of half `h`: k pair m / (MI NI) of the half, blocks in turn
     auto mfma_one = [&](auto h_tag, auto m_tag) {
         constexpr int H = decltype(h_tag)::value, MM = decltype(m_tag)::value;
         constexpr int I = MM / (MI * NI), BMI = (MM / NI) % MI, BNI = MM % NI;
-        acc[BMI][BNI] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[H][I][BMI], bf[H][I][BNI], acc[BMI][BNI], 0, 0, 0);
+        if constexpr (BLK == 32) acc[BMI][BNI] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[H][I][BMI], bf[H][I][BNI], acc[BMI][BNI], 0, 0, 0);
+        else acc[BMI][BNI] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[H][I][BMI], bf[H][I][BNI], acc[BMI][BNI], 0, 0, 0);
     };
     typedef std::integral_constant<int, 0> I0;
     typedef std::integral_constant<int, 1> I1;
@@ -241,21 +272,21 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restric
                 if (k + 2 >= K) v[2] = 0.f;
                 if (k + 3 >= K) v[3] = 0.f;
             }
-            *reinterpret_cast<f32x4*>(lds + (row * UA + (q ^ (row & 7))) * 4) = v;
+            *reinterpret_cast<f32x4*>(lds + (row * UA + S::a_slot(row, q)) * 4) = v;
         }
 #pragma unroll
         for (int p = 0; p < S::B_UNITS / S::NT; ++p) {
             const int id = tid + p * S::NT, kr = id / UB, u = id % UB, k = k0 + kr;
             f32x4 v = {0.f, 0.f, 0.f, 0.f};
             if (k < K) v = *reinterpret_cast<const f32x4*>(B + (size_t)k * ldb + clamp_group_col(bn0 + 4 * u, N, 4));
-            *reinterpret_cast<f32x4*>(lds + S::A_UNITS * 4 + (kr * UB + u) * 4) = v;
+            *reinterpret_cast<f32x4*>(lds + S::A_UNITS * 4 + (kr * UB + S::b_slot(kr, u)) * 4) = v;
         }
         lds_sync();
         static_for<0, 2>([&](auto h_tag) {
             constexpr int H = decltype(h_tag)::value;
             static_for<0, READS>([&](auto n) { read_one(I0{}, h_tag, n, 0); });
             static_for<0, MFMAS>([&](auto m_tag) {
-                if (2 * (H * HALF + decltype(m_tag)::value / (MI * NI)) < rem) mfma_one(h_tag, m_tag);
+                if (S::KI * (H * HALF + decltype(m_tag)::value / (MI * NI)) < rem) mfma_one(h_tag, m_tag);
             });
         });
     }
@@ -263,12 +294,12 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restric
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int m = bm0 + wm0 + 32 * mi + (r >> 2) * 8 + ls * 4 + (r & 3);
+        for (int r = 0; r < ACC; ++r) {
+            const int m = bm0 + acc_row(mi, r);
             if (m < M) {
 #pragma unroll
                 for (int ni = 0; ni < NI; ++ni) {
-                    const int n = bn0 + wn0 + 32 * ni + li;
+                    const int n = bn0 + wn0 + BLK * ni + li;
                     if (n < N) D[(size_t)m * ldd + n] = relu ? relu_by_sign(acc[mi][ni][r]) : acc[mi][ni][r];
                 }
             }

@@ -62,6 +62,7 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 // and, for dense GEMM only, the tiles fed by LDS-DMA loads of sgemm_dma_tile.hpp (2x2 waves, one per SIMD):
 //  18:  64x64, K steps of 32 in 4 LDS buffers     19:  64x64, K steps of 64 in 3 buffers
 //  20: 128x128 (2x2 blocks per wave), 21: 64x128, 22: 128x64, K steps of 32 in 4 buffers
+//  24:  32x32 on 16x16 blocks (v_mfma_f32_16x16x4_f32), K steps of 64 in 3 buffers     25: 64x32, two blocks per wave
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
 typedef SgemmShape<128, 128, 16, 2, 2, 2> SShapeSmall;
 typedef SgemmShape<256, 128, 16, 2, 2, 2> SShapeTall;
@@ -168,17 +169,30 @@ constexpr int kDmaMaxPitch = 1 << 23;
 // block-chain kernels fill more of the chip, above, the big tiles re-use their operands better.  Steps of 64 k in three
 // buffers (96 KiB: one workgroup per CU) are ahead on a long K with at most one tile per CU, steps of 32 k in four
 // buffers (64 KiB: two workgroups share a CU) everywhere else.  Shapes 20 - 22 are 128x128, 64x128 and 128x64 tiles of
-// the same kernel; only the first is chosen automatically.  All paths give the same bits.
+// the same kernel, 24 and 25 tiles of 32x32 and 64x32 on 16x16 blocks; 20 and 24 are chosen automatically.  All paths
+// give the same bits.
 inline int pick_dma_shape(int M, int N, int K, int batch) {
-    if (g_rt.sgemm_variant >= 18 && g_rt.sgemm_variant <= 22) return g_rt.sgemm_variant;
+    if ((g_rt.sgemm_variant >= 18 && g_rt.sgemm_variant <= 22) || (g_rt.sgemm_variant >= 24 && g_rt.sgemm_variant <= 25)) return g_rt.sgemm_variant;
     if (g_rt.sgemm_variant != 0) return 0;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch, tiles128 = (long)cdiv(M, 128) * cdiv(N, 128) * batch;
+    const long tiles32 = (long)cdiv(M, 32) * cdiv(N, 32) * batch;
     // one 128x128 tile (2 x 2 blocks a wave, each operand read once for two blocks) on nearly every CU:
     // 2048^3 128.5 -> 124.4 us, 2048x8192x2048 501 -> 476 us (144 TFLOP/s)
     if (tiles128 <= cus && 10 * tiles128 >= 9 * cus) return 20;
-    if (2 * tiles64 < cus || 4 * tiles64 > 25 * cus) return 0;
-    return tiles64 <= cus && K >= 1024 ? 19 : 18;
+    // Cycles per k of a launch, measured over squares of 384 .. 1792 at K = 1024 and 8192: a round of 64x64 tiles (one
+    // per CU) walks K at 34.2, a round of 32x32 tiles of 16x16 blocks at 9.7.  The small tiles win where the 64x64 ones
+    // fill their last round badly (1152^2: 324 tiles = 2 rounds against 1296 = 6 rounds: 235 -> 193 us at K = 8192;
+    // 768^2: 117 -> 95 us; 1536^2: 359 -> 311 us) and below half a 64x64 tile per CU (512x8192x512: 51 -> 36 us).
+    const double walk64 = 34.2 * (double)((tiles64 + cus - 1) / cus), walk32 = 9.7 * (double)((tiles32 + cus - 1) / cus);
+    if (2 * tiles64 >= cus && 4 * tiles64 <= 25 * cus) {
+        if (walk32 < 1.05 * walk64) return 24;      // (a tie goes to the small tiles: 1280^2 237 -> 230 us, 1664^2 379 -> 366 us)
+        return tiles64 <= cus && K >= 1024 ? 19 : 18;
+    }
+    // fewer tiles than that: the block-chain shapes 12 and 23 (pick_chain_shape) keep their results -- one chain per
+    // CU walks a very long K with less trouble from pitches of a power of two -- the 32x32 tiles take the rest
+    if (2 * tiles64 < cus && (long)cdiv(M, 16) * cdiv(N, 32) * batch > cus) return 24;
+    return 0;
 }
 
 }  // namespace decx_hip
