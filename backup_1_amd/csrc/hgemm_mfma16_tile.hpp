@@ -45,12 +45,6 @@ __device__ __forceinline__ int a16_unit_in_slot(int m, int s, int UA) {
 // dma_load16 with a tag in the instruction text.  Two branches of a dispatch that issue the same loads into different
 // stages are otherwise merged by the compiler into one sequence whose operands are selected per branch -- in vector
 // registers, which the scalar operands of this instruction do not accept.
-template <int TAG>
-__device__ __forceinline__ void dma_load16_tagged(const void* sbase, uint32_t lane_off, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 ; load %3"
-                 : : "v"(lane_off), "s"(sbase), "s"(lds_base), "n"(TAG) : "memory", "m0");
-}
-
 template <int BM_, int BN_, int BK_, int WAVES_M_, int WAVES_N_, int STAGES_>
 struct Hgemm16Shape {
     static constexpr int BM = BM_, BN = BN_, BK = BK_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, STAGES = STAGES_;

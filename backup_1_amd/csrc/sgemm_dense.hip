@@ -98,6 +98,7 @@ int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float*
         if (dma == 22) return launch_sgemm_dma<DmaTile<128, 64, 32, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
         if (dma == 24) return launch_sgemm_dma<DmaTile<32, 32, 64, 3, 16>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
         if (dma == 25) return launch_sgemm_dma<DmaTile<64, 32, 64, 3, 16>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+        if (dma == 26) return launch_sgemm_dma<DmaTile<256, 256, 16, 4, 32, 4, 2>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
     }
     if (vec_a && vec_b) {
         const int chain = pick_chain_shape(M, N, K, batch.count);

@@ -35,7 +35,9 @@
 // wave waits for its own loads of step t+1, after it nobody reads step t's buffer any more), then issues the loads of
 // step t+STAGES into that buffer and reads the first half of step t+1, all between its MFMAs.  Loads never run past
 // the last whole step: the source pointers stop there (later refills fetch that step again and are never read), which
-// keeps every step the same code with the same wait counts.  A ragged last step (K % BK) is staged through registers
+// keeps every step the same code with the same wait counts.  The walk is whole passes over the buffers, unrolled and free
+// of branches, then the steps that are left behind a test each; the loads of the two copies carry different tags in
+// their text (dma_load16_tagged), without which the compiler merges them and does not assemble.  A ragged last step (K % BK) is staged through registers
 // with zeros past K and only the MFMAs that hold a k < K are issued.
 //
 // Arithmetic: per output one fused multiply-add chain over ascending k -- slot 0 then slot 1 inside an instruction,
@@ -49,11 +51,12 @@ namespace decx_hip {
 // BLK_ = 32: blocks of 32x32 on v_mfma_f32_32x32x2_f32 (two k per instruction, 64 cycles); BLK_ = 16: blocks of 16x16 on
 // v_mfma_f32_16x16x4_f32 (four k per instruction, 32 cycles: a chain walks K twice as fast), for results with fewer
 // than four 32x32 blocks per CU.
-template <int BM_, int BN_, int BK_, int STAGES_, int BLK_ = 32>
+template <int BM_, int BN_, int BK_, int STAGES_, int BLK_ = 32, int WAVES_M_ = 2, int WAVES_N_ = 2>
 struct DmaTile {
     static constexpr bool APAIR = BLK_ == 32;                         // one read of A serves two MFMAs of a block
-    static constexpr int BM = BM_, BN = BN_, BK = BK_, STAGES = STAGES_, BLK = BLK_, NWAVES = 4, NT = 64 * NWAVES;
-    static constexpr int WM = BM / 2, WN = BN / 2, MI = WM / BLK, NI = WN / BLK;    // 2 x 2 waves of MI x NI blocks
+    static constexpr int BM = BM_, BN = BN_, BK = BK_, STAGES = STAGES_, BLK = BLK_;
+    static constexpr int WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, NWAVES = WAVES_M * WAVES_N, NT = 64 * NWAVES;
+    static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, MI = WM / BLK, NI = WN / BLK;    // waves of MI x NI blocks
     static constexpr int KI = BLK == 32 ? 2 : 4;                        // k per instruction
     static constexpr int UA = BK / 4;                                   // 16-byte units per row of A and step
     static constexpr int UB = BN / 4;                                   // 16-byte units per row of B
@@ -63,13 +66,14 @@ struct DmaTile {
     static constexpr int STAGE_FLOATS = (A_UNITS + B_UNITS) * 4;
     static constexpr size_t LDS_BYTES = (size_t)STAGES * STAGE_FLOATS * sizeof(float);
     // slot of unit q of row `row` of A inside its row, and of unit u of row k of B (see the header)
-    __device__ static constexpr int a_slot(int row, int q) { return q ^ (row & 7); }
+    __device__ static constexpr int a_slot(int row, int q) { return UA >= 8 ? q ^ (row & 7) : q ^ ((row >> 1) & 3); }
     __device__ static constexpr int b_slot(int k, int u) { return BLK == 32 ? u : u ^ (4 * (k & 1)); }
     static constexpr int HALF = BK / KI / 2;                            // MFMAs per block and half step
     static constexpr int READS = ((APAIR ? MI : 2 * MI) + NI) * HALF / 2, MFMAS = HALF * MI * NI;       // per half step and wave
-    static_assert((BLK == 32 || BLK == 16) && BM % (2 * BLK) == 0 && BN % (2 * BLK) == 0 && BN <= 256 && UB >= 8 && 64 % UB == 0,
+    static_assert((BLK == 32 || BLK == 16) && BM % (WAVES_M * BLK) == 0 && BN % (WAVES_N * BLK) == 0 && BN <= 256 && UB >= 8 && 64 % UB == 0,
                   "whole blocks per wave; a load covers whole rows of B");
-    static_assert(BK % 16 == 0 && UA >= 8 && 64 % UA == 0, "whole units per half step; the swizzle needs 8 slots a row");
+    static_assert(BK % 16 == 0 && (UA >= 8 || (UA == 4 && BLK == 32)) && 64 % UA == 0 && HALF % 2 == 0,
+                  "whole units per half step; the swizzle spreads a read over 8 slots (of one row, or of two rows of 4)");
     static_assert(A_UNITS % (64 * NWAVES) == 0 && B_UNITS % (64 * NWAVES) == 0, "loads divide over the waves");
     static_assert(STAGES >= 2 && LOADS * (STAGES - 1) <= 63, "vmcnt is a 6-bit counter");
     static_assert(LOADS <= MFMAS - 1, "the loads go out behind the MFMAs of a half step");
@@ -94,7 +98,7 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restric
     const int bm0 = tc.tm * S::BM, bn0 = tc.tn * S::BN;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
-    const int wm0 = (wave / 2) * S::WM, wn0 = (wave % 2) * S::WN;
+    const int wm0 = (wave / S::WAVES_N) * S::WM, wn0 = (wave % S::WAVES_N) * S::WN;
     const int li = lane % S::BLK, ls = lane / S::BLK;  // row (of A) or column (of B) inside a block, and k-slot
     const int full_steps = K / BK, rem = K - full_steps * BK;
 
@@ -119,13 +123,13 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restric
         b_off[j] = (uint32_t)(((size_t)kr * ldb + col) * sizeof(float));
     }
     int fetch_step = 0;                                // steps whose loads have gone out
-    auto issue_one = [&](int stage, auto j_tag) {
-        constexpr int J = decltype(j_tag)::value;
+    auto issue_one = [&](int stage, auto j_tag, auto site_tag) {       // site_tag: a number of its own for every place of call
+        constexpr int J = decltype(j_tag)::value, TAG = decltype(site_tag)::value * 64 + J;
         const uint32_t base = lds_base + (uint32_t)stage * (S::STAGE_FLOATS * 4u);
         if constexpr (J < S::A_LOADS) {
-            dma_load16(a_base, a_off[J], base + (uint32_t)(wave * S::A_LOADS + J) * 1024u);
+            dma_load16_tagged<TAG>(a_base, a_off[J], base + (uint32_t)(wave * S::A_LOADS + J) * 1024u);
         } else {
-            dma_load16(b_base, b_off[J - S::A_LOADS], base + (uint32_t)(S::A_UNITS * 16) + (uint32_t)(wave * S::B_LOADS + J - S::A_LOADS) * 1024u);
+            dma_load16_tagged<TAG>(b_base, b_off[J - S::A_LOADS], base + (uint32_t)(S::A_UNITS * 16) + (uint32_t)(wave * S::B_LOADS + J - S::A_LOADS) * 1024u);
         }
         if constexpr (J == S::LOADS - 1) {
             ++fetch_step;
@@ -175,7 +179,8 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restric
             }
 
     // fragment sets: set 0 feeds the first half of a step, set 1 the second
-    float af[2][HALF][MI], bf[2][HALF][NI];
+    // (the two operands one read brings lie side by side, as the read delivers them: no register moves)
+    float af[2][HALF / 2][MI][2], bf[2][HALF / 2][NI][2];
     // Read number n (0 .. READS-1) of half `h` of the step that lies `stage_floats` past the pointers of buffer ST.  The
     // reads come in groups that fetch the operands of MFMAs 2u and 2u + 1 (of every block) of the half: per row block one
     // read of A (32x32: both floats of a unit) or two (16x16: a float of each of two units), then two rows of B per
@@ -186,40 +191,33 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restric
         constexpr int U = NR / (AR + NI), W = NR % (AR + NI);
         if constexpr (W < AR && S::APAIR) {
             const float* p = pa[ST][W][H * (HALF / 2) + U] + stage_floats;        // floats s and s + 2 of a unit
-            af[H][2 * U][W] = p[0];
-            af[H][2 * U + 1][W] = p[2];
+            af[H][U][W][0] = p[0];
+            af[H][U][W][1] = p[2];
         } else if constexpr (W < AR) {                                           // float s of one unit
-            af[H][2 * U + W / MI][W % MI] = pa[ST][W % MI][H * HALF + 2 * U + W / MI][stage_floats];
+            af[H][U][W % MI][W / MI] = pa[ST][W % MI][H * HALF + 2 * U + W / MI][stage_floats];
         } else {
             const float* p = pb[ST][W - AR] + S::KI * (H * HALF + 2 * U) * S::BN + stage_floats;
-            bf[H][2 * U][W - AR] = p[0];
-            bf[H][2 * U + 1][W - AR] = p[S::KI * S::BN];
+            bf[H][U][W - AR][0] = p[0];
+            bf[H][U][W - AR][1] = p[S::KI * S::BN];
         }
     };
     // MFMA number m (0 .. MFMAS-1) of half `h`: k pair m / (MI NI) of the half, blocks in turn
     auto mfma_one = [&](auto h_tag, auto m_tag) {
         constexpr int H = decltype(h_tag)::value, MM = decltype(m_tag)::value;
         constexpr int I = MM / (MI * NI), BMI = (MM / NI) % MI, BNI = MM % NI;
-        if constexpr (BLK == 32) acc[BMI][BNI] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[H][I][BMI], bf[H][I][BNI], acc[BMI][BNI], 0, 0, 0);
-        else acc[BMI][BNI] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[H][I][BMI], bf[H][I][BNI], acc[BMI][BNI], 0, 0, 0);
+        if constexpr (BLK == 32) acc[BMI][BNI] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[H][I / 2][BMI][I % 2], bf[H][I / 2][BNI][I % 2], acc[BMI][BNI], 0, 0, 0);
+        else acc[BMI][BNI] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[H][I / 2][BMI][I % 2], bf[H][I / 2][BNI][I % 2], acc[BMI][BNI], 0, 0, 0);
     };
     typedef std::integral_constant<int, 0> I0;
     typedef std::integral_constant<int, 1> I1;
 
     if (full_steps > 0) {
-        // The walk below is ONE unrolled pass over the STAGES buffers, entered part-way the first time, so that the last
-        // step always ends a pass: step 0 lies in buffer `first`.
-        const int first = (STAGES - full_steps % STAGES) % STAGES;
-        static_for<0, STAGES>([&](auto s_tag) {
-            int stage = first + decltype(s_tag)::value;
-            stage -= stage >= STAGES ? STAGES : 0;
-            static_for<0, S::LOADS>([&](auto j) { issue_one(stage, j); });
-        });
+        static_for<0, STAGES>([&](auto s_tag) { static_for<0, S::LOADS>([&](auto j) { issue_one(decltype(s_tag)::value, j, std::integral_constant<int, 2 * STAGES + decltype(s_tag)::value>{}); }); });
         wait_dma_then_barrier<S::LOADS*(STAGES - 1)>();                      // step 0 has landed
-        static_for<0, READS>([&](auto n) { read_one(I0{}, I0{}, n, first * S::STAGE_FLOATS); });      // its first half
+        static_for<0, READS>([&](auto n) { read_one(I0{}, I0{}, n, 0); });  // its first half
 
-        auto k_step = [&](auto st_tag) {
-            constexpr int ST = decltype(st_tag)::value;
+        auto k_step = [&](auto st_tag, auto copy_tag) {
+            constexpr int ST = decltype(st_tag)::value, SITE = decltype(copy_tag)::value * STAGES + ST;
             typedef std::integral_constant<int, (ST + 1) % STAGES> NextStage;
             // first half: read n goes out behind MFMA n MFMAS / READS
             static_for<0, MFMAS>([&](auto m_tag) {
@@ -239,7 +237,7 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restric
                     __builtin_amdgcn_sched_barrier(0);
                     wait_dma_then_barrier<S::LOADS*(STAGES - 2)>();          // step t+1 has landed; step t's buffer is free
                 } else {
-                    if constexpr (MM - 1 < S::LOADS) issue_one(ST, std::integral_constant<int, MM - 1>{});
+                    if constexpr (MM - 1 < S::LOADS) issue_one(ST, std::integral_constant<int, MM - 1>{}, std::integral_constant<int, SITE>{});
                     static_for<0, READS>([&](auto n_tag) {
                         if constexpr (1 + decltype(n_tag)::value * (MFMAS - 1) / READS == MM) read_one(NextStage{}, I0{}, n_tag, 0);
                     });
@@ -247,13 +245,12 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restric
                 __builtin_amdgcn_sched_barrier(0);
             });
         };
-        int skip = first;
-        for (int t = -first; t < full_steps; t += STAGES) {
-            static_for<0, STAGES>([&](auto st) {
-                if (decltype(st)::value >= skip) k_step(st);
-            });
-            skip = 0;
-        }
+        // whole passes over the buffers, free of branches, then the steps that are left
+        int t0 = 0;
+        for (; t0 + STAGES <= full_steps; t0 += STAGES) static_for<0, STAGES>([&](auto st) { k_step(st, I0{}); });
+        static_for<0, STAGES>([&](auto st) {
+            if (t0 + decltype(st)::value < full_steps) k_step(st, I1{});
+        });
         wait_dma_then_barrier<0>();                                          // nothing is in flight into LDS any more
     }
 

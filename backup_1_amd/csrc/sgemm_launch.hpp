@@ -63,6 +63,7 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //  18:  64x64, K steps of 32 in 4 LDS buffers     19:  64x64, K steps of 64 in 3 buffers
 //  20: 128x128 (2x2 blocks per wave), 21: 64x128, 22: 128x64, K steps of 32 in 4 buffers
 //  24:  32x32 on 16x16 blocks (v_mfma_f32_16x16x4_f32), K steps of 64 in 3 buffers     25: 64x32, two blocks per wave
+//  26: 256x256 on 4x2 waves of 64x128 (two per SIMD), K steps of 16 in 4 buffers -- the large-problem default
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
 typedef SgemmShape<128, 128, 16, 2, 2, 2> SShapeSmall;
 typedef SgemmShape<256, 128, 16, 2, 2, 2> SShapeTall;
@@ -169,10 +170,10 @@ constexpr int kDmaMaxPitch = 1 << 23;
 // block-chain kernels fill more of the chip, above, the big tiles re-use their operands better.  Steps of 64 k in three
 // buffers (96 KiB: one workgroup per CU) are ahead on a long K with at most one tile per CU, steps of 32 k in four
 // buffers (64 KiB: two workgroups share a CU) everywhere else.  Shapes 20 - 22 are 128x128, 64x128 and 128x64 tiles of
-// the same kernel, 24 and 25 tiles of 32x32 and 64x32 on 16x16 blocks; 20 and 24 are chosen automatically.  All paths
-// give the same bits.
+// the same kernel, 24 and 25 tiles of 32x32 and 64x32 on 16x16 blocks, 26 the 256x256 tile on eight waves; 20, 24 and 26
+// are chosen automatically.  All paths give the same bits.
 inline int pick_dma_shape(int M, int N, int K, int batch) {
-    if ((g_rt.sgemm_variant >= 18 && g_rt.sgemm_variant <= 22) || (g_rt.sgemm_variant >= 24 && g_rt.sgemm_variant <= 25)) return g_rt.sgemm_variant;
+    if ((g_rt.sgemm_variant >= 18 && g_rt.sgemm_variant <= 22) || (g_rt.sgemm_variant >= 24 && g_rt.sgemm_variant <= 26)) return g_rt.sgemm_variant;
     if (g_rt.sgemm_variant != 0) return 0;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch, tiles128 = (long)cdiv(M, 128) * cdiv(N, 128) * batch;
@@ -185,6 +186,10 @@ inline int pick_dma_shape(int M, int N, int K, int batch) {
     // fill their last round badly (1152^2: 324 tiles = 2 rounds against 1296 = 6 rounds: 235 -> 193 us at K = 8192;
     // 768^2: 117 -> 95 us; 1536^2: 359 -> 311 us) and below half a 64x64 tile per CU (512x8192x512: 51 -> 36 us).
     const double walk64 = 34.2 * (double)((tiles64 + cus - 1) / cus), walk32 = 9.7 * (double)((tiles32 + cus - 1) / cus);
+    // where the register-staged kernel would run its 256x256 tiles on two waves per SIMD (shape 7), the same tile fed by
+    // LDS-DMA loads is 0.6 - 1 % ahead (8192^3: 150.5 -> 151.9 TFLOP/s, 4096^3: 148.9 -> 150.0, 8192x2048x8192: 147.9 -> 148.9):
+    // MFMA busy 98.3 % against 97.5 %
+    if (4 * tiles64 > 25 * cus && K >= 512 && pick_sgemm_variant(M, N, K, batch, true) == 7) return 26;
     if (2 * tiles64 >= cus && 4 * tiles64 <= 25 * cus) {
         if (walk32 < 1.05 * walk64) return 24;      // (a tie goes to the small tiles: 1280^2 237 -> 230 us, 1664^2 379 -> 366 us)
         return tiles64 <= cus && K >= 1024 ? 19 : 18;

@@ -68,6 +68,16 @@ __device__ __forceinline__ void dma_load16(const void* sbase, uint32_t lane_off,
                  : : "v"(lane_off), "s"(sbase), "s"(lds_base) : "memory", "m0");
 }
 
+// The same with a tag in the instruction text.  Copies of a code sequence that issue the same loads (two instances of an
+// unrolled pass, two branches of a dispatch) are otherwise merged by the compiler into one sequence whose operands are
+// selected per copy -- in vector registers, which the scalar operands of this instruction do not accept; texts that
+// differ cannot be merged.
+template <int TAG>
+__device__ __forceinline__ void dma_load16_tagged(const void* sbase, uint32_t lane_off, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 ; load %3"
+                 : : "v"(lane_off), "s"(sbase), "s"(lds_base), "n"(TAG) : "memory", "m0");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_dma_then_barrier() {
     // my loads older than the N most recent have landed; my LDS reads are done; then everybody meets

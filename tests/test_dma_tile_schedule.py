@@ -1,6 +1,6 @@
 """Host-side model of the K walk of sgemm_dma_kernel (backup_1_amd/csrc/sgemm_dma_tile.hpp): whole steps of BK travel
-through STAGES LDS buffers by loads whose completion the waves count (vmcnt), the walk is one unrolled pass over the
-buffers that is entered part-way the first time, the source pointers stop on the last whole step, and every step is
+through STAGES LDS buffers by loads whose completion the waves count (vmcnt), the walk is whole unrolled passes over the
+buffers followed by the steps that are left, the source pointers stop on the last whole step, and every step is
 computed in two halves whose operands are read half a step ahead.  The model replays prologue, walk and barriers for
 many K and checks what the kernel relies on: the wait before a barrier covers exactly the loads of the step about to
 be read, a buffer is refilled only after every half read from it, the operands of each half come from the buffer that
@@ -35,35 +35,36 @@ def replay(K, BK, STAGES, LOADS):
             buffer = issued.pop(0)
             lds[buffer] = pending.pop(buffer)
 
-    first = (STAGES - full % STAGES) % STAGES
     for s in range(STAGES):
-        issue((first + s) % STAGES)
+        issue(s)
     wait_until_outstanding(LOADS * (STAGES - 1))
-    frag = {0: lds[first], 1: None}                       # set 0: first half of step 0
-    t, skip = -first, first
-    while t < full:
+    frag = {0: lds[0], 1: None}                           # set 0: first half of step 0
+
+    def k_step(step, v):
+        assert frag[0] == step, "first half computed from another step's operands"
+        assert lds.get(v) == step, "the buffer of the pass does not hold the step"
+        frag[1] = lds[v]                                   # second half's operands, read during the first half
+        computed.append((step, 0))
+        assert frag[1] == step
+        computed.append((step, 1))                         # its first MFMA, then:
+        wait_until_outstanding(LOADS * (STAGES - 2))       # own loads of step t+1 have landed
+        # barrier: every wave has read both halves of buffer v
+        nxt = (v + 1) % STAGES
+        if step + 1 < full:
+            assert lds.get(nxt) == step + 1, "the next step has not landed behind the barrier"
+        del lds[v]
+        issue(v)                                           # refill with step t+STAGES (or the last whole step again)
+        frag[0] = lds.get(nxt)                             # first half of step t+1 (anything, once past the end)
+        reads.append(nxt)
+
+    t0 = 0
+    while t0 + STAGES <= full:                             # whole passes
         for v in range(STAGES):
-            if v < skip:
-                continue
-            step = t + v
-            assert frag[0] == step, "first half computed from another step's operands"
-            assert lds.get(v) == step, "the buffer of the pass does not hold the step"
-            frag[1] = lds[v]                               # second half's operands, read during the first half
-            computed.append((step, 0))
-            assert frag[1] == step
-            computed.append((step, 1))                     # its first MFMA, then:
-            wait_until_outstanding(LOADS * (STAGES - 2))   # own loads of step t+1 have landed
-            # barrier: every wave has read both halves of buffer v
-            nxt = (v + 1) % STAGES
-            if step + 1 < full:
-                assert lds.get(nxt) == step + 1, "the next step has not landed behind the barrier"
-            del lds[v]
-            issue(v)                                       # refill with step t+STAGES (or the last whole step again)
-            frag[0] = lds.get(nxt)                         # first half of step t+1 (anything, once past the end)
-            reads.append(nxt)
-        skip = 0
-        t += STAGES
-    assert t == full, "the last step must end a pass"
+            k_step(t0 + v, v)
+        t0 += STAGES
+    for v in range(STAGES):                                # the steps that are left
+        if t0 + v < full:
+            k_step(t0 + v, v)
     wait_until_outstanding(0)
     assert computed == [(s, h) for s in range(full) for h in (0, 1)]
     return full
