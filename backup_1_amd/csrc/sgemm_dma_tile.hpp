@@ -42,7 +42,7 @@
 //
 // Arithmetic: per output one fused multiply-add chain over ascending k -- slot 0 then slot 1 inside an instruction,
 // instructions in order -- exactly the chain of sgemm_tile_kernel and of the reference.
-// Requires 16-byte aligned A and B with lda, ldb multiples of 4 (and below 2^23 so that a tile's byte offsets fit 32 bits).
+// Requires 16-byte aligned A and B with lda, ldb multiples of 4 (and below 2^21 so that a tile's byte offsets fit 32 bits).
 #pragma once
 #include "sgemm_tile.hpp"
 

@@ -160,9 +160,9 @@ inline int pick_chain_shape(int M, int N, int K, int batch) {
     return tiles32 > tile_limit ? 0 : cost64 < cost32 ? 13 : 11;
 }
 
-// The 64x64 tiles fed by LDS-DMA loads (sgemm_dma_tile.hpp) address a tile's rows with 32-bit byte offsets from the
-// tile's first row: 63 rows of a pitch below 2^23 floats stay below 2^31.
-constexpr int kDmaMaxPitch = 1 << 23;
+// The tiles fed by LDS-DMA loads (sgemm_dma_tile.hpp) address a tile's rows with 32-bit byte offsets from the tile's
+// first row: 255 rows (the tallest tile has 256) of a pitch below 2^21 floats stay below 2^31 bytes.
+constexpr int kDmaMaxPitch = 1 << 21;
 
 // Which shape of the LDS-DMA kernel a result of M x N takes, or 0 for the other kernels.  Measured on 256 CUs against
 // the automatic choice among the others: ahead from about half a 64x64 tile per CU (768^2: 16.1 -> 14.5 us) to about six
