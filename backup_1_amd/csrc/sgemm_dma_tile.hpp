@@ -141,23 +141,37 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restric
 
     // ---- where this lane's operands lie: unit q of its row of every row block of A in every buffer, its column of every
     // column block of B in rows s, s+2, ...
+    // 32x32 blocks: a register per (buffer, row block, unit) -- ds_read2_b32 carries offsets of up to 255 floats only.
+    // 16x16 blocks: a register per unit -- the swizzle of A looks at the low bits of the row only, which blocks and
+    // waves do not change, so unit q of a lane's row lies at the same place in every row block and buffer, a whole
+    // number of rows further: an offset ds_read_b32 can carry.
     constexpr int BLK = S::BLK;
-    const float* pa[STAGES][MI][UA];
-    const float* pb[STAGES][NI];
+    const float* pa_all[BLK == 32 ? STAGES : 1][BLK == 32 ? MI : 1][UA];
+    const float* pb_all[BLK == 32 ? STAGES : 1][NI];
 #pragma unroll
-    for (int st = 0; st < STAGES; ++st) {
+    for (int st = 0; st < (BLK == 32 ? STAGES : 1); ++st) {
 #pragma unroll
-        for (int mi = 0; mi < MI; ++mi) {
+        for (int mi = 0; mi < (BLK == 32 ? MI : 1); ++mi) {
             const int row = wm0 + BLK * mi + li;
 #pragma unroll
-            for (int q = 0; q < UA; ++q) pa[st][mi][q] = lds + st * S::STAGE_FLOATS + (row * UA + S::a_slot(row, q)) * 4 + ls;
+            for (int q = 0; q < UA; ++q) pa_all[st][mi][q] = lds + st * S::STAGE_FLOATS + (row * UA + S::a_slot(li, q)) * 4 + ls;
         }
 #pragma unroll
         for (int ni = 0; ni < NI; ++ni) {
             const int col = wn0 + BLK * ni + li;                  // rows ls, ls + KI, ... of B: their parity is that of ls
-            pb[st][ni] = lds + st * S::STAGE_FLOATS + S::A_UNITS * 4 + ls * S::BN + S::b_slot(ls, col / 4) * 4 + col % 4;
+            pb_all[st][ni] = lds + st * S::STAGE_FLOATS + S::A_UNITS * 4 + ls * S::BN + S::b_slot(ls, col / 4) * 4 + col % 4;
         }
     }
+    auto pa = [&](auto st_tag, auto mi_tag, auto q_tag) {
+        constexpr int ST = decltype(st_tag)::value, MIV = decltype(mi_tag)::value, Q = decltype(q_tag)::value;
+        if constexpr (BLK == 32) return pa_all[ST][MIV][Q];
+        else return pa_all[0][0][Q] + ST * S::STAGE_FLOATS + BLK * MIV * UA * 4;
+    };
+    auto pb = [&](auto st_tag, auto ni_tag) {
+        constexpr int ST = decltype(st_tag)::value, NIV = decltype(ni_tag)::value;
+        if constexpr (BLK == 32) return pb_all[ST][NIV];
+        else return pb_all[0][NIV] + ST * S::STAGE_FLOATS;
+    };
 
     // accumulators: lane holds, of each of its blocks, D[8 (r / 4) + 4 ls + r % 4][li], r = 0 .. 15 (32x32), or
     // D[4 ls + r][li], r = 0 .. 3 (16x16); the chains start at C when there is one
@@ -190,13 +204,13 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restric
         constexpr int AR = S::APAIR ? MI : 2 * MI;      // reads of A per two k steps
         constexpr int U = NR / (AR + NI), W = NR % (AR + NI);
         if constexpr (W < AR && S::APAIR) {
-            const float* p = pa[ST][W][H * (HALF / 2) + U] + stage_floats;        // floats s and s + 2 of a unit
+            const float* p = pa(st_tag, std::integral_constant<int, W < MI ? W : 0>{}, std::integral_constant<int, (H * (HALF / 2) + U) % UA>{}) + stage_floats;   // floats s and s + 2 of a unit
             af[H][U][W][0] = p[0];
             af[H][U][W][1] = p[2];
         } else if constexpr (W < AR) {                                           // float s of one unit
-            af[H][U][W % MI][W / MI] = pa[ST][W % MI][H * HALF + 2 * U + W / MI][stage_floats];
+            af[H][U][W % MI][W / MI] = pa(st_tag, std::integral_constant<int, W % MI>{}, std::integral_constant<int, (H * HALF + 2 * U + W / MI) % UA>{})[stage_floats];
         } else {
-            const float* p = pb[ST][W - AR] + S::KI * (H * HALF + 2 * U) * S::BN + stage_floats;
+            const float* p = pb(st_tag, std::integral_constant<int, W >= AR ? W - AR : 0>{}) + S::KI * (H * HALF + 2 * U) * S::BN + stage_floats;
             bf[H][U][W - AR][0] = p[0];
             bf[H][U][W - AR][1] = p[S::KI * S::BN];
         }
