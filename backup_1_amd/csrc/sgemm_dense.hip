@@ -1,7 +1,6 @@
 // fp32 dense GEMM: argument checks, kernel choice and launch (sgemm_tile.hpp, sgemm_chain16.hpp), split-K.
 #include "sgemm_launch.hpp"
 #include "sgemm_chain16.hpp"
-#include "sgemm_dma_tile.hpp"
 
 namespace decx_hip {
 
@@ -58,30 +57,6 @@ int launch_sgemm_chain16(const float* A, int lda, const float* B, int ldb, const
     return 0;
 }
 
-// Tiles fed by LDS-DMA loads (sgemm_dma_tile.hpp): for results of a few tiles per CU.
-template <class S>
-int launch_sgemm_dma(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
-                       int N, int K, const Batch& batch, bool relu) {
-    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
-    const long total = (long)tiles_m * tiles_n;
-    if (total > 0x7fffffffL || batch.count > 65535) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
-    auto kern = Cin ? sgemm_dma_kernel<S, true> : sgemm_dma_kernel<S, false>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(sgemm_dma_kernel<S, true>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
-        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(sgemm_dma_kernel<S, false>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
-        attr_done = true;
-    }
-    const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
-    hipLaunchKernelGGL(kern, dim3((unsigned)total, (unsigned)batch.count), dim3(S::NT), S::LDS_BYTES, batch.stream, A, lda, B, ldb,
-                       Cin, ldc, D, ldd, M, N, K, tiles_m, tiles_n, group_m, relu, batch.stride_a, batch.stride_b, batch.stride_c,
-                       batch.stride_d);
-    HIP_TRY(hipGetLastError());
-    return 0;
-}
-
 int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
                   int N, int K, const Batch& batch, bool relu) {
     if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
@@ -91,14 +66,7 @@ int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float*
     DenseOut out{ldd, relu, aligned16(D) && ldd % 4 == 0 && batch.stride_d % 4 == 0};
     if (vec_a && vec_b && lda < kDmaMaxPitch && ldb < kDmaMaxPitch) {
         const int dma = pick_dma_shape(M, N, K, batch.count);
-        if (dma == 18) return launch_sgemm_dma<DmaTile<64, 64, 32, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
-        if (dma == 19) return launch_sgemm_dma<DmaTile<64, 64, 64, 3>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
-        if (dma == 20) return launch_sgemm_dma<DmaTile<128, 128, 32, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
-        if (dma == 21) return launch_sgemm_dma<DmaTile<64, 128, 32, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
-        if (dma == 22) return launch_sgemm_dma<DmaTile<128, 64, 32, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
-        if (dma == 24) return launch_sgemm_dma<DmaTile<32, 32, 64, 3, 16>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
-        if (dma == 25) return launch_sgemm_dma<DmaTile<64, 32, 64, 3, 16>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
-        if (dma == 26) return launch_sgemm_dma<DmaTile<256, 256, 16, 4, 32, 4, 2>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+        if (dma) return launch_sgemm_dma_shape(dma, A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
     }
     if (vec_a && vec_b) {
         const int chain = pick_chain_shape(M, N, K, batch.count);

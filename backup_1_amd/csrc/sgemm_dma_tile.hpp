@@ -59,7 +59,8 @@ struct DmaTile {
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, MI = WM / BLK, NI = WN / BLK;    // waves of MI x NI blocks
     static constexpr int KI = BLK == 32 ? 2 : 4;                        // k per instruction
     static constexpr int UA = BK / 4;                                   // 16-byte units per row of A and step
-    static constexpr int UB = BN / 4;                                   // 16-byte units per row of B
+    static constexpr int BN_LDS = (BN + 63) / 64 * 64;                  // columns of B staged per row: loads cover whole rows of 64 units' worth
+    static constexpr int UB = BN_LDS / 4;                               // 16-byte units per row of B in LDS
     static constexpr int A_UNITS = BM * UA, B_UNITS = BK * UB;
     static constexpr int A_LOADS = A_UNITS / 64 / NWAVES, B_LOADS = B_UNITS / 64 / NWAVES;   // per wave and step, 1 KiB each
     static constexpr int LOADS = A_LOADS + B_LOADS;
@@ -70,7 +71,7 @@ struct DmaTile {
     __device__ static constexpr int b_slot(int k, int u) { return BLK == 32 ? u : u ^ (4 * (k & 1)); }
     static constexpr int HALF = BK / KI / 2;                            // MFMAs per block and half step
     static constexpr int READS = ((APAIR ? MI : 2 * MI) + NI) * HALF / 2, MFMAS = HALF * MI * NI;       // per half step and wave
-    static_assert((BLK == 32 || BLK == 16) && BM % (WAVES_M * BLK) == 0 && BN % (WAVES_N * BLK) == 0 && BN <= 256 && UB >= 8 && 64 % UB == 0,
+    static_assert((BLK == 32 || BLK == 16) && BM % (WAVES_M * BLK) == 0 && BN % (WAVES_N * BLK) == 0 && BN_LDS <= 256 && UB >= 8 && 64 % UB == 0,
                   "whole blocks per wave; a load covers whole rows of B");
     static_assert(BK % 16 == 0 && (UA >= 8 || (UA == 4 && BLK == 32)) && 64 % UA == 0 && HALF % 2 == 0,
                   "whole units per half step; the swizzle spreads a read over 8 slots (of one row, or of two rows of 4)");
@@ -159,7 +160,7 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restric
 #pragma unroll
         for (int ni = 0; ni < NI; ++ni) {
             const int col = wn0 + BLK * ni + li;                  // rows ls, ls + KI, ... of B: their parity is that of ls
-            pb_all[st][ni] = lds + st * S::STAGE_FLOATS + S::A_UNITS * 4 + ls * S::BN + S::b_slot(ls, col / 4) * 4 + col % 4;
+            pb_all[st][ni] = lds + st * S::STAGE_FLOATS + S::A_UNITS * 4 + ls * S::BN_LDS + S::b_slot(ls, col / 4) * 4 + col % 4;
         }
     }
     auto pa = [&](auto st_tag, auto mi_tag, auto q_tag) {
@@ -210,9 +211,9 @@ __global__ __launch_bounds__(S::NT) void sgemm_dma_kernel(const float* __restric
         } else if constexpr (W < AR) {                                           // float s of one unit
             af[H][U][W % MI][W / MI] = pa(st_tag, std::integral_constant<int, W % MI>{}, std::integral_constant<int, (H * HALF + 2 * U + W / MI) % UA>{})[stage_floats];
         } else {
-            const float* p = pb(st_tag, std::integral_constant<int, W >= AR ? W - AR : 0>{}) + S::KI * (H * HALF + 2 * U) * S::BN + stage_floats;
+            const float* p = pb(st_tag, std::integral_constant<int, W >= AR ? W - AR : 0>{}) + S::KI * (H * HALF + 2 * U) * S::BN_LDS + stage_floats;
             bf[H][U][W - AR][0] = p[0];
-            bf[H][U][W - AR][1] = p[S::KI * S::BN];
+            bf[H][U][W - AR][1] = p[S::KI * S::BN_LDS];
         }
     };
     // MFMA number m (0 .. MFMAS-1) of half `h`: k pair m / (MI NI) of the half, blocks in turn

@@ -64,6 +64,7 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //  20: 128x128 (2x2 blocks per wave), 21: 64x128, 22: 128x64, K steps of 32 in 4 buffers
 //  24:  32x32 on 16x16 blocks (v_mfma_f32_16x16x4_f32), K steps of 64 in 3 buffers     25: 64x32, two blocks per wave
 //  26: 256x256 on 4x2 waves of 64x128 (two per SIMD), K steps of 16 in 4 buffers -- the large-problem default
+//  27: 256x224 on 8x1 waves of 32x224 -- for results that 224 columns tile better than 256
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
 typedef SgemmShape<128, 128, 16, 2, 2, 2> SShapeSmall;
 typedef SgemmShape<256, 128, 16, 2, 2, 2> SShapeTall;
@@ -86,7 +87,7 @@ typedef SgemmShape<128, 64, 16, 2, 2, 4> SShapeTiny2;    // 2x2 waves of 64x32
 // and a one-workgroup-per-CU build with deeper prefetch, better on long ones (224x128: shape 15, which measured 5-6 %
 // ahead of shape 6 on the 224x224x64 convolution under 128 filters; the same split of the 224x256 tile, and 256x128 on
 // 8 waves of 128x32, measured no better than shapes 10 and 5 and are not built).
-inline int pick_sgemm_variant(int M, int N, int K, int batch, bool dense = false) {
+inline int pick_sgemm_variant(int M, int N, int K, int batch, bool dense = false, double* cost_out = nullptr) {
     if ((g_rt.sgemm_variant >= 1 && g_rt.sgemm_variant <= 10) || (g_rt.sgemm_variant >= 15 && g_rt.sgemm_variant <= 17)) return g_rt.sgemm_variant;
     if (g_rt.sgemm_variant == 14) return dense ? 14 : 2;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
@@ -112,6 +113,7 @@ inline int pick_sgemm_variant(int M, int N, int K, int batch, bool dense = false
             best = one_per_cu && c.variant == 3 ? 5 : one_per_cu && c.variant == 4 ? 15 : c.variant == 2 ? 16 : c.variant;
         }
     }
+    if (cost_out) *cost_out = best_cost;
     return best;
 }
 
@@ -164,16 +166,27 @@ inline int pick_chain_shape(int M, int N, int K, int batch) {
 // first row: 255 rows (the tallest tile has 256) of a pitch below 2^21 floats stay below 2^31 bytes.
 constexpr int kDmaMaxPitch = 1 << 21;
 
+// The shapes of the LDS-DMA kernel are instantiated in three translation units (sgemm_dma_small.hip, sgemm_dma_blocks16.hip,
+// sgemm_dma_large.hip).
+int launch_sgemm_dma_small(int shape, const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M, int N, int K, const Batch& batch, bool relu);
+int launch_sgemm_dma_blocks16(int shape, const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M, int N, int K, const Batch& batch, bool relu);
+int launch_sgemm_dma_large(int shape, const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M, int N, int K, const Batch& batch, bool relu);
+inline int launch_sgemm_dma_shape(int shape, const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M, int N, int K, const Batch& batch, bool relu) {
+    if (shape >= 26) return launch_sgemm_dma_large(shape, A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+    if (shape == 20 || shape >= 24) return launch_sgemm_dma_blocks16(shape, A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+    return launch_sgemm_dma_small(shape, A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+}
+
 // Which shape of the LDS-DMA kernel a result of M x N takes, or 0 for the other kernels.  Measured on 256 CUs against
 // the automatic choice among the others: ahead from about half a 64x64 tile per CU (768^2: 16.1 -> 14.5 us) to about six
 // (2560^2: 270 -> 266 us), by most around one per CU (1024^3: 23.3 -> 18.3 us, 1024x8192x1024: 158 -> 122 us); below, the
 // block-chain kernels fill more of the chip, above, the big tiles re-use their operands better.  Steps of 64 k in three
 // buffers (96 KiB: one workgroup per CU) are ahead on a long K with at most one tile per CU, steps of 32 k in four
 // buffers (64 KiB: two workgroups share a CU) everywhere else.  Shapes 20 - 22 are 128x128, 64x128 and 128x64 tiles of
-// the same kernel, 24 and 25 tiles of 32x32 and 64x32 on 16x16 blocks, 26 the 256x256 tile on eight waves; 20, 24 and 26
+// the same kernel, 24 and 25 tiles of 32x32 and 64x32 on 16x16 blocks, 26 and 27 the 256x256 and 256x224 tiles on eight waves; 20, 24, 26 and 27
 // are chosen automatically.  All paths give the same bits.
 inline int pick_dma_shape(int M, int N, int K, int batch) {
-    if ((g_rt.sgemm_variant >= 18 && g_rt.sgemm_variant <= 22) || (g_rt.sgemm_variant >= 24 && g_rt.sgemm_variant <= 26)) return g_rt.sgemm_variant;
+    if ((g_rt.sgemm_variant >= 18 && g_rt.sgemm_variant <= 22) || (g_rt.sgemm_variant >= 24 && g_rt.sgemm_variant <= 27)) return g_rt.sgemm_variant;
     if (g_rt.sgemm_variant != 0) return 0;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch, tiles128 = (long)cdiv(M, 128) * cdiv(N, 128) * batch;
@@ -189,7 +202,16 @@ inline int pick_dma_shape(int M, int N, int K, int batch) {
     // where the register-staged kernel would run its 256x256 tiles on two waves per SIMD (shape 7), the same tile fed by
     // LDS-DMA loads is 0.6 - 1 % ahead (8192^3: 150.5 -> 151.9 TFLOP/s, 4096^3: 148.9 -> 150.0, 8192x2048x8192: 147.9 -> 148.9):
     // MFMA busy 98.3 % against 97.5 %
-    if (4 * tiles64 > 25 * cus && K >= 512 && pick_sgemm_variant(M, N, K, batch, true) == 7) return 26;
+    if (4 * tiles64 > 25 * cus && K >= 512) {
+        double cost = 0.0;
+        const int tiled = pick_sgemm_variant(M, N, K, batch, true, &cost);
+        // the 256x224 tile of the same kernel (eight waves of 32x224) in that cost model: 3000x1500x4500 (252 tiles either
+        // way) 311 -> 305 us against the register-staged 224x256 tile, 8192x8192x7168 6612 -> 6350 us
+        const long tiles224 = (long)cdiv(M, 256) * cdiv(N, 224) * batch;
+        const double cost224 = (double)((tiles224 + cus - 1) / cus) * 256 * 224 / 0.975;
+        if (cost > 0.0 && cost224 < cost) return 27;
+        if (tiled == 7) return 26;
+    }
     if (2 * tiles64 >= cus && 4 * tiles64 <= 25 * cus) {
         if (walk32 < 1.05 * walk64) return 24;      // (a tie goes to the small tiles: 1280^2 237 -> 230 us, 1664^2 379 -> 366 us)
         return tiles64 <= cus && K >= 1024 ? 19 : 18;
