@@ -1,5 +1,5 @@
 // Launch of one shape of the kernel of sgemm_dma_tile.hpp; instantiated in sgemm_dma_small.hip, sgemm_dma_blocks16.hip and
-// sgemm_dma_large.hip (the shapes compile for 15 - 30 s each, side by side in three translation units).
+// sgemm_dma_large.hip and sgemm_dma_wide.hip (the shapes compile for 15 - 30 s each, side by side in four translation units).
 #pragma once
 #include "sgemm_launch.hpp"
 #include "sgemm_dma_tile.hpp"

@@ -59,7 +59,7 @@ struct DmaTile {
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, MI = WM / BLK, NI = WN / BLK;    // waves of MI x NI blocks
     static constexpr int KI = BLK == 32 ? 2 : 4;                        // k per instruction
     static constexpr int UA = BK / 4;                                   // 16-byte units per row of A and step
-    static constexpr int BN_LDS = (BN + 63) / 64 * 64;                  // columns of B staged per row: loads cover whole rows of 64 units' worth
+    static constexpr int BN_LDS = BN <= 32 ? 32 : BN <= 64 ? 64 : BN <= 128 ? 128 : 256;    // columns of B staged per row: a load of 64 units covers whole rows
     static constexpr int UB = BN_LDS / 4;                               // 16-byte units per row of B in LDS
     static constexpr int A_UNITS = BM * UA, B_UNITS = BK * UB;
     static constexpr int A_LOADS = A_UNITS / 64 / NWAVES, B_LOADS = B_UNITS / 64 / NWAVES;   // per wave and step, 1 KiB each

@@ -64,7 +64,7 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //  20: 128x128 (2x2 blocks per wave), 21: 64x128, 22: 128x64, K steps of 32 in 4 buffers
 //  24:  32x32 on 16x16 blocks (v_mfma_f32_16x16x4_f32), K steps of 64 in 3 buffers     25: 64x32, two blocks per wave
 //  26: 256x256 on 4x2 waves of 64x128 (two per SIMD), K steps of 16 in 4 buffers -- the large-problem default
-//  27: 256x224 on 8x1 waves of 32x224 -- for results that 224 columns tile better than 256
+//  27: 256x224 on 8x1 waves of 32x224 -- for results that 224 columns tile better than 256     28: 256x192, likewise
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
 typedef SgemmShape<128, 128, 16, 2, 2, 2> SShapeSmall;
 typedef SgemmShape<256, 128, 16, 2, 2, 2> SShapeTall;
@@ -166,12 +166,14 @@ inline int pick_chain_shape(int M, int N, int K, int batch) {
 // first row: 255 rows (the tallest tile has 256) of a pitch below 2^21 floats stay below 2^31 bytes.
 constexpr int kDmaMaxPitch = 1 << 21;
 
-// The shapes of the LDS-DMA kernel are instantiated in three translation units (sgemm_dma_small.hip, sgemm_dma_blocks16.hip,
-// sgemm_dma_large.hip).
+// The shapes of the LDS-DMA kernel are instantiated in four translation units (sgemm_dma_small.hip, sgemm_dma_blocks16.hip,
+// sgemm_dma_large.hip, sgemm_dma_wide.hip).
 int launch_sgemm_dma_small(int shape, const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M, int N, int K, const Batch& batch, bool relu);
 int launch_sgemm_dma_blocks16(int shape, const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M, int N, int K, const Batch& batch, bool relu);
 int launch_sgemm_dma_large(int shape, const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M, int N, int K, const Batch& batch, bool relu);
+int launch_sgemm_dma_wide(int shape, const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M, int N, int K, const Batch& batch, bool relu);
 inline int launch_sgemm_dma_shape(int shape, const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M, int N, int K, const Batch& batch, bool relu) {
+    if (shape >= 28) return launch_sgemm_dma_wide(shape, A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
     if (shape >= 26) return launch_sgemm_dma_large(shape, A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
     if (shape == 20 || shape >= 24) return launch_sgemm_dma_blocks16(shape, A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
     return launch_sgemm_dma_small(shape, A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
@@ -183,10 +185,10 @@ inline int launch_sgemm_dma_shape(int shape, const float* A, int lda, const floa
 // block-chain kernels fill more of the chip, above, the big tiles re-use their operands better.  Steps of 64 k in three
 // buffers (96 KiB: one workgroup per CU) are ahead on a long K with at most one tile per CU, steps of 32 k in four
 // buffers (64 KiB: two workgroups share a CU) everywhere else.  Shapes 20 - 22 are 128x128, 64x128 and 128x64 tiles of
-// the same kernel, 24 and 25 tiles of 32x32 and 64x32 on 16x16 blocks, 26 and 27 the 256x256 and 256x224 tiles on eight waves; 20, 24, 26 and 27
+// the same kernel, 24 and 25 tiles of 32x32 and 64x32 on 16x16 blocks, 26, 27 and 28 the 256x256, 256x224 and 256x192 tiles on eight waves; 20, 24 and 26 - 28
 // are chosen automatically.  All paths give the same bits.
 inline int pick_dma_shape(int M, int N, int K, int batch) {
-    if ((g_rt.sgemm_variant >= 18 && g_rt.sgemm_variant <= 22) || (g_rt.sgemm_variant >= 24 && g_rt.sgemm_variant <= 27)) return g_rt.sgemm_variant;
+    if ((g_rt.sgemm_variant >= 18 && g_rt.sgemm_variant <= 22) || (g_rt.sgemm_variant >= 24 && g_rt.sgemm_variant <= 28)) return g_rt.sgemm_variant;
     if (g_rt.sgemm_variant != 0) return 0;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch, tiles128 = (long)cdiv(M, 128) * cdiv(N, 128) * batch;
@@ -207,8 +209,11 @@ inline int pick_dma_shape(int M, int N, int K, int batch) {
         const int tiled = pick_sgemm_variant(M, N, K, batch, true, &cost);
         // the 256x224 tile of the same kernel (eight waves of 32x224) in that cost model: 3000x1500x4500 (252 tiles either
         // way) 311 -> 305 us against the register-staged 224x256 tile, 8192x8192x7168 6612 -> 6350 us
-        const long tiles224 = (long)cdiv(M, 256) * cdiv(N, 224) * batch;
+        const long tiles224 = (long)cdiv(M, 256) * cdiv(N, 224) * batch, tiles192 = (long)cdiv(M, 256) * cdiv(N, 192) * batch;
         const double cost224 = (double)((tiles224 + cus - 1) / cus) * 256 * 224 / 0.975;
+        // and the 256x192 tile (eight waves of 32x192): 6144^3 is 768 of them, three whole rounds: 3186 -> 3075 us (150.8 TFLOP/s)
+        const double cost192 = (double)((tiles192 + cus - 1) / cus) * 256 * 192 / 0.975;
+        if (cost > 0.0 && cost192 < cost && cost192 < cost224) return 28;
         if (cost > 0.0 && cost224 < cost) return 27;
         if (tiled == 7) return 26;
     }

@@ -20,7 +20,7 @@ def test_random_gemms_bit_exact(gpu, oracle, seed):
     for case in range(10):
         M, N = int(rng.integers(1, 420)), int(rng.integers(1, 420))
         K = int(rng.choice([int(rng.integers(1, 70)), int(rng.integers(1, 700))]))
-        variant = int(rng.integers(0, 28))
+        variant = int(rng.integers(0, 29))
         align = int(rng.choice([8, 8, 4, 1]))          # DECX pitch, a 16-byte pitch, an unaligned pitch
         with_c, relu = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
         A, B = workloads.normal((M, K), 100 * seed + case), workloads.normal((K, N), 100 * seed + case + 50)

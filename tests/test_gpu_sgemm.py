@@ -28,7 +28,7 @@ SHAPES = [(1, 1, 1), (3, 5, 7), (31, 17, 33), (32, 16, 32), (128, 16, 128), (129
           (300, 70, 500), (257, 1500, 255), (64, 8, 1000), (1000, 3, 64), (513, 129, 259)]
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28])
 @pytest.mark.parametrize("shape", SHAPES)
 def test_integer_exact_all_tiles(gpu, shape, variant):
     M, K, N = shape
@@ -46,7 +46,7 @@ def test_unaligned_pitch_uses_elementwise_loader(gpu, shape):
     assert np.array_equal(gpu_sgemm(A, B, align=1), exact_int_product(A, B))
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28])
 def test_a_times_b_plus_c(gpu, oracle, variant):
     M, K, N = 200, 150, 300
     A, B, C = workloads.small_ints((M, K), 21), workloads.small_ints((K, N), 22), workloads.small_ints((M, N), 23, -100, 100)
@@ -61,7 +61,7 @@ def test_a_times_b_plus_c(gpu, oracle, variant):
                           oracle.sgemm_chain(Ar, Br, Cr).view(np.uint32))
 
 
-@pytest.mark.parametrize("variant", [11, 12, 13, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27])
+@pytest.mark.parametrize("variant", [11, 12, 13, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28])
 def test_block_chain_kernel_walks_every_k_layout(gpu, oracle, variant):
     # sgemm_chain16.hpp: chunks of 64 k through 2, 4 or 8 register sets and 3 LDS buffers, a ragged last chunk apart;
     # sgemm_dma_tile.hpp: steps of 32 or 64 k through 4 or 3 LDS buffers walked in one unrolled pass entered part-way;
@@ -106,7 +106,7 @@ def test_permutation_matrix_moves_columns_exactly(gpu):
 def test_config1_1024_cube_vs_chain(gpu, oracle):
     A, B = workloads.gemm_square(1024)
     ref = oracle.sgemm_chain(A, B)
-    for variant in range(0, 28):
+    for variant in range(0, 29):
         assert np.array_equal(gpu_sgemm(A, B, variant=variant).view(np.uint32), ref.view(np.uint32)), variant
 
 

@@ -19,7 +19,7 @@ def parent_with_view(view, c0, parent_cols, nan):
 
 # (M, K, N, c0 of B, parent pitch of B): the last shape is a scaled-down copy of the pipeline's case (last panel of a
 # 3000-wide B); variants cover the 32x32x2 tiles, the block-chain shapes, the LDS-DMA tiles and the automatic choice
-@pytest.mark.parametrize("variant", [0, 2, 7, 9, 11, 12, 13, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27])
+@pytest.mark.parametrize("variant", [0, 2, 7, 9, 11, 12, 13, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28])
 @pytest.mark.parametrize("shape", [(96, 64, 40, 24, 64), (130, 72, 100, 8, 108), (256, 128, 952, 2048, 3000)])
 def test_fp32_b_is_a_column_range(gpu, oracle, variant, shape):
     M, K, N, c0, pb = shape
