@@ -63,7 +63,7 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //  18:  64x64, K steps of 32 in 4 LDS buffers     19:  64x64, K steps of 64 in 3 buffers
 //  20: 128x128 (2x2 blocks per wave), 21: 64x128, 22: 128x64, K steps of 32 in 4 buffers
 //  24:  32x32 on 16x16 blocks (v_mfma_f32_16x16x4_f32), K steps of 64 in 3 buffers     25: 64x32, two blocks per wave
-//  26: 256x256 on 4x2 waves of 64x128 (two per SIMD), K steps of 16 in 4 buffers -- the large-problem default
+//  26: 256x256 on 4x2 waves of 64x128 (two per SIMD), K steps of 16 in 2 buffers -- the large-problem default
 //  27: 256x224 on 8x1 waves of 32x224 -- for results that 224 columns tile better than 256     28: 256x192, likewise
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
 typedef SgemmShape<128, 128, 16, 2, 2, 2> SShapeSmall;
