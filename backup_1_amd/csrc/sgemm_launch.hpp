@@ -61,7 +61,7 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //  23:  16x32x64,  2 computing + 2 moving waves, one per SIMD -- at most one such tile per CU
 // and, for dense GEMM only, the tiles fed by LDS-DMA loads of sgemm_dma_tile.hpp (2x2 waves, one per SIMD):
 //  18:  64x64, K steps of 32 in 4 LDS buffers     19:  64x64, K steps of 64 in 3 buffers
-//  20: 128x128 (2x2 blocks per wave), 21: 64x128, 22: 128x64, K steps of 32 in 4 buffers
+//  20: 128x128 on 4x2 waves of 32x64 (two per SIMD), K steps of 16 in 2 buffers; 21: 64x128, 22: 128x64 (four waves), K steps of 32 in 4 buffers
 //  24:  32x32 on 16x16 blocks (v_mfma_f32_16x16x4_f32), K steps of 64 in 3 buffers     25: 64x32, two blocks per wave
 //  26: 256x256 on 4x2 waves of 64x128 (two per SIMD), K steps of 16 in 2 buffers -- the large-problem default
 //  27: 256x224 on 8x1 waves of 32x224 -- for results that 224 columns tile better than 256     28: 256x192, likewise
@@ -193,9 +193,13 @@ inline int pick_dma_shape(int M, int N, int K, int batch) {
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch, tiles128 = (long)cdiv(M, 128) * cdiv(N, 128) * batch;
     const long tiles32 = (long)cdiv(M, 32) * cdiv(N, 32) * batch;
-    // one 128x128 tile (2 x 2 blocks a wave, each operand read once for two blocks) on nearly every CU:
-    // 2048^3 128.5 -> 124.4 us, 2048x8192x2048 501 -> 476 us (144 TFLOP/s)
-    if (tiles128 <= cus && 10 * tiles128 >= 9 * cus) return 20;
+    // 128x128 tiles on eight waves (4 x 2 of 32x64, two per SIMD) in one or two rounds whose last is at least 88 % full:
+    // 2048^3 128.5 -> 118.2 us (145 TFLOP/s), 2048x8192x2048 501 -> 456 us (151 TFLOP/s), 1920^2 x 4096 245 -> 231 us,
+    // 2816^2 x 4096 482 -> 459 us
+    {
+        const long last = tiles128 % cus == 0 ? cus : tiles128 % cus;
+        if (tiles128 <= 2 * cus && 100 * last >= 88 * cus) return 20;
+    }
     // Cycles per k of a launch, measured over squares of 384 .. 1792 at K = 1024 and 8192: a round of 64x64 tiles (one
     // per CU) walks K at 34.2, a round of 32x32 tiles of 16x16 blocks at 9.7.  The small tiles win where the 64x64 ones
     // fill their last round badly (1152^2: 324 tiles = 2 rounds against 1296 = 6 rounds: 235 -> 193 us at K = 8192;
