@@ -40,21 +40,6 @@ struct HconvDmaShape {
     static_assert(BN % 8 == 0 && (BM * (BN / 8)) % NT == 0, "the result tile leaves in whole 16-byte units");
 };
 
-typedef int i32x4 __attribute__((ext_vector_type(4)));
-
-// raw buffer resource over [base, base + bytes): stride 0, offsets in bytes, out-of-range reads give zeros
-__device__ __forceinline__ i32x4 raw_buffer_words(const void* base, unsigned bytes) {
-    const uint64_t b = reinterpret_cast<uint64_t>(base);
-    return i32x4{(int)(uint32_t)b, (int)(uint32_t)((b >> 32) & 0xffffu), (int)bytes, 0x00020000};
-}
-
-// One 16-byte-per-lane load from a buffer (per-lane byte offset + wave-uniform byte offset) straight into LDS at
-// lds_base + 16*lane (lds_base wave-uniform).
-__device__ __forceinline__ void dma_buffer_load16(i32x4 rsrc, uint32_t lane_off, uint32_t uniform_off, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
-                 : : "v"(lane_off), "s"(rsrc), "s"(uniform_off), "s"(lds_base) : "memory", "m0");
-}
-
 template <class S>
 __global__ __launch_bounds__(S::NT) void hconv_dma_kernel(HalfImage img, HalfFilters fb, HalfTensorOut out, int M, int N,
                                                           int Kw /* K in words, a multiple of 32 */, int tiles_n) {

@@ -14,6 +14,10 @@ int conv_dispatch_paired(int variant, const Im2colA<true>& a, const FilterB<true
 int conv_dispatch_plain(int variant, const Im2colA<false>& a, const FilterB<false>& b, const float* bias, float* dst,
                         const TensorOut& out, int M, int N, int K, const Batch& batch);
 
+// the convolution on LDS-DMA loads and 16x16 blocks (sconv_dma.hpp), instantiated in sconv_dma.hip
+int launch_sconv_dma_shape(int shape, const Im2colA<true>& img, const FilterB<true>& fb, const float* bias, float* dst,
+                           const TensorOut& out, int M, int N, int K);
+
 template <class S>
 int launch_conv_chain16(const Im2colA<false>& img, const FilterB<false>& fb, const float* bias, float* dst, const TensorOut& out,
                         int M, int N, int K) {
@@ -78,6 +82,18 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
         if (chain == 12) return launch_conv_chain16<Chain16<1, 1, 8, 2>>(a, b, bias, dst, out, M, N, K);
         if (chain == 23) return launch_conv_chain16<Chain16Rect<1, 2, 1, 6, 2>>(a, b, bias, dst, out, M, N, K);
         return launch_conv_chain16<Chain16<4, 2, 2, 3>>(a, b, bias, dst, out, M, N, K);
+    }
+    // a K step of 32 inside one tap, results leaving as 16-byte units: the LDS-DMA kernel on 16x16 blocks.  Forced by
+    // shapes 29 and 30; by itself it takes a result that its 208x128 tiles cover in one round
+    if (dpitch % 32 == 0 && N % 4 == 0 && aligned16(dst) && dst_dpitch % 4 == 0 && dst_row_stride % 4 == 0) {
+        const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+        int shape = g_rt.sgemm_variant >= 29 && g_rt.sgemm_variant <= 30 ? g_rt.sgemm_variant : 0;
+        if (g_rt.sgemm_variant == 0 && (long)cdiv(M, 208) * cdiv(N, 128) <= cus && 4 * (long)cdiv(M, 208) * cdiv(N, 128) >= 3 * cus) shape = 29;
+        if (shape) {
+            Im2colA<true> a{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
+            FilterB<true> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
+            return launch_sconv_dma_shape(shape, a, b, bias, dst, out, M, N, K);
+        }
     }
     if (dpitch % 16 == 0) {      // a whole K step inside one tap: the tap walk runs on the scalar unit
         Im2colAUniform a{{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes}};

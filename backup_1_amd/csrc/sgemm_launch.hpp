@@ -65,6 +65,10 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //  24:  32x32 on 16x16 blocks (v_mfma_f32_16x16x4_f32), K steps of 64 in 3 buffers     25: 64x32, two blocks per wave
 //  26: 256x256 on 4x2 waves of 64x128 (two per SIMD), K steps of 16 in 2 buffers -- the large-problem default
 //  27: 256x224 on 8x1 waves of 32x224 -- for results that 224 columns tile better than 256     28: 256x192, likewise
+// and, for convolutions with a channel pitch that is a multiple of 32 and filters in fours, the LDS-DMA kernel on 16x16
+// blocks of sconv_dma.hpp (K steps of 32 in 2 buffers, eight waves, two per SIMD):
+//  29: 208x128 on 1x8 waves of 13x1 blocks -- 6 1/2 block rows of 32 for results of 196 rows per CU (224x224 pixels)
+//  30: 256x256 on 2x4 waves of 8x4 blocks -- measured behind shape 7 (512x512x256 under 256 filters: 145.6 against 149 TFLOP/s), not chosen by itself
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
 typedef SgemmShape<128, 128, 16, 2, 2, 2> SShapeSmall;
 typedef SgemmShape<256, 128, 16, 2, 2, 2> SShapeTall;

@@ -7,7 +7,8 @@ be read, a buffer is refilled only after every half read from it, the operands o
 holds that step, the loads never leave the whole steps, and every step is computed once, in ascending order."""
 import pytest
 
-SHAPES = ((32, 4, 4), (64, 3, 8), (32, 4, 8), (64, 3, 4), (64, 3, 6), (16, 2, 4), (16, 2, 2))      # (BK, STAGES, LOADS per wave and step) of the shapes that are built
+SHAPES = ((32, 4, 4), (64, 3, 8), (32, 4, 8), (64, 3, 4), (64, 3, 6), (16, 2, 4), (16, 2, 2),      # (BK, STAGES, LOADS per wave and step) of the shapes that are built
+          (32, 2, 6), (32, 2, 8))      # the convolution kernel of sconv_dma.hpp: same buffers, waits and barriers (its refills past the end fetch nothing instead of the last step again)
 
 
 def replay(K, BK, STAGES, LOADS):

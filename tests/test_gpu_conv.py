@@ -34,6 +34,27 @@ def test_real_valued_data_bit_exact_with_the_chain(gpu, oracle, case, variant):
                           oracle.conv2_chain(src, filt, flag).view(np.uint32))
 
 
+DMA_CASES = [  # H, W, C, N, kh, kw, flag: channel pitch a multiple of 32 and filter counts in fours, which the LDS-DMA kernel takes
+    (30, 30, 64, 128, 3, 3, 1), (64, 64, 32, 64, 5, 5, 0), (50, 47, 32, 12, 3, 3, 1), (19, 300, 64, 132, 1, 1, 1),
+    (40, 40, 96, 200, 3, 3, 0), (33, 31, 32, 4, 7, 5, 1), (17, 19, 32, 8, 17, 17, 1), (9, 11, 32, 260, 1, 1, 0),
+    (61, 67, 128, 36, 3, 3, 1), (5, 4, 32, 16, 3, 3, 1),
+]
+
+
+@pytest.mark.parametrize("variant", [29, 30])
+@pytest.mark.parametrize("case", DMA_CASES)
+def test_lds_dma_kernel_bit_exact_with_the_chain(gpu, oracle, case, variant):
+    # K steps of 32: 3x3x32 is an odd count (the step behind the whole passes), 1x1x32 a single one; taps left, right, above
+    # and below the image; filter counts that leave 16x16 blocks and 128-wide tiles partly empty; bias and ReLU on the sum
+    H, W, C, N, kh, kw, flag = case
+    src, filt = workloads.normal((H, W, C), 500 + H), workloads.normal((N, kh, kw, C), 600 + N)
+    ref = oracle.conv2_chain(src, filt, flag)
+    assert np.array_equal(gpu_conv(src, filt, flag, variant=variant).view(np.uint32), ref.view(np.uint32))
+    bias = workloads.normal((N,), 700 + N)
+    want = oracle.relu(ref + bias[None, None, :])
+    assert np.array_equal(gpu_conv(src, filt, flag, variant=variant, bias=bias, relu=True).view(np.uint32), want.view(np.uint32))
+
+
 def test_all_ones_counts_taps(gpu):
     H, W, C, N = 20, 24, 64, 8
     d = gpu_conv(np.ones((H, W, C), np.float32), np.ones((N, 3, 3, C), np.float32), 1)
@@ -56,7 +77,7 @@ def test_config4_224x224x64_128_filters(gpu, oracle):
     src, filt = workloads.conv_case()
     ref = oracle.conv2_chain(src, filt, 1)
     # same arithmetic as the reference's lowered GEMM (single fused chain over k = (ki*kw + kj)*dpitch + c): same bits
-    for variant in (0, 1, 2, 3, 4, 7, 11, 13, 15, 17, 23):
+    for variant in (0, 1, 2, 3, 4, 7, 11, 13, 15, 17, 23, 29, 30):
         assert np.array_equal(gpu_conv(src, filt, 1, variant=variant).view(np.uint32), ref.view(np.uint32)), variant
     si, fi = workloads.small_ints((224, 224, 64), 71, -4, 4), workloads.small_ints((128, 3, 3, 64), 72, -4, 4)
     assert np.array_equal(gpu_conv(si, fi, 1), oracle.conv2_chain(si, fi, 1))

@@ -39,7 +39,9 @@ def test_random_convolutions_bit_exact(gpu, oracle, seed):
         kh, kw = int(rng.choice([1, 3, 5, 7])), int(rng.choice([1, 3, 5, 7]))
         H, W = int(rng.integers(kh, 40)), int(rng.integers(kw, 40))
         C, N = int(rng.integers(1, 40)), int(rng.integers(1, 150))
-        flag, variant = int(rng.integers(0, 2)), int(rng.choice(list(range(14)) + [15, 16, 17, 23]))
+        if rng.integers(0, 3) == 0:
+            C, N = int(rng.choice([32, 64, 96])), 4 * int(rng.integers(1, 40))      # what the LDS-DMA kernel (29, 30) takes
+        flag, variant = int(rng.integers(0, 2)), int(rng.choice(list(range(14)) + [15, 16, 17, 23, 29, 30]))
         src = workloads.normal((H, W, C), 300 * seed + case)
         filt = workloads.normal((N, kh, kw, C), 300 * seed + case + 150)
         ref = oracle.conv2_chain(src, filt, flag)
