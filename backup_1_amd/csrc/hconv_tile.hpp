@@ -68,16 +68,6 @@ struct HalfTensorOut {
     bool relu;
 };
 
-// m / d and m % d for 0 <= m < 2^22 and d > 0 by a float reciprocal and one correction step either way
-__device__ __forceinline__ void small_divmod(int m, int d, float rcp_d, int& quot, int& rem) {
-    int qv = (int)((float)m * rcp_d);
-    int r = m - qv * d;
-    if (r < 0) { r += d; --qv; }
-    if (r >= d) { r -= d; ++qv; }
-    quot = qv;
-    rem = r;
-}
-
 // Epilogue of the fp16 convolution kernels.  Lane (li, lh) holds for pixel wm0 + 32 mi + li the filters
 // wn0 + 32 ni + 8 j + 4 lh + e (e = 0..3) in acc[mi][ni][4 j + e]: bias, ReLU and one rounding to binary16 per run of
 // four, then through LDS (which must be free: no reader of the operand buffers left, no load into them in flight) so

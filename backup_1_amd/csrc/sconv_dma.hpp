@@ -35,7 +35,8 @@
 // Arithmetic: per output one fused multiply-add chain over ascending k = (ki*kw + kj)*dpitch + c, taps outside the image
 // and padding channels entering as zeros -- the chain of sgemm_tile_kernel's convolution and of the reference
 // (conv2_mk_im2col.h:167-274, eq_GEMM.cuh:109-209).  Bias and ReLU join the finished sum.
-// The result tile leaves through LDS, one block row at a time, as 16-byte non-temporal stores of whole output rows.
+// The result tile leaves through LDS, up to four block rows at a time, as 16-byte non-temporal stores of whole output
+// rows (the 25.7 MB of the 224x224x128 result, written by all CUs at once when the single round ends, take about 4 us).
 #pragma once
 #include "sgemm_tile.hpp"
 
@@ -61,6 +62,8 @@ struct SconvDmaShape {
     static_assert(MI * BLOCK_BYTES <= 65536 && NI * BLOCK_BYTES <= 65536, "a fragment read reaches every block and buffer by its offset field");
     static_assert(LOADS <= MFMAS - 1 && LOADS * (STAGES - 1) <= 63, "loads go out behind the MFMAs of a k-group; vmcnt is a 6-bit counter");
     static_assert(2 * OUT_FLOATS * 4 <= LDS_BYTES && BN % 4 == 0, "two block rows of the result fit the operand buffers");
+    // block rows of the result that go through LDS between two barriers (two such groups lie in LDS side by side)
+    static constexpr int OUT_GROUP = LDS_BYTES / (2 * OUT_FLOATS * 4) >= 4 ? 4 : LDS_BYTES / (2 * OUT_FLOATS * 4) >= 2 ? 2 : 1;
 };
 
 template <class S>
@@ -84,13 +87,17 @@ __global__ __launch_bounds__(S::NT) void sconv_dma_kernel(Im2colA<true> img, Fil
     const i32x4 img_rsrc = raw_buffer_words(img.src, img.bytes), filt_rsrc = raw_buffer_words(fb.filt, fb.bytes);
     int a_x[S::A_LOADS];
     uint32_t a_off[S::A_LOADS], b_off[S::B_LOADS];
+    const bool small_m = M < (1 << 22);
+    const float rcp_wout = 1.0f / (float)img.Wout;
 #pragma unroll
     for (int j = 0; j < S::A_LOADS; ++j) {
         const int r = (wave * S::A_LOADS + j) * 8 + lane / 8;
         const int unit = (lane % 8) ^ (lane / 8);
         int m = bm0 + r;
         if (m >= M) m = M - 1;                                       // rows past the end are computed and never stored
-        const int y = m / img.Wout, x = m - y * img.Wout;
+        int y, x;
+        if (small_m) small_divmod(m, img.Wout, rcp_wout, y, x);
+        else { y = m / img.Wout; x = m - y * img.Wout; }
         a_x[j] = r < S::BM ? x - img.ox : -(1 << 30);                // rows past the tile: every tap "outside"
         a_off[j] = (uint32_t)(4 * ((y - img.oy) * img.row_stride + (x - img.ox) * img.dpitch) + 16 * unit);
     }
@@ -246,8 +253,10 @@ __global__ __launch_bounds__(S::NT) void sconv_dma_kernel(Im2colA<true> img, Fil
     // the refills past the end of K still write (zeros) when they land: wait for them before LDS becomes the result tile
     wait_dma_then_barrier<0>();
 
-    // ---- result: block row p of every wave goes to LDS (bias and ReLU applied), then leaves as whole rows of 16-byte
-    // stores; two LDS tiles in turn, so one barrier per block row
+    // ---- result: OUT_GROUP block rows of every wave go to LDS (bias and ReLU applied), then leave as whole rows of
+    // 16-byte stores; two such LDS tiles in turn, so one barrier per group
+    // (bias and ReLU are the same for the whole launch: one instance of the loop per combination, chosen by scalar
+    // branches, instead of selects per element -- vector instructions here are time with nothing behind them to hide in)
     float bv[NI];
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni) {
@@ -256,29 +265,52 @@ __global__ __launch_bounds__(S::NT) void sconv_dma_kernel(Im2colA<true> img, Fil
     }
     float* out_lds = reinterpret_cast<float*>(lds_raw);
     const int wave_m = wave / S::WAVES_N;
+    constexpr int UNITS = 16 * S::WAVES_M * (S::BN / 4);
+    static_assert(UNITS % S::NT == 0, "the stores of a block row divide over the threads");
+    // where this thread's 16-byte units of a block row go: row `srow` of the LDS tile, pixel sm0 (+ 16 per block row)
+    int srow[UNITS / S::NT], sm0[UNITS / S::NT], sc4[UNITS / S::NT];
 #pragma unroll
-    for (int p = 0; p < MI; ++p) {
-        float* ot = out_lds + (p & 1) * S::OUT_FLOATS;
+    for (int it = 0; it < UNITS / S::NT; ++it) {
+        const int id = tid + it * S::NT;
+        srow[it] = id / (S::BN / 4);
+        sc4[it] = id % (S::BN / 4);
+        sm0[it] = bm0 + (srow[it] / 16) * S::WM + srow[it] % 16;
+    }
+    auto store_tile = [&](auto bias_tag, auto relu_tag) {
+        constexpr bool BIAS = decltype(bias_tag)::value, RELU = decltype(relu_tag)::value;
 #pragma unroll
-        for (int ni = 0; ni < NI; ++ni)
+        for (int p0 = 0; p0 < MI; p0 += S::OUT_GROUP) {
+            float* ot = out_lds + ((p0 / S::OUT_GROUP) & 1) * (S::OUT_GROUP * S::OUT_FLOATS);
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float v = bias != nullptr ? acc[p][ni][r] + bv[ni] : acc[p][ni][r];      // (adding 0 would turn -0 into +0)
-                ot[(wave_m * 16 + 4 * ls + r) * S::OUT_ROW + wn0 + 16 * ni + li] = out.finish(v);
-            }
-        lds_sync();
-        constexpr int UNITS = 16 * S::WAVES_M * (S::BN / 4);
-        static_assert(UNITS % S::NT == 0, "the stores of a block row divide over the threads");
+            for (int pp = 0; pp < S::OUT_GROUP && p0 + pp < MI; ++pp)
 #pragma unroll
-        for (int it = 0; it < UNITS / S::NT; ++it) {
-            const int id = tid + it * S::NT;
-            const int row = id / (S::BN / 4), c4 = id % (S::BN / 4);
-            const int m = bm0 + (row / 16) * S::WM + 16 * p + row % 16, n = bn0 + 4 * c4;
-            if (m < M && n < N) {      // N is a multiple of 4: a quad is inside or outside as a whole
-                const f32x4 v = *reinterpret_cast<const f32x4*>(ot + row * S::OUT_ROW + 4 * c4);
-                __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(dst + out.offset(m) + n));
-            }
+                for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const float v = BIAS ? acc[p0 + pp][ni][r] + bv[ni] : acc[p0 + pp][ni][r];      // (adding 0 would turn -0 into +0)
+                        ot[pp * S::OUT_FLOATS + (wave_m * 16 + 4 * ls + r) * S::OUT_ROW + wn0 + 16 * ni + li] = RELU ? relu_by_sign(v) : v;
+                    }
+            lds_sync();
+#pragma unroll
+            for (int pp = 0; pp < S::OUT_GROUP && p0 + pp < MI; ++pp)
+#pragma unroll
+                for (int it = 0; it < UNITS / S::NT; ++it) {
+                    const int m = sm0[it] + 16 * (p0 + pp), n = bn0 + 4 * sc4[it];
+                    if (m < M && n < N) {      // N is a multiple of 4: a quad is inside or outside as a whole
+                        const f32x4 v = *reinterpret_cast<const f32x4*>(ot + pp * S::OUT_FLOATS + srow[it] * S::OUT_ROW + 4 * sc4[it]);
+                        __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(dst + out.offset(m) + n));
+                    }
+                }
         }
+    };
+    typedef std::integral_constant<bool, false> No;
+    typedef std::integral_constant<bool, true> Yes;
+    if (bias != nullptr) {
+        if (out.relu) store_tile(Yes{}, Yes{});
+        else store_tile(Yes{}, No{});
+    } else {
+        if (out.relu) store_tile(No{}, Yes{});
+        else store_tile(No{}, No{});
     }
 }
 

@@ -35,6 +35,16 @@ __host__ __device__ __forceinline__ constexpr int clamp_group_col(int col, int N
     return col < last ? col : last;
 }
 
+// m / d and m % d for 0 <= m < 2^22 and d > 0 by a float reciprocal and one correction step either way
+__device__ __forceinline__ void small_divmod(int m, int d, float rcp_d, int& quot, int& rem) {
+    int qv = (int)((float)m * rcp_d);
+    int r = m - qv * d;
+    if (r < 0) { r += d; --qv; }
+    if (r >= d) { r -= d; ++qv; }
+    quot = qv;
+    rem = r;
+}
+
 // f(integral_constant<int, I>) for I = I0 .. N-1, unrolled at compile time
 template <int I, int N, class F>
 __device__ __forceinline__ void static_for(F&& f) {
