@@ -37,7 +37,7 @@ def test_real_valued_data_bit_exact_with_the_chain(gpu, oracle, case, variant):
 DMA_CASES = [  # H, W, C, N, kh, kw, flag: channel pitch a multiple of 32 and filter counts in fours, which the LDS-DMA kernel takes
     (30, 30, 64, 128, 3, 3, 1), (64, 64, 32, 64, 5, 5, 0), (50, 47, 32, 12, 3, 3, 1), (19, 300, 64, 132, 1, 1, 1),
     (40, 40, 96, 200, 3, 3, 0), (33, 31, 32, 4, 7, 5, 1), (17, 19, 32, 8, 17, 17, 1), (9, 11, 32, 260, 1, 1, 0),
-    (61, 67, 128, 36, 3, 3, 1), (5, 4, 32, 16, 3, 3, 1),
+    (61, 67, 128, 36, 3, 3, 1), (5, 4, 32, 16, 3, 3, 1), (40, 1, 32, 8, 3, 3, 1), (1, 50, 64, 8, 3, 3, 1), (48, 52, 32, 20, 1, 5, 0),
 ]
 
 
