@@ -7,7 +7,8 @@ namespace decx_hip {
 template <class S>
 static int launch_sconv_dma(const Im2colA<true>& img, const FilterB<true>& fb, const float* bias, float* dst, const TensorOut& out,
                             int M, int N, int K) {
-    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    // tiles are patches of 16 output rows x BM / 16 columns (sconv_tiles counts them the same way)
+    const int Hout = M / out.Wout, tiles_x = cdiv(out.Wout, S::BM / 16), tiles_m = cdiv(Hout, 16) * tiles_x, tiles_n = cdiv(N, S::BN);
     const long total = (long)tiles_m * tiles_n;
     if (total > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
     static bool attr_done = false;
@@ -15,7 +16,7 @@ static int launch_sconv_dma(const Im2colA<true>& img, const FilterB<true>& fb, c
         HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(sconv_dma_kernel<S>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
         attr_done = true;
     }
-    hipLaunchKernelGGL(sconv_dma_kernel<S>, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, bias, dst, out, M, N, K, tiles_m, tiles_n);
+    hipLaunchKernelGGL(sconv_dma_kernel<S>, dim3((unsigned)total), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, bias, dst, out, Hout, N, K, tiles_x, tiles_m, tiles_n);
     HIP_TRY(hipGetLastError());
     return 0;
 }

@@ -5,6 +5,8 @@
 // them with 224 rows on 224 CUs or with 208 rows by mixing block sizes; on 16x16 blocks a tile of 208 rows x 128 filters
 // is 13 x 8 blocks -- 6 1/2 block rows of 32 where 6 1/8 is all the work there is -- on eight waves, two per SIMD, each
 // wave owning all 13 row blocks of one 16-filter column.  Both instructions retire 32 multiply-adds per cycle.
+// The 208 rows are a patch of 16 output rows x 13 columns, column by column: a block of 16 rows is 16 pixels of one image
+// column, and so is each group of 8 rows that one load instruction fetches (224x224: 14 x 18 = 252 patches, one round).
 //
 // Why LDS-DMA: with the im2col lowering a K step lies inside one tap, and per output pixel it is 128 contiguous bytes of
 // the image -- eight 16-byte units -- exactly as a row of A in the dense kernel (sgemm_dma_tile.hpp).  The filter bank
@@ -17,8 +19,8 @@
 // The swizzle is applied on the global side (the lane whose place is slot t of row r fetches unit t ^ (r % 8)).
 // buffer_load_dwordx4 ... lds takes a 32-bit offset into a buffer resource and answers an offset outside the buffer
 // with zeros, written to LDS like data: image rows above and below the tensor fall out of range by themselves (negative
-// or past the end), a tap left or right of the image gets an out-of-range offset by one compare and select per load,
-// and refills past the end of K fetch nothing.
+// or past the end).  Whether a tap lies left or right of the image is the same for all pixels of a load -- they share
+// their column -- so the scalar unit decides it and adds 2^31 to the load's offset, which throws every lane out of range.
 //
 // Pipeline: two LDS buffers, one barrier per K step (eight k-groups of MI x NI MFMAs per wave).  Fragments are read one
 // k-group ahead into the other of two register sets, between the MFMAs.  The barrier sits behind the first MFMA of the
@@ -26,11 +28,14 @@
 // more; the loads of step t+2 into that buffer and the reads of step t+1's first k-group follow between the remaining
 // MFMAs.  The walk is whole passes over the two buffers, then one more step if the count is odd; the loads of every
 // copy carry their own tag in the instruction text (dma_load16_tagged explains why).
-// A 16x16x4 MFMA lasts 32 cycles, half of a 32x32x2, and what a wave issues between two of them shows: the offsets of a
-// step's loads (tap walk on the scalar unit, column test and select per image load) are worked out in pieces of at most
-// two dependent instructions spread over the step (208x128 tile, 224x224x64 under 128 filters: 62.6 -> 61.4 us).
-// Measured on that shape: 18 K steps at 3.04 us where the 208 MFMAs of a SIMD take 2.77 us at 2.4 GHz, plus 7.3 us of launch,
-// first loads and 25.7 MB of stores; the same kernel with loads that fetch one and the same step every time runs its steps in 2.83 us.
+// A 16x16x4 MFMA lasts 32 cycles, half of a 32x32x2, and what a wave issues between two of them shows: a vector
+// instruction takes the matrix pipe's issue slot (probed: one v_add_u32 behind every 16x16x4 MFMA, two waves per SIMD,
+// 152.6 -> 126 TFLOP/s; scalar instructions cost a tenth of that), a chain of dependent ones its latency besides.  Per
+// step a wave therefore issues, beside its 104 MFMAs, 112 LDS reads and 6 loads, four vector instructions (one
+// addition per image load) and the tap walk on the scalar unit, in pieces spread over the step.  With the pixels of a
+// tile in raster order (a compare and a select per lane and image load, 14 vector instructions per step) the same kernel
+// took 61.1 us on 224x224x64 under 128 filters; as patches 59.7 us: 18 K steps at 2.93 us where the 208 MFMAs of a SIMD
+// take 2.77 us at 2.4 GHz, plus 7 us of launch, first loads and 25.7 MB of stores.
 //
 // Arithmetic: per output one fused multiply-add chain over ascending k = (ki*kw + kj)*dpitch + c, taps outside the image
 // and padding channels entering as zeros -- the chain of sgemm_tile_kernel's convolution and of the reference
@@ -68,14 +73,18 @@ struct SconvDmaShape {
 
 template <class S>
 __global__ __launch_bounds__(S::NT) void sconv_dma_kernel(Im2colA<true> img, FilterB<true> fb, const float* __restrict__ bias,
-                                                          float* __restrict__ dst, TensorOut out, int M, int N, int K,
-                                                          int tiles_m, int tiles_n) {
+                                                          float* __restrict__ dst, TensorOut out, int Hout, int N, int K,
+                                                          int tiles_x, int tiles_m, int tiles_n) {
     constexpr int MI = S::MI, NI = S::NI, U = S::U, STAGES = S::STAGES, GROUPS = S::GROUPS, MFMAS = S::MFMAS, READS = S::READS;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];   // [STAGES][A_ROWS x U units] [STAGES][BN x U units]
     const uint32_t lds_base = lds_byte_address(lds_raw);
 
     const TileCoord tc = xcd_grouped_tile((int)blockIdx.x, tiles_m, tiles_n, 8);
-    const int bm0 = tc.tm * S::BM, bn0 = tc.tn * S::BN;
+    // a tile is a patch of 16 output rows x TILE_X columns: row 16 bx + yy of the lowered product is pixel (y0 + yy, x0 + bx),
+    // so a block of 16 rows -- and each of the two loads that fetch it -- lies in one image column
+    constexpr int TILE_X = S::BM / 16;
+    const int tile_y = tc.tm / tiles_x, tile_x = tc.tm - tile_y * tiles_x;
+    const int y0 = 16 * tile_y, x0 = TILE_X * tile_x, bn0 = tc.tn * S::BN;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
     const int wm0 = (wave / S::WAVES_N) * S::WM, wn0 = (wave % S::WAVES_N) * S::WN;
@@ -85,20 +94,15 @@ __global__ __launch_bounds__(S::NT) void sconv_dma_kernel(Im2colA<true> img, Fil
     // ---- sources of this wave's loads.  A load moves 64 units = 8 rows; lane L moves, for row 8c + L/8, the unit whose
     // slot in the row is L%8.
     const i32x4 img_rsrc = raw_buffer_words(img.src, img.bytes), filt_rsrc = raw_buffer_words(fb.filt, fb.bytes);
-    int a_x[S::A_LOADS];
+    int a_x[S::A_LOADS];                                   // image column of tap column 0 of the load's pixels: the same for all lanes
     uint32_t a_off[S::A_LOADS], b_off[S::B_LOADS];
-    const bool small_m = M < (1 << 22);
-    const float rcp_wout = 1.0f / (float)img.Wout;
 #pragma unroll
     for (int j = 0; j < S::A_LOADS; ++j) {
-        const int r = (wave * S::A_LOADS + j) * 8 + lane / 8;
+        const int chunk = wave * S::A_LOADS + j;             // rows 8 chunk .. 8 chunk + 7: column x0 + chunk / 2, rows y0 + 8 (chunk % 2) ...
         const int unit = (lane % 8) ^ (lane / 8);
-        int m = bm0 + r;
-        if (m >= M) m = M - 1;                                       // rows past the end are computed and never stored
-        int y, x;
-        if (small_m) small_divmod(m, img.Wout, rcp_wout, y, x);
-        else { y = m / img.Wout; x = m - y * img.Wout; }
-        a_x[j] = r < S::BM ? x - img.ox : -(1 << 30);                // rows past the tile: every tap "outside"
+        const int y = y0 + 8 * (chunk % 2) + lane / 8, x = x0 + chunk / 2;
+        // pixels below or right of the output are computed and never stored; what they load is range-checked like everything else
+        a_x[j] = chunk < 2 * TILE_X ? x - img.ox : -(1 << 30);      // rows past the tile: every tap "outside"
         a_off[j] = (uint32_t)(4 * ((y - img.oy) * img.row_stride + (x - img.ox) * img.dpitch) + 16 * unit);
     }
 #pragma unroll
@@ -119,23 +123,21 @@ __global__ __launch_bounds__(S::NT) void sconv_dma_kernel(Im2colA<true> img, Fil
     const uint32_t wrap_a = 4u * (uint32_t)(img.row_stride - img.kw * img.dpitch), wrap_b = 4u * (uint32_t)(fb.filt_row_stride - fb.kw * fb.dpitch);
     // Offsets of the next batch of loads, worked out ahead of time in pieces that are spread between the MFMAs of a step:
     // every instruction a wave issues between two MFMAs delays its next MFMA by its own latency when it depends on the one
-    // before (measured: 12 dependent additions per step cost 0.11 us of 2.8), so no piece holds more than two dependent
-    // instructions.  Pieces 3j, 3j+1, 3j+2: column test operand, offset sum and select of image load j; then one select per
-    // filter load.
-    uint32_t a_next[S::A_LOADS], b_next[S::B_LOADS], b_soff_next = 0;
-    int a_col[S::A_LOADS];
-    constexpr int PREPARE_PIECES = 3 * S::A_LOADS + S::B_LOADS, ADVANCE_PIECES = 3;
+    // before (measured: 12 dependent additions per step cost 0.11 us of 2.8), and a vector instruction takes the matrix
+    // pipe's issue slot besides.  An image load's pixels share their column, so whether the tap lies beside the image is
+    // the scalar unit's to decide: it adds 2^31 to the walk's offset of such a load, which throws every lane out of the
+    // buffer's range (tensors stay below 2 GiB less the apron, checked by the launcher).  That leaves one vector addition
+    // per image load and step.  A filter load needs none: the walk is its scalar offset, and past the end of K it
+    // fetches the filter's first step again (never read).
+    uint32_t a_next[S::A_LOADS], a_add[S::A_LOADS], b_soff_next = 0;
+    constexpr int PREPARE_PIECES = 2 * S::A_LOADS, ADVANCE_PIECES = 3;
     auto prepare_piece = [&](auto p_tag) {
-        constexpr int P = decltype(p_tag)::value;
-        if constexpr (P < 3 * S::A_LOADS) {
-            constexpr int J = P / 3;
-            if constexpr (P % 3 == 0) a_col[J] = a_x[J] + walk_kj;
-            else if constexpr (P % 3 == 1) a_next[J] = a_off[J] + walk_off_a;
-            else a_next[J] = (uint32_t)a_col[J] < walk_w ? a_next[J] : kOutOfRange;
+        constexpr int P = decltype(p_tag)::value, J = P / 2;
+        if constexpr (P % 2 == 0) {
+            a_add[J] = (uint32_t)(a_x[J] + walk_kj) < walk_w ? walk_off_a : walk_off_a + kOutOfRange;
+            if constexpr (P == 0) b_soff_next = walk_w != 0u ? walk_off_b : 0u;
         } else {
-            constexpr int JB = P - 3 * S::A_LOADS;
-            b_next[JB] = walk_w != 0u ? b_off[JB] : kOutOfRange;
-            if constexpr (JB == 0) b_soff_next = walk_off_b;
+            a_next[J] = a_off[J] + a_add[J];
         }
     };
     auto advance_piece = [&](auto q_tag) {
@@ -161,7 +163,7 @@ __global__ __launch_bounds__(S::NT) void sconv_dma_kernel(Im2colA<true> img, Fil
             dma_buffer_load16_tagged<TAG>(img_rsrc, a_next[J], 0u, lds_base + (uint32_t)(ST * S::A_BYTES) + (uint32_t)((wave * S::A_LOADS + J) * S::CHUNK));
         } else {
             constexpr int JB = J - S::A_LOADS;
-            dma_buffer_load16_tagged<TAG>(filt_rsrc, b_next[JB], b_soff_next,
+            dma_buffer_load16_tagged<TAG>(filt_rsrc, b_off[JB], b_soff_next,
                                           lds_base + (uint32_t)(STAGES * S::A_BYTES + ST * S::B_BYTES) + (uint32_t)((wave * S::B_LOADS + JB) * S::CHUNK));
         }
     };
@@ -267,14 +269,16 @@ __global__ __launch_bounds__(S::NT) void sconv_dma_kernel(Im2colA<true> img, Fil
     const int wave_m = wave / S::WAVES_N;
     constexpr int UNITS = 16 * S::WAVES_M * (S::BN / 4);
     static_assert(UNITS % S::NT == 0, "the stores of a block row divide over the threads");
-    // where this thread's 16-byte units of a block row go: row `srow` of the LDS tile, pixel sm0 (+ 16 per block row)
-    int srow[UNITS / S::NT], sm0[UNITS / S::NT], sc4[UNITS / S::NT];
+    // where this thread's 16-byte units of a block row go: row `srow` of the LDS tile = output row sy of column sx0 (+ 1
+    // per block row)
+    int srow[UNITS / S::NT], sy[UNITS / S::NT], sx0[UNITS / S::NT], sc4[UNITS / S::NT];
 #pragma unroll
     for (int it = 0; it < UNITS / S::NT; ++it) {
         const int id = tid + it * S::NT;
         srow[it] = id / (S::BN / 4);
         sc4[it] = id % (S::BN / 4);
-        sm0[it] = bm0 + (srow[it] / 16) * S::WM + srow[it] % 16;
+        sy[it] = y0 + srow[it] % 16;
+        sx0[it] = x0 + (srow[it] / 16) * MI;
     }
     auto store_tile = [&](auto bias_tag, auto relu_tag) {
         constexpr bool BIAS = decltype(bias_tag)::value, RELU = decltype(relu_tag)::value;
@@ -295,10 +299,10 @@ __global__ __launch_bounds__(S::NT) void sconv_dma_kernel(Im2colA<true> img, Fil
             for (int pp = 0; pp < S::OUT_GROUP && p0 + pp < MI; ++pp)
 #pragma unroll
                 for (int it = 0; it < UNITS / S::NT; ++it) {
-                    const int m = sm0[it] + 16 * (p0 + pp), n = bn0 + 4 * sc4[it];
-                    if (m < M && n < N) {      // N is a multiple of 4: a quad is inside or outside as a whole
+                    const int x = sx0[it] + p0 + pp, n = bn0 + 4 * sc4[it];
+                    if (sy[it] < Hout && x < out.Wout && n < N) {      // N is a multiple of 4: a quad is inside or outside as a whole
                         const f32x4 v = *reinterpret_cast<const f32x4*>(ot + pp * S::OUT_FLOATS + srow[it] * S::OUT_ROW + 4 * sc4[it]);
-                        __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(dst + out.offset(m) + n));
+                        __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(dst + (size_t)sy[it] * out.row_stride + (size_t)x * out.dpitch + n));
                     }
                 }
         }

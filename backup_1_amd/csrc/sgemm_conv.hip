@@ -83,12 +83,17 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
         if (chain == 23) return launch_conv_chain16<Chain16Rect<1, 2, 1, 6, 2>>(a, b, bias, dst, out, M, N, K);
         return launch_conv_chain16<Chain16<4, 2, 2, 3>>(a, b, bias, dst, out, M, N, K);
     }
-    // a K step of 32 inside one tap, results leaving as 16-byte units: the LDS-DMA kernel on 16x16 blocks.  Forced by
-    // shapes 29 and 30; by itself it takes a result that its 208x128 tiles cover in one round
-    if (dpitch % 32 == 0 && N % 4 == 0 && aligned16(dst) && dst_dpitch % 4 == 0 && dst_row_stride % 4 == 0) {
+    // a K step of 32 inside one tap, results leaving as 16-byte units: the LDS-DMA kernel on 16x16 blocks.  Its column
+    // test adds 2^31 to an offset, which must throw it out of the tensor's range even from the apron's negative offsets.
+    // Forced by shapes 29 and 30; by itself it takes a result that its patches of 16 x 13 pixels x 128 filters cover in
+    // one round that fills at least three quarters of the CUs
+    const size_t apron_bytes = ((size_t)oy * src_row_stride + (size_t)ox * dpitch + 4) * sizeof(float);
+    if (dpitch % 32 == 0 && N % 4 == 0 && aligned16(dst) && dst_dpitch % 4 == 0 && dst_row_stride % 4 == 0 &&
+        src_bytes + apron_bytes + (size_t)(16 + kh) * src_row_stride * sizeof(float) < 0x80000000ull) {
         const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+        const long patches = (long)cdiv(Hout, 16) * cdiv(Wout, 13) * cdiv(N, 128);
         int shape = g_rt.sgemm_variant >= 29 && g_rt.sgemm_variant <= 30 ? g_rt.sgemm_variant : 0;
-        if (g_rt.sgemm_variant == 0 && (long)cdiv(M, 208) * cdiv(N, 128) <= cus && 4 * (long)cdiv(M, 208) * cdiv(N, 128) >= 3 * cus) shape = 29;
+        if (g_rt.sgemm_variant == 0 && patches <= cus && 4 * patches >= 3 * cus) shape = 29;
         if (shape) {
             Im2colA<true> a{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
             FilterB<true> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};

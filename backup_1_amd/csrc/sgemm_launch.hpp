@@ -67,8 +67,8 @@ int launch_sgemm_tile(const ASrc& a, const BSrc& b, const float* Cin, int ldc, f
 //  27: 256x224 on 8x1 waves of 32x224 -- for results that 224 columns tile better than 256     28: 256x192, likewise
 // and, for convolutions with a channel pitch that is a multiple of 32 and filters in fours, the LDS-DMA kernel on 16x16
 // blocks of sconv_dma.hpp (K steps of 32 in 2 buffers, eight waves, two per SIMD):
-//  29: 208x128 on 1x8 waves of 13x1 blocks -- 6 1/2 block rows of 32 for results of 196 rows per CU (224x224 pixels)
-//  30: 256x256 on 2x4 waves of 8x4 blocks -- measured behind shape 7 (512x512x256 under 256 filters: 145.6 against 149 TFLOP/s), not chosen by itself
+//  29: 208x128 (a patch of 16 x 13 pixels) on 1x8 waves of 13x1 blocks -- 6 1/2 block rows of 32 for results of 196 rows per CU (224x224 pixels)
+//  30: 256x256 (16 x 16 pixels) on 2x4 waves of 8x4 blocks -- measured behind shape 7 (512x512x256 under 256 filters: 148.1 against 149 TFLOP/s), not chosen by itself
 typedef SgemmShape<256, 256, 16, 2, 2> SShapeBig;
 typedef SgemmShape<128, 128, 16, 2, 2, 2> SShapeSmall;
 typedef SgemmShape<256, 128, 16, 2, 2, 2> SShapeTall;
