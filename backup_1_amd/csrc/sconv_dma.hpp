@@ -168,6 +168,16 @@ __global__ __launch_bounds__(S::NT) void sconv_dma_kernel(Im2colA<true> img, Fil
         }
     };
 
+    // the first STAGES steps go out before anything else is set up: the rest of the preparation runs under their latency
+    if (steps > 0) {
+        static_for<0, STAGES>([&](auto s_tag) {
+            static_for<0, PREPARE_PIECES>([&](auto p) { prepare_piece(p); });
+            static_for<0, S::LOADS>([&](auto j) { issue_one(s_tag, j, std::integral_constant<int, 2 * STAGES + decltype(s_tag)::value>{}); });
+            static_for<0, ADVANCE_PIECES>([&](auto q) { advance_piece(q); });
+        });
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
     // ---- where this lane's operands lie: float ls of unit g of row li of a block, one register per unit and operand;
     // block and buffer are whole rows further, in the offset field of the read
     const float* pa[STAGES][GROUPS];
@@ -204,11 +214,6 @@ __global__ __launch_bounds__(S::NT) void sconv_dma_kernel(Im2colA<true> img, Fil
     typedef std::integral_constant<int, 1> I1;
 
     if (steps > 0) {
-        static_for<0, STAGES>([&](auto s_tag) {
-            static_for<0, PREPARE_PIECES>([&](auto p) { prepare_piece(p); });
-            static_for<0, S::LOADS>([&](auto j) { issue_one(s_tag, j, std::integral_constant<int, 2 * STAGES + decltype(s_tag)::value>{}); });
-            static_for<0, ADVANCE_PIECES>([&](auto q) { advance_piece(q); });
-        });
         wait_dma_then_barrier<S::LOADS*(STAGES - 1)>();                      // step 0 has landed
         static_for<0, READS>([&](auto n) { read_one(I0{}, I0{}, n); });     // its first k-group
 
