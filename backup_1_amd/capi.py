@@ -20,11 +20,11 @@ SYMBOLS = [
     "decx_hip_host_malloc", "decx_hip_host_free", "decx_hip_memcpy2d", "decx_hip_memcpy", "decx_hip_sync",
     "decx_hip_sgemm", "decx_hip_sgemm_async", "decx_hip_hgemm_f32acc", "decx_hip_hgemm_f32acc_async",
     "decx_hip_conv2_im2col_f32", "decx_hip_conv2_im2col_f32_async", "decx_hip_timer_start", "decx_hip_timer_stop",
-    "decx_hip_last_error", "decx_hip_set_sgemm_variant", "decx_hip_set_hgemm_variant", "decx_hip_copy_kernel",
+    "decx_hip_last_error", "decx_hip_set_sgemm_variant", "decx_hip_set_hgemm_variant", "decx_hip_stream",
     "decx_hip_sgemm_splitk", "decx_hip_sgemm_batched", "decx_hip_hgemm_f32acc_batched", "decx_hip_gemm3_host_f32", "decx_hip_gemm3_host_f16",
     "decx_hip_conv2_im2col_f32_fused", "decx_hip_conv2_im2col_f16", "decx_hip_conv2_im2col_f16_async", "decx_hip_sgemm_relu", "decx_hip_relu_f32", "decx_hip_relu_f32_async",
     "decx_hip_relu_f32_rec", "decx_hip_relu_f32_backward", "decx_hip_gemm_host_f32", "decx_hip_gemm_host_f16",
-    "decx_hip_b_read_extent", "decx_hip_set_splitk_mode", "decx_hip_hgemm_f32acc_noalloc", "decx_hip_hgemm_probe",
+    "decx_hip_b_read_extent", "decx_hip_set_splitk_mode", "decx_hip_hgemm_f32acc_noalloc",
 ]
 
 
@@ -59,7 +59,7 @@ def lib():
             "decx_hip_hgemm_f32acc_async": ([P, I, P, I, P, I, P, I, I, I, I], I),
             "decx_hip_conv2_im2col_f32": ([P, I, I, I, Z, P, I, I, I, Z, Z, P, I, Z, I], I),
             "decx_hip_conv2_im2col_f32_async": ([P, I, I, I, Z, P, I, I, I, Z, Z, P, I, Z, I], I),
-            "decx_hip_copy_kernel": ([P, P, Z], I),
+            "decx_hip_stream": ([], P),
             "decx_hip_sgemm_splitk": ([P, I, P, I, P, I, P, I, I, I, I, I], I),
             "decx_hip_sgemm_batched": ([P, I, Z, P, I, Z, P, I, Z, P, I, Z, I, I, I, I], I),
             "decx_hip_hgemm_f32acc_batched": ([P, I, Z, P, I, Z, P, I, Z, P, I, Z, I, I, I, I], I),
@@ -78,7 +78,6 @@ def lib():
             "decx_hip_set_sgemm_variant": ([I], I), "decx_hip_set_hgemm_variant": ([I], I),
             "decx_hip_b_read_extent": ([I, I, I], I),
             "decx_hip_set_splitk_mode": ([I], I),
-            "decx_hip_hgemm_probe": ([I, P, I, P, I, P, I, I, I, I], I),
             "decx_hip_hgemm_f32acc_noalloc": ([P, I, P, I, P, I, P, I, I, I, I, I], I),
         }
         for name, (args, res) in sig.items():
@@ -86,6 +85,29 @@ def lib():
             fn.argtypes, fn.restype = args, res
         _lib = L
     return _lib
+
+
+PROBE_LIB_PATH = os.path.join(_HERE, "libdecx_hip_probe.so")
+_probe = None
+
+
+def probe_lib():
+    """Load libdecx_hip_probe.so, the measurement instruments (`make -C backup_1_amd/csrc probes`): ablation builds of
+    the large fp16 tile kernel and the calibration copy kernel.  Only bench.py's `ladder` and `copy` legs use it."""
+    global _probe
+    if _probe is None:
+        if not os.path.exists(PROBE_LIB_PATH):
+            raise FileNotFoundError("%s is missing: build it with `make -C backup_1_amd/csrc probes`" % PROBE_LIB_PATH)
+        L = ctypes.CDLL(PROBE_LIB_PATH)
+        P, I, Z = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+        L.decx_probe_hgemm.argtypes, L.decx_probe_hgemm.restype = [I, I, P, P, I, P, I, P, I, I, I, I, I, I], I
+        L.decx_probe_copy.argtypes, L.decx_probe_copy.restype = [P, P, P, Z], I
+        _probe = L
+    return _probe
+
+
+def stream():
+    return lib().decx_hip_stream()
 
 
 def last_error():

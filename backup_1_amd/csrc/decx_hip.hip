@@ -3,6 +3,7 @@
 // Declarations and the reference interface each entry point stands in for: include/decx_hip.h.
 #include "runtime.hpp"
 
+#include <chrono>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -57,7 +58,9 @@ int check_gemm_args(const void* A, int lda, const void* B, int ldb, const void* 
     return 0;
 }
 
-// the fp32 workspace of the fp16 split-K paths: grown on demand, kept until the process ends
+// the fp32 workspace of the fp16 split-K paths: reserved by decx_hip_init for every split the library chooses by itself
+// (at most one 128x128 tile and range per CU, twice that in the atomic mode's tile count), grown only for larger forced
+// splits, kept until the process ends
 int ensure_partial(size_t need) {
     if (need <= g_rt.partial_bytes) return 0;
     HIP_TRY(hipDeviceSynchronize());               // earlier launches may still use the old workspace
@@ -273,13 +276,6 @@ int gemm_host_pipeline(const T* hA, int lda, const T* hB, int ldb, const T* hC, 
     return 0;
 }
 
-// Plain streaming copy, 16 bytes per lane and iteration: the known-size kernel that hardware traffic counters
-// (FETCH_SIZE / WRITE_SIZE) are calibrated against.
-__global__ __launch_bounds__(256) void copy_kernel(f32x4* __restrict__ dst, const f32x4* __restrict__ src, size_t quads) {
-    const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < quads; i += stride) dst[i] = src[i];
-}
-
 // Element-wise ReLU family of nn/operators/ReLU.h.  MODE 0: forward; 1: forward + record; 2: backward (dst = src where
 // the recorded bit is set, else 0 * src; ReLU.h:131-165).  The bit map has one byte per 8 consecutive floats: bits 4..7
 // = the first 16-byte quad's x,y,z,w, bits 0..3 = the second quad's (ReLU.h:86-123).
@@ -343,10 +339,44 @@ int relu_enqueue(const float* src, float* dst, unsigned char* rec_map, size_t n)
     return 0;
 }
 
-int finish(int rc) {
-    if (rc != 0) return rc;
+// One lane stores `value` to a word of pinned, host-coherent memory (system scope, release).
+__global__ __launch_bounds__(64) void completion_flag_kernel(unsigned* host_flag, unsigned value) {
+    if (threadIdx.x == 0) __atomic_store_n(host_flag, value, __ATOMIC_RELEASE);
+}
+
+// Waits until the compute work enqueued on the library's stream is complete.  Every call of the reference's API blocks
+// (cudaDeviceSynchronize, GEMM.h:122, :450; conv2_mk_im2col.h:268), so this is on the path of every drop-in call, and
+// most of them are kernels of tens of microseconds.  Measured on an MI355X around a 60 us kernel: launch +
+// hipStreamSynchronize returns 11.4 us after the kernel's own time, polling hipStreamQuery or an event no sooner; a
+// one-lane kernel enqueued behind it that stores a sequence number to a word of host-coherent pinned memory, which
+// the host polls, 7.9 us.  The stream runs kernels in order, each starting after the one before has completed and
+// released its writes, so when the number arrives every kernel enqueued before it is complete.  The host polls for
+// a bounded time only (spin_wait_us; a faulting kernel never delivers the number) and then, as for spin_wait_us = 0,
+// waits in hipStreamSynchronize.
+int wait_compute() {
+    if (g_rt.spin_wait_us > 0 && g_rt.done_flag) {
+        const unsigned seq = ++g_rt.done_seq;
+        hipLaunchKernelGGL(completion_flag_kernel, dim3(1), dim3(64), 0, g_rt.stream, g_rt.done_flag, seq);
+        HIP_TRY(hipGetLastError());
+        const auto t0 = std::chrono::steady_clock::now();
+        for (unsigned polls = 1;; ++polls) {
+            if (__atomic_load_n(g_rt.done_flag, __ATOMIC_ACQUIRE) == seq) return 0;
+            if ((polls & 255u) == 0 && std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(g_rt.spin_wait_us)) break;
+        }
+    }
     HIP_TRY(hipStreamSynchronize(g_rt.stream));
     return 0;
+}
+
+// copies and fills: the host may read what they wrote the moment the call returns, so these wait in the runtime
+int wait_stream() {
+    HIP_TRY(hipStreamSynchronize(g_rt.stream));
+    return 0;
+}
+
+int finish(int rc) {
+    if (rc != 0) return rc;
+    return wait_compute();
 }
 
 }  // namespace
@@ -373,7 +403,21 @@ int decx_hip_init(int* device) {
         HIP_TRY(hipEventCreate(&g_rt.ev_start));
         HIP_TRY(hipEventCreate(&g_rt.ev_stop));
         if (const char* gm = getenv("DECX_HIP_GROUP_M")) { int v = atoi(gm); if (v > 0) g_rt.group_m = v; }
+        if (const char* sw = getenv("DECX_HIP_SPIN_WAIT_US")) { int v = atoi(sw); if (v >= 0) g_rt.spin_wait_us = v; }
+        {
+            void* flag = nullptr;                              // the word the completion kernel writes and wait_compute polls
+            if (hipHostMalloc(&flag, 64, hipHostMallocCoherent) != hipSuccess) {
+                (void)hipGetLastError();
+                flag = nullptr;                                // blocking calls then wait in hipStreamSynchronize
+            } else {
+                *static_cast<unsigned*>(flag) = 0;
+            }
+            g_rt.done_flag = static_cast<unsigned*>(flag);
+            g_rt.done_seq = 0;
+        }
         if (int rc = hgemm_static_scratch_init(dev)) return rc;
+        // so that the _async fp16 entry points never synchronise the device to grow the workspace
+        if (int rc = ensure_partial((size_t)2 * (size_t)(g_rt.compute_units > 0 ? g_rt.compute_units : 256) * 128 * 128 * sizeof(float))) return rc;
         g_rt.is_init = true;
     }
     if (device) *device = g_rt.device;
@@ -410,8 +454,7 @@ int decx_hip_free(void* dptr) {
 int decx_hip_memset(void* dptr, int value, size_t bytes) {
     if (!g_rt.is_init) return need_init();
     HIP_TRY(hipMemsetAsync(dptr, value, bytes, g_rt.stream));
-    HIP_TRY(hipStreamSynchronize(g_rt.stream));
-    return 0;
+    return wait_stream();
 }
 
 int decx_hip_host_malloc(void** hptr, size_t bytes) {
@@ -448,8 +491,7 @@ int decx_hip_memcpy2d(void* dst, size_t dst_pitch_bytes, const void* src, size_t
         return fail(DECX_HIP_FAIL_ERROR_PARAMS, "pitch smaller than the row width\n");
     HIP_TRY(hipMemcpy2DAsync(dst, dst_pitch_bytes, src, src_pitch_bytes, width_bytes, rows, copy_kind(direction),
                              g_rt.stream));
-    HIP_TRY(hipStreamSynchronize(g_rt.stream));
-    return 0;
+    return wait_stream();
 }
 
 int decx_hip_memcpy(void* dst, const void* src, size_t bytes, int direction) {
@@ -457,8 +499,7 @@ int decx_hip_memcpy(void* dst, const void* src, size_t bytes, int direction) {
     if (direction < DECX_HIP_H2D || direction > DECX_HIP_D2D) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "bad copy direction\n");
     if (bytes == 0) return 0;
     HIP_TRY(hipMemcpyAsync(dst, src, bytes, copy_kind(direction), g_rt.stream));
-    HIP_TRY(hipStreamSynchronize(g_rt.stream));
-    return 0;
+    return wait_stream();
 }
 
 int decx_hip_sync(void) {
@@ -583,17 +624,7 @@ int decx_hip_relu_f32_backward(const float* src, float* dst, const unsigned char
     return finish(relu_enqueue<2>(src, dst, const_cast<unsigned char*>(rec_map), n));
 }
 
-int decx_hip_copy_kernel(void* dst, const void* src, size_t bytes) {
-    if (!g_rt.is_init) return need_init();
-    if (!dst || !src || bytes % 16 != 0 || !aligned16(dst) || !aligned16(src))
-        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "copy needs 16-byte aligned pointers and a multiple of 16 bytes\n");
-    if (bytes == 0) return 0;
-    const int blocks = g_rt.compute_units > 0 ? g_rt.compute_units * 8 : 2048;
-    hipLaunchKernelGGL(copy_kernel, dim3(blocks), dim3(256), 0, g_rt.stream, static_cast<f32x4*>(dst),
-                       static_cast<const f32x4*>(src), bytes / 16);
-    HIP_TRY(hipGetLastError());
-    return finish(0);
-}
+void* decx_hip_stream(void) { return g_rt.is_init ? static_cast<void*>(g_rt.stream) : nullptr; }
 
 int decx_hip_timer_start(void) {
     if (!g_rt.is_init) return need_init();
@@ -622,10 +653,6 @@ int decx_hip_set_hgemm_variant(int variant) {
     int prev = g_rt.hgemm_variant;
     g_rt.hgemm_variant = variant;
     return prev;
-}
-
-int decx_hip_hgemm_probe(int ablate, const uint16_t* A, int lda, const uint16_t* B, int ldb, uint16_t* D, int ldd, int M, int N, int K) {
-    return hgemm_probe_enqueue(ablate, A, lda, B, ldb, D, ldd, M, N, K);
 }
 
 int decx_hip_set_splitk_mode(int mode) {

@@ -29,6 +29,8 @@ namespace decx_hip {
 //      loads is not what the kernel loses time to (4 waves of 128x128, a quarter fewer LDS reads, measured 1387 too: on
 //      uniform[-1,1] data every arrangement ends at the same power-limited rate); kept as the second instantiation of
 //      the kernel's stage arithmetic
+//  17: as 15 with one workgroup per compute unit that walks its tiles as one stream of K steps (no prologue after the
+//      first tile, the epilogue under the next tile's loads); products of whole tiles only, others fall back to 15
 //  11: split-K on shape 8 through an fp32 workspace (hgemm_splitk_enqueue) -- few tiles and a long K
 // and, for the fp16 convolution only: 12 keeps its register-staged kernels, 13 takes its LDS-DMA kernel for any image
 // whose channel pitch allows it, 14 its tap-row kernel; each switches its split over K off (experiments and tests)
@@ -70,33 +72,36 @@ int launch_hgemm_mfma16(const uint16_t* A, int lda, const uint16_t* B, int ldb, 
     return 0;
 }
 
-// Measurement variants of the kernel above (decx_hip_hgemm_probe): same launch, parts of the K walk left out.
-int hgemm_probe_enqueue(int ablate, const uint16_t* A, int lda, const uint16_t* B, int ldb, uint16_t* D, int ldd, int M, int N, int K) {
-    typedef HShape16 S;
-    Batch batch;
-    batch.stream = g_rt.stream;
-    if (int rc = check_gemm_args(A, lda, B, ldb, nullptr, 0, D, ldd, M, N, K, batch)) return rc;
-    if (!aligned16(A) || !aligned16(B) || lda % 8 || ldb % 8 || (size_t)lda * 512 >= ((size_t)1 << 32) || (size_t)ldb * 128 >= ((size_t)1 << 32))
-        return fail(DECX_HIP_FAIL_ERROR_PARAMS, "the probe needs 16-byte aligned A, B with lda, ldb multiples of 8\n");
-    void (*kern)(const _Float16*, int, const _Float16*, int, const _Float16*, int, _Float16*, int, int, int, int, int, int, int, size_t,
-                 size_t, size_t, size_t) = nullptr;
-    switch (ablate) {
-        case 0: kern = hgemm_mfma16_kernel<S, false, 0>; break;
-        case 1: kern = hgemm_mfma16_kernel<S, false, 1>; break;
-        case 3: kern = hgemm_mfma16_kernel<S, false, 3>; break;
-        case 4: kern = hgemm_mfma16_kernel<S, false, 4>; break;
-        case 5: kern = hgemm_mfma16_kernel<S, false, 5>; break;
-        case 6: kern = hgemm_mfma16_kernel<S, false, 6>; break;
-        case 7: kern = hgemm_mfma16_kernel<S, false, 7>; break;
-        default: return fail(DECX_HIP_FAIL_ERROR_PARAMS, "probe variants: 0, 1, 3, 4, 5, 6, 7\n");
+// The same tile as one workgroup per compute unit that walks its tiles as one stream of K steps (PERSIST build of the
+// kernel): whole tiles only, one problem per launch.
+template <class S>
+bool hgemm_mfma16_persistent_fits(int M, int N, int K, const Batch& batch) {
+    const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+    return batch.count == 1 && M % S::BM == 0 && N % S::BN == 0 && K % (S::BK * S::WALK) == 0 && K >= S::BK * S::STAGES &&
+           (long)(M / S::BM) * (N / S::BN) > cus;                  // with at most one tile per CU there is nothing to chain
+}
+
+template <class S>
+int launch_hgemm_mfma16_persistent(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
+                                   int ldd, int M, int N, int K, const Batch& batch) {
+    auto kern = Cin ? hgemm_mfma16_kernel<S, true, 0, true> : hgemm_mfma16_kernel<S, false, 0, true>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hgemm_mfma16_kernel<S, true, 0, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::PERSIST_LDS_BYTES));
+        HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hgemm_mfma16_kernel<S, false, 0, true>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::PERSIST_LDS_BYTES));
+        attr_done = true;
     }
-    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)S::LDS_BYTES));
-    const int tiles_m = cdiv(M, S::BM), tiles_n = cdiv(N, S::BN);
+    const int tiles_m = M / S::BM, tiles_n = N / S::BN;
+    const long total = (long)tiles_m * tiles_n;
+    if (total > 0x7fffffffL) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "problem too large for one launch\n");
+    const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     const int group_m = tiles_m < g_rt.group_m ? tiles_m : g_rt.group_m;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tiles_m * tiles_n)), dim3(S::NT), S::LDS_BYTES, batch.stream,
+    hipLaunchKernelGGL(kern, dim3((unsigned)(total < cus ? total : cus)), dim3(S::NT), S::PERSIST_LDS_BYTES, batch.stream,
                        reinterpret_cast<const _Float16*>(A), lda, reinterpret_cast<const _Float16*>(B), ldb,
-                       static_cast<const _Float16*>(nullptr), 0, reinterpret_cast<_Float16*>(D), ldd, M, N, K, tiles_m, tiles_n, group_m,
-                       (size_t)0, (size_t)0, (size_t)0, (size_t)0);
+                       reinterpret_cast<const _Float16*>(Cin), ldc, reinterpret_cast<_Float16*>(D), ldd, M, N, K,
+                       tiles_m, tiles_n, group_m, (size_t)0, (size_t)0, (size_t)0, (size_t)0);
     HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -235,7 +240,7 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
     int variant = g_rt.hgemm_variant;
     {
         // few 128x128 tiles and a long K: split K (variant 11 forces it, any other fixed variant switches it off)
-        if (batch.count == 1 && (variant < 1 || variant > 10) && (variant < 15 || variant > 16)) {
+        if (batch.count == 1 && (variant < 1 || variant > 10) && (variant < 15 || variant > 17)) {
             int splits = auto_hgemm_splits(M, N, K);
             if (variant == 11 && splits == 0 && K >= 1024 && (size_t)M * N <= ((size_t)1 << 26)) {
                 const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
@@ -248,7 +253,7 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
         }
         if (variant == 11) variant = 0;
     }
-    if (variant < 1 || (variant > 10 && (variant < 15 || variant > 16))) {
+    if (variant < 1 || (variant > 10 && (variant < 15 || variant > 17))) {
         // same cost model as the fp32 picker: rounds of tiles per CU x tile area / measured shape efficiency
         const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
         const long big = (long)cdiv(M, 256) * cdiv(N, 256) * batch.count, small = (long)cdiv(M, 128) * cdiv(N, 128) * batch.count;
@@ -256,6 +261,11 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
         const double cost_small = (double)((small + cus - 1) / cus) * 16384.0 / 0.75;
         // the small tile with three LDS stages holds one workgroup per CU: only worth it when there is at most one to hold
         variant = cost_big <= cost_small ? 15 : (small <= cus ? 9 : 8);
+    }
+    if (variant == 17) {
+        if (hgemm_mfma16_persistent_fits<HShape16>(M, N, K, batch))
+            return launch_hgemm_mfma16_persistent<HShape16>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+        variant = 15;
     }
     if (variant == 15) return launch_hgemm_mfma16<HShape16>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     if (variant == 16) return launch_hgemm_mfma16<HShape16K32S4>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
@@ -273,7 +283,7 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
 
 // ---------------------------------------------------------------------------------------------------------------
 // The K-range route on a workspace that is part of the library's code object instead of an allocation: for callers
-// that must not allocate device memory (code under graph capture, serving loops, harnesses that forbid it).  Every GPU
+// that must not allocate device memory (serving loops, harnesses that forbid it).  Every GPU
 // the library is loaded on holds its own copy of the array until the process ends; host code reaches it only through
 // the address hipGetSymbolAddress returns for the current device.
 // ---------------------------------------------------------------------------------------------------------------

@@ -57,6 +57,9 @@ struct Hgemm16Shape {
     static constexpr int A_UNITS = BM * UA, B_UNITS = BK * UB;
     static constexpr int A_BYTES = A_UNITS * 16, B_BYTES = B_UNITS * 16;
     static constexpr size_t LDS_BYTES = (size_t)STAGES * (A_BYTES + B_BYTES);
+    // the many-tiles-per-workgroup build parks results in chunks of PARK_ROWS rows per wave behind the stages
+    static constexpr int PARK_ROWS = 32;
+    static constexpr size_t PERSIST_LDS_BYTES = LDS_BYTES + (size_t)WAVES_M_ * WAVES_N_ * PARK_ROWS * (BN_ / WAVES_N_) * 2;
     static constexpr int A_LOADS = A_UNITS / 64 / NWAVES, B_LOADS = B_UNITS / 64 / NWAVES, LOADS = A_LOADS + B_LOADS;
     static constexpr int A_PASSES = A_UNITS / NT, B_PASSES = B_UNITS / NT;
     static_assert(BK == 32 || BK == 64, "one or two k-blocks of 32 per K step");
@@ -79,8 +82,22 @@ struct Hgemm16Shape {
 // ABLATE != 0 builds measurement variants that leave work out of the K walk and produce no meaningful result (the cost of
 // each part of the kernel is the difference between two of them): bit 0 = the K walk issues no DMA loads (LDS keeps
 // the first two K steps), bit 1 = it issues no LDS reads (the registers keep the first fragments), bit 2 = the result
-// is not stored.  Only decx_hip_hgemm_probe launches them.
-template <class S, bool HAS_C, int ABLATE = 0>
+// is not stored, bit 3 = the loads of the K walk never move on (every step fetches the tile's first K step again, which
+// the caches then hold: the loads without their misses).  Bits 4-5 pick the order of the 16 matrix instructions of a
+// unit: 0 = row block by row block with the column order reversed on every other one, so that exactly one operand
+// changes between any two instructions of a k-block (the product's order: on uniform[-1,1] operands the matrix pipe
+// draws measurably less power than when both operands change at every row block, and the chip clocks 2 % higher);
+// 1 = row block by row block, columns always ascending; 2 = column block by column block (the B fragment stays).
+// The sums do not depend on the order: every accumulator sees its k-blocks ascending.  Only the probe library
+// launches variants with any of these bits set.
+//
+// PERSIST: the grid holds one workgroup per compute unit and a workgroup walks the tiles blockIdx.x, blockIdx.x +
+// gridDim.x, ... as one stream of K steps: the loads that refill the stages during a tile's last STAGES steps fetch the
+// first steps of the next tile (where the one-tile kernel repeats the last step), so no tile after the first has a
+// prologue, and the epilogue -- through a parking area of its own behind the stages, 4 KB per wave -- runs while
+// those loads are in flight.  For whole tiles only: M % BM == 0, N % BN == 0, K % (BK * WALK) == 0, K >= BK * STAGES,
+// one problem per launch (the host checks).
+template <class S, bool HAS_C, int ABLATE = 0, bool PERSIST = false>
 __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __restrict__ A, int lda,
                                                              const _Float16* __restrict__ B, int ldb, const _Float16* Cin,
                                                              int ldc, _Float16* D, int ldd, int M, int N, int K, int tiles_m,
@@ -90,6 +107,7 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
     constexpr int UM = S::UM, MH = S::MH, KS = S::KS, UNITS = S::UNITS, STAGES = S::STAGES, WALK = S::WALK;
     constexpr int A_BYTES = S::A_BYTES, B_BYTES = S::B_BYTES;
     constexpr int BLK = UM * NI;                                // MFMAs per unit
+    constexpr int ORDER = (ABLATE >> 4) & 3;
     A += (size_t)blockIdx.y * a_batch_stride;
     B += (size_t)blockIdx.y * b_batch_stride;
     if (HAS_C) Cin += (size_t)blockIdx.y * c_batch_stride;
@@ -97,8 +115,10 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];   // [A stages][B stages]
     const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char*)lds_raw;
 
-    const TileCoord tc = xcd_grouped_tile(blockIdx.x, tiles_m, tiles_n, group_m);
-    const int bm0 = tc.tm * BM, bn0 = tc.tn * BN;
+    const int total_tiles = tiles_m * tiles_n;
+    int tile = blockIdx.x;
+    const TileCoord tc = xcd_grouped_tile(tile, tiles_m, tiles_n, group_m);
+    int bm0 = tc.tm * BM, bn0 = tc.tn * BN;
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / kWave), lane = tid % kWave;
     const int wm0 = (wave / S::WAVES_N) * S::WM, wn0 = (wave % S::WAVES_N) * S::WN;
@@ -107,7 +127,7 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
     // ---- DMA sources: wave-uniform bases that advance by one K step per fetched step + loop-invariant lane offsets
     const int m_first = bm0 < M ? bm0 : M - 1;
     const _Float16* a_base = A + (size_t)m_first * lda;
-    const _Float16* b_base = B;
+    const _Float16* b_base = PERSIST ? B + bn0 : B;              // PERSIST: lane offsets are the same for every (whole) tile
     uint32_t a_off[S::A_LOADS], b_off[S::B_LOADS];
 #pragma unroll
     for (int j = 0; j < S::A_LOADS; ++j) {
@@ -123,7 +143,7 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
         const int chunk = wave * S::B_LOADS + j;                // 64 units = 64 / UB k-rows
         const int kr = chunk * (64 / UB) + lane / UB;
         const int u = (lane % UB) ^ (((kr & 3) << 2) | (((kr >> 3) & 1) << 1));
-        const int col = clamp_group_col(bn0 + 8 * u, N, 8);     // stay inside the operand; such columns are never stored
+        const int col = PERSIST ? 8 * u : clamp_group_col(bn0 + 8 * u, N, 8);     // stay inside the operand; such columns are never stored
         b_off[j] = (uint32_t)(((size_t)kr * ldb + col) * sizeof(_Float16));
     }
     // Every K step fetches the step STAGES ahead of it into the stage it leaves, also the last STAGES, which have nothing
@@ -132,6 +152,18 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
     const int full_steps = K / BK;
     int steps_fetched = 0;
     const size_t b_step = (size_t)BK * ldb;
+    // PERSIST: where the fetches go on once the current tile's steps are all out (set before each tile's walk)
+    const _Float16* a_next = a_base;
+    const _Float16* b_next = b_base;
+    bool has_next = false;
+    auto plan_next_tile = [&]() {
+        const int nt = tile + (int)gridDim.x;
+        has_next = nt < total_tiles;
+        const TileCoord nc = xcd_grouped_tile(has_next ? nt : tile, tiles_m, tiles_n, group_m);
+        a_next = A + (size_t)(nc.tm * BM) * lda;
+        b_next = B + nc.tn * BN;
+    };
+    if constexpr (PERSIST) plan_next_tile();
     auto issue_one = [&](auto stage_tag, auto j_tag, auto in_walk_tag) {
         constexpr int STG = decltype(stage_tag)::value, J = decltype(j_tag)::value;
         if constexpr ((ABLATE & 1) && decltype(in_walk_tag)::value) return;
@@ -141,11 +173,18 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
             constexpr int JB = J - S::A_LOADS;
             dma_load16_tagged<STG * 64 + J>(b_base, b_off[JB], lds_base + (uint32_t)(STAGES * A_BYTES + STG * B_BYTES) + (uint32_t)(wave * S::B_LOADS + JB) * 1024u);
         }
-        if constexpr (J == S::LOADS - 1) {
+        if constexpr (J == S::LOADS - 1 && !(ABLATE & 8)) {
             ++steps_fetched;
-            const bool more = steps_fetched < full_steps;        // scalar: the next fetch is a new step
-            a_base += more ? BK : 0;
-            b_base += more ? b_step : (size_t)0;
+            const bool more = steps_fetched < full_steps;        // scalar: the next fetch is a new step of this tile
+            if constexpr (PERSIST) {
+                const bool wrap = !more && has_next && steps_fetched == full_steps;      // ... or the first of the next
+                a_base = more ? a_base + BK : (wrap ? a_next : a_base);
+                b_base = more ? b_base + b_step : (wrap ? b_next : b_base);
+                steps_fetched = wrap ? 0 : (more ? steps_fetched : full_steps);
+            } else {
+                a_base += more ? BK : 0;
+                b_base += more ? b_step : (size_t)0;
+            }
         }
     };
 
@@ -217,10 +256,12 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
     // MFMA number I of unit U of walk step V: row block (U % MH) * UM + I / NI, column block I % NI
     auto mfma_one = [&](auto v_tag, auto u_tag, auto i_tag) {
         constexpr int U = decltype(u_tag)::value, I = decltype(i_tag)::value;
-        constexpr int KB = U / MH, MIX = (U % MH) * UM + I / NI, NIX = I % NI, BS = DECX_BSET(decltype(v_tag)::value, KB);
+        constexpr int ROWB = ORDER == 2 ? I % UM : I / NI;                              // row block within the unit
+        constexpr int NIX = ORDER == 2 ? I / UM : (ORDER == 0 && (ROWB & 1) ? NI - 1 - I % NI : I % NI);
+        constexpr int KB = U / MH, MIX = (U % MH) * UM + ROWB, BS = DECX_BSET(decltype(v_tag)::value, KB);
         const i16x4 lo = blo[BS][NIX], hi = bhi[BS][NIX];
         const i16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        acc[MIX][NIX] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, both), af[U & 1][I / NI], acc[MIX][NIX], 0, 0, 0);
+        acc[MIX][NIX] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, both), af[U & 1][ROWB], acc[MIX][NIX], 0, 0, 0);
     };
 #define DECX_PIN() __builtin_amdgcn_sched_barrier(0)
 
@@ -277,29 +318,33 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
     };
 
     typedef std::integral_constant<int, 0> I0;
+    bool first_tile = true;                                     // PERSIST: later tiles find their first steps fetched already
+    for (;;) {
     if (full_steps > 0) {
         // The walk starts at walk step `first` such that it ends with step WALK - 1: a first pass that begins at `first`,
         // then whole passes.  The prologue fills all stages, K step j into stage (first + j) % STAGES.
-        const int first = (WALK - full_steps % WALK) % WALK;
-        static_for<0, WALK>([&](auto v0) {
-            if (first == decltype(v0)::value) {
-                static_for<0, STAGES>([&](auto j) {
-                    typedef std::integral_constant<int, (decltype(v0)::value + decltype(j)::value) % STAGES> Stg;
-                    static_for<0, S::LOADS>([&](auto l) { issue_one(Stg{}, l, std::false_type{}); });
-                });
-                wait_dma_then_barrier<S::LOADS*(STAGES - 1)>();          // step 0 has landed
-                static_for<0, FIRST_READS>([&](auto r) { read_first(v0, r); });
-            }
-        });
-        DECX_PIN();
-        if constexpr (ABLATE & 2) {                              // the sets the walk would have filled
+        const int first = PERSIST ? 0 : (WALK - full_steps % WALK) % WALK;
+        if (first_tile) {
+            static_for<0, WALK>([&](auto v0) {
+                if (first == decltype(v0)::value) {
+                    static_for<0, STAGES>([&](auto j) {
+                        typedef std::integral_constant<int, (decltype(v0)::value + decltype(j)::value) % STAGES> Stg;
+                        static_for<0, S::LOADS>([&](auto l) { issue_one(Stg{}, l, std::false_type{}); });
+                    });
+                    wait_dma_then_barrier<S::LOADS*(STAGES - 1)>();          // step 0 has landed
+                    static_for<0, FIRST_READS>([&](auto r) { read_first(v0, r); });
+                }
+            });
+            DECX_PIN();
+            if constexpr (ABLATE & 2) {                              // the sets the walk would have filled
 #pragma unroll
-            for (int x = 0; x < UM; ++x) af[1][x] = af[0][x];
+                for (int x = 0; x < UM; ++x) af[1][x] = af[0][x];
 #pragma unroll
-            for (int x = 0; x < NI; ++x) {
-                const i16x4 lo = blo[0][x] | blo[1][x], hi = bhi[0][x] | bhi[1][x];      // whichever set was read
-                blo[0][x] = blo[1][x] = lo;
-                bhi[0][x] = bhi[1][x] = hi;
+                for (int x = 0; x < NI; ++x) {
+                    const i16x4 lo = blo[0][x] | blo[1][x], hi = bhi[0][x] | bhi[1][x];      // whichever set was read
+                    blo[0][x] = blo[1][x] = lo;
+                    bhi[0][x] = bhi[1][x] = hi;
+                }
             }
         }
         // the first pass skips the walk steps before `first` (a scalar branch around each step)
@@ -313,7 +358,7 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
     }
 
     // ---- partial last K step: through registers into stage 0 (zero-filled beyond K), then all of its units
-    if (full_steps * BK < K) {
+    if (!PERSIST && full_steps * BK < K) {
         const int k0 = full_steps * BK;
         u32x4 a_stage[S::A_PASSES], b_stage[S::B_PASSES];
 #pragma unroll
@@ -370,59 +415,84 @@ __global__ __launch_bounds__(S::NT) void hgemm_mfma16_kernel(const _Float16* __r
             static_for<0, BLK>([&](auto i_tag) { mfma_one(I0{}, u_tag, i_tag); });
         });
     }
-#undef DECX_BSET
-#undef DECX_PIN
 
     // ---- epilogue.  acc[mi][ni][e] is element (row 16 mi + li, column 16 ni + 4 lg + e) of the wave's piece.  dst = A*B + C
-    // adds C in fp32; one rounding to binary16; the piece goes to LDS (rows of WN halves, 16-byte pieces XOR-swizzled by
-    // the row) and leaves as 16-byte stores.
-    wait_dma_then_barrier<0>();                                 // nobody reads operands any more, and the last (redundant) stage loads have landed
-    constexpr int ROW_BYTES = S::WN * 2, PIECES = S::WN / 8, ROWS_PER_PASS = kWave / PIECES, PASSES = S::WM / ROWS_PER_PASS;
+    // adds C in fp32; one rounding to binary16; the piece goes to LDS in chunks of CH_ROWS rows (rows of WN halves, 16-byte
+    // pieces XOR-swizzled by the row) and leaves as 16-byte stores.  One chunk in the operand buffers, which are free by
+    // then; PERSIST: chunks of 32 rows in the wave's own 4 KB behind the stages, which are being refilled meanwhile.
+    if constexpr (!PERSIST) wait_dma_then_barrier<0>();         // nobody reads operands any more, and the last (redundant) stage loads have landed
+    constexpr int ROW_BYTES = S::WN * 2, PIECES = S::WN / 8, ROWS_PER_PASS = kWave / PIECES;
+    constexpr int CH_ROWS = PERSIST ? S::PARK_ROWS : S::WM, CHUNKS = S::WM / CH_ROWS, PASSES = CH_ROWS / ROWS_PER_PASS;
     static_assert(PIECES >= 8 && (PIECES & (PIECES - 1)) == 0 && kWave % PIECES == 0, "piece swizzle");
-    unsigned char* park = lds_raw + (size_t)wave * (S::WM * ROW_BYTES);
+    static_assert(CH_ROWS % 16 == 0 && S::WM % CH_ROWS == 0 && CH_ROWS % ROWS_PER_PASS == 0, "chunks of whole row blocks");
+    unsigned char* park = PERSIST ? lds_raw + S::LDS_BYTES + (size_t)wave * (CH_ROWS * ROW_BYTES) : lds_raw + (size_t)wave * (S::WM * ROW_BYTES);
     const int m_wave = bm0 + wm0, n_wave = bn0 + wn0;
-#pragma unroll
-    for (int mi = 0; mi < MI; ++mi)
-#pragma unroll
-        for (int ni = 0; ni < NI; ++ni) {
-            const int row = 16 * mi + li, col = 16 * ni + 4 * lg;
-            f32x4v v = acc[mi][ni];
-            if (HAS_C) {
-                const int m = m_wave + row, n = n_wave + col;
-                if (m < M) {
-                    const _Float16* crow = Cin + (size_t)m * ldc + n;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (n + e < N) v[e] += (float)crow[e];
-                }
-            }
-            const f16x4 h = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-            const int piece = col >> 3;
-            *reinterpret_cast<u32x2*>(park + row * ROW_BYTES + ((piece ^ (row & 7)) << 4) + ((lg & 1) << 3)) = __builtin_bit_cast(u32x2, h);
-        }
     // the wave reads back what it wrote itself: LDS operations of a wave complete in order, no barrier needed
     const bool vec_d = ((reinterpret_cast<uintptr_t>(D) | (uintptr_t)(ldd * 2)) & 15) == 0;
     const bool whole = bm0 + BM <= M && bn0 + BN <= N && vec_d;     // one scalar test instead of checks around every store
 #pragma unroll
-    for (int pass = 0; pass < PASSES; ++pass) {
-        const int row = pass * ROWS_PER_PASS + lane / PIECES, piece = lane % PIECES;
-        const u32x4 v = *reinterpret_cast<const u32x4*>(park + row * ROW_BYTES + ((piece ^ (row & 7)) << 4));
-        const int m = m_wave + row, n = n_wave + 8 * piece;
-        _Float16* dp = D + (size_t)m * ldd + n;
-        if ((ABLATE & 4) && K >= 0) continue;                    // (a condition the compiler cannot fold, so the sums stay live)
-        if (whole) {
-            __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dp));      // written once, not read by this launch
-        } else if (m < M) {
-            if (vec_d && n + 8 <= N) {
-                *reinterpret_cast<u32x4*>(dp) = v;
-            } else {
-                const f16x8 h = __builtin_bit_cast(f16x8, v);
+    for (int ch = 0; ch < CHUNKS; ++ch) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (n + e < N) dp[e] = h[e];
+        for (int mc = 0; mc < CH_ROWS / 16; ++mc)
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni) {
+                const int mi = ch * (CH_ROWS / 16) + mc;
+                const int row = 16 * mc + li, col = 16 * ni + 4 * lg;           // row within the chunk
+                f32x4v v = acc[mi][ni];
+                if (HAS_C) {
+                    const int m = m_wave + ch * CH_ROWS + row, n = n_wave + col;
+                    if (m < M) {
+                        const _Float16* crow = Cin + (size_t)m * ldc + n;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (n + e < N) v[e] += (float)crow[e];
+                    }
+                }
+                const f16x4 h = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+                const int piece = col >> 3;
+                *reinterpret_cast<u32x2*>(park + row * ROW_BYTES + ((piece ^ (row & 7)) << 4) + ((lg & 1) << 3)) = __builtin_bit_cast(u32x2, h);
+            }
+#pragma unroll
+        for (int pass = 0; pass < PASSES; ++pass) {
+            const int row = pass * ROWS_PER_PASS + lane / PIECES, piece = lane % PIECES;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(park + row * ROW_BYTES + ((piece ^ (row & 7)) << 4));
+            const int m = m_wave + ch * CH_ROWS + row, n = n_wave + 8 * piece;
+            _Float16* dp = D + (size_t)m * ldd + n;
+            if ((ABLATE & 4) && K >= 0) continue;                    // (a condition the compiler cannot fold, so the sums stay live)
+            if (whole) {
+                __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dp));      // written once, not read by this launch
+            } else if (m < M) {
+                if (vec_d && n + 8 <= N) {
+                    *reinterpret_cast<u32x4*>(dp) = v;
+                } else {
+                    const f16x8 h = __builtin_bit_cast(f16x8, v);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (n + e < N) dp[e] = h[e];
+                }
             }
         }
     }
+    if constexpr (!PERSIST) {
+        break;
+    } else {
+        if (!has_next) break;
+        tile += (int)gridDim.x;
+        const TileCoord nc = xcd_grouped_tile(tile, tiles_m, tiles_n, group_m);
+        bm0 = nc.tm * BM;
+        bn0 = nc.tn * BN;
+        plan_next_tile();
+        first_tile = false;
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni) acc[mi][ni] = f32x4v{0.f, 0.f, 0.f, 0.f};
+    }
+    }   // tiles of this workgroup
+    // PERSIST: the loads of the last steps (repeats, nobody reads them) must have landed before the workgroup gives up its LDS
+    if constexpr (PERSIST) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#undef DECX_BSET
+#undef DECX_PIN
 }
 
 }  // namespace decx_hip

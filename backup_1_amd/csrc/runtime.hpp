@@ -24,6 +24,10 @@ struct Runtime {
     size_t partial_bytes = 0;
     int splitk_atomic = 0;         // fp16 split-K: 0 = one workspace plane per K range, added in range order (the same
                                    // result on every run); 1 = all ranges add into one plane with atomics
+    int spin_wait_us = 2000;       // a blocking compute call polls its completion word this long before it waits in
+                                   // hipStreamSynchronize (env DECX_HIP_SPIN_WAIT_US overrides; 0 = wait there at once)
+    unsigned* done_flag = nullptr; // pinned, host-coherent word a one-lane kernel behind the work stores done_seq to
+    unsigned done_seq = 0;
     int group_m = 8;   // tile-rows per raster group of the XCD-aware tile walk (env DECX_HIP_GROUP_M overrides, for tuning)
 };
 extern Runtime g_rt;
@@ -72,8 +76,6 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
                  int flag, const float* bias = nullptr, bool relu = false);
 int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                   int ldd, int M, int N, int K, const Batch& batch);
-// measurement variants of the large fp16 tile with parts of its K walk left out (no meaningful result)
-int hgemm_probe_enqueue(int ablate, const uint16_t* A, int lda, const uint16_t* B, int ldb, uint16_t* D, int ldd, int M, int N, int K);
 // the K-range route of hgemm_enqueue on the library's static device workspace (no allocation); splits <= 0: automatic
 int hgemm_splitk_static_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
                                 uint16_t* D, int ldd, int M, int N, int K, int splits);

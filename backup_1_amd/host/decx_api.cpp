@@ -109,11 +109,28 @@ de::DH gemm_device(de::GPU_Matrix<T>& A_, de::GPU_Matrix<T>& B_, de::GPU_Matrix<
     if (!decx_hip_is_init()) return not_init();                                           // GEMM.h:403
     if (A->width != B->height) return de::DH{decx::DECX_FAIL_DimsNotMatching, kGemmDims}; // GEMM.h:408
     if (C && (C->width != B->width || C->height != A->height)) return de::DH{decx::DECX_FAIL_DimsNotMatching, kMDims};
-    if (C != dst && !dst->re_construct(B->width, A->height))                              // GEMM.h:414 (fp16 too: defect D7 not kept)
+    // A dst that is A or B, or shares its payload with one of them (operator= shares, GPU_Matrix.h:441-451), would be
+    // written by some workgroups while others still read it: such a product goes into a fresh matrix whose payload dst
+    // then takes over.  A dst that is C, or shares C's payload, is used in place (each element of C is read by the
+    // workgroup that writes it, before it writes it).
+    const bool over_operand = dst == A || dst == B || dst->shares_block_with(*A) || dst->shares_block_with(*B);
+    const bool over_c = C && (dst == C || dst->shares_block_with(*C));
+    decx::_GPU_Matrix<T> fresh;
+    decx::_GPU_Matrix<T>* out = dst;
+    if (over_operand) {
+        if (!fresh.construct(B->width, A->height))
+            return fresh.last_status == DECX_HIP_FAIL_ALLOCATION ? alloc_fail() : from_status(fresh.last_status);
+        out = &fresh;
+    } else if (over_c) {
+        if (dst->width != B->width || dst->height != A->height || !dst->Mat.ptr) return de::DH{decx::DECX_FAIL_DimsNotMatching, kMDims};
+    } else if (!dst->re_construct(B->width, A->height)) {                                 // GEMM.h:414 (fp16 too: defect D7 not kept)
         return dst->last_status == DECX_HIP_FAIL_ALLOCATION ? alloc_fail() : from_status(dst->last_status);
-    return from_status(GemmCall<T>::run(A->Mat.ptr, (int)A->pitch, B->Mat.ptr, (int)B->pitch, C ? C->Mat.ptr : nullptr,
-                                        C ? (int)C->pitch : 0, dst->Mat.ptr, (int)dst->pitch, (int)A->height,
-                                        (int)B->width, (int)A->width));
+    }
+    const int rc = GemmCall<T>::run(A->Mat.ptr, (int)A->pitch, B->Mat.ptr, (int)B->pitch, C ? C->Mat.ptr : nullptr,
+                                    C ? (int)C->pitch : 0, out->Mat.ptr, (int)out->pitch, (int)A->height, (int)B->width,
+                                    (int)A->width);
+    if (rc == 0 && out != dst) dst->share_from(fresh);
+    return from_status(rc);
 }
 
 template <typename T> struct Gemm3Call;
@@ -145,11 +162,27 @@ de::DH gemm3_host(de::MatrixArray<T>& A_, de::MatrixArray<T>& B_, de::MatrixArra
     if (A->ArrayNumber != B->ArrayNumber || (C && C->ArrayNumber != A->ArrayNumber))
         return de::DH{decx::DECX_FAIL_MNumNotMatching, num_msg};
     if (C && (C->width != B->width || C->height != A->height)) return de::DH{decx::DECX_FAIL_DimsNotMatching, kMDims};
-    if (C != dst && !dst->re_construct(B->width, A->height, (uint)A->ArrayNumber, decx::Page_Locked)) return alloc_fail();
-    return from_status(Gemm3Call<T>::run(A->MatArr.ptr, (int)A->pitch, A->_plane, B->MatArr.ptr, (int)B->pitch, B->_plane,
-                                         C ? C->MatArr.ptr : nullptr, C ? (int)C->pitch : 0, C ? C->_plane : 0, dst->MatArr.ptr,
-                                         (int)dst->pitch, dst->_plane, (int)A->height, (int)B->width, (int)A->width,
-                                         (int)A->ArrayNumber));
+    // the pipeline downloads result i-1 while matrix i+1 is uploaded: a dst that is (or shares its payload with) A or B
+    // is computed into a fresh array that dst then takes over; one that shares C's is used in place (as gemm_host)
+    const bool over_operand = dst == A || dst == B || dst->shares_block_with(*A) || dst->shares_block_with(*B);
+    const bool over_c = C && (dst == C || dst->shares_block_with(*C));
+    decx::_MatrixArray<T> fresh;
+    decx::_MatrixArray<T>* out = dst;
+    if (over_operand) {
+        if (!fresh.construct(B->width, A->height, (uint)A->ArrayNumber, decx::Page_Locked)) return alloc_fail();
+        out = &fresh;
+    } else if (over_c) {
+        if (dst->width != B->width || dst->height != A->height || dst->ArrayNumber != A->ArrayNumber || !dst->MatArr.ptr)
+            return de::DH{decx::DECX_FAIL_DimsNotMatching, kMDims};
+    } else if (!dst->re_construct(B->width, A->height, (uint)A->ArrayNumber, decx::Page_Locked)) {
+        return alloc_fail();
+    }
+    const int rc = Gemm3Call<T>::run(A->MatArr.ptr, (int)A->pitch, A->_plane, B->MatArr.ptr, (int)B->pitch, B->_plane,
+                                     C ? C->MatArr.ptr : nullptr, C ? (int)C->pitch : 0, C ? C->_plane : 0, out->MatArr.ptr,
+                                     (int)out->pitch, out->_plane, (int)A->height, (int)B->width, (int)A->width,
+                                     (int)A->ArrayNumber);
+    if (rc == 0 && out != dst) dst->share_from(fresh);
+    return from_status(rc);
 }
 
 }  // namespace
@@ -364,11 +397,14 @@ DH conv_host(Tensor<T>& src_, TensorArray<T>& kernel_, Tensor<T>& dst_, const in
     if (rc) return from_status(rc);
     rc = decx_hip_memcpy(dK.ptr, ker->TensArr.ptr, ker->total_bytes, DECX_HIP_H2D);
     if (rc) return from_status(rc);
-    // sized (and zero-filled) only now that the operands are on the device: dst may be src or share its payload
+    // dst may be src (or share its payload): it is sized (and zero-filled) only now that the operands are on the device,
+    // and what the kernel needs of src's layout is taken down before that, since re_construct may rewrite those fields
+    const int src_dpitch = (int)src->dpitch;
+    const size_t src_row = src->dp_x_wp;
     if (!dst->re_construct((uint)Wout, (uint)Hout, ker->tensor_num, decx::Page_Locked)) return alloc_fail();   // :178
     rc = decx_hip_memset(dD.ptr, 0, dst->total_bytes);   // the width / channel padding of dst stays zero
     if (rc) return from_status(rc);
-    rc = ConvCall<T>::run(static_cast<const T*>(dS.ptr), H, W, (int)src->dpitch, src->dp_x_wp, static_cast<const T*>(dK.ptr),
+    rc = ConvCall<T>::run(static_cast<const T*>(dS.ptr), H, W, src_dpitch, src_row, static_cast<const T*>(dK.ptr),
                           (int)ker->tensor_num, kh, kw, ker->_gap, ker->dp_x_wp, static_cast<T*>(dD.ptr), (int)dst->dpitch,
                           dst->dp_x_wp, flag);
     if (rc) return from_status(rc);
@@ -385,11 +421,22 @@ DH conv_device(GPU_Tensor<T>& src_, GPU_TensorArray<T>& kernel_, GPU_Tensor<T>& 
     int Hout = 0, Wout = 0;
     DH pre = conv_precheck(src->depth, ker->depth, H, W, kh, kw, flag, Hout, Wout);
     if (pre.error_type != decx::DECX_SUCCESS) return pre;
-    if (!dst->re_construct((uint)Wout, (uint)Hout, ker->tensor_num))
+    // a dst that is src or shares its payload would be overwritten while neighbouring outputs still read it (or be
+    // freed by re_construct before the kernel runs): such a result goes into a fresh tensor that dst then takes over
+    decx::_GPU_Tensor<T> fresh;
+    decx::_GPU_Tensor<T>* out = dst;
+    if (dst == src || dst->shares_block_with(*src)) {
+        if (!fresh.construct((uint)Wout, (uint)Hout, ker->tensor_num))
+            return fresh.last_status == DECX_HIP_FAIL_ALLOCATION ? alloc_fail() : from_status(fresh.last_status);
+        out = &fresh;
+    } else if (!dst->re_construct((uint)Wout, (uint)Hout, ker->tensor_num)) {
         return dst->last_status == DECX_HIP_FAIL_ALLOCATION ? alloc_fail() : from_status(dst->last_status);
-    return from_status(ConvCall<T>::run(src->Tens.ptr, H, W, (int)src->dpitch, src->dp_x_wp, ker->TensArr.ptr,
-                                        (int)ker->tensor_num, kh, kw, ker->_gap, ker->dp_x_wp, dst->Tens.ptr,
-                                        (int)dst->dpitch, dst->dp_x_wp, flag));
+    }
+    const int rc = ConvCall<T>::run(src->Tens.ptr, H, W, (int)src->dpitch, src->dp_x_wp, ker->TensArr.ptr,
+                                    (int)ker->tensor_num, kh, kw, ker->_gap, ker->dp_x_wp, out->Tens.ptr, (int)out->dpitch,
+                                    out->dp_x_wp, flag);
+    if (rc == 0 && out != dst) dst->share_from(fresh);
+    return from_status(rc);
 }
 }  // namespace
 

@@ -199,13 +199,15 @@ public:
         block_.reset();
         Mat.ptr = nullptr;
     }
+    bool shares_block_with(const _GPU_Matrix<T>& o) const { return block_ && block_ == o.block_; }
+    void share_from(_GPU_Matrix<T>& s) {
+        if (&s == this) return;
+        block_ = s.block_;
+        attribute_assign(s.width, s.height);
+        Mat.ptr = s.Mat.ptr;
+    }
     de::GPU_Matrix<T>& operator=(de::GPU_Matrix<T>& src) override {   // shares src's block (GPU_Matrix.h:441-451)
-        _GPU_Matrix<T>& s = dynamic_cast<_GPU_Matrix<T>&>(src);
-        if (&s != this) {
-            block_ = s.block_;
-            attribute_assign(s.width, s.height);
-            Mat.ptr = s.Mat.ptr;
-        }
+        share_from(dynamic_cast<_GPU_Matrix<T>&>(src));
         return *this;
     }
     ~_GPU_Matrix() override { release(); }
@@ -373,13 +375,14 @@ public:
     uint MatrixNumber() override { return (uint)ArrayNumber; }
     bool shares_block_with(const _MatrixArray<T>& o) const { return block_ && block_ == o.block_; }
     T& index(uint row, uint col, size_t seq) override { return MatArr.ptr[seq * _plane + (size_t)row * pitch + col]; }
+    void share_from(_MatrixArray<T>& s) {
+        if (&s == this) return;
+        block_ = s.block_;
+        attribute_assign(s.width, s.height, (uint)s.ArrayNumber, s._store_type);
+        MatArr.ptr = s.MatArr.ptr;
+    }
     de::MatrixArray<T>& operator=(de::MatrixArray<T>& src) override {   // shares src's block (MatrixArray.h:473-498)
-        _MatrixArray<T>& s = dynamic_cast<_MatrixArray<T>&>(src);
-        if (&s != this) {
-            block_ = s.block_;
-            attribute_assign(s.width, s.height, (uint)s.ArrayNumber, s._store_type);
-            MatArr.ptr = s.MatArr.ptr;
-        }
+        share_from(dynamic_cast<_MatrixArray<T>&>(src));
         return *this;
     }
     void release() override {
@@ -429,13 +432,15 @@ public:
     uint Width() override { return width; }
     uint Height() override { return height; }
     uint Depth() override { return depth; }
+    bool shares_block_with(const _GPU_Tensor<T>& o) const { return block_ && block_ == o.block_; }
+    void share_from(_GPU_Tensor<T>& s) {
+        if (&s == this) return;
+        block_ = s.block_;
+        attribute_assign(s.width, s.height, s.depth);
+        Tens.ptr = s.Tens.ptr;
+    }
     de::GPU_Tensor<T>& operator=(de::GPU_Tensor<T>& src) override {   // shares src's block (GPU_Tensor.h)
-        _GPU_Tensor<T>& s = dynamic_cast<_GPU_Tensor<T>&>(src);
-        if (&s != this) {
-            block_ = s.block_;
-            attribute_assign(s.width, s.height, s.depth);
-            Tens.ptr = s.Tens.ptr;
-        }
+        share_from(dynamic_cast<_GPU_Tensor<T>&>(src));
         return *this;
     }
     void Load_from_host(de::Tensor<T>& src) override {

@@ -148,23 +148,36 @@ def bench_hgemm(capi, workloads, n, steps, warmup, seed, shape=None, verify_rows
     return out
 
 
+LADDER_BUILDS = [(0, "2 LDS stages of 64 k, one tile per workgroup"), (1, "4 LDS stages of 32 k"), (2, "5 LDS stages of 32 k"),
+                 (3, "2 LDS stages of 64 k, one workgroup per CU walks its tiles as one stream of K steps")]
+LADDER_RUNGS = [(7, "matrix instructions only"), (5, "+ LDS fragment reads"), (12, "+ global->LDS loads that never move on (cache hits)"),
+                (4, "+ global->LDS loads (whole K walk, no stores)"), (0, "whole kernel")]
+LADDER_ORDERS = [(16, "whole kernel, matrix instructions row block by row block, columns ascending"),
+                 (32, "whole kernel, matrix instructions column block by column block")]
+
+
 def bench_fp16_ladder(capi, workloads, steps, warmup, n=8192):
-    """The large fp16 tile kernel with parts of its K walk left out (decx_hip_hgemm_probe), on uniform[-1,1] operands
-    and on all-zero ones: what each part costs, and what the operand values cost (the same instructions on zeros draw
-    less power, so the chip clocks higher).  Every rung issues the same matrix instructions: 2 n^3 flop."""
+    """The large fp16 tile kernel in several builds with parts of its K walk left out (libdecx_hip_probe.so), on
+    uniform[-1,1] operands and on all-zero ones: what each part costs, and what the operand values cost (the same
+    instructions on zeros draw less power, so the chip clocks higher).  Every rung issues the same matrix
+    instructions: 2 n^3 flop."""
+    probe, stream = capi.probe_lib(), capi.stream()
     A = workloads.uniform_pm1((n, n), 5).astype(np.float16).view(np.uint16)
     B = workloads.uniform_pm1((n, n), 6).astype(np.float16).view(np.uint16)
     dA, dB = capi.DeviceBuffer.from_numpy(A), capi.DeviceBuffer.from_numpy(B)
     dZ = capi.DeviceBuffer(n * n * 2)
     dZ.fill(0)
     dD = capi.DeviceBuffer(n * n * 2)
-    rungs = [(7, "matrix instructions only"), (5, "+ LDS fragment reads"), (4, "+ global->LDS loads (whole K walk, no stores)"),
-             (0, "whole kernel")]
     out = []
-    for ablate, what in rungs:
-        row = {"ablate": ablate, "what": what}
+    cases = [(kind, kname, ab, what) for kind, kname in LADDER_BUILDS for ab, what in LADDER_RUNGS]
+    cases += [(0, LADDER_BUILDS[0][1], ab, what) for ab, what in LADDER_ORDERS]
+    for kind, kname, ablate, what in cases:
+        row = {"build": kind, "build_what": kname, "ablate": ablate, "what": what}
         for tag, a, b in (("uniform", dA, dB), ("zeros", dZ, dZ)):
-            launch = lambda: capi.check(capi.lib().decx_hip_hgemm_probe(ablate, a.ptr, n, b.ptr, n, dD.ptr, n, n, n, n))
+            def launch():
+                rc = probe.decx_probe_hgemm(kind, ablate, stream, a.ptr, n, b.ptr, n, dD.ptr, n, n, n, n, 8, 0)
+                if rc != 0:
+                    raise RuntimeError("decx_probe_hgemm(kind %d, ablate %d) returned %d" % (kind, ablate, rc))
             wall, ev = time_launches(capi, launch, steps, warmup)
             row["tflops_" + tag] = round(2.0 * n ** 3 / (ev * 1e-3) / 1e12, 1)
             row["ms_" + tag] = round(ev, 4)
@@ -325,6 +338,55 @@ def bench_conv_fused(capi, workloads, steps, warmup):
     return {"ms_wall": best, "tflops": flops / (best * 1e-3) / 1e12}
 
 
+def time_blocking_calls(call, steps, warmup):
+    """(min, median) wall milliseconds of whole synchronous calls, one after the other."""
+    ms = []
+    for i in range(warmup + steps):
+        t0 = time.perf_counter()
+        call()
+        if i >= warmup:
+            ms.append((time.perf_counter() - t0) * 1e3)
+    ms.sort()
+    return ms[0], ms[len(ms) // 2]
+
+
+def bench_blocking_calls(capi, workloads, steps, warmup):
+    """What a caller of the synchronous drop-in API (every call of the reference's API blocks) sees on kernels of tens of
+    microseconds: whole calls of decx_hip_sgemm at 1024^3 beside the same kernel enqueued back to back, and the floor
+    of a blocking call (a 64-float ReLU: launch + wait, next to nothing to compute)."""
+    n = 1024
+    A, B = workloads.uniform_pm1((n, n), 77), workloads.uniform_pm1((n, n), 78)
+    dA, dB, dD = capi.DeviceBuffer.from_numpy(A), capi.DeviceBuffer.from_numpy(B), capi.DeviceBuffer(n * n * 4)
+    steps = max(steps, 200)
+    best, med = time_blocking_calls(lambda: capi.sgemm(dA.ptr, n, dB.ptr, n, dD.ptr, n, n, n, n, blocking=True), steps, warmup)
+    _, ev = time_launches(capi, lambda: capi.sgemm(dA.ptr, n, dB.ptr, n, dD.ptr, n, n, n, n, blocking=False), steps, warmup)
+    tiny = capi.DeviceBuffer(256)
+    tiny.fill(0)
+    fbest, fmed = time_blocking_calls(lambda: capi.check(capi.lib().decx_hip_relu_f32(tiny.ptr, tiny.ptr, 64)), steps, warmup)
+    flops = 2.0 * n ** 3
+    return {"fp32_1024_blocking_call": {"ms_per_call_min": round(best, 4), "ms_per_call_median": round(med, 4),
+                                        "tflops": round(flops / (best * 1e-3) / 1e12, 2),
+                                        "ms_per_launch_enqueued": round(ev, 4)},
+            "blocking_call_floor_relu_64_floats": {"ms_per_call_min": round(fbest, 4), "ms_per_call_median": round(fmed, 4)}}
+
+
+def cpp_api_blocking_calls():
+    """The same two blocking calls made from C++ through the DECX-named API (tests/build/test_decx_api timing, built by
+    backup_1_amd/host/Makefile): what a DECX program sees, without the ctypes call overhead of this script."""
+    import re
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests", "build", "test_decx_api")
+    if not os.path.exists(exe):
+        return None
+    r = subprocess.run([exe, "timing"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    out = {}
+    for line in r.stdout.splitlines():
+        m = re.match(r"(.+?)\s+min\s+([0-9.]+) us\s+median\s+([0-9.]+) us", line)
+        if m:
+            out[m.group(1).strip()] = {"us_per_call_min": float(m.group(2)), "us_per_call_median": float(m.group(3))}
+    return out or None
+
+
 def cpu_baseline(workloads, A, B, rows):
     """The restated DECX_cpu thread-pool SGEMM (oracle/, kind "port") on the first `rows` rows of the headline A times
     the full B: B re-pack included, 12 tasks on a pool of min(hardware threads, 16) workers, as the reference sizes it."""
@@ -409,7 +471,7 @@ def main():
     if "ladder" in only:
         also["fp16_8192_ladder"] = bench_fp16_ladder(capi, workloads, side_steps, side_warmup)
         for row in also["fp16_8192_ladder"]:
-            log("fp16 ladder, %-48s %7.1f TFLOP/s on uniform[-1,1], %7.1f on zeros" % (row["what"], row["tflops_uniform"], row["tflops_zeros"]))
+            log("fp16 ladder, build %d, %-52s %7.1f TFLOP/s on uniform[-1,1], %7.1f on zeros" % (row["build"], row["what"], row["tflops_uniform"], row["tflops_zeros"]))
     if want("sq4096"):
         r = bench_sgemm(capi, workloads, 4096, 4096, 4096, side_steps, side_warmup, 1234)
         also["fp32_4096"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
@@ -476,6 +538,15 @@ def main():
         r = bench_conv_fused(capi, workloads, side_steps, side_warmup)
         also["fp32_conv_bias_relu_fused_blocking_call"] = {"tflops": round(r["tflops"], 2), "ms_per_call": round(r["ms_wall"], 4)}
         log("conv + bias + relu (one kernel, blocking call): %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+        also.update(bench_blocking_calls(capi, workloads, side_steps, side_warmup))
+        cpp = cpp_api_blocking_calls()
+        if cpp:
+            also["cpp_api_blocking_calls"] = cpp
+            for what, v in cpp.items():
+                log("C++ API, blocking %s: %.1f us per call (median %.1f)" % (what, v["us_per_call_min"], v["us_per_call_median"]))
+        log("fp32 1024^3 blocking call: %.4f ms (enqueued: %.4f ms per launch); floor of a blocking call: %.4f ms"
+            % (also["fp32_1024_blocking_call"]["ms_per_call_min"], also["fp32_1024_blocking_call"]["ms_per_launch_enqueued"],
+               also["blocking_call_floor_relu_64_floats"]["ms_per_call_min"]))
 
     if "copy" in only:
         # calibration launch for the traffic counters: 1 GiB read + 1 GiB written by a plain copy kernel
@@ -483,7 +554,9 @@ def main():
         src, dst = capi.DeviceBuffer(nbytes), capi.DeviceBuffer(nbytes)
         src.fill(1)
         for _ in range(3):
-            capi.check(capi.lib().decx_hip_copy_kernel(dst.ptr, src.ptr, nbytes))
+            rc = capi.probe_lib().decx_probe_copy(capi.stream(), dst.ptr, src.ptr, nbytes)
+            if rc != 0:
+                raise RuntimeError("decx_probe_copy returned %d" % rc)
         also["copy_1GiB"] = {"bytes_read": nbytes, "bytes_written": nbytes}
 
     if want("host"):

@@ -93,10 +93,10 @@ int decx_hip_sgemm_async(const float* A, int lda, const float* B, int ldb, const
  * in binary16 (GEMM_kernel_def.cuh:100-121), which this library deliberately does not reproduce.
  * Fast path needs A, B 16-byte aligned with lda, ldb multiples of 8 (DECX pitch is a multiple of 16 halves).
  * Results with very few 128x128 tiles and a long K (say 64 x 65536 x 1024) are computed by K ranges in parallel: each
- * range writes its fp32 partial sums into a plane of its own in a workspace the library allocates on first use (M*N
- * floats per range, kept for later calls; growing it synchronises the device -- so the _async entry points must not be
- * called from two host threads at once), the planes are added in range order and the sum is rounded to binary16
- * once.  Like every reference path the result is therefore the same on every run; decx_hip_set_splitk_mode selects
+ * range writes its fp32 partial sums into a plane of its own in a workspace of the library (M*N floats per range;
+ * decx_hip_init reserves 2 x CUs x 128 x 128 floats, 32 MiB on an MI355X, which covers every split the library chooses
+ * by itself; only a larger forced split grows it, which synchronises the device), the planes are added in range order
+ * and the sum is rounded to binary16 once.  Like every reference path the result is therefore the same on every run; decx_hip_set_splitk_mode selects
  * the older scheme in which all ranges add into one plane with atomics, in no fixed order. */
 int decx_hip_hgemm_f32acc(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                           int ldd, int M, int N, int K);
@@ -111,7 +111,8 @@ int decx_hip_hgemm_f32acc_async(const uint16_t* A, int lda, const uint16_t* B, i
 int decx_hip_set_splitk_mode(int mode);
 
 /* decx_hip_hgemm_f32acc for callers that cannot allocate device memory.  It has no counterpart in the reference: it is
- * for code under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  Same arguments, arithmetic
+ * for tight serving loops and harnesses that forbid hipMalloc (it launches on the library's own stream and waits for the
+ * result, so it is not for a stream under graph capture).  Same arguments, arithmetic
  * and result as decx_hip_hgemm_f32acc on its K-range route (`splits` ranges of K; <= 0: the count decx_hip_hgemm_f32acc
  * would choose, 1 if it would not split), but the fp32 planes of the ranges live in a fixed array inside the library's
  * code object, DECX_HIP_STATIC_WORKSPACE_BYTES per GPU, held until the process ends.  It calls no allocating routine.
@@ -240,19 +241,11 @@ int decx_hip_relu_f32_async(const float* src, float* dst, size_t n);
 int decx_hip_relu_f32_rec(const float* src, float* dst, unsigned char* rec_map, size_t n);
 int decx_hip_relu_f32_backward(const float* src, float* dst, const unsigned char* rec_map, size_t n);
 
-/* A plain device-to-device streaming copy kernel of `bytes` bytes (16-byte aligned, multiple of 16).  It has no
- * counterpart in the reference: it exists so that hardware traffic counters read for the kernels above can be scaled
- * by what the same counters read for a kernel whose traffic is known exactly.  Blocks until complete. */
-int decx_hip_copy_kernel(void* dst, const void* src, size_t bytes);
-
-/* A measurement instrument like the copy kernel above, with no counterpart in the reference: launches (without waiting)
- * the large fp16 GEMM tile kernel of decx_hip_hgemm_f32acc with parts of its K walk left out, so that the cost of each
- * part can be read off as the difference between two variants.  `ablate` is a sum of: 1 = no global -> LDS loads inside
- * the K walk, 2 = no LDS -> register reads inside it (the matrix instructions keep running on the first fragments),
- * 4 = the result is not stored; allowed values 0 (the whole kernel), 1, 3, 4, 5, 6, 7.  Every variant issues the same
- * matrix instructions; all but 0 leave D meaningless or untouched.  Arguments as decx_hip_hgemm_f32acc without C; A, B
- * 16-byte aligned with lda, ldb multiples of 8. */
-int decx_hip_hgemm_probe(int ablate, const uint16_t* A, int lda, const uint16_t* B, int ldb, uint16_t* D, int ldd, int M, int N, int K);
+/* The HIP stream (a hipStream_t) on which every _async entry point enqueues and on which the blocking ones wait: for
+ * callers that order work of their own behind the library's (the reference keeps its streams to itself; no
+ * counterpart).  NULL before decx_hip_init.  The stream has default priority and does not synchronise with the NULL
+ * stream. */
+void* decx_hip_stream(void);
 
 /* Timing on the library's own stream (the reference's demos time with clock(), CUDA_GEMM.cpp:43-46, :93-96).
  * start records an event, stop records another, waits for it and returns the elapsed milliseconds. */

@@ -2,6 +2,8 @@
 // (test/test/CUDA_GEMM/CUDA_GEMM.cpp, test/test/"generating classes"/*.h), but with assertions, and checks results
 // against the CPU oracle (liboracle.so).  Usage: test_decx_api cpu | cpu-small | gpu   (cpu-small: what the sanitizer
 // builds of backup_1_amd/host/Makefile run)
+#include <algorithm>
+#include <chrono>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -560,6 +562,133 @@ static void conv_flavours_and_flags() {
     CHECK(de::cuda::Conv2_MK_im2col(s, k2, d, 1).error_type == decx::DECX_FAIL_DimsNotMatching);
 }
 
+
+// A result container that is one of the operands, or shares its payload with one (operator= shares: Matrix.h:510-530
+// and its twins): every path must deliver the product of the operands as they were before the call.
+static void results_that_alias_operands() {
+    // device-resident GEMM: D = A (shared payload), square so that re_construct alone would be a no-op
+    {
+        const int S = 160;
+        de::Matrix<float>& A = de::CreateMatrixRef<float>(S, S, 0);
+        de::Matrix<float>& B = de::CreateMatrixRef<float>(S, S, 0);
+        de::Matrix<float>& R = de::CreateMatrixRef<float>(S, S, 0);
+        fill(A, unif); fill(B, unif);
+        const std::vector<float> want = chain(A, B);
+        de::GPU_Matrix<float>& dA = de::CreateGPUMatrixRef<float>(S, S);
+        de::GPU_Matrix<float>& dB = de::CreateGPUMatrixRef<float>(S, S);
+        de::GPU_Matrix<float>& dD = de::CreateGPUMatrixRef<float>();
+        dA.Load_from_host(A); dB.Load_from_host(B);
+        dD = dA;                                                       // shares A's device block
+        CHECK(de::cuda::GEMM(dA, dB, dD).error_type == decx::DECX_SUCCESS);
+        dD.Load_to_host(R);
+        CHECK(dense(R) == want);
+        dA.Load_to_host(R);
+        CHECK(dense(R) == dense(A));                                   // A itself is untouched
+        CHECK(de::cuda::GEMM(dA, dB, dA).error_type == decx::DECX_SUCCESS);      // dst IS A
+        dA.Load_to_host(R);
+        CHECK(dense(R) == want);
+        dA.Load_from_host(A);
+        CHECK(de::cuda::GEMM(dA, dB, dB).error_type == decx::DECX_SUCCESS);      // dst IS B
+        dB.Load_to_host(R);
+        CHECK(dense(R) == want);
+    }
+    // GEMM3 over arrays: dst shares A's payload, and dst is B
+    {
+        const int S = 96, NUM = 3;
+        de::MatrixArray<float>& A = de::CreateMatrixArrayRef<float>(S, S, NUM, 0);
+        de::MatrixArray<float>& B = de::CreateMatrixArrayRef<float>(S, S, NUM, 0);
+        de::MatrixArray<float>& D = de::CreateMatrixArrayRef<float>();
+        for (int s = 0; s < NUM; ++s)
+            for (int i = 0; i < S; ++i) for (int j = 0; j < S; ++j) { A.index(i, j, s) = small_int(); B.index(i, j, s) = small_int(); }
+        std::vector<std::vector<float>> want(NUM);
+        for (int s = 0; s < NUM; ++s) {
+            want[s].resize((size_t)S * S);
+            oracle_sgemm_chain_fast(&A.index(0, 0, s), S, &B.index(0, 0, s), S, nullptr, 0, want[s].data(), S, S, S, S, 0);
+        }
+        auto same_as_want = [&](de::MatrixArray<float>& R) {
+            bool same = R.Width() == (uint)S && R.Height() == (uint)S && R.MatrixNumber() == (uint)NUM;
+            for (int s = 0; s < NUM && same; ++s)
+                for (int i = 0; i < S; ++i) for (int j = 0; j < S; ++j) same = same && R.index(i, j, s) == want[s][(size_t)i * S + j];
+            return same;
+        };
+        D = A;
+        const float a00 = A.index(0, 0, 0);
+        CHECK(de::cuda::GEMM3(A, B, D).error_type == decx::DECX_SUCCESS);
+        CHECK(same_as_want(D));
+        CHECK(A.index(0, 0, 0) == a00 && &A.index(0, 0, 0) != &D.index(0, 0, 0));   // A kept its payload, D has a new one
+        CHECK(de::cuda::GEMM3(A, B, B).error_type == decx::DECX_SUCCESS);
+        CHECK(same_as_want(B));
+    }
+    // convolution on host tensors with dst == src: as many filters as channels (same shape), and a different count
+    for (int N : {8, 5, 12}) {
+        const int H = 14, W = 12, C = 8, kh = 3, kw = 3;
+        de::Tensor<float>& src = de::CreateTensorRef<float>(W, H, C, 0);
+        de::Tensor<float>& copy = de::CreateTensorRef<float>(W, H, C, 0);
+        de::TensorArray<float>& ker = de::CreateTensorArrayRef<float>(kw, kh, C, N, 0);
+        de::Tensor<float>& want = de::CreateTensorRef<float>();
+        for (int y = 0; y < H; ++y) for (int x = 0; x < W; ++x) for (int c = 0; c < C; ++c) copy.index(y, x, c) = src.index(y, x, c) = small_int();
+        for (int n = 0; n < N; ++n) for (int i = 0; i < kh; ++i) for (int j = 0; j < kw; ++j) for (int c = 0; c < C; ++c) ker.index(i, j, c, n) = small_int();
+        CHECK(de::cuda::Conv2_MK_im2col(copy, ker, want, 1).error_type == decx::DECX_SUCCESS);
+        CHECK(de::cuda::Conv2_MK_im2col(src, ker, src, 1).error_type == decx::DECX_SUCCESS);
+        bool same = src.Depth() == (uint)N && src.Width() == (uint)W && src.Height() == (uint)H;
+        for (int y = 0; y < H && same; ++y) for (int x = 0; x < W; ++x) for (int n = 0; n < N; ++n) same = same && src.index(y, x, n) == want.index(y, x, n);
+        CHECK(same);
+        // device-resident tensors: dst shares src's block
+        de::GPU_Tensor<float>& dsrc = de::CreateGPUTensorRef<float>(W, H, C);
+        de::GPU_TensorArray<float>& dker = de::CreateGPUTensorArrayRef<float>(kw, kh, C, N);
+        de::GPU_Tensor<float>& ddst = de::CreateGPUTensorRef<float>();
+        dsrc.Load_from_host(copy); dker.Load_from_host(ker);
+        ddst = dsrc;
+        CHECK(de::cuda::Conv2_MK_im2col(dsrc, dker, ddst, 1).error_type == decx::DECX_SUCCESS);
+        de::Tensor<float>& got = de::CreateTensorRef<float>(W, H, N, 0);
+        ddst.Load_to_host(got);
+        same = ddst.Depth() == (uint)N;
+        for (int y = 0; y < H && same; ++y) for (int x = 0; x < W; ++x) for (int n = 0; n < N; ++n) same = same && got.index(y, x, n) == want.index(y, x, n);
+        CHECK(same);
+        CHECK(de::cuda::Conv2_MK_im2col(dsrc, dker, dsrc, 1).error_type == decx::DECX_SUCCESS);   // dst IS src
+        de::Tensor<float>& got2 = de::CreateTensorRef<float>(W, H, N, 0);
+        dsrc.Load_to_host(got2);
+        same = dsrc.Depth() == (uint)N;
+        for (int y = 0; y < H && same; ++y) for (int x = 0; x < W; ++x) for (int n = 0; n < N; ++n) same = same && got2.index(y, x, n) == want.index(y, x, n);
+        CHECK(same);
+        src.release(); copy.release(); ker.release(); want.release(); got.release(); got2.release(); dsrc.release(); dker.release(); ddst.release();
+    }
+}
+
+// What a caller of the synchronous C++ API sees on kernels of tens of microseconds (mode "timing", not a test): whole
+// calls of de::cuda::Conv2_MK_im2col on device-resident tensors at 224x224x64 under 128 filters of 3x3x64, and of
+// de::cuda::GEMM on device-resident 1024^3 matrices.
+static void blocking_call_timing() {
+    auto report = [](const char* what, std::vector<double>& us) {
+        std::sort(us.begin(), us.end());
+        std::printf("%-56s min %8.2f us  median %8.2f us\n", what, us.front(), us[us.size() / 2]);
+    };
+    {
+        de::GPU_Tensor<float>& s = de::CreateGPUTensorRef<float>(224, 224, 64);
+        de::GPU_TensorArray<float>& k = de::CreateGPUTensorArrayRef<float>(3, 3, 64, 128);
+        de::GPU_Tensor<float>& d = de::CreateGPUTensorRef<float>(224, 224, 128);
+        std::vector<double> us;
+        for (int i = 0; i < 700; ++i) {
+            const auto t0 = std::chrono::steady_clock::now();
+            de::cuda::Conv2_MK_im2col(s, k, d, 1);
+            if (i >= 200) us.push_back(std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count());
+        }
+        report("Conv2_MK_im2col(GPU_Tensor) 224x224x64, 128 x 3x3x64", us);
+    }
+    {
+        de::GPU_Matrix<float>& A = de::CreateGPUMatrixRef<float>(1024, 1024);
+        de::GPU_Matrix<float>& B = de::CreateGPUMatrixRef<float>(1024, 1024);
+        de::GPU_Matrix<float>& D = de::CreateGPUMatrixRef<float>(1024, 1024);
+        std::vector<double> us;
+        for (int i = 0; i < 1500; ++i) {
+            const auto t0 = std::chrono::steady_clock::now();
+            de::cuda::GEMM(A, B, D);
+            if (i >= 500) us.push_back(std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count());
+        }
+        report("GEMM(GPU_Matrix<float>) 1024^3", us);
+    }
+}
+
 int main(int argc, char** argv) {
     std::string mode = argc > 1 ? argv[1] : "cpu";
     if (mode == "cpu" || mode == "cpu-small") {
@@ -571,6 +700,9 @@ int main(int argc, char** argv) {
         RUN(half_conversion);
         RUN(gemm_refuses_before_init);
         RUN(cpu_sgemm_matches_chain_bit_for_bit);
+    } else if (mode == "timing") {
+        de::InitCuda();
+        blocking_call_timing();
     } else {
         de::InitCuda();
         RUN(reference_demo_known_answer);
@@ -582,6 +714,7 @@ int main(int argc, char** argv) {
         RUN(gemm3_matrix_arrays);
         RUN(gemm_long_lr);
         RUN(nn_relu_family);
+        RUN(results_that_alias_operands);
     }
     std::printf("%s: %d failure(s)\n", mode.c_str(), g_fail);
     return g_fail ? 1 : 0;

@@ -27,7 +27,7 @@ SHAPES = [(1, 1, 1), (3, 5, 7), (31, 17, 33), (32, 32, 32), (128, 32, 128), (129
           (300, 70, 500), (257, 1500, 255), (64, 8, 1000), (1000, 3, 64), (513, 129, 259)]
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 15, 16])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 15, 16, 17])
 @pytest.mark.parametrize("shape", SHAPES)
 def test_integer_exact_all_tiles(gpu, shape, variant):
     M, K, N = shape
@@ -98,8 +98,37 @@ def test_split_k_is_the_same_on_every_run(gpu, oracle):
     finally:
         assert capi.lib().decx_hip_set_splitk_mode(prev) == 1
     assert np.max((np.abs(atomic - ref) - np.abs(ref) / 2048.0) / scale) < TOL
-    # a product that is not split must not care about the mode
-    assert np.array_equal(gpu_hgemm(A[:, :512], B[:512], variant=8), gpu_hgemm(A[:, :512], B[:512], variant=8))
+    # a product that is not split must not care about the mode: the same bits under either
+    unsplit = gpu_hgemm(A[:, :512], B[:512], variant=8)
+    prev = capi.lib().decx_hip_set_splitk_mode(1)
+    try:
+        assert np.array_equal(gpu_hgemm(A[:, :512], B[:512], variant=8), unsplit)
+    finally:
+        capi.lib().decx_hip_set_splitk_mode(prev)
+
+
+@pytest.mark.parametrize("shape", [(4352, 128, 4352), (4352, 384, 4608), (1024, 256, 69632 + 256)])
+def test_one_workgroup_per_cu_walking_its_tiles(gpu, oracle, shape):
+    # variant 17: more whole 256x256 tiles than compute units, one workgroup per CU walks several of them as one stream
+    # of K steps (the next tile's first loads are issued during the last steps of the tile before).  Every accumulator
+    # sees the same k-blocks in the same order as in the one-tile-per-workgroup build: the same bits, with and without C;
+    # integer data exact; real data within the fp16 rule against fp64.
+    M, K, N = shape
+    info = capi.device_info()
+    assert (M // 256) * (N // 256) > info["compute_units"]
+    Ai, Bi = workloads.small_ints((M, K), 51, -3, 3), workloads.small_ints((K, N), 52, -3, 3)
+    want = (Ai.astype(np.float64) @ Bi.astype(np.float64)).astype(np.float16).view(np.uint16)
+    assert np.array_equal(gpu_hgemm(to_bits(Ai), to_bits(Bi), variant=17), want)
+    del Ai, Bi, want
+    A, B = to_bits(workloads.uniform_pm1((M, K), 53)), to_bits(workloads.uniform_pm1((K, N), 54))
+    C = to_bits(workloads.uniform_pm1((M, N), 55))
+    one_tile = gpu_hgemm(A, B, variant=15)
+    walked = gpu_hgemm(A, B, variant=17)
+    assert np.array_equal(walked, one_tile)
+    assert np.array_equal(gpu_hgemm(A, B, C, variant=17), gpu_hgemm(A, B, C, variant=15))
+    rows = np.random.Generator(np.random.PCG64(56)).choice(M, size=24, replace=False).astype(np.int32)
+    ref, scale = oracle.gemm_f64_rows_f16(A, B, rows)
+    assert rel_err_vs_abs_scale(from_bits(walked[rows]), ref, scale) < TOL
 
 
 def test_rounding_to_half_is_nearest_even(gpu):

@@ -37,6 +37,30 @@ def bits(x):
     return x.astype(np.float16).view(np.uint16)
 
 
+def free_device_bytes():
+    """hipMemGetInfo, read straight from the HIP runtime the library is linked against."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
+def test_the_entry_point_allocates_no_device_memory(gpu):
+    # operands and result are the caller's; between their allocation and their release the free device memory must not
+    # move, whatever the number of K ranges, on the first call of the process on this entry point as on later ones
+    shapes = [(200, 16384, 520, 0), (40, 4096, 136, 0), (256, 8192, 512, 16), (64, 65536, 1024, 0)]
+    bufs = []
+    for M, K, N, _ in shapes:
+        A, B = bits(workloads.uniform_pm1((M, K), 7)), bits(workloads.uniform_pm1((K, N), 8))
+        bufs.append((capi.DeviceBuffer.from_numpy(A), capi.DeviceBuffer.from_numpy(B), capi.DeviceBuffer(M * N * 2)))
+    capi.sync()
+    before = free_device_bytes()
+    for (M, K, N, splits), (dA, dB, dD) in zip(shapes, bufs):
+        capi.check(capi.lib().decx_hip_hgemm_f32acc_noalloc(dA.ptr, K, dB.ptr, N, None, 0, dD.ptr, N, M, N, K, splits))
+        assert free_device_bytes() == before, (M, K, N, splits)
+
+
 def test_two_calls_in_a_row_match_the_allocating_entry_point(gpu, oracle):
     # first a product that takes many K ranges and most of a plane, then a smaller one with fewer ranges
     for (M, K, N), seed in (((200, 16384, 520), 70), ((40, 4096, 130), 80)):
