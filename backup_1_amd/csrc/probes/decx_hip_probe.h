@@ -19,7 +19,8 @@ extern "C" {
  *   kind  : 0 = 2 LDS stages of 64 k, one tile per workgroup (the product's build for ragged and batched products)
  *           1 = 4 stages of 32 k          2 = 5 stages of 32 k
  *           3 = kind 0 as one workgroup per compute unit that walks its tiles as one stream of K steps (the product's
- *               build for large products of whole tiles)          4 = kind 1 in that form
+ *               opt-in build for large products of whole tiles, variant 17)          4 = kind 1 in that form
+ *           5 = kind 0 on 4 waves of 128 x 128 (one per SIMD, a third fewer LDS fragment reads)          6 = kind 1 on those waves
  *   ablate: a sum of 1 = no global -> LDS loads inside the K walk, 2 = no LDS -> register reads inside it (the matrix
  *           instructions keep running on the first fragments), 4 = the result is not stored, 8 = the loads never move on
  *           (they fetch the tile's first K step over and over: loads that hit the caches), 16 / 32 = the matrix

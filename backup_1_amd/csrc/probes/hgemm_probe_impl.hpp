@@ -55,6 +55,8 @@ int launch(int ablate, hipStream_t stream, const uint16_t* A, int lda, const uin
 typedef Hgemm16Shape<256, 256, 64, 2, 4, 2> Shape2x64;
 typedef Hgemm16Shape<256, 256, 32, 2, 4, 4> Shape4x32;
 typedef Hgemm16Shape<256, 256, 32, 2, 4, 5> Shape5x32;
+typedef Hgemm16Shape<256, 256, 32, 2, 2, 4> ShapeFat4x32;
+typedef Hgemm16Shape<256, 256, 64, 2, 2, 2> ShapeFat;     // 4 waves of 128 x 128, one per SIMD
 
 int probe_kind0(int, hipStream_t, const uint16_t*, int, const uint16_t*, int, uint16_t*, int, int, int, int, int, int);
 int probe_kind0_orders(int, hipStream_t, const uint16_t*, int, const uint16_t*, int, uint16_t*, int, int, int, int, int, int);
@@ -62,6 +64,8 @@ int probe_kind1(int, hipStream_t, const uint16_t*, int, const uint16_t*, int, ui
 int probe_kind2(int, hipStream_t, const uint16_t*, int, const uint16_t*, int, uint16_t*, int, int, int, int, int, int);
 int probe_kind3(int, hipStream_t, const uint16_t*, int, const uint16_t*, int, uint16_t*, int, int, int, int, int, int);
 int probe_kind4(int, hipStream_t, const uint16_t*, int, const uint16_t*, int, uint16_t*, int, int, int, int, int, int);
+int probe_kind6(int, hipStream_t, const uint16_t*, int, const uint16_t*, int, uint16_t*, int, int, int, int, int, int);
+int probe_kind5(int, hipStream_t, const uint16_t*, int, const uint16_t*, int, uint16_t*, int, int, int, int, int, int);
 
 #define DECX_PROBE_DEFINE(NAME, SHAPE, PERSIST, ...)                                                                              \
     int NAME(int ablate, hipStream_t stream, const uint16_t* A, int lda, const uint16_t* B, int ldb, uint16_t* D, int ldd, int M, \

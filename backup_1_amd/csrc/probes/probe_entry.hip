@@ -24,6 +24,8 @@ int decx_probe_hgemm(int kind, int ablate, void* stream, const uint16_t* A, int 
         case 2: return probe_kind2(ablate, s, A, lda, B, ldb, D, ldd, M, N, K, group_m, grid);
         case 3: return probe_kind3(ablate, s, A, lda, B, ldb, D, ldd, M, N, K, group_m, grid);
         case 4: return probe_kind4(ablate, s, A, lda, B, ldb, D, ldd, M, N, K, group_m, grid);
+        case 6: return probe_kind6(ablate, s, A, lda, B, ldb, D, ldd, M, N, K, group_m, grid);
+        case 5: return probe_kind5(ablate, s, A, lda, B, ldb, D, ldd, M, N, K, group_m, grid);
         default: return 0x0d;
     }
 }

@@ -149,7 +149,9 @@ def bench_hgemm(capi, workloads, n, steps, warmup, seed, shape=None, verify_rows
 
 
 LADDER_BUILDS = [(0, "2 LDS stages of 64 k, one tile per workgroup"), (1, "4 LDS stages of 32 k"), (2, "5 LDS stages of 32 k"),
-                 (3, "2 LDS stages of 64 k, one workgroup per CU walks its tiles as one stream of K steps")]
+                 (3, "2 LDS stages of 64 k, one workgroup per CU walks its tiles as one stream of K steps"),
+                 (5, "2 LDS stages of 64 k, 4 waves of 128 x 128 (one per SIMD) instead of 8 of 128 x 64"),
+                 (6, "4 LDS stages of 32 k, 4 waves of 128 x 128")]
 LADDER_RUNGS = [(7, "matrix instructions only"), (5, "+ LDS fragment reads"), (12, "+ global->LDS loads that never move on (cache hits)"),
                 (4, "+ global->LDS loads (whole K walk, no stores)"), (0, "whole kernel")]
 LADDER_ORDERS = [(16, "whole kernel, matrix instructions row block by row block, columns ascending"),
