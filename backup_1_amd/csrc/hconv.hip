@@ -1,9 +1,11 @@
-// fp16 fused im2col convolution with fp32 accumulation: kernel choice and launch (hconv_tile.hpp, hconv_dma.hpp,
-// hconv_taprow.hpp), split over K for small images.
+// fp16 fused im2col convolution with fp32 accumulation: kernel choice and launch (hconv_mfma16.hpp for images that give
+// at least a quarter of the CUs a tile and have a channel pitch in 64s, else hconv_taprow.hpp, hconv_dma.hpp,
+// hconv_tile.hpp), split over K for small images.
 #include "runtime.hpp"
 #include "hconv_tile.hpp"
 #include "hconv_dma.hpp"
 #include "hconv_taprow.hpp"
+#include "hconv_mfma16.hpp"
 
 namespace decx_hip {
 
@@ -11,6 +13,10 @@ namespace decx_hip {
 typedef HconvShape<128, 128, 2, 2, 4> HconvSquare;   // 2x2 waves of 64x64
 typedef HconvShape<256, 128, 4, 2, 4> HconvTall;     // 4x2 waves of 64x64, two per SIMD: half the filter reads per pixel
 typedef HconvDmaShape<256, 128, 4, 2, 3> HconvDma;   // the tall tile fed by LDS-DMA loads, three K steps in LDS
+// at most 64 filters: the 128-wide tiles of the 16x16x32 kernel would spend half of their matrix instructions on
+// filters that do not exist
+static bool narrow16(int N) { return N <= 64; }
+
 int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_stride, const uint16_t* filt, int N, int kh,
                   int kw, size_t filt_stride, size_t filt_row_stride, uint16_t* dst, int dst_dpitch, size_t dst_row_stride,
                   int flag, const uint16_t* bias, bool relu) {
@@ -66,7 +72,7 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
     const int all_steps = cdiv(Kw, 32);
     const long square_tiles = (long)cdiv(M, 128) * tiles_n;
     int splits = 1;
-    const bool kernel_forced = g_rt.hgemm_variant >= 12 && g_rt.hgemm_variant <= 14;      // experiments and tests: no split
+    const bool kernel_forced = (g_rt.hgemm_variant >= 12 && g_rt.hgemm_variant <= 14) || g_rt.hgemm_variant == 18;      // experiments and tests: no split
     if (!kernel_forced && !tall && 2 * square_tiles <= cus && all_steps >= 8 && (size_t)M * N <= ((size_t)1 << 26)) {
         const double t_whole = 4.0 + 0.75 * all_steps;
         double best = 0.85 * t_whole;
@@ -105,6 +111,37 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
                            out, M, N);
         HIP_TRY(hipGetLastError());
         return 0;
+    }
+    // a K step of 64 halves inside one tap: the kernel on v_mfma_f32_16x16x32_f16 with patch-shaped tiles (hconv_mfma16.hpp),
+    // 256 filters wide where there are more than 128.  Its column test adds 2^31 to an offset, which must throw it out of
+    // the tensor's range even from the apron's negative offsets, and its patches reach up to 15 rows and 15 columns past
+    // the output: those offsets must stay below 2^31 as well.  hgemm variant 18 takes it for any image it can run on; by
+    // itself it takes the images whose patches give at least a quarter of the CUs a tile.
+    {
+        const size_t apron_bytes = ((size_t)oy * src_row_stride + (size_t)ox * dpitch + 8) * 2;
+        const bool fits = tap_uniform && src_bytes + apron_bytes + ((size_t)(16 + kh) * src_row_stride + (size_t)(16 + kw) * dpitch) * 2 < 0x80000000ull;
+        const bool wide = N > 128;
+        const long patches = (long)cdiv(Hout, 16) * cdiv(Wout, 16);
+        const long tiles16 = patches * cdiv(N, wide ? 256 : 128);
+        const bool by_itself = !kernel_forced && !narrow16(N) && tiles16 >= cus / 4 && g_rt.hgemm_variant != 19;
+        if (fits && tiles16 <= 0x7fffffffL && (g_rt.hgemm_variant == 18 || by_itself)) {
+            auto launch16 = [&](auto shape) -> int {
+                typedef decltype(shape) S;
+                static bool attr_done = false;           // one per shape: the lambda's body is instantiated per S
+                if (!attr_done) {
+                    HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(hconv_mfma16_kernel<S>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                (int)S::LDS_BYTES));
+                    attr_done = true;
+                }
+                const int tn = cdiv(N, S::BN), tx = cdiv(Wout, S::PATCH_X);
+                hipLaunchKernelGGL(hconv_mfma16_kernel<S>, dim3((unsigned)(patches * tn)), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, out,
+                                   Hout, N, tx, (int)patches, tn);
+                HIP_TRY(hipGetLastError());
+                return 0;
+            };
+            if (wide) return launch16(Hconv16Shape<256, 2, 4>{});      // 2x4 waves of 128 pixels x 64 filters
+            return launch16(Hconv16Shape<128, 4, 2>{});                // 4x2 waves of 64 pixels x 64 filters
+        }
     }
     // filters 3, 5 or 7 wide: the LDS-DMA kernel that loads a tap row's pixels once for all of its taps, if a tile's patch
     // fits its 320 rows (255 + kw positions plus kw - 1 per image row the tile touches).  hgemm variant 14 takes it for

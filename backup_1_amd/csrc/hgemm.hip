@@ -33,7 +33,9 @@ namespace decx_hip {
 //      first tile, the epilogue under the next tile's loads); products of whole tiles only, others fall back to 15
 //  11: split-K on shape 8 through an fp32 workspace (hgemm_splitk_enqueue) -- few tiles and a long K
 // and, for the fp16 convolution only: 12 keeps its register-staged kernels, 13 takes its LDS-DMA kernel for any image
-// whose channel pitch allows it, 14 its tap-row kernel; each switches its split over K off (experiments and tests)
+// whose channel pitch allows it, 14 its tap-row kernel, 18 its kernel on 16x16x32 matrix instructions with patch-shaped
+// tiles (hconv_mfma16.hpp); each switches its split over K off.  19 keeps kernel 18 out of the automatic choice.
+// (experiments and tests)
 typedef HgemmShape<256, 256, 32, 2, 2> HShapeBig;
 typedef HgemmShape<128, 128, 32, 2, 2> HShapeSmall;
 typedef HgemmDmaShape<256, 256, 32, 2, 2, 4> HShapeDma;

@@ -101,7 +101,7 @@ def test_headline_shape_sampled(gpu, oracle):
     assert check_against_f64(oracle, got, sbuf, fb, 1) < TOL
     # the library's choice is the tap-row kernel; the LDS-DMA and the register-staged kernels must agree with it to the
     # rounding of the result (they add the same fp32 products in another order)
-    for variant in (12, 13, 14):
+    for variant in (12, 13, 14, 18, 19):
         other, _, _ = gpu_hconv(src, filt, 1, variant=variant)
         diff = np.abs(other.astype(np.float64) - got.astype(np.float64))
         assert np.all(diff <= 2.0 ** -9 * np.maximum(np.abs(got.astype(np.float64)), 1.0)), variant
@@ -166,9 +166,10 @@ DMA_CASES = [(20, 22, 64, 6, 3, 3), (16, 16, 64, 128, 3, 3), (33, 17, 128, 130, 
              (300, 20, 128, 140, 3, 5)]
 
 
-@pytest.mark.parametrize("variant", [14, 13, 12])
+# 18 takes the kernel on 16x16x32 matrix instructions with patch-shaped tiles (256 filters wide above 128 filters), 19 keeps it out
+@pytest.mark.parametrize("variant", [18, 14, 13, 12, 19])
 @pytest.mark.parametrize("flag", [1, 0])
-@pytest.mark.parametrize("case", DMA_CASES)
+@pytest.mark.parametrize("case", DMA_CASES + [(50, 35, 64, 300, 3, 3), (17, 90, 128, 257, 1, 3)])
 def test_dma_kernel_and_register_kernel_on_the_same_cases(gpu, oracle, case, flag, variant):
     H, W, C, N, kh, kw = case
     if flag == 0 and (H <= 2 * (kh // 2) or W <= 2 * (kw // 2)):

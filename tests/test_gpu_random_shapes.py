@@ -50,7 +50,7 @@ def test_random_convolutions_bit_exact(gpu, oracle, seed):
 
 @pytest.mark.parametrize("seed", range(8))
 def test_random_fp16_convolutions_exact_on_small_integers(gpu, oracle, seed):
-    # every fp16 convolution kernel (12: register-staged, 13: LDS-DMA, 14: tap rows in LDS, 0: the library's choice,
+    # every fp16 convolution kernel (12: register-staged, 13: LDS-DMA, 14: tap rows in LDS, 18: 16x16x32 blocks on patches, 0: the library's choice,
     # which includes the split over K) on random shapes; channel counts that make the channel pitch a multiple of 64 halves
     # half of the time, since only those reach kernels 13 and 14.  Values in {-1, 0, 1}: sums stay exact in binary16.
     rng = np.random.Generator(np.random.PCG64(9000 + seed))
@@ -59,7 +59,7 @@ def test_random_fp16_convolutions_exact_on_small_integers(gpu, oracle, seed):
         H, W = int(rng.integers(kh, 70)), int(rng.integers(kw, 70))
         C = int(rng.choice([64, 128, 57])) if rng.integers(0, 2) else int(rng.integers(1, 70))
         N = int(rng.integers(1, 200))
-        flag, variant = int(rng.integers(0, 2)), int(rng.choice([0, 12, 13, 14]))
+        flag, variant = int(rng.integers(0, 2)), int(rng.choice([0, 12, 13, 14, 18]))
         if flag == 0 and (H <= 2 * (kh // 2) or W <= 2 * (kw // 2)):
             flag = 1
         src = workloads.small_ints((H, W, C), 500 * seed + case, -1, 1).astype(np.float16)
