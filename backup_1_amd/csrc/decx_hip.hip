@@ -661,6 +661,23 @@ int decx_hip_set_splitk_mode(int mode) {
     return prev;
 }
 
+int decx_hip_sgemm_plan(int M, int N, int K, int batch, long lda, long ldb, int aligned) {
+    if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || lda < K || ldb < N) return -1;
+    return sgemm_plan(M, N, K, batch, lda, ldb, aligned != 0);
+}
+
+int decx_hip_hgemm_plan(int M, int N, int K, int batch, long lda, long ldb, int aligned, int* splits) {
+    if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || lda < K || ldb < N) return -1;
+    return hgemm_plan(M, N, K, batch, lda, ldb, aligned != 0, splits);
+}
+
+int decx_hip_conv_patch_offsets_fit(int H, int W, int dpitch, size_t src_row_stride, int kh, int kw, int flag, int elem_bytes) {
+    if (H <= 0 || W <= 0 || dpitch <= 0 || kh <= 0 || kw <= 0 || (elem_bytes != 2 && elem_bytes != 4) || src_row_stride < (size_t)W * dpitch) return -1;
+    const size_t src_bytes = ((size_t)(H - 1) * src_row_stride + (size_t)W * dpitch) * elem_bytes;
+    if (src_bytes >= 0x80000000ull) return 0;
+    return conv_patch_offsets_fit(src_bytes, src_row_stride, (size_t)dpitch, kh, kw, flag ? kh / 2 : 0, flag ? kw / 2 : 0, (size_t)elem_bytes) ? 1 : 0;
+}
+
 int decx_hip_b_read_extent(int N, int tile_n, int unit) {
     if (N <= 0 || tile_n <= 0 || unit <= 0 || tile_n % unit) return -1;
     int last = -1;

@@ -118,8 +118,7 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
     // the output: those offsets must stay below 2^31 as well.  hgemm variant 18 takes it for any image it can run on; by
     // itself it takes the images whose patches give at least a quarter of the CUs a tile.
     {
-        const size_t apron_bytes = ((size_t)oy * src_row_stride + (size_t)ox * dpitch + 8) * 2;
-        const bool fits = tap_uniform && src_bytes + apron_bytes + ((size_t)(16 + kh) * src_row_stride + (size_t)(16 + kw) * dpitch) * 2 < 0x80000000ull;
+        const bool fits = tap_uniform && conv_patch_offsets_fit(src_bytes, src_row_stride, (size_t)dpitch, kh, kw, oy, ox, 2);
         const bool wide = N > 128;
         const long patches = (long)cdiv(Hout, 16) * cdiv(Wout, 16);
         const long tiles16 = patches * cdiv(N, wide ? 256 : 128);

@@ -227,43 +227,62 @@ int hgemm_splitk_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb,
     return hgemm_splitk_launch(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, plan, g_rt.partial, ordered, stream);
 }
 
+// the LDS-DMA tiles address a tile's rows with 32-bit byte offsets from the tile's first row: 256 rows of A, 64 of B
+static bool hgemm_pitches_fit(long lda, long ldb) {
+    return lda % 8 == 0 && ldb % 8 == 0 && ldb >= 8 && (size_t)lda * 256 * sizeof(uint16_t) < ((size_t)1 << 32) &&
+           (size_t)ldb * 64 * sizeof(uint16_t) < ((size_t)1 << 32);
+}
 static bool hgemm_vector_path(const uint16_t* A, int lda, const uint16_t* B, int ldb, const Batch& batch) {
-    // the LDS-DMA tiles address a tile's rows with 32-bit byte offsets from the tile's first row: 256 rows of A, 64 of B
-    const bool narrow = (size_t)lda * 256 * sizeof(uint16_t) < ((size_t)1 << 32) && (size_t)ldb * 64 * sizeof(uint16_t) < ((size_t)1 << 32);
-    return aligned16(A) && aligned16(B) && lda % 8 == 0 && ldb % 8 == 0 && ldb >= 8 && batch.stride_a % 8 == 0 &&
-           batch.stride_b % 8 == 0 && narrow;
+    return aligned16(A) && aligned16(B) && batch.stride_a % 8 == 0 && batch.stride_b % 8 == 0 && hgemm_pitches_fit(lda, ldb);
 }
 
-int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
-                  int ldd, int M, int N, int K, const Batch& batch) {
-    if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
-    const bool vec = hgemm_vector_path(A, lda, B, ldb, batch);
-    if (!vec) return launch_hgemm_tile<HShapeSmall, false>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+// The kernel decx_hip_hgemm_f32acc takes for a product, as the number decx_hip_set_hgemm_variant would force it with
+// (the table at the top of this file); 0 = operands the vector loaders cannot take (the 128x128 tile with element-wise
+// loaders); 11 = split over K, *splits ranges.
+static int plan_hgemm(int M, int N, int K, int batch_count, bool vec, int* splits_out) {
+    if (splits_out) *splits_out = 0;
+    if (!vec) return 0;
     int variant = g_rt.hgemm_variant;
-    {
-        // few 128x128 tiles and a long K: split K (variant 11 forces it, any other fixed variant switches it off)
-        if (batch.count == 1 && (variant < 1 || variant > 10) && (variant < 15 || variant > 17)) {
-            int splits = auto_hgemm_splits(M, N, K);
-            if (variant == 11 && splits == 0 && K >= 1024 && (size_t)M * N <= ((size_t)1 << 26)) {
-                const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
-                const long tiles = (long)cdiv(M, 128) * cdiv(N, 128);
-                long s = (2 * cus + tiles - 1) / tiles;
-                if (s > K / 512) s = K / 512;
-                splits = s >= 2 ? (int)s : 0;
-            }
-            if (splits >= 2) return hgemm_splitk_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, splits, batch.stream);
+    // few 128x128 tiles and a long K: split K (variant 11 forces it, any other fixed variant switches it off)
+    if (batch_count == 1 && (variant < 1 || variant > 10) && (variant < 15 || variant > 17)) {
+        int splits = auto_hgemm_splits(M, N, K);
+        if (variant == 11 && splits == 0 && K >= 1024 && (size_t)M * N <= ((size_t)1 << 26)) {
+            const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+            const long tiles = (long)cdiv(M, 128) * cdiv(N, 128);
+            long s = (2 * cus + tiles - 1) / tiles;
+            if (s > K / 512) s = K / 512;
+            splits = s >= 2 ? (int)s : 0;
         }
-        if (variant == 11) variant = 0;
+        if (splits >= 2) {
+            if (splits_out) *splits_out = splits;
+            return 11;
+        }
     }
+    if (variant == 11) variant = 0;
     if (variant < 1 || (variant > 10 && (variant < 15 || variant > 17))) {
         // same cost model as the fp32 picker: rounds of tiles per CU x tile area / measured shape efficiency
         const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
-        const long big = (long)cdiv(M, 256) * cdiv(N, 256) * batch.count, small = (long)cdiv(M, 128) * cdiv(N, 128) * batch.count;
+        const long big = (long)cdiv(M, 256) * cdiv(N, 256) * batch_count, small = (long)cdiv(M, 128) * cdiv(N, 128) * batch_count;
         const double cost_big = (double)((big + cus - 1) / cus) * 65536.0;
         const double cost_small = (double)((small + cus - 1) / cus) * 16384.0 / 0.75;
         // the small tile with three LDS stages holds one workgroup per CU: only worth it when there is at most one to hold
         variant = cost_big <= cost_small ? 15 : (small <= cus ? 9 : 8);
     }
+    return variant;
+}
+
+// host-only: the choice above for a product described by its sizes and pitches (decx_hip_hgemm_plan)
+int hgemm_plan(int M, int N, int K, int batch, long lda, long ldb, bool aligned, int* splits) {
+    return plan_hgemm(M, N, K, batch, aligned && hgemm_pitches_fit(lda, ldb), splits);
+}
+
+int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
+                  int ldd, int M, int N, int K, const Batch& batch) {
+    if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
+    int splits = 0;
+    int variant = plan_hgemm(M, N, K, batch.count, hgemm_vector_path(A, lda, B, ldb, batch), &splits);
+    if (variant == 0) return launch_hgemm_tile<HShapeSmall, false>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
+    if (variant == 11) return hgemm_splitk_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, splits, batch.stream);
     if (variant == 17) {
         if (hgemm_mfma16_persistent_fits<HShape16>(M, N, K, batch))
             return launch_hgemm_mfma16_persistent<HShape16>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);

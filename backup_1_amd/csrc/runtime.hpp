@@ -48,6 +48,18 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 inline int cdiv(int a, int b) { return (a + b - 1) / b; }
 
+// The convolution kernels on patch-shaped tiles (sconv_dma.hpp, hconv_mfma16.hpp) address the image with 32-bit byte
+// offsets through a buffer resource and throw a load out of the tensor's range by adding 2^31 to its offset.  That works
+// while every offset they form stays below 2^31 before the addition and wraps past 2^32 - (apron) after it: the tensor's
+// bytes, plus the apron's negative offsets (oy rows and ox pixels before the first, and a 16-byte unit), plus the
+// patches' reach past the output (up to 16 rows and 16 columns) and the taps' (kh rows, kw pixels) must stay below 2^31.
+// Strides and pitches in elements of elem_bytes.
+inline bool conv_patch_offsets_fit(size_t src_bytes, size_t row_stride, size_t dpitch, int kh, int kw, int oy, int ox, size_t elem_bytes) {
+    const size_t apron_bytes = ((size_t)oy * row_stride + (size_t)ox * dpitch) * elem_bytes + 16;
+    const size_t reach_bytes = ((size_t)(16 + kh) * row_stride + (size_t)(16 + kw) * dpitch) * elem_bytes;
+    return src_bytes + apron_bytes + reach_bytes < 0x80000000ull;
+}
+
 // A batch of `count` independent, equally shaped problems; the strides are in elements between consecutive problems.
 // Every launcher enqueues on `stream`.
 struct Batch {
@@ -76,6 +88,9 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
                  int flag, const float* bias = nullptr, bool relu = false);
 int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc, uint16_t* D,
                   int ldd, int M, int N, int K, const Batch& batch);
+// host-only: which kernel the two entry points above take for a product of these sizes and pitches (no device call)
+int sgemm_plan(int M, int N, int K, int batch, long lda, long ldb, bool aligned);
+int hgemm_plan(int M, int N, int K, int batch, long lda, long ldb, bool aligned, int* splits);
 // the K-range route of hgemm_enqueue on the library's static device workspace (no allocation); splits <= 0: automatic
 int hgemm_splitk_static_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
                                 uint16_t* D, int ldd, int M, int N, int K, int splits);

@@ -88,9 +88,8 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
     // and its patches reach up to 15 rows and 12 columns past the output: those offsets must stay below 2^31 as well.
     // Forced by shapes 29 and 30; by itself it takes a result that its patches of 16 x 13 pixels x 128 filters cover in
     // one round that fills at least three quarters of the CUs
-    const size_t apron_bytes = ((size_t)oy * src_row_stride + (size_t)ox * dpitch + 4) * sizeof(float);
     if (dpitch % 32 == 0 && N % 4 == 0 && aligned16(dst) && dst_dpitch % 4 == 0 && dst_row_stride % 4 == 0 &&
-        src_bytes + apron_bytes + ((size_t)(16 + kh) * src_row_stride + (size_t)(16 + kw) * dpitch) * sizeof(float) < 0x80000000ull) {
+        conv_patch_offsets_fit(src_bytes, src_row_stride, (size_t)dpitch, kh, kw, oy, ox, sizeof(float))) {
         const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
         const long patches = (long)cdiv(Hout, 16) * cdiv(Wout, 13) * cdiv(N, 128);
         int shape = g_rt.sgemm_variant >= 29 && g_rt.sgemm_variant <= 30 ? g_rt.sgemm_variant : 0;

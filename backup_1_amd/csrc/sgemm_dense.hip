@@ -60,31 +60,29 @@ int launch_sgemm_chain16(const float* A, int lda, const float* B, int ldb, const
 int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float* Cin, int ldc, float* D, int ldd, int M,
                   int N, int K, const Batch& batch, bool relu) {
     if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
-    const int variant = pick_sgemm_variant(M, N, K, batch.count, true);
     const bool vec_a = aligned16(A) && lda % 4 == 0 && batch.stride_a % 4 == 0;
     const bool vec_b = aligned16(B) && ldb % 4 == 0 && ldb >= 4 && batch.stride_b % 4 == 0;
     DenseOut out{ldd, relu, aligned16(D) && ldd % 4 == 0 && batch.stride_d % 4 == 0};
-    if (vec_a && vec_b && lda < kDmaMaxPitch && ldb < kDmaMaxPitch) {
-        const int dma = pick_dma_shape(M, N, K, batch.count);
-        if (dma) return launch_sgemm_dma_shape(dma, A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+    const int plan = plan_sgemm(M, N, K, batch.count, vec_a, vec_b, lda, ldb);
+    if (plan == 0) {     // unaligned operands: element-wise loaders, one tile shape only
+        DenseA<false> a{A, lda, M, K, batch.stride_a};
+        DenseB<false> b{B, ldb, N, K, batch.stride_b};
+        return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K, batch);
     }
-    if (vec_a && vec_b) {
-        const int chain = pick_chain_shape(M, N, K, batch.count);
-        if (chain == 11) return launch_sgemm_chain16<Chain16<2, 1, 4, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
-        if (chain == 12) return launch_sgemm_chain16<Chain16<1, 1, 8, 2>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
-        if (chain == 13) return launch_sgemm_chain16<Chain16<4, 2, 2, 3>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
-        if (chain == 23) return launch_sgemm_chain16<Chain16Rect<1, 2, 1, 6, 2>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
-    }
-    if (vec_a && vec_b) {
-        DenseA<true> a{A, lda, M, K, batch.stride_a};
-        DenseB<true> b{B, ldb, N, K, batch.stride_b};
-        if (variant == 14) return launch_sgemm_tile<SShape192>(a, b, Cin, ldc, D, out, M, N, K, batch);
-        return dispatch_sgemm(variant, a, b, Cin, ldc, D, out, M, N, K, batch);
-    }
-    // unaligned operands: element-wise loaders, one tile shape only
-    DenseA<false> a{A, lda, M, K, batch.stride_a};
-    DenseB<false> b{B, ldb, N, K, batch.stride_b};
-    return launch_sgemm_tile<SShapeSmall>(a, b, Cin, ldc, D, out, M, N, K, batch);
+    if ((plan >= 18 && plan <= 22) || (plan >= 24 && plan <= 28)) return launch_sgemm_dma_shape(plan, A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+    if (plan == 11) return launch_sgemm_chain16<Chain16<2, 1, 4, 4>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+    if (plan == 12) return launch_sgemm_chain16<Chain16<1, 1, 8, 2>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+    if (plan == 13) return launch_sgemm_chain16<Chain16<4, 2, 2, 3>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+    if (plan == 23) return launch_sgemm_chain16<Chain16Rect<1, 2, 1, 6, 2>>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch, relu);
+    DenseA<true> a{A, lda, M, K, batch.stride_a};
+    DenseB<true> b{B, ldb, N, K, batch.stride_b};
+    if (plan == 14) return launch_sgemm_tile<SShape192>(a, b, Cin, ldc, D, out, M, N, K, batch);
+    return dispatch_sgemm(plan, a, b, Cin, ldc, D, out, M, N, K, batch);
+}
+
+// host-only: the choice above for a product described by its sizes and pitches (decx_hip_sgemm_plan)
+int sgemm_plan(int M, int N, int K, int batch, long lda, long ldb, bool aligned) {
+    return plan_sgemm(M, N, K, batch, aligned && lda % 4 == 0, aligned && ldb % 4 == 0 && ldb >= 4, lda, ldb);
 }
 
 // Split-K GEMM for problems whose M x N tile count leaves most CUs idle while K is long (the short-M / long-K shapes of

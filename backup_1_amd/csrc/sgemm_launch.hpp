@@ -197,12 +197,12 @@ inline int pick_dma_shape(int M, int N, int K, int batch) {
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch, tiles128 = (long)cdiv(M, 128) * cdiv(N, 128) * batch;
     const long tiles32 = (long)cdiv(M, 32) * cdiv(N, 32) * batch;
-    // 128x128 tiles on eight waves (4 x 2 of 32x64, two per SIMD) in one or two rounds whose last is at least 88 % full:
+    // 128x128 tiles on eight waves (4 x 2 of 32x64, two per SIMD) in one or two rounds whose last is at least 7/8 full:
     // 2048^3 128.5 -> 118.2 us (145 TFLOP/s), 2048x8192x2048 501 -> 456 us (151 TFLOP/s), 1920^2 x 4096 245 -> 231 us,
     // 2816^2 x 4096 482 -> 459 us
     {
         const long last = tiles128 % cus == 0 ? cus : tiles128 % cus;
-        if (tiles128 <= 2 * cus && 100 * last >= 88 * cus) return 20;
+        if (tiles128 <= 2 * cus && 8 * last >= 7 * cus) return 20;     // (1920^2: 225 tiles of 256)
     }
     // Cycles per k of a launch, measured over squares of 384 .. 1792 at K = 1024 and 8192: a round of 64x64 tiles (one
     // per CU) walks K at 34.2, a round of 32x32 tiles of 16x16 blocks at 9.7.  The small tiles win where the 64x64 ones
@@ -233,6 +233,21 @@ inline int pick_dma_shape(int M, int N, int K, int batch) {
     // CU walks a very long K with less trouble from pitches of a power of two -- the 32x32 tiles take the rest
     if (2 * tiles64 < cus && (long)cdiv(M, 16) * cdiv(N, 32) * batch > cus) return 24;
     return 0;
+}
+
+// The kernel decx_hip_sgemm takes for a product, as the number decx_hip_set_sgemm_variant would force it with: a shape
+// of the LDS-DMA tiles (18 - 22, 24 - 28) where both pitches leave a tile's byte offsets in 32 bits, else a shape of the
+// one-wave-per-block kernel (11 - 13, 23), else a register-staged tile (1 - 10, 14 - 17); 0 = operands that the vector
+// loaders cannot take (not 16-byte aligned, pitch not in fours): the 128x128 tile with element-wise loaders.
+inline int plan_sgemm(int M, int N, int K, int batch, bool vec_a, bool vec_b, long lda, long ldb) {
+    if (!(vec_a && vec_b)) return 0;
+    if (lda < kDmaMaxPitch && ldb < kDmaMaxPitch) {
+        const int dma = pick_dma_shape(M, N, K, batch);
+        if (dma) return dma;
+    }
+    const int chain = pick_chain_shape(M, N, K, batch);
+    if (chain) return chain;
+    return pick_sgemm_variant(M, N, K, batch, true);
 }
 
 }  // namespace decx_hip

@@ -372,6 +372,90 @@ def bench_blocking_calls(capi, workloads, steps, warmup):
             "blocking_call_floor_relu_64_floats": {"ms_per_call_min": round(fbest, 4), "ms_per_call_median": round(fmed, 4)}}
 
 
+SWEEP_FP32 = [(1024, 1024, 1024), (1536, 1536, 1536), (2048, 2048, 2048), (2560, 2560, 2560), (3072, 3072, 3072), (4096, 4096, 4096),
+              (6144, 6144, 6144), (640, 640, 640), (768, 768, 768), (896, 896, 896), (1152, 1152, 1152), (1280, 1280, 1280),
+              (1664, 1664, 1664), (3000, 1500, 4500), (2816, 4096, 2816), (1920, 4096, 1920), (8192, 1024, 256), (4096, 4096, 64),
+              (8192, 64, 8192), (4096, 128, 4096), (8192, 2048, 8192), (2048, 8192, 2048), (1024, 8192, 1024), (512, 8192, 512),
+              (384, 8192, 384), (64, 65536, 1024), (128, 16384, 1024), (196, 4608, 512), (300, 200, 260), (8192, 8192, 8192)]
+SWEEP_FP32_VARIANTS = [2, 3, 4, 5, 7, 8, 9, 10, 14, 15, 16, 11, 12, 13, 23, 18, 19, 20, 21, 22, 24, 25, 26, 27, 28]
+SWEEP_CONV = [(224, 224, 64, 128, 3), (112, 112, 128, 128, 3), (56, 56, 256, 256, 3), (28, 28, 512, 512, 3), (128, 128, 128, 128, 5),
+              (512, 512, 256, 256, 3)]
+SWEEP_CONV_VARIANTS = [2, 3, 4, 5, 7, 9, 10, 15, 16, 17, 11, 12, 13, 23, 29, 30]
+SWEEP_FP16 = [(8192, 8192, 8192), (4096, 4096, 4096), (2048, 2048, 2048), (1024, 1024, 1024), (3000, 1500, 4500), (64, 65536, 1024),
+              (512, 8192, 512), (128, 16384, 2048)]
+SWEEP_FP16_VARIANTS = [1, 2, 7, 8, 9, 10, 15, 16, 17, 11]
+
+
+def sweep_one(capi, launch, set_variant, variants, budget_ms=25.0):
+    """ms per launch of `launch` under the automatic choice and under every forced variant; a variant that takes more than
+    eight times the automatic choice's time is timed on one launch only."""
+    def timed(n):
+        capi.timer_start()
+        for _ in range(n):
+            launch()
+        return capi.timer_stop() / n
+    out = {}
+    for v in [0] + list(variants) + [0]:                # the automatic choice first and last: the better of the two
+        set_variant(v)
+        launch()
+        capi.sync()
+        one = timed(1)
+        if v != 0 and one > 8.0 * out[0]:
+            out[v] = one
+            continue
+        n = max(3, min(200, int(budget_ms / max(one, 1e-3))))
+        timed(n)                                        # the chip's clock settles over the first milliseconds
+        t = min(timed(n), timed(n))
+        out[v] = min(t, out[v]) if v in out else t
+    set_variant(0)
+    return out
+
+
+def bench_shape_sweep(capi, workloads):
+    """The automatic kernel choice against every forced variant, shape by shape (the evidence behind the pickers of
+    sgemm_launch.hpp, hgemm.hip and the convolution launchers)."""
+    L = capi.lib()
+    rows = []
+    def padded(x, unit):                                # the pitch of a DECX container: 8 floats, 16 halves (Matrix.h:24-27)
+        return (x + unit - 1) // unit * unit
+    def row_of(what, auto_variant, t):
+        best = min((v for v in t if v), key=lambda v: t[v])
+        return {"what": what, "auto_variant": auto_variant, "auto_ms": round(t[0], 5), "best_variant": best, "best_ms": round(t[best], 5),
+                "auto_over_best": round(t[0] / t[best], 4), "ms_by_variant": {str(v): round(ms, 5) for v, ms in t.items()}}
+    for M, K, N in SWEEP_FP32:
+        lda, ldb = padded(K, 8), padded(N, 8)
+        A, B = np.zeros((M, lda), np.float32), np.zeros((K, ldb), np.float32)
+        A[:, :K], B[:, :N] = workloads.uniform_pm1((M, K), 31), workloads.uniform_pm1((K, N), 32)
+        dA, dB, dD = capi.DeviceBuffer.from_numpy(A), capi.DeviceBuffer.from_numpy(B), capi.DeviceBuffer(M * ldb * 4)
+        t = sweep_one(capi, lambda: capi.sgemm(dA.ptr, lda, dB.ptr, ldb, dD.ptr, ldb, M, N, K, blocking=False), L.decx_hip_set_sgemm_variant,
+                      SWEEP_FP32_VARIANTS)
+        rows.append(row_of("fp32 GEMM %dx%dx%d (MxKxN)" % (M, K, N), L.decx_hip_sgemm_plan(M, N, K, 1, lda, ldb, 1), t))
+        for b in (dA, dB, dD):
+            b.free()
+    for H, W, C, N, k in SWEEP_CONV:
+        src, filt = workloads.conv_case(H=H, W=W, C=C, N=N, kh=k, kw=k)
+        kp = (k + 3) // 4 * 4
+        fb = np.zeros((N, k, kp, C), np.float32); fb[:, :, :k, :] = filt
+        dS, dF, dD = capi.DeviceBuffer.from_numpy(src), capi.DeviceBuffer.from_numpy(fb), capi.DeviceBuffer(H * W * N * 4)
+        t = sweep_one(capi, lambda: capi.conv2_im2col(dS.ptr, H, W, C, W * C, dF.ptr, N, k, k, k * kp * C, kp * C, dD.ptr, N, W * N, 1, blocking=False),
+                      L.decx_hip_set_sgemm_variant, SWEEP_CONV_VARIANTS)
+        rows.append(row_of("fp32 conv %dx%dx%d under %d filters %dx%d" % (H, W, C, N, k, k), "auto", t))
+        for b in (dS, dF, dD):
+            b.free()
+    for M, K, N in SWEEP_FP16:
+        lda, ldb = padded(K, 16), padded(N, 16)
+        A, B = np.zeros((M, lda), np.uint16), np.zeros((K, ldb), np.uint16)
+        A[:, :K] = workloads.uniform_pm1((M, K), 33).astype(np.float16).view(np.uint16)
+        B[:, :N] = workloads.uniform_pm1((K, N), 34).astype(np.float16).view(np.uint16)
+        dA, dB, dD = capi.DeviceBuffer.from_numpy(A), capi.DeviceBuffer.from_numpy(B), capi.DeviceBuffer(M * ldb * 2)
+        t = sweep_one(capi, lambda: capi.hgemm(dA.ptr, lda, dB.ptr, ldb, dD.ptr, ldb, M, N, K, blocking=False), L.decx_hip_set_hgemm_variant,
+                      SWEEP_FP16_VARIANTS)
+        rows.append(row_of("fp16 GEMM %dx%dx%d (MxKxN)" % (M, K, N), L.decx_hip_hgemm_plan(M, N, K, 1, lda, ldb, 1, None), t))
+        for b in (dA, dB, dD):
+            b.free()
+    return rows
+
+
 def cpp_api_blocking_calls():
     """The same two blocking calls made from C++ through the DECX-named API (tests/build/test_decx_api timing, built by
     backup_1_amd/host/Makefile): what a DECX program sees, without the ctypes call overhead of this script."""
@@ -430,7 +514,7 @@ def main():
     ap.add_argument("--sgemm-variant", type=int, default=0, help="force a fp32 tile shape (0 = automatic)")
     ap.add_argument("--hgemm-variant", type=int, default=0, help="force a fp16 tile shape (0 = automatic)")
     ap.add_argument("--no-verify", action="store_true", help="skip the post-run comparison of sampled rows with the oracle")
-    ap.add_argument("--only", default="", help="comma list of: headline,fp16,sq4096,small,ragged,conv,relu,host,cpu (default all); extra: ladder, copy")
+    ap.add_argument("--only", default="", help="comma list of: headline,fp16,sq4096,small,ragged,conv,relu,host,cpu (default all); extra: ladder, copy, sweep")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); --gpus %d is not supported. "
@@ -550,6 +634,11 @@ def main():
             % (also["fp32_1024_blocking_call"]["ms_per_call_min"], also["fp32_1024_blocking_call"]["ms_per_launch_enqueued"],
                also["blocking_call_floor_relu_64_floats"]["ms_per_call_min"]))
 
+    if "sweep" in only:
+        also["shape_choice_sweep"] = bench_shape_sweep(capi, workloads)
+        for row in also["shape_choice_sweep"]:
+            log("sweep, %-46s auto %-4s %9.5f ms | best forced %-3s %9.5f ms | auto / best %.3f"
+                % (row["what"], row["auto_variant"], row["auto_ms"], row["best_variant"], row["best_ms"], row["auto_over_best"]))
     if "copy" in only:
         # calibration launch for the traffic counters: 1 GiB read + 1 GiB written by a plain copy kernel
         nbytes = 1 << 30

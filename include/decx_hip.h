@@ -262,6 +262,22 @@ const char* decx_hip_last_error(void);
 int decx_hip_set_sgemm_variant(int variant);
 int decx_hip_set_hgemm_variant(int variant);
 
+/* Host-only (no device call, no counterpart in the reference; usable before decx_hip_init, when 256 compute units are
+ * assumed): which kernel decx_hip_sgemm / decx_hip_hgemm_f32acc take for `batch` products of M x N x K with these pitches
+ * (elements), computed by the very functions the entry points use -- the number decx_hip_set_*_variant would force that
+ * kernel with (tables in backup_1_amd/csrc/sgemm_launch.hpp and hgemm.hip), 0 for operands the vector loaders cannot take
+ * (`aligned` = 0: a pointer off the 16-byte grid; or a pitch not in fours / eights), -1 on bad sizes.  The fp16 variant
+ * stores the number of K ranges to *splits (nullable) when the answer is 11 (split over K), else 0.  Tests walk these
+ * over grids of shapes; nothing in the compute path depends on them. */
+int decx_hip_sgemm_plan(int M, int N, int K, int batch, long lda, long ldb, int aligned);
+int decx_hip_hgemm_plan(int M, int N, int K, int batch, long lda, long ldb, int aligned, int* splits);
+
+/* Host-only: 1 if the convolution kernels that work on patch-shaped tiles may run on a source tensor of these dimensions
+ * (their 32-bit byte offsets, the apron's negative ones and the patches' reach past the output included, stay on the
+ * right side of 2^31: see conv_patch_offsets_fit in backup_1_amd/csrc/runtime.hpp), 0 if the library takes its other
+ * kernels for it, -1 on bad arguments.  elem_bytes 4 (fp32) or 2 (binary16); strides in elements. */
+int decx_hip_conv_patch_offsets_fit(int H, int W, int dpitch, size_t src_row_stride, int kh, int kw, int flag, int elem_bytes);
+
 /* Host-only arithmetic check (no device call, no counterpart in the reference): the largest column index, relative to
  * the B pointer passed to a GEMM entry point, that the vector loaders of a kernel with tile_n-wide tiles fetch when B
  * has N valid columns and is read in groups of `unit` columns (4 for fp32, 8 for fp16) -- computed with the very

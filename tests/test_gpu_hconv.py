@@ -156,6 +156,11 @@ def test_split_walk_over_k_is_the_same_on_every_run(gpu, oracle):
     finally:
         capi.lib().decx_hip_set_splitk_mode(prev)
     assert check_against_f64(oracle, atomic, sbuf, fb, 1) < TOL
+    # the two ways of combining the ranges add the same fp32 partial sums in another order: a few fp32 ulps of the sum's
+    # scale apart at most, which the one rounding to binary16 turns into at most one binary16 ulp of the result
+    ref, scale = oracle.conv2_f64_f16(sbuf, fb, 1)
+    diff = np.abs(atomic.astype(np.float64) - first.astype(np.float64))
+    assert np.all(diff <= 2.0 ** -10 * np.abs(ref) + 1e-5 * scale + 2.0 ** -24)
 
 
 # channel pitch a multiple of 64 halves: a K step lies inside one tap, which is what the LDS-DMA kernel needs.  It is the

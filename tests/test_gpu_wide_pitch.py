@@ -59,3 +59,23 @@ def test_fp16_wide_pitch(gpu, pitch, variant):
         capi.lib().decx_hip_set_hgemm_variant(prev)
     want = (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float16).view(np.uint16)
     assert np.array_equal(get(dD, M, N, pitch, np.uint16), want)
+
+
+@pytest.mark.parametrize("variant", [26, 27, 28, 20, 18, 0])
+def test_fp32_lds_dma_tiles_at_their_widest_pitch(gpu, oracle, variant):
+    # pitches of 2^21 - 4 floats, the widest the LDS-DMA tiles take: row 255 of a 256-row tile of A starts 2^31 - 4080 bytes
+    # after the tile's first row, the last 32-bit byte offset these kernels form.  (One float wider and the library takes
+    # another kernel: tests/test_kernel_choice.py.)  Two tile rows, so that the second tile's base lies beyond 2 GiB.
+    M, K, N, pitch = 300, 72, 260, (1 << 21) - 4
+    A = workloads.normal((M, K), 921)
+    B = workloads.normal((K, N), 922)
+    dA, dB = put(A, pitch), put(B, pitch)
+    dD = capi.DeviceBuffer(M * 264 * 4)
+    prev = capi.lib().decx_hip_set_sgemm_variant(variant)
+    try:
+        if variant:
+            assert capi.lib().decx_hip_sgemm_plan(M, N, K, 1, pitch, pitch, 1) == variant      # the tile under test does run
+        capi.sgemm(dA.ptr, pitch, dB.ptr, pitch, dD.ptr, 264, M, N, K)
+    finally:
+        capi.lib().decx_hip_set_sgemm_variant(prev)
+    assert np.array_equal(get(dD, M, N, 264, np.float32).view(np.uint32), oracle.sgemm_chain(A, B).view(np.uint32))
