@@ -13,10 +13,6 @@ namespace decx_hip {
 typedef HconvShape<128, 128, 2, 2, 4> HconvSquare;   // 2x2 waves of 64x64
 typedef HconvShape<256, 128, 4, 2, 4> HconvTall;     // 4x2 waves of 64x64, two per SIMD: half the filter reads per pixel
 typedef HconvDmaShape<256, 128, 4, 2, 3> HconvDma;   // the tall tile fed by LDS-DMA loads, three K steps in LDS
-// at most 64 filters: the 128-wide tiles of the 16x16x32 kernel would spend half of their matrix instructions on
-// filters that do not exist
-static bool narrow16(int N) { return N <= 64; }
-
 int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_stride, const uint16_t* filt, int N, int kh,
                   int kw, size_t filt_stride, size_t filt_row_stride, uint16_t* dst, int dst_dpitch, size_t dst_row_stride,
                   int flag, const uint16_t* bias, bool relu) {
@@ -119,10 +115,15 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
     // itself it takes the images whose patches give at least a quarter of the CUs a tile.
     {
         const bool fits = tap_uniform && conv_patch_offsets_fit(src_bytes, src_row_stride, (size_t)dpitch, kh, kw, oy, ox, 2);
-        const bool wide = N > 128;
         const long patches = (long)cdiv(Hout, 16) * cdiv(Wout, 16);
-        const long tiles16 = patches * cdiv(N, wide ? 256 : 128);
-        const bool by_itself = !kernel_forced && !narrow16(N) && tiles16 >= cus / 4 && g_rt.hgemm_variant != 19;
+        // tiles 256 filters wide (half the image traffic per filter) where they still give half of the CUs a tile (measured:
+        // 224x224x64 under 256 filters, 196 patches, 18.6 us against 21.1 on 392 tiles of 128 filters; 112x112x128 under
+        // 256, 49 patches, 24.9 against 15.6), 64 wide for at most 64 filters (the wider ones would spend their matrix
+        // instructions on filters that do not exist: 1024x512x64 under 64 filters 65.9 -> 49.1 us against the tap-row kernel)
+        const bool wide = N > 128 && 2 * patches * cdiv(N, 256) >= cus;
+        const bool slim = N <= 64;
+        const long tiles16 = patches * cdiv(N, wide ? 256 : slim ? 64 : 128);
+        const bool by_itself = !kernel_forced && tiles16 >= cus / 4 && g_rt.hgemm_variant != 19;
         if (fits && tiles16 <= 0x7fffffffL && (g_rt.hgemm_variant == 18 || by_itself)) {
             auto launch16 = [&](auto shape) -> int {
                 typedef decltype(shape) S;
@@ -139,6 +140,7 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
                 return 0;
             };
             if (wide) return launch16(Hconv16Shape<256, 2, 4>{});      // 2x4 waves of 128 pixels x 64 filters
+            if (slim) return launch16(Hconv16Shape<64, 8, 1>{});       // 8x1 waves of 32 pixels x 64 filters
             return launch16(Hconv16Shape<128, 4, 2>{});                // 4x2 waves of 64 pixels x 64 filters
         }
     }
