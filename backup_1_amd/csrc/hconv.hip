@@ -61,6 +61,26 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
         HIP_TRY(allow(reinterpret_cast<const void*>(hconv_tile_kernel<HconvSquare, false>), HconvSquare::LDS_BYTES));
         attr_done = true;
     }
+    // a K step of 64 halves inside one tap: the kernel on v_mfma_f32_16x16x32_f16 with patch-shaped tiles (hconv_mfma16.hpp).
+    // Its column test adds 2^31 to an offset, which must throw it out of the tensor's range even from the apron's negative
+    // offsets, and its patches reach up to 15 rows and 15 columns past the output: those offsets must stay below 2^31 as
+    // well.  hgemm variant 18 takes it for any image it can run on; by itself it takes the images whose patches give at
+    // least a sixth of the CUs a tile (56x56x256 under 256 filters: 64 tiles of 64 filters 17.2 us, split over K 22.8;
+    // 112x112x64 under 64 filters: 49 tiles 6.9 us against 7.9), and then before the split over K is considered.
+    const bool kernel_forced = (g_rt.hgemm_variant >= 12 && g_rt.hgemm_variant <= 14) || g_rt.hgemm_variant == 18;      // experiments and tests: no split
+    const bool fits16 = tap_uniform && conv_patch_offsets_fit(src_bytes, src_row_stride, (size_t)dpitch, kh, kw, oy, ox, 2);
+    const long patches = (long)cdiv(Hout, 16) * cdiv(Wout, 16);
+    // tiles 256 filters wide (half the image traffic per filter) where they still give half of the CUs a tile (measured:
+    // 224x224x64 under 256 filters, 196 patches, 18.6 us against 21.1 on 392 tiles of 128 filters; 112x112x128 under
+    // 256, 49 patches, 24.9 against 15.6), 64 wide for at most 64 filters (the wider ones would spend their matrix
+    // instructions on filters that do not exist: 1024x512x64 under 64 filters 65.9 -> 49.1 us against the tap-row kernel)
+    const bool wide = N > 128 && 2 * patches * cdiv(N, 256) >= cus;
+    // ... and also where tiles of 128 filters would leave half of the CUs without one (measured: 112x112x128 under 256
+    // filters 15.0 -> 11.6 us, 128x128x128 under 128 filters 14.9 -> 10.8 us; at 196 patches under 128 filters 10.5 -> 14.5)
+    const bool slim = N <= 64 || 2 * patches * cdiv(N, 128) <= cus;
+    const long tiles16 = patches * cdiv(N, wide ? 256 : slim ? 64 : 128);
+    bool take16 = fits16 && tiles16 <= 0x7fffffffL &&
+                  (g_rt.hgemm_variant == 18 || (!kernel_forced && 6 * tiles16 >= cus && g_rt.hgemm_variant != 19));
     // small image: few tiles and many K steps -> ranges of K steps as separate workgroups, fp32 partial sums in the
     // workspace, bias / ReLU / rounding in a finishing kernel
     // Measured model, in us: a workgroup walks a K step of 64 halves in 0.75 us (1.3 x that once two workgroups share a
@@ -68,8 +88,7 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
     const int all_steps = cdiv(Kw, 32);
     const long square_tiles = (long)cdiv(M, 128) * tiles_n;
     int splits = 1;
-    const bool kernel_forced = (g_rt.hgemm_variant >= 12 && g_rt.hgemm_variant <= 14) || g_rt.hgemm_variant == 18;      // experiments and tests: no split
-    if (!kernel_forced && !tall && 2 * square_tiles <= cus && all_steps >= 8 && (size_t)M * N <= ((size_t)1 << 26)) {
+    if (!kernel_forced && !take16 && !tall && 2 * square_tiles <= cus && all_steps >= 8 && (size_t)M * N <= ((size_t)1 << 26)) {
         const double t_whole = 4.0 + 0.75 * all_steps;
         double best = 0.85 * t_whole;
         const long most = (2 * cus + square_tiles - 1) / square_tiles;
@@ -77,6 +96,12 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
             const double share = square_tiles * s > cus ? 1.3 : 1.0;
             const double t = 9.0 + 3.1e-6 * M * N * s + 0.75 * share * cdiv(all_steps, s);
             if (t < best) best = t, splits = s;
+        }
+        // the 16x16x32 kernel on a single round of tiles, in the same model: 5 us fixed + 0.34 us per K step (measured at
+        // 16 - 64 tiles: 64x64x256 under 128 filters 17.1 us against 20.0 for the split, 28x28x512 under 512 30.8 against 21.7)
+        if (fits16 && tiles16 <= cus && g_rt.hgemm_variant != 19 && 5.0 + 0.34 * all_steps < best) {
+            take16 = true;
+            splits = 1;
         }
     }
     if (splits > 1) {
@@ -108,23 +133,8 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
         HIP_TRY(hipGetLastError());
         return 0;
     }
-    // a K step of 64 halves inside one tap: the kernel on v_mfma_f32_16x16x32_f16 with patch-shaped tiles (hconv_mfma16.hpp),
-    // 256 filters wide where there are more than 128.  Its column test adds 2^31 to an offset, which must throw it out of
-    // the tensor's range even from the apron's negative offsets, and its patches reach up to 15 rows and 15 columns past
-    // the output: those offsets must stay below 2^31 as well.  hgemm variant 18 takes it for any image it can run on; by
-    // itself it takes the images whose patches give at least a quarter of the CUs a tile.
     {
-        const bool fits = tap_uniform && conv_patch_offsets_fit(src_bytes, src_row_stride, (size_t)dpitch, kh, kw, oy, ox, 2);
-        const long patches = (long)cdiv(Hout, 16) * cdiv(Wout, 16);
-        // tiles 256 filters wide (half the image traffic per filter) where they still give half of the CUs a tile (measured:
-        // 224x224x64 under 256 filters, 196 patches, 18.6 us against 21.1 on 392 tiles of 128 filters; 112x112x128 under
-        // 256, 49 patches, 24.9 against 15.6), 64 wide for at most 64 filters (the wider ones would spend their matrix
-        // instructions on filters that do not exist: 1024x512x64 under 64 filters 65.9 -> 49.1 us against the tap-row kernel)
-        const bool wide = N > 128 && 2 * patches * cdiv(N, 256) >= cus;
-        const bool slim = N <= 64;
-        const long tiles16 = patches * cdiv(N, wide ? 256 : slim ? 64 : 128);
-        const bool by_itself = !kernel_forced && tiles16 >= cus / 4 && g_rt.hgemm_variant != 19;
-        if (fits && tiles16 <= 0x7fffffffL && (g_rt.hgemm_variant == 18 || by_itself)) {
+        if (take16) {
             auto launch16 = [&](auto shape) -> int {
                 typedef decltype(shape) S;
                 static bool attr_done = false;           // one per shape: the lambda's body is instantiated per S

@@ -300,6 +300,22 @@ __global__ __launch_bounds__(S::NT) void hconv_mfma16_kernel(HalfImage img, Half
     }
     // the wave reads back what it wrote itself: LDS operations of a wave complete in order, no barrier needed
     const bool vec = out.dpitch % 8 == 0 && out.row_stride % 8 == 0 && (reinterpret_cast<size_t>(out.dst) & 15) == 0;
+    static_assert(ROWS_PER_PASS == 8 && S::PATCH_Y == 16 && S::WM % 16 == 0, "a pass is the upper or the lower half of one image column of the patch");
+    if (vec && y0 + S::PATCH_Y <= Hout && x0 + S::PATCH_X <= out.Wout && bn0 + BN <= N) {
+        // a patch that lies inside the output as a whole (one scalar test): no checks around the stores, and the address
+        // moves from pass to pass by one of two wave-uniform steps -- 8 rows down, or up again and one column on
+        const int row0 = lane / PIECES, piece = lane % PIECES;
+        _Float16* dp = out.dst + (size_t)(y0 + row0) * out.row_stride + (size_t)(x0 + wm0 / S::PATCH_Y) * out.dpitch + n_wave + 8 * piece;
+        const ptrdiff_t down = (ptrdiff_t)(8 * out.row_stride), over = (ptrdiff_t)out.dpitch - down;
+        const unsigned char* src = park + row0 * ROW_BYTES + ((piece ^ row0) << 4);
+#pragma unroll
+        for (int pass = 0; pass < PASSES; ++pass) {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(src + pass * ROWS_PER_PASS * ROW_BYTES);
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dp));      // written once, not read by this launch
+            dp += (pass & 1) ? over : down;
+        }
+        return;
+    }
 #pragma unroll
     for (int pass = 0; pass < PASSES; ++pass) {
         const int row = pass * ROWS_PER_PASS + lane / PIECES, piece = lane % PIECES;
@@ -308,7 +324,7 @@ __global__ __launch_bounds__(S::NT) void hconv_mfma16_kernel(HalfImage img, Half
         if (y < Hout && x < out.Wout && n < N) {
             _Float16* dp = out.dst + (size_t)y * out.row_stride + (size_t)x * out.dpitch + n;
             if (vec && n + 8 <= N) {
-                __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dp));      // written once, not read by this launch
+                __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dp));
             } else {
                 const f16x8 h = __builtin_bit_cast(f16x8, v);
 #pragma unroll
