@@ -388,14 +388,18 @@ SWEEP_FP16_VARIANTS = [1, 2, 7, 8, 9, 10, 15, 16, 17, 11]
 
 def sweep_one(capi, launch, set_variant, variants, budget_ms=25.0):
     """ms per launch of `launch` under the automatic choice and under every forced variant; a variant that takes more than
-    eight times the automatic choice's time is timed on one launch only."""
+    eight times the automatic choice's time is timed on one launch only.  (Interleaved A/B runs of the automatic choice and
+    the same variant forced agree to 0.1 %; in a sweep the order of the variants shows as a few percent on kernels of
+    tens of microseconds, hence the three placements of the automatic choice.)"""
     def timed(n):
         capi.timer_start()
         for _ in range(n):
             launch()
         return capi.timer_stop() / n
     out = {}
-    for v in [0] + list(variants) + [0]:                # the automatic choice first and last: the better of the two
+    variants = list(variants)
+    half = len(variants) // 2
+    for v in [0] + variants[:half] + [0] + variants[half:] + [0]:      # the automatic choice three times: the best of them
         set_variant(v)
         launch()
         capi.sync()
@@ -405,6 +409,8 @@ def sweep_one(capi, launch, set_variant, variants, budget_ms=25.0):
             continue
         n = max(3, min(200, int(budget_ms / max(one, 1e-3))))
         timed(n)                                        # the chip's clock settles over the first milliseconds
+        if v == 0:
+            timed(n)
         t = min(timed(n), timed(n))
         out[v] = min(t, out[v]) if v in out else t
     set_variant(0)
