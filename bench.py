@@ -328,26 +328,37 @@ def bench_conv_fused(capi, workloads, steps, warmup):
     dS, dF = capi.DeviceBuffer.from_numpy(src), capi.DeviceBuffer.from_numpy(fb)
     dB = capi.DeviceBuffer.from_numpy(workloads.normal((N,), 78))
     dD = capi.DeviceBuffer(H * W * N * 4)
-    launch = lambda: capi.check(capi.lib().decx_hip_conv2_im2col_f32_fused(
-        dS.ptr, H, W, C, W * C, dF.ptr, N, kh, kw, kh * 4 * C, 4 * C, dD.ptr, N, W * N, 1, dB.ptr, 1))
-    ms = []
-    for i in range(warmup + steps):          # the fused entry point is synchronous: time whole calls
-        t0 = time.perf_counter()
-        launch()
-        if i >= warmup: ms.append((time.perf_counter() - t0) * 1e3)
+    import ctypes
+    fn = capi.lib().decx_hip_conv2_im2col_f32_fused
+    # the arguments converted once, as a C or C++ caller's are: ctypes otherwise spends a microsecond per call on them
+    args = tuple(t(v) for t, v in zip(fn.argtypes, (dS.ptr, H, W, C, W * C, dF.ptr, N, kh, kw, kh * 4 * C, 4 * C, dD.ptr, N, W * N,
+                                                    1, dB.ptr, 1)))
+    capi.check(fn(*args))
+
+    def launch():
+        rc = fn(*args)
+        if rc:
+            capi.check(rc)
+    best, med = time_blocking_calls(launch, steps, warmup)   # the fused entry point is synchronous: time whole calls
     flops = 2.0 * H * W * N * kh * kw * C
-    best = min(ms)
-    return {"ms_wall": best, "tflops": flops / (best * 1e-3) / 1e12}
+    return {"ms_wall": best, "ms_median": med, "tflops": flops / (best * 1e-3) / 1e12}
 
 
 def time_blocking_calls(call, steps, warmup):
-    """(min, median) wall milliseconds of whole synchronous calls, one after the other."""
+    """(min, median) wall milliseconds of whole synchronous calls, one after the other: like every side workload, after
+    at least SIDE_MIN_WARM_MS of calls (the chip clocks up over the first tens of milliseconds) and over at least
+    SIDE_MIN_TIMED_MS of them."""
+    t_end = time.perf_counter() + SIDE_MIN_WARM_MS * 1e-3
+    done = 0
+    while done < warmup or time.perf_counter() < t_end:
+        call()
+        done += 1
     ms = []
-    for i in range(warmup + steps):
+    t_end = time.perf_counter() + SIDE_MIN_TIMED_MS * 1e-3
+    while len(ms) < steps or time.perf_counter() < t_end:
         t0 = time.perf_counter()
         call()
-        if i >= warmup:
-            ms.append((time.perf_counter() - t0) * 1e3)
+        ms.append((time.perf_counter() - t0) * 1e3)
     ms.sort()
     return ms[0], ms[len(ms) // 2]
 
@@ -628,7 +639,8 @@ def main():
                                       "frac_of_hbm_peak": round(r["gbps"] / PEAK_HBM_GBPS, 4)}
         log("relu 8192x8192: %.4f ms -> %.0f GB/s" % (r["ms_wall"], r["gbps"]))
         r = bench_conv_fused(capi, workloads, side_steps, side_warmup)
-        also["fp32_conv_bias_relu_fused_blocking_call"] = {"tflops": round(r["tflops"], 2), "ms_per_call": round(r["ms_wall"], 4)}
+        also["fp32_conv_bias_relu_fused_blocking_call"] = {"tflops": round(r["tflops"], 2), "ms_per_call": round(r["ms_wall"], 4),
+                                                           "ms_per_call_median": round(r["ms_median"], 4)}
         log("conv + bias + relu (one kernel, blocking call): %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
         also.update(bench_blocking_calls(capi, workloads, side_steps, side_warmup))
         cpp = cpp_api_blocking_calls()
