@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from backup_1_amd import workloads
-from gpu_helpers import gpu_conv, gpu_hconv, gpu_sgemm
+from gpu_helpers import gpu_conv, gpu_hconv, gpu_hgemm, gpu_sgemm
 
 pytestmark = pytest.mark.gpu
 
@@ -72,3 +72,27 @@ def test_random_fp16_convolutions_exact_on_small_integers(gpu, oracle, seed):
         assert scale.max() < 2048
         want = np.maximum(ref, 0.0) if relu else ref
         assert np.array_equal(got.astype(np.float64), want), (H, W, C, N, kh, kw, flag, variant, relu)
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_fp16_gemms_exact_on_small_integers(gpu, seed):
+    # every fp16 GEMM kernel (register-staged 1, 2; LDS-DMA tiles on 32x32x16 blocks 3 - 10; on 16x16x32 blocks 15, 16, and 17,
+    # the walk over several tiles per workgroup, which falls back to 15 on ragged products; 11: split over K; 0: the
+    # library's choice) on ragged M / N / K, with K shorter than one, two or three K steps among them, DECX pitches,
+    # 16-byte pitches and unaligned ones, with and without "+ C".  Values in {-2 .. 2} and K <= 500: every sum is an
+    # integer below 2048 in magnitude, exact in binary16, so the bits must equal the fp64 product's.
+    rng = np.random.Generator(np.random.PCG64(9500 + seed))
+    for case in range(10):
+        M, N = int(rng.integers(1, 600)), int(rng.integers(1, 600))
+        K = int(rng.choice([int(rng.integers(1, 100)), int(rng.integers(1, 500))]))
+        variant = int(rng.choice([0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 15, 16, 17]))
+        align = int(rng.choice([16, 16, 8, 1]))
+        with_c = bool(rng.integers(0, 2))
+        A = workloads.small_ints((M, K), 700 * seed + case, -2, 2)
+        B = workloads.small_ints((K, N), 700 * seed + case + 350, -2, 2)
+        C = workloads.small_ints((M, N), 700 * seed + case + 500, -40, 40) if with_c else None
+        want = A.astype(np.float64) @ B.astype(np.float64) + (C if with_c else 0.0)
+        assert np.abs(want).max() <= 2048
+        h = lambda x: x.astype(np.float16).view(np.uint16)
+        got = gpu_hgemm(h(A), h(B), h(C) if with_c else None, align=align, variant=variant)
+        assert np.array_equal(got.view(np.float16).astype(np.float64), want), (M, K, N, variant, align, with_c)
