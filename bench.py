@@ -363,6 +363,25 @@ def time_blocking_calls(call, steps, warmup):
     return ms[0], ms[len(ms) // 2]
 
 
+def bench_batched(capi, workloads, fp16, batch, n):
+    """`batch` independent n^3 products in one launch of the batched entry point (the kernel step of GEMM3 over a
+    MatrixArray); the entry point blocks, so whole calls are timed."""
+    es = 2 if fp16 else 4
+    mats_a, mats_b = [], []
+    for i in range(batch):
+        a, b = workloads.uniform_pm1((n, n), 900 + 2 * i), workloads.uniform_pm1((n, n), 901 + 2 * i)
+        if fp16:
+            a, b = a.astype(np.float16).view(np.uint16), b.astype(np.float16).view(np.uint16)
+        mats_a.append(a); mats_b.append(b)
+    dA, dB = capi.DeviceBuffer.from_numpy(np.stack(mats_a)), capi.DeviceBuffer.from_numpy(np.stack(mats_b))
+    dD = capi.DeviceBuffer(batch * n * n * es)
+    fn = capi.lib().decx_hip_hgemm_f32acc_batched if fp16 else capi.lib().decx_hip_sgemm_batched
+    call = lambda: capi.check(fn(dA.ptr, n, n * n, dB.ptr, n, n * n, None, 0, 0, dD.ptr, n, n * n, n, n, n, batch))
+    best, med = time_blocking_calls(call, 20, 5)
+    flops = 2.0 * batch * n ** 3
+    return {"tflops": round(flops / (best * 1e-3) / 1e12, 2), "ms_per_call_min": round(best, 4), "ms_per_call_median": round(med, 4)}
+
+
 def bench_blocking_calls(capi, workloads, steps, warmup):
     """What a caller of the synchronous drop-in API (every call of the reference's API blocks) sees on kernels of tens of
     microseconds: whole calls of decx_hip_sgemm at 1024^3 beside the same kernel enqueued back to back, and the floor
@@ -601,6 +620,11 @@ def main():
         r = bench_hgemm(capi, workloads, 0, side_steps, side_warmup, 79, shape=(64, 65536, 1024))
         also["fp16_long_k_64x65536x1024_split_k"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4)}
         log("fp16 64x65536x1024 (split-K, fp32 workspace): %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+        # GEMM3's kernel step: 16 products of 1024^3 in one launch (256 tiles of 256 x 256 where one product has 16)
+        also["fp32_batched_16x1024_one_launch_blocking_call"] = bench_batched(capi, workloads, False, 16, 1024)
+        also["fp16_batched_16x1024_one_launch_blocking_call"] = bench_batched(capi, workloads, True, 16, 1024)
+        log("16 x 1024^3 in one launch: fp32 %.1f TFLOP/s, fp16 %.1f TFLOP/s" %
+            (also["fp32_batched_16x1024_one_launch_blocking_call"]["tflops"], also["fp16_batched_16x1024_one_launch_blocking_call"]["tflops"]))
     if want("ragged"):
         r = bench_sgemm(capi, workloads, 3000, 1500, 4500, side_steps, side_warmup, 4321, dist="normal")
         also["fp32_ragged_3000x1500x4500"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
