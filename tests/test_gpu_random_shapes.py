@@ -96,3 +96,19 @@ def test_random_fp16_gemms_exact_on_small_integers(gpu, seed):
         h = lambda x: x.astype(np.float16).view(np.uint16)
         got = gpu_hgemm(h(A), h(B), h(C) if with_c else None, align=align, variant=variant)
         assert np.array_equal(got.view(np.float16).astype(np.float64), want), (M, K, N, variant, align, with_c)
+
+
+@pytest.mark.parametrize("shape", [(3_000_000, 8, 8), (8, 8, 3_000_000), (16, 1_000_000, 16), (1, 1, 70_000), (70_000, 1, 1),
+                                   (1, 500_000, 1), (100_000, 40, 1), (1, 40, 100_000), (65_537, 3, 129), (250, 70_000, 6)])
+def test_extreme_aspect_ratios_exact_on_small_integers(gpu, shape):
+    # millions of rows or columns under a few k, one row under a million k: tile counts, grids and chain lengths far from
+    # the squares.  Values in {-1, 0, 1} with at most a third of them non-zero in A keep every sum exact in both precisions.
+    M, K, N = shape
+    A = workloads.small_ints((M, K), 41, -1, 1)
+    B = workloads.small_ints((K, N), 42, -1, 1)
+    if K > 2000:
+        A[:, 2000:] = 0                                 # |sum| <= 2000: exact in binary16 as well
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    assert np.array_equal(gpu_sgemm(A, B).astype(np.float64), want), shape
+    h = lambda x: x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(gpu_hgemm(h(A), h(B)).view(np.float16).astype(np.float64), want), shape
