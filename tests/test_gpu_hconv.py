@@ -192,6 +192,27 @@ def test_dma_kernel_and_register_kernel_on_the_same_cases(gpu, oracle, case, fla
     assert check_against_f64(oracle, got, sbuf, fb, flag, bias16=bias, relu=True) < TOL
 
 
+@pytest.mark.parametrize("variant", [0, 18, 14, 13, 12])
+@pytest.mark.parametrize("case", [(20, 21, 64, 40, 17, 17, 1), (40, 38, 64, 130, 17, 17, 0), (30, 18, 64, 130, 9, 11, 1),
+                                  (24, 24, 128, 64, 11, 3, 1), (19, 40, 64, 24, 2, 4, 1), (33, 33, 24, 10, 17, 1, 1)])
+def test_large_and_even_filter_extents(gpu, oracle, case, variant):
+    # the reference's lowering takes filters of up to 17 x 17 (conv2_mk_im2col.h:278-306); even extents centre on
+    # element kh / 2, kw / 2 like the odd ones.  Only four channels of the filters are non-zero, so that sums of {-1, 0, 1}
+    # products stay exact in binary16 under 289 taps.
+    H, W, C, N, kh, kw, flag = case
+    si = workloads.small_ints((H, W, C), 881, -1, 1).astype(np.float16)
+    fi = workloads.small_ints((N, kh, kw, C), 882, -1, 1).astype(np.float16)
+    fi[:, :, :, 4:] = 0
+    got, sbuf, fb = gpu_hconv(si, fi, flag, variant=variant)
+    ref, scale = oracle.conv2_f64_f16(sbuf, fb, flag)
+    assert scale.max() < 2048
+    assert np.array_equal(got.astype(np.float64), ref)
+    src = workloads.uniform_01((H, W, C), 883).astype(np.float16)
+    filt = workloads.normal((N, kh, kw, C), 884, sigma=0.02).astype(np.float16)
+    got, sbuf, fb = gpu_hconv(src, filt, flag, variant=variant)
+    assert check_against_f64(oracle, got, sbuf, fb, flag) < TOL
+
+
 def test_error_codes(gpu):
     L = capi.lib()
     d = capi.DeviceBuffer(1 << 16)
