@@ -12,6 +12,7 @@ CASES = [  # H, W, C, N, kh, kw, flag
     (6, 7, 4, 3, 3, 3, 1), (6, 7, 4, 3, 3, 3, 0), (5, 9, 8, 2, 5, 3, 1), (8, 8, 4, 5, 1, 1, 1), (9, 6, 4, 2, 3, 5, 0),
     (33, 31, 3, 7, 3, 3, 1), (40, 50, 16, 130, 3, 3, 1), (21, 23, 6, 5, 7, 7, 1), (21, 23, 6, 5, 7, 7, 0),
     (30, 30, 64, 128, 3, 3, 1), (17, 19, 4, 1, 17, 17, 1), (64, 64, 32, 64, 5, 5, 0),
+    (12, 14, 8, 6, 2, 4, 1), (12, 14, 8, 6, 4, 2, 0),          # even extents centre on element kh / 2, kw / 2 like the odd ones
 ]
 
 
@@ -38,6 +39,7 @@ DMA_CASES = [  # H, W, C, N, kh, kw, flag: channel pitch a multiple of 32 and fi
     (30, 30, 64, 128, 3, 3, 1), (64, 64, 32, 64, 5, 5, 0), (50, 47, 32, 12, 3, 3, 1), (19, 300, 64, 132, 1, 1, 1),
     (40, 40, 96, 200, 3, 3, 0), (33, 31, 32, 4, 7, 5, 1), (17, 19, 32, 8, 17, 17, 1), (9, 11, 32, 260, 1, 1, 0),
     (61, 67, 128, 36, 3, 3, 1), (5, 4, 32, 16, 3, 3, 1), (40, 1, 32, 8, 3, 3, 1), (1, 50, 64, 8, 3, 3, 1), (48, 52, 32, 20, 1, 5, 0),
+    (20, 22, 32, 8, 4, 2, 1), (20, 22, 32, 8, 2, 6, 0),
 ]
 
 
