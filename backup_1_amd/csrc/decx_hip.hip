@@ -98,6 +98,81 @@ Batch batch_on_library_stream(int count, size_t sa, size_t sb, size_t sc, size_t
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// What the host-matrix pipelines keep between calls, like the reference keeps its device blocks in a pool
+// (core/memory_management/MemoryPool_D.h) until de::release_all_tmp (Memory_pool.h:23-37): device blocks, the copy
+// streams and the events.  Allocating and freeing three 256 MiB blocks and creating the streams costs 2 ms of a
+// 14 ms call at 8192^3.  Every pipeline call ends with all of its work complete, so whatever it used is free again
+// when it returns; decx_hip_release_tmp gives the blocks back to the runtime.
+// ---------------------------------------------------------------------------------------------------------------
+struct TmpBlock {
+    void* ptr;
+    size_t bytes;
+    bool in_use;
+};
+constexpr int kMaxTmpBlocks = 16, kPipeEvents = 40;
+TmpBlock g_tmp[kMaxTmpBlocks];
+int g_tmp_count = 0;
+struct PipeObjects {
+    hipStream_t up = nullptr, down = nullptr;                    // uploads, downloads (kernels run on the library's stream)
+    hipEvent_t ev[kPipeEvents] = {};
+    bool ready = false;
+} g_pipe;
+
+int free_idle_tmp_blocks() {
+    int kept = 0;
+    hipError_t first = hipSuccess;
+    for (int i = 0; i < g_tmp_count; ++i) {
+        if (g_tmp[i].in_use) {
+            g_tmp[kept++] = g_tmp[i];
+        } else {
+            const hipError_t e = hipFree(g_tmp[i].ptr);
+            if (e != hipSuccess && first == hipSuccess) first = e;
+        }
+    }
+    g_tmp_count = kept;
+    return first == hipSuccess ? 0 : hip_fail(first, "hipFree");
+}
+
+// the smallest idle block that holds `bytes` without being more than twice as large (+ 16 MiB); else a new one
+void* tmp_acquire(size_t bytes) {
+    int best = -1;
+    for (int i = 0; i < g_tmp_count; ++i)
+        if (!g_tmp[i].in_use && g_tmp[i].bytes >= bytes && g_tmp[i].bytes <= 2 * bytes + ((size_t)16 << 20) &&
+            (best < 0 || g_tmp[i].bytes < g_tmp[best].bytes))
+            best = i;
+    if (best >= 0) {
+        g_tmp[best].in_use = true;
+        return g_tmp[best].ptr;
+    }
+    if (g_tmp_count == kMaxTmpBlocks) (void)free_idle_tmp_blocks();
+    if (g_tmp_count == kMaxTmpBlocks) return nullptr;
+    void* p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        (void)free_idle_tmp_blocks();                  // make room and try once more
+        if (hipMalloc(&p, bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+    }
+    g_tmp[g_tmp_count++] = TmpBlock{p, bytes, true};
+    return p;
+}
+void tmp_release(void* p) {
+    for (int i = 0; i < g_tmp_count; ++i)
+        if (g_tmp[i].ptr == p) g_tmp[i].in_use = false;
+}
+
+int pipe_objects() {
+    if (g_pipe.ready) return 0;
+    HIP_TRY(hipStreamCreateWithFlags(&g_pipe.up, hipStreamNonBlocking));
+    HIP_TRY(hipStreamCreateWithFlags(&g_pipe.down, hipStreamNonBlocking));
+    for (hipEvent_t& e : g_pipe.ev) HIP_TRY(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+    g_pipe.ready = true;
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
 // Host-resident batches (the MatrixArray GEMM3 of the reference): one matrix triple per pipeline step, two device
 // buffer sets, uploads / kernel / downloads on three streams chained by events, so that the copies of steps i+1 and
 // i-1 run under the kernel of step i.
@@ -112,38 +187,33 @@ int gemm3_host_pipeline(const T* hA, int lda, size_t plane_a, const T* hB, int l
         return fail(DECX_HIP_FAIL_ERROR_PARAMS, "leading dimension smaller than the row length\n");
     const size_t bytes_a = (size_t)M * lda * sizeof(T), bytes_b = (size_t)K * ldb * sizeof(T), bytes_d = (size_t)M * ldd * sizeof(T);
     struct Set { T *a = nullptr, *b = nullptr, *d = nullptr; hipEvent_t up = nullptr, done = nullptr, down = nullptr; } set[2];
-    hipStream_t s_up = nullptr, s_down = nullptr;
+    if (int rc0 = pipe_objects()) return rc0;
+    const hipStream_t s_up = g_pipe.up, s_down = g_pipe.down;
     int rc = 0;
     auto cleanup = [&] {
         (void)hipDeviceSynchronize();
         for (Set& s : set) {
-            if (s.a) (void)hipFree(s.a);
-            if (s.b) (void)hipFree(s.b);
-            if (s.d) (void)hipFree(s.d);
-            if (s.up) (void)hipEventDestroy(s.up);
-            if (s.done) (void)hipEventDestroy(s.done);
-            if (s.down) (void)hipEventDestroy(s.down);
+            if (s.a) tmp_release(s.a);
+            if (s.b) tmp_release(s.b);
+            if (s.d) tmp_release(s.d);
         }
-        if (s_up) (void)hipStreamDestroy(s_up);
-        if (s_down) (void)hipStreamDestroy(s_down);
     };
 #define PIPE_TRY(expr)                                   \
     do {                                                 \
         hipError_t e_ = (expr);                          \
         if (e_ != hipSuccess) { rc = hip_fail(e_, #expr); cleanup(); return rc; } \
     } while (0)
-    for (Set& s : set) {
-        if (hipMalloc(&s.a, bytes_a) != hipSuccess || hipMalloc(&s.b, bytes_b) != hipSuccess || hipMalloc(&s.d, bytes_d) != hipSuccess) {
-            (void)hipGetLastError();
+    for (int i = 0; i < 2; ++i) {
+        Set& s = set[i];
+        s.a = static_cast<T*>(tmp_acquire(bytes_a));
+        s.b = static_cast<T*>(tmp_acquire(bytes_b));
+        s.d = static_cast<T*>(tmp_acquire(bytes_d));
+        if (!s.a || !s.b || !s.d) {
             cleanup();
             return fail(DECX_HIP_FAIL_ALLOCATION, "Fail to allocate memory\n");
         }
-        PIPE_TRY(hipEventCreateWithFlags(&s.up, hipEventDisableTiming));
-        PIPE_TRY(hipEventCreateWithFlags(&s.done, hipEventDisableTiming));
-        PIPE_TRY(hipEventCreateWithFlags(&s.down, hipEventDisableTiming));
+        s.up = g_pipe.ev[3 * i], s.done = g_pipe.ev[3 * i + 1], s.down = g_pipe.ev[3 * i + 2];
     }
-    PIPE_TRY(hipStreamCreateWithFlags(&s_up, hipStreamNonBlocking));
-    PIPE_TRY(hipStreamCreateWithFlags(&s_down, hipStreamNonBlocking));
     auto upload = [&](int i) -> hipError_t {
         Set& s = set[i & 1];
         hipError_t e;
@@ -173,8 +243,13 @@ int gemm3_host_pipeline(const T* hA, int lda, size_t plane_a, const T* hB, int l
     }
     PIPE_TRY(hipStreamSynchronize(s_down));
     PIPE_TRY(hipStreamSynchronize(g_rt.stream));
+    PIPE_TRY(hipStreamSynchronize(s_up));
 #undef PIPE_TRY
-    cleanup();
+    for (Set& s_ : set) {
+        tmp_release(s_.a);
+        tmp_release(s_.b);
+        tmp_release(s_.d);
+    }
     return 0;
 }
 
@@ -202,38 +277,33 @@ int gemm_host_pipeline(const T* hA, int lda, const T* hB, int ldb, const T* hC, 
     };
     const int pm = panel_extent(M), pn = panel_extent(N);
     const int panels_a = cdiv(M, pm), panels_b = cdiv(N, pn), steps = panels_a + panels_b;
+    static_assert(2 * MAX_STEPS <= kPipeEvents, "an upload and a kernel event per step");
+    if (int rc0 = pipe_objects()) return rc0;
     T *dA = nullptr, *dB = nullptr, *dD = nullptr;
-    hipStream_t s_up = nullptr, s_down = nullptr;
-    hipEvent_t up[MAX_STEPS] = {}, done[MAX_STEPS] = {};
+    const hipStream_t s_up = g_pipe.up, s_down = g_pipe.down;
+    hipEvent_t* const up = g_pipe.ev;
+    hipEvent_t* const done = g_pipe.ev + MAX_STEPS;
     int rc = 0;
-    auto cleanup = [&] {
+    auto release_blocks = [&] {
+        if (dA) tmp_release(dA);
+        if (dB) tmp_release(dB);
+        if (dD) tmp_release(dD);
+    };
+    auto cleanup = [&] {           // after an error: whatever was enqueued must be over before the blocks are used again
         (void)hipDeviceSynchronize();
-        if (dA) (void)hipFree(dA);
-        if (dB) (void)hipFree(dB);
-        if (dD) (void)hipFree(dD);
-        for (int p = 0; p < MAX_STEPS; ++p) {
-            if (up[p]) (void)hipEventDestroy(up[p]);
-            if (done[p]) (void)hipEventDestroy(done[p]);
-        }
-        if (s_up) (void)hipStreamDestroy(s_up);
-        if (s_down) (void)hipStreamDestroy(s_down);
+        release_blocks();
     };
 #define PIPE_TRY(expr)                                   \
     do {                                                 \
         hipError_t e_ = (expr);                          \
         if (e_ != hipSuccess) { rc = hip_fail(e_, #expr); cleanup(); return rc; } \
     } while (0)
-    if (hipMalloc(&dA, (size_t)M * lda * sizeof(T)) != hipSuccess || hipMalloc(&dB, (size_t)K * ldb * sizeof(T)) != hipSuccess ||
-        hipMalloc(&dD, (size_t)M * ldd * sizeof(T)) != hipSuccess) {
-        (void)hipGetLastError();
+    dA = static_cast<T*>(tmp_acquire((size_t)M * lda * sizeof(T)));
+    dB = static_cast<T*>(tmp_acquire((size_t)K * ldb * sizeof(T)));
+    dD = static_cast<T*>(tmp_acquire((size_t)M * ldd * sizeof(T)));
+    if (!dA || !dB || !dD) {
         cleanup();
         return fail(DECX_HIP_FAIL_ALLOCATION, "Fail to allocate memory\n");
-    }
-    PIPE_TRY(hipStreamCreateWithFlags(&s_up, hipStreamNonBlocking));
-    PIPE_TRY(hipStreamCreateWithFlags(&s_down, hipStreamNonBlocking));
-    for (int p = 0; p < steps; ++p) {
-        PIPE_TRY(hipEventCreateWithFlags(&up[p], hipEventDisableTiming));
-        PIPE_TRY(hipEventCreateWithFlags(&done[p], hipEventDisableTiming));
     }
     int a_up = 0, b_up = 0;      // panels of A / B on the device (or on their way, in stream order)
     for (int step = 0; step < steps; ++step) {
@@ -258,6 +328,8 @@ int gemm_host_pipeline(const T* hA, int lda, const T* hB, int ldb, const T* hC, 
             PIPE_TRY(hipMemcpy2DAsync(dD + (size_t)r0 * ldd + c0, (size_t)ldd * sizeof(T), hC + (size_t)r0 * ldc + c0,
                                       (size_t)ldc * sizeof(T), (size_t)cols * sizeof(T), rows, hipMemcpyHostToDevice, s_up));
         PIPE_TRY(hipEventRecord(up[step], s_up));
+        // (the strips of consecutive steps are disjoint and could run side by side on two streams; measured, two
+        // kernels sharing the chip slow each other by what the overlap gains)
         PIPE_TRY(hipStreamWaitEvent(g_rt.stream, up[step], 0));
         Batch one;
         one.stream = g_rt.stream;
@@ -269,10 +341,10 @@ int gemm_host_pipeline(const T* hA, int lda, const T* hB, int ldb, const T* hC, 
         PIPE_TRY(hipMemcpy2DAsync(hD + (size_t)r0 * ldd + c0, (size_t)ldd * sizeof(T), d_region, (size_t)ldd * sizeof(T),
                                   (size_t)cols * sizeof(T), rows, hipMemcpyDeviceToHost, s_down));
     }
-    PIPE_TRY(hipStreamSynchronize(s_down));
+    PIPE_TRY(hipStreamSynchronize(s_down));            // every download waits for its kernel, every kernel for its uploads
     PIPE_TRY(hipStreamSynchronize(g_rt.stream));
 #undef PIPE_TRY
-    cleanup();
+    release_blocks();
     return 0;
 }
 
@@ -622,6 +694,12 @@ int decx_hip_relu_f32_rec(const float* src, float* dst, unsigned char* rec_map, 
 }
 int decx_hip_relu_f32_backward(const float* src, float* dst, const unsigned char* rec_map, size_t n) {
     return finish(relu_enqueue<2>(src, dst, const_cast<unsigned char*>(rec_map), n));
+}
+
+int decx_hip_release_tmp(void) {
+    if (!g_rt.is_init) return need_init();
+    HIP_TRY(hipDeviceSynchronize());
+    return free_idle_tmp_blocks();
 }
 
 void* decx_hip_stream(void) { return g_rt.is_init ? static_cast<void*>(g_rt.stream) : nullptr; }

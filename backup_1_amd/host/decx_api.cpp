@@ -193,7 +193,8 @@ void InitCuda() {
     int dev = -1;
     (void)decx_hip_init(&dev);   // failures surface as DECX_FAIL_not_init on the first compute call
 }
-void release_all_tmp() {}
+// Memory_pool.h:23-37: gives back what the pools hold; here the device blocks the host-matrix pipelines keep
+void release_all_tmp() { (void)decx_hip_release_tmp(); }
 
 // IEEE binary32 -> binary16, round to nearest even
 Half Float2Half(const float& x) {

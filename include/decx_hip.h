@@ -154,7 +154,8 @@ int decx_hip_hgemm_f32acc_batched(const uint16_t* A, int lda, size_t stride_a, c
  * kernel, the download -- without the reference's padded device copies (GEMM.h:80-104).  The rows of the result are
  * processed in panels so that the upload of the next panel of A, the kernel and the download of the previous result
  * panel overlap (the reference runs them back to back on one stream).  hA, hB, hC (nullable, may equal hD), hD are
- * HOST pointers; pinned memory (decx_hip_host_malloc) is needed for the overlap, pageable memory works serially. */
+ * HOST pointers; pinned memory (decx_hip_host_malloc) is needed for the overlap, pageable memory works serially.
+ * The device blocks stay with the library for the next call (decx_hip_release_tmp gives them back). */
 int decx_hip_gemm_host_f32(const float* hA, int lda, const float* hB, int ldb, const float* hC, int ldc, float* hD, int ldd,
                            int M, int N, int K);
 int decx_hip_gemm_host_f16(const uint16_t* hA, int lda, const uint16_t* hB, int ldb, const uint16_t* hC, int ldc, uint16_t* hD,
@@ -240,6 +241,11 @@ int decx_hip_relu_f32(const float* src, float* dst, size_t n);
 int decx_hip_relu_f32_async(const float* src, float* dst, size_t n);
 int decx_hip_relu_f32_rec(const float* src, float* dst, unsigned char* rec_map, size_t n);
 int decx_hip_relu_f32_backward(const float* src, float* dst, const unsigned char* rec_map, size_t n);
+
+/* de::release_all_tmp (core/memory_management/Memory_pool.h:23-37: releases the blocks its memory pools hold).  The
+ * host-matrix entry points (decx_hip_gemm_host_*, decx_hip_gemm3_host_*) keep their device blocks for the next call, as
+ * the reference's device pool does (MemoryPool_D.h); this waits for the device and frees them. */
+int decx_hip_release_tmp(void);
 
 /* The HIP stream (a hipStream_t) on which every _async entry point enqueues and on which the blocking ones wait: for
  * callers that order work of their own behind the library's (the reference keeps its streams to itself; no

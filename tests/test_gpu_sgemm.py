@@ -228,6 +228,46 @@ def test_host_resident_gemm_pipeline_fp16(gpu, oracle):
     assert np.array_equal(oracle.half_to_float(D), (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32))
 
 
+def test_host_pipelines_keep_their_device_blocks_until_release_tmp(gpu):
+    # the device blocks of the host-matrix entry points stay with the library between calls (the reference's device pool,
+    # MemoryPool_D.h) and go back to the runtime with decx_hip_release_tmp (de::release_all_tmp, Memory_pool.h:23-37);
+    # a call of another size in between takes blocks of its own or a larger idle one, and results stay right throughout
+    import ctypes
+    import time
+    hip = ctypes.CDLL("libamdhip64.so")
+
+    def free_bytes():
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+        return free.value
+
+    L = gpu.lib()
+    p = lambda a: a.ctypes.data
+
+    def call(M, K, N):
+        A, B = workloads.small_ints((M, K), 96), workloads.small_ints((K, N), 97)
+        D = np.zeros((M, N), np.float32)
+        gpu.check(L.decx_hip_gemm_host_f32(p(A), K, p(B), N, None, 0, p(D), N, M, N, K))
+        assert np.array_equal(D, (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32))
+        return free_bytes()
+
+    gpu.check(L.decx_hip_release_tmp())
+    big = (4000, 64, 4000)
+    first = call(*big)
+    assert call(*big) == first                          # the same call again allocates nothing
+    assert call(1500, 24, 1200) < first                 # much smaller operands: blocks of their own
+    assert call(*big) == call(*big)
+    held = free_bytes()
+    gpu.check(L.decx_hip_release_tmp())
+    kept_at_least = 4 * (4000 * 64 + 64 * 4000 + 4000 * 4000)
+    deadline = time.time() + 2.0                        # the runtime reports freed memory with a delay
+    while free_bytes() - held < kept_at_least and time.time() < deadline:
+        time.sleep(0.05)
+    assert free_bytes() - held >= kept_at_least
+    gpu.check(L.decx_hip_release_tmp())                 # nothing left to give back: still fine
+    assert call(*big) <= first + kept_at_least          # and the pipelines work on after a release
+
+
 def _splitk(gpu, A, B, C=None, splits=0, inplace=False):
     M, K = A.shape
     _, N = B.shape
