@@ -24,7 +24,7 @@ SYMBOLS = [
     "decx_hip_sgemm_splitk", "decx_hip_sgemm_batched", "decx_hip_hgemm_f32acc_batched", "decx_hip_gemm3_host_f32", "decx_hip_gemm3_host_f16",
     "decx_hip_conv2_im2col_f32_fused", "decx_hip_conv2_im2col_f16", "decx_hip_conv2_im2col_f16_async", "decx_hip_sgemm_relu", "decx_hip_relu_f32", "decx_hip_relu_f32_async",
     "decx_hip_relu_f32_rec", "decx_hip_relu_f32_backward", "decx_hip_gemm_host_f32", "decx_hip_gemm_host_f16",
-    "decx_hip_b_read_extent", "decx_hip_sgemm_plan", "decx_hip_hgemm_plan", "decx_hip_conv_patch_offsets_fit", "decx_hip_set_splitk_mode", "decx_hip_hgemm_f32acc_noalloc", "decx_hip_release_tmp",
+    "decx_hip_b_read_extent", "decx_hip_sgemm_plan", "decx_hip_hgemm_plan", "decx_hip_conv_patch_offsets_fit", "decx_hip_set_splitk_mode", "decx_hip_hgemm_f32acc_noalloc", "decx_hip_release_tmp", "decx_hip_tmp_malloc", "decx_hip_tmp_free",
 ]
 
 
@@ -59,7 +59,8 @@ def lib():
             "decx_hip_hgemm_f32acc_async": ([P, I, P, I, P, I, P, I, I, I, I], I),
             "decx_hip_conv2_im2col_f32": ([P, I, I, I, Z, P, I, I, I, Z, Z, P, I, Z, I], I),
             "decx_hip_conv2_im2col_f32_async": ([P, I, I, I, Z, P, I, I, I, Z, Z, P, I, Z, I], I),
-            "decx_hip_stream": ([], P), "decx_hip_release_tmp": ([], I),
+            "decx_hip_stream": ([], P), "decx_hip_release_tmp": ([], I), "decx_hip_tmp_malloc": ([ctypes.POINTER(ctypes.c_void_p), Z], I),
+            "decx_hip_tmp_free": ([P], I),
             "decx_hip_sgemm_splitk": ([P, I, P, I, P, I, P, I, I, I, I, I], I),
             "decx_hip_sgemm_batched": ([P, I, Z, P, I, Z, P, I, Z, P, I, Z, I, I, I, I], I),
             "decx_hip_hgemm_f32acc_batched": ([P, I, Z, P, I, Z, P, I, Z, P, I, Z, I, I, I, I], I),

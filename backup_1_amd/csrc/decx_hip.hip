@@ -696,6 +696,24 @@ int decx_hip_relu_f32_backward(const float* src, float* dst, const unsigned char
     return finish(relu_enqueue<2>(src, dst, const_cast<unsigned char*>(rec_map), n));
 }
 
+int decx_hip_tmp_malloc(void** dptr, size_t bytes) {
+    if (!g_rt.is_init) return need_init();
+    if (!dptr || bytes == 0) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "null pointer or empty block\n");
+    *dptr = tmp_acquire(bytes);
+    if (!*dptr) return fail(DECX_HIP_FAIL_ALLOCATION, "Fail to allocate memory\n");
+    return 0;
+}
+
+int decx_hip_tmp_free(void* dptr) {
+    if (!dptr) return 0;
+    for (int i = 0; i < g_tmp_count; ++i)
+        if (g_tmp[i].ptr == dptr && g_tmp[i].in_use) {
+            g_tmp[i].in_use = false;
+            return 0;
+        }
+    return fail(DECX_HIP_FAIL_ERROR_PARAMS, "not a block of decx_hip_tmp_malloc in use\n");
+}
+
 int decx_hip_release_tmp(void) {
     if (!g_rt.is_init) return need_init();
     HIP_TRY(hipDeviceSynchronize());

@@ -31,10 +31,10 @@ de::DH alloc_fail() {
     return de::DH{decx::DECX_FAIL_ALLOCATION, msg};
 }
 
-struct DeviceTemp {   // a device buffer freed on scope exit
+struct DeviceTemp {   // a device block from the library's pool of temporaries, given back to it on scope exit
     void* ptr = nullptr;
-    int alloc(size_t bytes) { return decx_hip_malloc(&ptr, bytes); }
-    ~DeviceTemp() { if (ptr) decx_hip_free(ptr); }
+    int alloc(size_t bytes) { return decx_hip_tmp_malloc(&ptr, bytes); }
+    ~DeviceTemp() { if (ptr) decx_hip_tmp_free(ptr); }
 };
 
 template <typename T> struct GemmCall;
@@ -402,7 +402,9 @@ DH conv_host(Tensor<T>& src_, TensorArray<T>& kernel_, Tensor<T>& dst_, const in
     // and what the kernel needs of src's layout is taken down before that, since re_construct may rewrite those fields
     const int src_dpitch = (int)src->dpitch;
     const size_t src_row = src->dp_x_wp;
-    if (!dst->re_construct((uint)Wout, (uint)Hout, ker->tensor_num, decx::Page_Locked)) return alloc_fail();   // :178
+    // (:178; every byte of dst, padding included, then comes down from the device block, which is zero where the
+    // kernel does not write: the zero fill of re_construct would be written over)
+    if (!dst->re_construct_for_overwrite((uint)Wout, (uint)Hout, ker->tensor_num, decx::Page_Locked)) return alloc_fail();
     rc = decx_hip_memset(dD.ptr, 0, dst->total_bytes);   // the width / channel padding of dst stays zero
     if (rc) return from_status(rc);
     rc = ConvCall<T>::run(static_cast<const T*>(dS.ptr), H, W, src_dpitch, src_row, static_cast<const T*>(dK.ptr),

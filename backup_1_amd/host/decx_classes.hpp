@@ -254,6 +254,12 @@ public:
         }
         return construct(w, h, d, store_type);
     }
+    // re_construct for a caller that writes all total_bytes itself right away (padding included): a tensor that
+    // already has the shape is left as it is instead of zero-filled (Tensor.h:350-355 fills; 25.7 MB take 0.3 ms)
+    bool re_construct_for_overwrite(uint w, uint h, uint d, int store_type) {
+        if (Tens.ptr && w == width && h == height && d == depth && store_type == _store_type) return true;
+        return construct(w, h, d, store_type);
+    }
     uint Width() override { return width; }
     uint Height() override { return height; }
     uint Depth() override { return depth; }

@@ -247,6 +247,13 @@ int decx_hip_relu_f32_backward(const float* src, float* dst, const unsigned char
  * the reference's device pool does (MemoryPool_D.h); this waits for the device and frees them. */
 int decx_hip_release_tmp(void);
 
+/* Temporary device blocks from that pool: what decx::alloc::_device_malloc / _device_dealloc are to the reference's host
+ * overloads, whose device temporaries come from and go back to decx::mem_pool_D (core/allocators.h:184-189, :137-140;
+ * conv2_mk_im2col.h:167-274 takes ker_buf, src_buf, I2C_buf and dst_buf that way).  tmp_free keeps the block for the next
+ * tmp_malloc of a similar size; the work that used it must be complete.  Not for blocks a caller keeps: decx_hip_malloc. */
+int decx_hip_tmp_malloc(void** dptr, size_t bytes);
+int decx_hip_tmp_free(void* dptr);
+
 /* The HIP stream (a hipStream_t) on which every _async entry point enqueues and on which the blocking ones wait: for
  * callers that order work of their own behind the library's (the reference keeps its streams to itself; no
  * counterpart).  NULL before decx_hip_init.  The stream has default priority and does not synchronise with the NULL

@@ -678,6 +678,30 @@ static void blocking_call_timing() {
         }
         report("Conv2_MK_im2col(GPU_Tensor) 224x224x64, 128 x 3x3x64", us);
     }
+    {   // the reference's own convolution entry: host tensors in, host tensor out (conv2_mk_im2col.h:25)
+        de::Tensor<float>& s = de::CreateTensorRef<float>(224, 224, 64, decx::Page_Locked);
+        de::TensorArray<float>& k = de::CreateTensorArrayRef<float>(3, 3, 64, 128, decx::Page_Locked);
+        de::Tensor<float>& d = de::CreateTensorRef<float>(224, 224, 128, decx::Page_Locked);
+        std::vector<double> us;
+        for (int i = 0; i < 150; ++i) {
+            const auto t0 = std::chrono::steady_clock::now();
+            de::cuda::Conv2_MK_im2col(s, k, d, 1);
+            if (i >= 30) us.push_back(std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count());
+        }
+        report("Conv2_MK_im2col(Tensor) 224x224x64, 128 x 3x3x64, host tensors", us);
+    }
+    {   // host matrices in, host matrix out (GEMM.h:56-131)
+        de::Matrix<float>& A = de::CreateMatrixRef<float>(4096, 4096, decx::Page_Locked);
+        de::Matrix<float>& B = de::CreateMatrixRef<float>(4096, 4096, decx::Page_Locked);
+        de::Matrix<float>& D = de::CreateMatrixRef<float>(4096, 4096, decx::Page_Locked);
+        std::vector<double> us;
+        for (int i = 0; i < 24; ++i) {
+            const auto t0 = std::chrono::steady_clock::now();
+            de::cuda::GEMM(A, B, D);
+            if (i >= 4) us.push_back(std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count());
+        }
+        report("GEMM(Matrix<float>) 4096^3, host matrices", us);
+    }
     {
         de::GPU_Matrix<float>& A = de::CreateGPUMatrixRef<float>(1024, 1024);
         de::GPU_Matrix<float>& B = de::CreateGPUMatrixRef<float>(1024, 1024);
