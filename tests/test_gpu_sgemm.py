@@ -265,6 +265,16 @@ def test_host_pipelines_keep_their_device_blocks_until_release_tmp(gpu):
         time.sleep(0.05)
     assert free_bytes() - held >= kept_at_least
     gpu.check(L.decx_hip_release_tmp())                 # nothing left to give back: still fine
+    # temporaries of the C++ layer's host overloads: the same pool
+    blk, blk2 = ctypes.c_void_p(), ctypes.c_void_p()
+    gpu.check(L.decx_hip_tmp_malloc(ctypes.byref(blk), 5 << 20))
+    gpu.check(L.decx_hip_tmp_free(blk))
+    gpu.check(L.decx_hip_tmp_malloc(ctypes.byref(blk2), 4 << 20))
+    assert blk2.value == blk.value                      # a block of a similar size is taken again
+    gpu.check(L.decx_hip_tmp_free(blk2))
+    assert L.decx_hip_tmp_free(blk2) == 0x0d and L.decx_hip_tmp_free(None) == 0
+    assert L.decx_hip_tmp_malloc(None, 16) == 0x0d and L.decx_hip_tmp_malloc(ctypes.byref(blk), 0) == 0x0d
+    gpu.check(L.decx_hip_release_tmp())
     assert call(*big) <= first + kept_at_least          # and the pipelines work on after a release
 
 
