@@ -195,7 +195,7 @@ def test_gemm3_host_pipeline(gpu):
 @pytest.mark.parametrize("shape", [(96, 40, 120), (2048 + 300, 72, 264), (5000, 33, 100), (2100, 40, 2300), (300, 24, 5000),
                                    (9000, 16, 3100)])
 def test_host_resident_gemm_pipeline(gpu, shape):
-    # decx_hip_gemm_host_f32: pitched host matrices in, pitched host matrix out; above 1024 rows of A / columns of B the
+    # decx_hip_gemm_host_f32: pitched host matrices in, pitched host matrix out; above 512 rows of A / columns of B the
     # operands go up as several panels, and the result is computed and brought back region by region
     M, K, N = shape
     A, B = workloads.small_ints((M, K), 91), workloads.small_ints((K, N), 92)
