@@ -259,6 +259,22 @@ def bench_host_resident_gemm(capi, A, B, reps):
     return {"ms": best * 1e3, "tflops": 2.0 * M * N * K / best / 1e12, "pcie_bytes": 4.0 * (M * K + K * N + M * N)}
 
 
+def bench_host_resident_gemm3(capi, workloads, count, n, reps):
+    """de::cuda::GEMM3(MatrixArray...) equivalent (GEMM3.h:27-36) through decx_hip_gemm3_host_f32: `count` products of n^3
+    between pinned host arrays; uploads, kernels and downloads of consecutive matrices overlap on three streams."""
+    hA, hB, hD = (PinnedArray(capi, (count, n, n), np.float32) for _ in range(3))
+    for i in range(count):
+        hA.array[i], hB.array[i] = workloads.uniform_pm1((n, n), 700 + 2 * i), workloads.uniform_pm1((n, n), 701 + 2 * i)
+    best = None
+    for _ in range(reps + 1):
+        t0 = time.perf_counter()
+        capi.check(capi.lib().decx_hip_gemm3_host_f32(hA.ptr, n, n * n, hB.ptr, n, n * n, None, 0, 0, hD.ptr, n, n * n, n, n, n, count))
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    for h in (hA, hB, hD): h.free()
+    return {"ms": best * 1e3, "tflops": 2.0 * count * n ** 3 / best / 1e12, "pcie_bytes": 12.0 * count * n * n}
+
+
 def bench_host_resident_conv(capi, workloads, reps):
     """de::cuda::Conv2_MK_im2col(Tensor, TensorArray, Tensor) equivalent (conv2_mk_im2col.h:278-306): upload the
     tensor and the filters, fused kernel, download the result."""
@@ -697,6 +713,10 @@ def main():
         also["host_resident_gemm_%d_pcie_inclusive" % n] = {"tflops": round(r["tflops"], 2), "ms_per_call": round(r["ms"], 2),
                                                             "pcie_bytes": r["pcie_bytes"]}
         log("host-resident GEMM %d^3 (H2D + kernel + D2H): %.1f ms -> %.1f TFLOP/s" % (n, r["ms"], r["tflops"]))
+        r = bench_host_resident_gemm3(capi, workloads, 8, 2048, 3)
+        also["host_resident_gemm3_8x2048_pcie_inclusive"] = {"tflops": round(r["tflops"], 2), "ms_per_call": round(r["ms"], 2),
+                                                              "pcie_bytes": r["pcie_bytes"]}
+        log("host-resident GEMM3, 8 x 2048^3 (H2D + kernels + D2H): %.2f ms -> %.1f TFLOP/s" % (r["ms"], r["tflops"]))
         r = bench_host_resident_conv(capi, workloads, 5)
         also["host_resident_conv_pcie_inclusive"] = {"tflops": round(r["tflops"], 2), "ms_per_call": round(r["ms"], 3)}
         log("host-resident conv (H2D + kernel + D2H): %.3f ms -> %.1f TFLOP/s" % (r["ms"], r["tflops"]))
