@@ -17,6 +17,9 @@ int conv_dispatch_plain(int variant, const Im2colA<false>& a, const FilterB<fals
 // the convolution on LDS-DMA loads and 16x16 blocks (sconv_dma.hpp), instantiated in sconv_dma.hip
 int launch_sconv_dma_shape(int shape, const Im2colA<true>& img, const FilterB<true>& fb, const float* bias, float* dst,
                            const TensorOut& out, int M, int N, int K);
+// the convolution of small images on tiles of 32 x 32 fed by LDS-DMA loads (sconv_small.hpp), instantiated in sconv_small.hip
+int launch_sconv_small_shape(const Im2colA<true>& img, const FilterB<true>& fb, const float* bias, float* dst, const TensorOut& out,
+                             int M, int N, int K);
 
 template <class S>
 int launch_conv_chain16(const Im2colA<false>& img, const FilterB<false>& fb, const float* bias, float* dst, const TensorOut& out,
@@ -36,10 +39,22 @@ int launch_conv_chain16(const Im2colA<false>& img, const FilterB<false>& fb, con
     return 0;
 }
 
+namespace {
+// shape 33 is the automatic choice with the small-image kernel kept out of it (experiments and tests): the rest of the
+// function sees shape 0
+struct ShapeForThisCall {
+    int saved;
+    explicit ShapeForThisCall(int shape) : saved(g_rt.sgemm_variant) { g_rt.sgemm_variant = shape; }
+    ~ShapeForThisCall() { g_rt.sgemm_variant = saved; }
+};
+}  // namespace
+
 int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt, int N, int kh,
                  int kw, size_t filt_stride, size_t filt_row_stride, float* dst, int dst_dpitch, size_t dst_row_stride,
                  int flag, const float* bias, bool relu) {
     if (!g_rt.is_init) return need_init();
+    const bool small_kept_out = g_rt.sgemm_variant == 33;
+    const ShapeForThisCall shape_for_this_call(small_kept_out ? 0 : g_rt.sgemm_variant);
     if (flag != DECX_HIP_CONV_NO_COMPENSATE && flag != DECX_HIP_CONV_ZERO_COMPENSATE)
         return fail(DECX_HIP_FAIL_ERROR_FLAG, "This flag is meaningless in current context\n");   // core/error.h:67
     if (!src || !filt || !dst) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "null tensor pointer\n");
@@ -72,6 +87,35 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
     // (its 64x64 shape walks a convolution 14 % slower than a dense product of the same size -- the moving waves do the
     // im2col addressing -- so once 128x64 tiles cover three quarters of the CUs the tiles are ahead: 112x112x128 under 128
     // filters 57.1 -> 50.6 us)
+    // Small images with a channel pitch in 32s (a K step inside one tap): tiles of 32 pixels x 32 filters on 16x16 blocks fed
+    // by LDS-DMA loads (sconv_small.hpp; forced by shape 31).  Taken where a measured model of its time is below that of
+    // the kernel the rest of this function would take (microseconds; fitted on 38 layer shapes from 7x7x512 to
+    // 512x512x256, on which the choice is within 4 % of the better kernel everywhere): every SIMD walks K once per
+    // 16x16 block it owns, at 8 cycles per k and 72 % of the matrix pipe's pace, after 4 us of launch, first loads and
+    // stores; the patch kernel's single round takes 7 us + 2.93 us per 32 k; the register-staged tiles 8 us + their
+    // tile cost at the matrix peak of one CU.
+    if (!small_kept_out && (g_rt.sgemm_variant == 0 || g_rt.sgemm_variant == 31) && dpitch % 32 == 0 &&
+        conv_patch_offsets_fit(src_bytes, src_row_stride, (size_t)dpitch, kh, kw, oy, ox, sizeof(float))) {
+        bool take = g_rt.sgemm_variant == 31;
+        if (!take) {
+            const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+            const double blocks = 4.0 * (double)cdiv(Hout, 8) * cdiv(Wout, 4) * cdiv(N, 32);
+            const double rounds = blocks / (4.0 * cus) > 1.0 ? blocks / (4.0 * cus) : 1.0;
+            const double t_small = 4.0 + rounds * K * 8.0 / 2400.0 / 0.72;
+            const long patches = (long)cdiv(Hout, 16) * cdiv(Wout, 13) * cdiv(N, 128);
+            const bool patch_kernel = N % 4 == 0 && aligned16(dst) && dst_dpitch % 4 == 0 && dst_row_stride % 4 == 0 &&
+                                      patches <= cus && 4 * patches >= 3 * cus;
+            double tile_cost = 0.0;
+            (void)pick_sgemm_variant(M, N, K, 1, false, &tile_cost);
+            const double t_other = patch_kernel ? 7.0 + K / 32 * 2.93 : 8.0 + tile_cost * K * 2.0 / 614.5e3;
+            take = 0.9 * t_small < t_other;
+        }
+        if (take) {
+            Im2colA<true> a{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
+            FilterB<true> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
+            return launch_sconv_small_shape(a, b, bias, dst, out, M, N, K);
+        }
+    }
     int chain = pick_chain_shape(M, N, K, 1);
     if (chain == 13 && g_rt.sgemm_variant == 0 && (long)cdiv(M, 128) * cdiv(N, 64) >= 3 * (g_rt.compute_units > 0 ? g_rt.compute_units : 256) / 4)
         chain = 0;

@@ -425,8 +425,9 @@ SWEEP_FP32 = [(1024, 1024, 1024), (1536, 1536, 1536), (2048, 2048, 2048), (2560,
               (384, 8192, 384), (64, 65536, 1024), (128, 16384, 1024), (196, 4608, 512), (300, 200, 260), (8192, 8192, 8192)]
 SWEEP_FP32_VARIANTS = [2, 3, 4, 5, 7, 8, 9, 10, 14, 15, 16, 11, 12, 13, 23, 18, 19, 20, 21, 22, 24, 25, 26, 27, 28]
 SWEEP_CONV = [(224, 224, 64, 128, 3), (112, 112, 128, 128, 3), (56, 56, 256, 256, 3), (28, 28, 512, 512, 3), (128, 128, 128, 128, 5),
-              (512, 512, 256, 256, 3)]
-SWEEP_CONV_VARIANTS = [2, 3, 4, 5, 7, 9, 10, 15, 16, 17, 11, 12, 13, 23, 29, 30]
+              (512, 512, 256, 256, 3), (224, 224, 64, 64, 3), (96, 96, 128, 256, 3), (28, 28, 256, 256, 3), (14, 14, 512, 512, 3),
+              (180, 180, 128, 128, 3), (208, 208, 64, 128, 3), (256, 256, 64, 128, 3), (56, 56, 64, 256, 1)]
+SWEEP_CONV_VARIANTS = [2, 3, 4, 5, 7, 9, 10, 15, 16, 17, 11, 12, 13, 23, 29, 30, 31, 33]
 SWEEP_FP16 = [(8192, 8192, 8192), (4096, 4096, 4096), (2048, 2048, 2048), (1024, 1024, 1024), (3000, 1500, 4500), (64, 65536, 1024),
               (512, 8192, 512), (128, 16384, 2048)]
 SWEEP_FP16_VARIANTS = [1, 2, 7, 8, 9, 10, 15, 16, 17, 11]
@@ -667,6 +668,18 @@ def main():
             "tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
             "frac_of_fp32_matrix_peak": round(r["tflops_kernel"] / PEAK_FP32_MATRIX_TFLOPS, 4)}
         log("conv 512x512x256 -> 256: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+        # and a CNN layer on a small image (the use the reference names this convolution for): few outputs, long K
+        small = dict(H=56, W=56, C=256, N=256)
+        r = bench_conv(capi, workloads, side_steps, side_warmup, **small)
+        also["fp32_conv_56x56x256_256f3x3_fused_im2col"] = {
+            "tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
+            "frac_of_fp32_matrix_peak": round(r["tflops_kernel"] / PEAK_FP32_MATRIX_TFLOPS, 4)}
+        log("conv 56x56x256 -> 256: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+        r = bench_hconv(capi, workloads, side_steps, side_warmup, **small)
+        also["fp16_conv_56x56x256_256f3x3_f32acc_fused_im2col"] = {
+            "tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
+            "frac_of_fp16_dense_peak": round(r["tflops_kernel"] / PEAK_FP16_MATRIX_TFLOPS, 4)}
+        log("fp16 conv 56x56x256 -> 256: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
         r = bench_hconv(capi, workloads, side_steps, side_warmup, **big)
         also["fp16_conv_512x512x256_256f3x3_f32acc_fused_im2col"] = {
             "tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),

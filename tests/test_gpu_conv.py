@@ -43,7 +43,7 @@ DMA_CASES = [  # H, W, C, N, kh, kw, flag: channel pitch a multiple of 32 and fi
 ]
 
 
-@pytest.mark.parametrize("variant", [29, 30])
+@pytest.mark.parametrize("variant", [29, 30, 31])      # 31: the small-image kernel (tiles of 32 pixels x 32 filters)
 @pytest.mark.parametrize("case", DMA_CASES)
 def test_lds_dma_kernel_bit_exact_with_the_chain(gpu, oracle, case, variant):
     # K steps of 32: 3x3x32 is an odd count (the step behind the whole passes), 1x1x32 a single one; taps left, right, above

@@ -40,8 +40,8 @@ def test_random_convolutions_bit_exact(gpu, oracle, seed):
         H, W = int(rng.integers(kh, 40)), int(rng.integers(kw, 40))
         C, N = int(rng.integers(1, 40)), int(rng.integers(1, 150))
         if rng.integers(0, 3) == 0:
-            C, N = int(rng.choice([32, 64, 96])), 4 * int(rng.integers(1, 40))      # what the LDS-DMA kernel (29, 30) takes
-        flag, variant = int(rng.integers(0, 2)), int(rng.choice(list(range(14)) + [15, 16, 17, 23, 29, 30]))
+            C, N = int(rng.choice([32, 64, 96])), 4 * int(rng.integers(1, 40))      # what the LDS-DMA kernels (29, 30, 31) take
+        flag, variant = int(rng.integers(0, 2)), int(rng.choice(list(range(14)) + [15, 16, 17, 23, 29, 30, 31]))
         src = workloads.normal((H, W, C), 300 * seed + case)
         filt = workloads.normal((N, kh, kw, C), 300 * seed + case + 150)
         ref = oracle.conv2_chain(src, filt, flag)
