@@ -89,8 +89,8 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
     // filters 57.1 -> 50.6 us)
     // Small images with a channel pitch in 32s (a K step inside one tap): tiles of 32 pixels x 32 filters on 16x16 blocks fed
     // by LDS-DMA loads (sconv_small.hpp; forced by shape 31).  Taken where a measured model of its time is below that of
-    // the kernel the rest of this function would take (microseconds; fitted on 38 layer shapes from 7x7x512 to
-    // 512x512x256, on which the choice is within 4 % of the better kernel everywhere): every SIMD walks K once per
+    // the kernel the rest of this function would take (microseconds; fitted on 48 layer shapes from 7x7x512 to
+    // 1024x1024x32, on which the choice is within 2 % of the better kernel everywhere): every SIMD walks K once per
     // 16x16 block it owns, at 8 cycles per k and 72 % of the matrix pipe's pace, after 4 us of launch, first loads and
     // stores; the patch kernel's single round takes 7 us + 2.93 us per 32 k; the register-staged tiles 8 us + their
     // tile cost at the matrix peak of one CU.
@@ -107,8 +107,11 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
                                       patches <= cus && 4 * patches >= 3 * cus;
             double tile_cost = 0.0;
             (void)pick_sgemm_variant(M, N, K, 1, false, &tile_cost);
-            const double t_other = patch_kernel ? 7.0 + K / 32 * 2.93 : 8.0 + tile_cost * K * 2.0 / 614.5e3;
-            take = 0.9 * t_small < t_other;
+            // (the tile model is optimistic where its tiles come in at most two rounds -- they do not fill the chip and
+            // their prologue and epilogue lie open: there it counts for a tenth more)
+            const bool few_rounds = (long)cdiv(M, 128) * cdiv(N, 128) <= 2 * cus;
+            const double t_other = patch_kernel ? 7.0 + K / 32 * 2.93 : (8.0 + tile_cost * K * 2.0 / 614.5e3) * (few_rounds ? 1.0 / 0.9 : 1.0);
+            take = t_small < t_other;
         }
         if (take) {
             Im2colA<true> a{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
