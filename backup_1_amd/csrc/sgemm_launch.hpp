@@ -98,7 +98,9 @@ inline int pick_sgemm_variant(int M, int N, int K, int batch, bool dense = false
     // At most 8 K steps and several rounds of tiles: the launch is bound by writing the result, and two small workgroups
     // per CU overlap one tile's stores with the other's K walk (8192x64x8192: 0.100 -> 0.091 ms, 4096x128x4096: 0.0430
     // -> 0.0417 ms against the big tiles).
-    if (K <= 128 && (long)cdiv(M, 128) * cdiv(N, 128) * batch >= 2 * cus) return 2;
+    // (a result at most 64 wide: 128x64 tiles -- 400000x32x64: 52.1 -> 29.3 us, 500000x64x48: 52.8 us against 64.7 on the
+    // 64x64 LDS-DMA tiles)
+    if (K <= 128 && (long)cdiv(M, 128) * cdiv(N, 128) * batch >= 2 * cus) return N <= 64 ? 9 : 2;
     struct Cand { int variant, bm, bn; double eff; };
     const Cand cands[] = {{7, 256, 256, 1.00}, {10, 224, 256, 0.96}, {3, 256, 128, 0.95}, {4, 224, 128, 0.94}, {2, 128, 128, 0.92},
                           {9, 128, 64, 0.83}, {8, 64, 64, 0.78}, {14, 192, 192, 0.93}, {17, 208, 128, 0.90}};
@@ -189,7 +191,7 @@ inline int launch_sgemm_dma_shape(int shape, const float* A, int lda, const floa
 // block-chain kernels fill more of the chip, above, the big tiles re-use their operands better.  Steps of 64 k in three
 // buffers (96 KiB: one workgroup per CU) are ahead on a long K with at most one tile per CU, steps of 32 k in four
 // buffers (64 KiB: two workgroups share a CU) everywhere else.  Shapes 20 - 22 are 128x128, 64x128 and 128x64 tiles of
-// the same kernel, 24 and 25 tiles of 32x32 and 64x32 on 16x16 blocks, 26, 27 and 28 the 256x256, 256x224 and 256x192 tiles on eight waves; 20, 24 and 26 - 28
+// the same kernel, 24 and 25 tiles of 32x32 and 64x32 on 16x16 blocks, 26, 27 and 28 the 256x256, 256x224 and 256x192 tiles on eight waves; all but 21 and 22
 // are chosen automatically.  All paths give the same bits.
 inline int pick_dma_shape(int M, int N, int K, int batch) {
     if ((g_rt.sgemm_variant >= 18 && g_rt.sgemm_variant <= 22) || (g_rt.sgemm_variant >= 24 && g_rt.sgemm_variant <= 28)) return g_rt.sgemm_variant;
@@ -202,7 +204,10 @@ inline int pick_dma_shape(int M, int N, int K, int batch) {
     // 2816^2 x 4096 482 -> 459 us
     {
         const long last = tiles128 % cus == 0 ? cus : tiles128 % cus;
-        if (tiles128 <= 2 * cus && 8 * last >= 7 * cus) return 20;     // (1920^2: 225 tiles of 256)
+        // ... and whose tiles are at least 85 % result (30000x512x48: a tile 128 wide is 5/8 padding, 32.7 us against 19.6
+        // on 64x64 tiles)
+        const bool mostly_result = 100.0 * M * N * batch >= 85.0 * 16384.0 * tiles128;
+        if (tiles128 <= 2 * cus && 8 * last >= 7 * cus && mostly_result) return 20;     // (1920^2: 225 tiles of 256)
     }
     // Cycles per k of a launch, measured over squares of 384 .. 1792 at K = 1024 and 8192: a round of 64x64 tiles (one
     // per CU) walks K at 34.2, a round of 32x32 tiles of 16x16 blocks at 9.7.  The small tiles win where the 64x64 ones
@@ -212,18 +217,53 @@ inline int pick_dma_shape(int M, int N, int K, int batch) {
     // where the register-staged kernel would run its 256x256 tiles on two waves per SIMD (shape 7), the same tile fed by
     // LDS-DMA loads is 0.6 - 1 % ahead (8192^3: 150.5 -> 151.9 TFLOP/s, 4096^3: 148.9 -> 150.0, 8192x2048x8192: 147.9 -> 148.9):
     // MFMA busy 98.3 % against 97.5 %
-    if (4 * tiles64 > 25 * cus && K >= 512) {
+    if (4 * tiles64 > 25 * cus) {
         double cost = 0.0;
         const int tiled = pick_sgemm_variant(M, N, K, batch, true, &cost);
-        // the 256x224 tile of the same kernel (eight waves of 32x224) in that cost model: 3000x1500x4500 (252 tiles either
-        // way) 311 -> 305 us against the register-staged 224x256 tile, 8192x8192x7168 6612 -> 6350 us
-        const long tiles224 = (long)cdiv(M, 256) * cdiv(N, 224) * batch, tiles192 = (long)cdiv(M, 256) * cdiv(N, 192) * batch;
-        const double cost224 = (double)((tiles224 + cus - 1) / cus) * 256 * 224 / 0.975;
-        // and the 256x192 tile (eight waves of 32x192): 6144^3 is 768 of them, three whole rounds: 3186 -> 3075 us (150.8 TFLOP/s)
-        const double cost192 = (double)((tiles192 + cus - 1) / cus) * 256 * 192 / 0.975;
-        if (cost > 0.0 && cost192 < cost && cost192 < cost224) return 28;
-        if (cost > 0.0 && cost224 < cost) return 27;
-        if (tiled == 7) return 26;
+        if (K >= 512) {
+            // the 256x224 tile of the same kernel (eight waves of 32x224) in that cost model: 3000x1500x4500 (252 tiles either
+            // way) 311 -> 305 us against the register-staged 224x256 tile, 8192x8192x7168 6612 -> 6350 us
+            const long tiles224 = (long)cdiv(M, 256) * cdiv(N, 224) * batch, tiles192 = (long)cdiv(M, 256) * cdiv(N, 192) * batch;
+            const double cost224 = (double)((tiles224 + cus - 1) / cus) * 256 * 224 / 0.975;
+            // and the 256x192 tile (eight waves of 32x192): 6144^3 is 768 of them, three whole rounds: 3186 -> 3075 us (150.8 TFLOP/s)
+            const double cost192 = (double)((tiles192 + cus - 1) / cus) * 256 * 192 / 0.975;
+            if (cost > 0.0 && cost192 < cost && cost192 < cost224) return 28;
+            if (cost > 0.0 && cost224 < cost) return 27;
+            if (tiled == 7) return 26;
+        }
+        // A tall result at most 32 wide: the 64x32 tiles of 16x16 blocks are the only ones that do not pad it to 64 columns
+        // (200000x1024x32: 271 -> 172 us, 150000x2304x32: 407 -> 269, 400000x128x32: 128 -> 54, 600000x576x16: 401 -> 285)
+        if (N <= 32) return 25;
+        if (N <= 256) {
+            // At most 256 wide on a short K: bound by the epilogue.  Up to 64 columns the register-staged 128x64 tiles
+            // (pick_sgemm_variant) up to K = 128, the 64x64 LDS-DMA tiles from there (200000x256x64: 68.1 -> 65.7 us);
+            // beyond 64 columns the 128x128 LDS-DMA tiles (200000x128x128: 67.4 -> 62.9 us, 200000x96x96: 60.3 -> 49.7,
+            // 60000x256x100: 45.6 -> 35.4)
+            if (K <= 128 && N <= 64) return 0;
+            if (K <= 256) return N <= 64 ? 18 : 20;
+            // On a longer K, in microseconds: the tile cost at one CU's matrix peak after 8 us, against
+            //  - the 64x32 tiles of 16x16 blocks, which every SIMD walks at 8 cycles per k and block, at 0.93 K / (K + 280)
+            //    of the matrix pipe's pace, but at most 0.75 (launches of several hundred microseconds on real-valued data
+            //    run into the power limit, where the small tiles' extra LDS traffic costs clock: 100000x4096x128 runs at
+            //    0.88 on zeros and 0.77 on uniform data), after 4 us: ahead where the wide tiles pad the columns heavily
+            //    (82944x864x96: 165.6 -> 134.5 us; 64 rows per tile are ahead of 32 in this many rounds: 144.7 -> 134.5).
+            //    The tile model's efficiencies are those of a long K; against these tiles the big tiles' prologue and
+            //    epilogue weigh 150 k more (82944x864x224 on 224x128 tiles: 358 us against the model's 265);
+            //  - the 64x64 tiles fed by LDS-DMA loads, at 85 % in the tile model, for one or two of them across: ahead of
+            //    the register-staged 128x64 and 64x64 ones (409600x576x64: 301.7 -> 291.5 us, 200704x288x64: 79.7 -> 74.9);
+            //  - the 128x128 tiles fed by LDS-DMA loads where at least 85 % of them is result, at 96 % in the tile model
+            //    (147456x1152x128: 352 us on the 64x64 tiles -> 340, 150000x2048x256: 1219 on the 256x128 tile -> 1167).
+            const double us_per_cost = K * 2.0 / 614.5e3;
+            const double t_tiles = cost > 0.0 ? 8.0 + cost * us_per_cost : 1e30;
+            const double small_pace = std::min(0.75, 0.93 * K / (K + 280.0));
+            const double t_small = K >= 512 ? 4.0 + (double)tiles32 / cus * K * 8.0 / 2400.0 / small_pace : 1e30;
+            const double t_64 = N <= 128 ? 8.0 + (double)((tiles64 + cus - 1) / cus) * 4096.0 / 0.85 * us_per_cost : 1e30;
+            const bool mostly_result128 = 100.0 * M * N * batch >= 85.0 * 16384.0 * tiles128;
+            const double t_128 = mostly_result128 ? 8.0 + (double)((tiles128 + cus - 1) / cus) * 16384.0 / 0.96 * us_per_cost : 1e30;
+            if (t_small < t_tiles * (K + 150.0) / K && t_small < t_64 && t_small < t_128) return 25;
+            if (t_128 < t_tiles && t_128 < t_64) return 20;
+            if (t_64 < t_tiles) return 18;
+        }
     }
     if (2 * tiles64 >= cus && 4 * tiles64 <= 25 * cus) {
         if (walk32 < 1.05 * walk64) return 24;      // (a tie goes to the small tiles: 1280^2 237 -> 230 us, 1664^2 379 -> 366 us)

@@ -422,7 +422,10 @@ SWEEP_FP32 = [(1024, 1024, 1024), (1536, 1536, 1536), (2048, 2048, 2048), (2560,
               (6144, 6144, 6144), (640, 640, 640), (768, 768, 768), (896, 896, 896), (1152, 1152, 1152), (1280, 1280, 1280),
               (1664, 1664, 1664), (3000, 1500, 4500), (2816, 4096, 2816), (1920, 4096, 1920), (8192, 1024, 256), (4096, 4096, 64),
               (8192, 64, 8192), (4096, 128, 4096), (8192, 2048, 8192), (2048, 8192, 2048), (1024, 8192, 1024), (512, 8192, 512),
-              (384, 8192, 384), (64, 65536, 1024), (128, 16384, 1024), (196, 4608, 512), (300, 200, 260), (8192, 8192, 8192)]
+              (384, 8192, 384), (64, 65536, 1024), (128, 16384, 1024), (196, 4608, 512), (300, 200, 260), (8192, 8192, 8192),
+              # tall results at most 256 wide (the shape of a lowered convolution)
+              (409600, 576, 64), (147456, 1152, 128), (82944, 864, 96), (82944, 864, 224), (100000, 4096, 128), (300000, 128, 64),
+              (200000, 128, 128), (30000, 512, 48), (262144, 288, 32), (150000, 2048, 256), (200000, 1024, 32), (400000, 32, 64)]
 SWEEP_FP32_VARIANTS = [2, 3, 4, 5, 7, 8, 9, 10, 14, 15, 16, 11, 12, 13, 23, 18, 19, 20, 21, 22, 24, 25, 26, 27, 28]
 SWEEP_CONV = [(224, 224, 64, 128, 3), (112, 112, 128, 128, 3), (56, 56, 256, 256, 3), (28, 28, 512, 512, 3), (128, 128, 128, 128, 5),
               (512, 512, 256, 256, 3), (224, 224, 64, 64, 3), (96, 96, 128, 256, 3), (28, 28, 256, 256, 3), (14, 14, 512, 512, 3),

@@ -99,7 +99,10 @@ def test_random_fp16_gemms_exact_on_small_integers(gpu, seed):
 
 
 @pytest.mark.parametrize("shape", [(3_000_000, 8, 8), (8, 8, 3_000_000), (16, 1_000_000, 16), (1, 1, 70_000), (70_000, 1, 1),
-                                   (1, 500_000, 1), (100_000, 40, 1), (1, 40, 100_000), (65_537, 3, 129), (250, 70_000, 6)])
+                                   (1, 500_000, 1), (100_000, 40, 1), (1, 40, 100_000), (65_537, 3, 129), (250, 70_000, 6),
+                                   # tall results at most 256 wide, each on the tile the picker has for that width and K
+                                   (70_001, 600, 96), (60_003, 100, 100), (60_000, 130, 64), (45_000, 1030, 128), (33_333, 520, 200),
+                                   (52_000, 515, 250), (41_000, 300, 33), (120_000, 520, 24), (90_000, 70, 50)])
 def test_extreme_aspect_ratios_exact_on_small_integers(gpu, shape):
     # millions of rows or columns under a few k, one row under a million k: tile counts, grids and chain lengths far from
     # the squares.  Values in {-1, 0, 1} with at most a third of them non-zero in A keep every sum exact in both precisions.

@@ -67,6 +67,23 @@ def test_fp32_headline_and_config_shapes(lib):
     assert lib.decx_hip_sgemm_plan(0, 8, 8, 1, 8, 8, 1) == -1 and lib.decx_hip_sgemm_plan(8, 8, 8, 1, 4, 8, 1) == -1
 
 
+def test_fp32_tall_results_take_the_tiles_that_pad_them_least(lib):
+    """Many rows under at most 256 columns (the shape of a lowered convolution): the measured choices."""
+    plan = lambda M, K, N: lib.decx_hip_sgemm_plan(M, N, K, 1, pad(K, 8), pad(N, 8), 1)
+    assert plan(30000, 512, 48) == 18             # not the 128x128 tile, which would be 5/8 padding
+    assert plan(82944, 864, 96) == 25 and plan(82944, 864, 160) == 25      # 96 = 3 x 32, 160 = 5 x 32 columns
+    assert plan(409600, 576, 64) == 18 and plan(200000, 256, 64) == 18     # one 64x64 tile across
+    assert plan(300000, 128, 64) == 9 and plan(400000, 32, 64) == 9        # a few K steps only: 128x64 register-staged tiles
+    assert plan(147456, 1152, 128) == 20 and plan(200000, 128, 128) == 20 and plan(150000, 2048, 256) == 20
+    assert plan(262144, 288, 32) == 25 and plan(150000, 2304, 32) == 25 and plan(600000, 576, 16) == 25    # tiles 32 wide
+    assert plan(100000, 4096, 128) in FP32_TILES  # 782 tiles of 128x128 would be 3.05 rounds
+    for N in range(1, 257):                       # every width: a kernel the dispatch builds; on a long K never a 128-wide tile that is mostly padding
+        for M, K in ((100000, 128), (100000, 600), (250000, 2048)):
+            v = plan(M, K, N)
+            assert v in FP32_TILES | FP32_DMA, (M, K, N, v)
+            assert not (K > 256 and v == 20 and N % 128 != 0 and N % 128 < 100), (M, K, N)
+
+
 def test_forced_fp32_variants_stay_where_they_can_run(lib):
     for forced in sorted(FP32_TILES | FP32_CHAINS | FP32_DMA):
         lib.decx_hip_set_sgemm_variant(forced)
