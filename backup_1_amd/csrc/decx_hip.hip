@@ -763,6 +763,16 @@ int decx_hip_sgemm_plan(int M, int N, int K, int batch, long lda, long ldb, int 
     return sgemm_plan(M, N, K, batch, lda, ldb, aligned != 0);
 }
 
+int decx_hip_sgemm_plan_split(int M, int N, int K, int batch, long lda, long ldb, int aligned, int* shape, int* by_columns) {
+    if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || lda < K || ldb < N) return -1;
+    return sgemm_plan_split(M, N, K, batch, lda, ldb, aligned != 0, shape, by_columns);
+}
+
+int decx_hip_hgemm_plan_split(int M, int N, int K, int batch, long lda, long ldb, int aligned, int* by_columns) {
+    if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || lda < K || ldb < N) return -1;
+    return hgemm_plan_split(M, N, K, batch, lda, ldb, aligned != 0, by_columns);
+}
+
 int decx_hip_hgemm_plan(int M, int N, int K, int batch, long lda, long ldb, int aligned, int* splits) {
     if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || lda < K || ldb < N) return -1;
     return hgemm_plan(M, N, K, batch, lda, ldb, aligned != 0, splits);

@@ -35,6 +35,7 @@ namespace decx_hip {
 // and, for the fp16 convolution only: 12 keeps its register-staged kernels, 13 takes its LDS-DMA kernel for any image
 // whose channel pitch allows it, 14 its tap-row kernel, 18 its kernel on 16x16x32 matrix instructions with patch-shaped
 // tiles (hconv_mfma16.hpp); each switches its split over K off.  19 keeps kernel 18 out of the automatic choice.
+// 20: the automatic choice, every product in one launch (plan_hgemm_whole_rounds_split switched off).
 // (experiments and tests)
 typedef HgemmShape<256, 256, 32, 2, 2> HShapeBig;
 typedef HgemmShape<128, 128, 32, 2, 2> HShapeSmall;
@@ -242,7 +243,7 @@ static bool hgemm_vector_path(const uint16_t* A, int lda, const uint16_t* B, int
 static int plan_hgemm(int M, int N, int K, int batch_count, bool vec, int* splits_out) {
     if (splits_out) *splits_out = 0;
     if (!vec) return 0;
-    int variant = g_rt.hgemm_variant;
+    int variant = g_rt.hgemm_variant == 20 ? 0 : g_rt.hgemm_variant;
     // few 128x128 tiles and a long K: split K (variant 11 forces it, any other fixed variant switches it off)
     if (batch_count == 1 && (variant < 1 || variant > 10) && (variant < 15 || variant > 17)) {
         int splits = auto_hgemm_splits(M, N, K);
@@ -271,6 +272,50 @@ static int plan_hgemm(int M, int N, int K, int batch_count, bool vec, int* split
     return variant;
 }
 
+// A result whose 256x256 tiles come in whole rounds plus a part of one (a round = one tile per CU) pays a whole round
+// for the part, and five rounds of 128x128 tiles where four and a bit would do.  The rows -- or columns -- that fill
+// whole rounds of the 256x256 tile go to one launch of it, the rest to a second launch that picks its own kernel
+// (4352^2: 289 tiles; 3840 rows in one round, 512 rows on 136 tiles of 128x128): taken where whole rounds plus the
+// one-launch cost of the rest plus 4 us for the second launch stay under 96 % of the one-launch cost of the whole.
+// Costs in tile area per CU / efficiency, the unit of plan_hgemm; 5.5e6 of it per microsecond and k.  Variant 20 keeps
+// every product in one launch (experiments and tests).
+struct HgemmWholeRoundsSplit {
+    bool by_columns = false;
+    int first = 0;          // rows (columns) of the first launch; 0 = one launch
+};
+static double hgemm_one_launch_cost(int M, int N) {
+    const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+    const long big = (long)cdiv(M, 256) * cdiv(N, 256), small = (long)cdiv(M, 128) * cdiv(N, 128);
+    return std::min((double)((big + cus - 1) / cus) * 65536.0, (double)((small + cus - 1) / cus) * 16384.0 / 0.75);
+}
+static HgemmWholeRoundsSplit plan_hgemm_whole_rounds_split(int M, int N, int K, int batch_count, bool vec) {
+    HgemmWholeRoundsSplit plan;
+    if (!vec || g_rt.hgemm_variant != 0 || batch_count != 1 || K < 512) return plan;
+    const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+    const long tiles_m = cdiv(M, 256), tiles_n = cdiv(N, 256), whole = tiles_m * tiles_n / cus;
+    if (whole < 1 || tiles_m * tiles_n % cus == 0) return plan;
+    double best = 0.96 * hgemm_one_launch_cost(M, N);
+    const double second_launch = 4.0 * 5.5e6 / (2.0 * K);
+    for (int by_columns = 0; by_columns < 2; ++by_columns) {
+        const long lines = whole * cus / (by_columns ? tiles_m : tiles_n);          // whole tile rows (columns) in the whole rounds
+        if (lines < 1 || lines >= (by_columns ? tiles_n : tiles_m)) continue;
+        const int first = (int)lines * 256;
+        const double cost = (double)whole * 65536.0 + (by_columns ? hgemm_one_launch_cost(M, N - first) : hgemm_one_launch_cost(M - first, N)) + second_launch;
+        if (cost < best) {
+            best = cost;
+            plan.by_columns = by_columns != 0, plan.first = first;
+        }
+    }
+    return plan;
+}
+
+// host-only: the two-launch plan for a product (decx_hip_hgemm_plan_split)
+int hgemm_plan_split(int M, int N, int K, int batch, long lda, long ldb, bool aligned, int* by_columns) {
+    const HgemmWholeRoundsSplit split = plan_hgemm_whole_rounds_split(M, N, K, batch, aligned && hgemm_pitches_fit(lda, ldb));
+    if (by_columns) *by_columns = split.by_columns ? 1 : 0;
+    return split.first;
+}
+
 // host-only: the choice above for a product described by its sizes and pitches (decx_hip_hgemm_plan)
 int hgemm_plan(int M, int N, int K, int batch, long lda, long ldb, bool aligned, int* splits) {
     return plan_hgemm(M, N, K, batch, aligned && hgemm_pitches_fit(lda, ldb), splits);
@@ -280,7 +325,19 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
                   int ldd, int M, int N, int K, const Batch& batch) {
     if (int rc = check_gemm_args(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch)) return rc;
     int splits = 0;
-    int variant = plan_hgemm(M, N, K, batch.count, hgemm_vector_path(A, lda, B, ldb, batch), &splits);
+    const bool vec = hgemm_vector_path(A, lda, B, ldb, batch);
+    const HgemmWholeRoundsSplit split = plan_hgemm_whole_rounds_split(M, N, K, batch.count, vec);
+    if (split.first > 0 && !split.by_columns) {
+        if (int rc = launch_hgemm_mfma16<HShape16>(A, lda, B, ldb, Cin, ldc, D, ldd, split.first, N, K, batch)) return rc;
+        return hgemm_enqueue(A + (size_t)split.first * lda, lda, B, ldb, Cin ? Cin + (size_t)split.first * ldc : nullptr, ldc,
+                             D + (size_t)split.first * ldd, ldd, M - split.first, N, K, batch);
+    }
+    if (split.first > 0) {
+        if (int rc = launch_hgemm_mfma16<HShape16>(A, lda, B, ldb, Cin, ldc, D, ldd, M, split.first, K, batch)) return rc;
+        return hgemm_enqueue(A, lda, B + split.first, ldb, Cin ? Cin + split.first : nullptr, ldc, D + split.first, ldd, M,
+                             N - split.first, K, batch);
+    }
+    int variant = plan_hgemm(M, N, K, batch.count, vec, &splits);
     if (variant == 0) return launch_hgemm_tile<HShapeSmall, false>(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, batch);
     if (variant == 11) return hgemm_splitk_enqueue(A, lda, B, ldb, Cin, ldc, D, ldd, M, N, K, splits, batch.stream);
     if (variant == 17) {

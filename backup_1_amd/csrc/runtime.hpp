@@ -90,7 +90,9 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
                   int ldd, int M, int N, int K, const Batch& batch);
 // host-only: which kernel the two entry points above take for a product of these sizes and pitches (no device call)
 int sgemm_plan(int M, int N, int K, int batch, long lda, long ldb, bool aligned);
+int sgemm_plan_split(int M, int N, int K, int batch, long lda, long ldb, bool aligned, int* shape, int* by_columns);
 int hgemm_plan(int M, int N, int K, int batch, long lda, long ldb, bool aligned, int* splits);
+int hgemm_plan_split(int M, int N, int K, int batch, long lda, long ldb, bool aligned, int* by_columns);
 // the K-range route of hgemm_enqueue on the library's static device workspace (no allocation); splits <= 0: automatic
 int hgemm_splitk_static_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const uint16_t* Cin, int ldc,
                                 uint16_t* D, int ldd, int M, int N, int K, int splits);

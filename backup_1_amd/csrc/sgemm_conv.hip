@@ -39,22 +39,12 @@ int launch_conv_chain16(const Im2colA<false>& img, const FilterB<false>& fb, con
     return 0;
 }
 
-namespace {
-// shape 33 is the automatic choice with the small-image kernel kept out of it (experiments and tests): the rest of the
-// function sees shape 0
-struct ShapeForThisCall {
-    int saved;
-    explicit ShapeForThisCall(int shape) : saved(g_rt.sgemm_variant) { g_rt.sgemm_variant = shape; }
-    ~ShapeForThisCall() { g_rt.sgemm_variant = saved; }
-};
-}  // namespace
-
 int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt, int N, int kh,
                  int kw, size_t filt_stride, size_t filt_row_stride, float* dst, int dst_dpitch, size_t dst_row_stride,
                  int flag, const float* bias, bool relu) {
     if (!g_rt.is_init) return need_init();
     const bool small_kept_out = g_rt.sgemm_variant == 33;
-    const ShapeForThisCall shape_for_this_call(small_kept_out ? 0 : g_rt.sgemm_variant);
+    const ShapeForThisCall shape_for_this_call(small_kept_out || g_rt.sgemm_variant == 34 ? 0 : g_rt.sgemm_variant);
     if (flag != DECX_HIP_CONV_NO_COMPENSATE && flag != DECX_HIP_CONV_ZERO_COMPENSATE)
         return fail(DECX_HIP_FAIL_ERROR_FLAG, "This flag is meaningless in current context\n");   // core/error.h:67
     if (!src || !filt || !dst) return fail(DECX_HIP_FAIL_ERROR_PARAMS, "null tensor pointer\n");

@@ -63,7 +63,22 @@ int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float*
     const bool vec_a = aligned16(A) && lda % 4 == 0 && batch.stride_a % 4 == 0;
     const bool vec_b = aligned16(B) && ldb % 4 == 0 && ldb >= 4 && batch.stride_b % 4 == 0;
     DenseOut out{ldd, relu, aligned16(D) && ldd % 4 == 0 && batch.stride_d % 4 == 0};
+    const bool one_launch = g_rt.sgemm_variant == 34;
+    const ShapeForThisCall shape_for_this_call(one_launch ? 0 : g_rt.sgemm_variant);
     const int plan = plan_sgemm(M, N, K, batch.count, vec_a, vec_b, lda, ldb);
+    if (!one_launch && plan != 0) {
+        const WholeRoundsSplit split = plan_whole_rounds_split(M, N, K, batch.count, lda, ldb);
+        if (split.shape && !split.by_columns) {
+            if (int rc = launch_sgemm_dma_shape(split.shape, A, lda, B, ldb, Cin, ldc, D, ldd, split.first, N, K, batch, relu)) return rc;
+            return sgemm_enqueue(A + (size_t)split.first * lda, lda, B, ldb, Cin ? Cin + (size_t)split.first * ldc : nullptr, ldc,
+                                 D + (size_t)split.first * ldd, ldd, M - split.first, N, K, batch, relu);
+        }
+        if (split.shape) {
+            if (int rc = launch_sgemm_dma_shape(split.shape, A, lda, B, ldb, Cin, ldc, D, ldd, M, split.first, K, batch, relu)) return rc;
+            return sgemm_enqueue(A, lda, B + split.first, ldb, Cin ? Cin + split.first : nullptr, ldc, D + split.first, ldd, M,
+                                 N - split.first, K, batch, relu);
+        }
+    }
     if (plan == 0) {     // unaligned operands: element-wise loaders, one tile shape only
         DenseA<false> a{A, lda, M, K, batch.stride_a};
         DenseB<false> b{B, ldb, N, K, batch.stride_b};
@@ -82,7 +97,17 @@ int sgemm_enqueue(const float* A, int lda, const float* B, int ldb, const float*
 
 // host-only: the choice above for a product described by its sizes and pitches (decx_hip_sgemm_plan)
 int sgemm_plan(int M, int N, int K, int batch, long lda, long ldb, bool aligned) {
+    const ShapeForThisCall shape_for_this_call(g_rt.sgemm_variant == 34 ? 0 : g_rt.sgemm_variant);
     return plan_sgemm(M, N, K, batch, aligned && lda % 4 == 0, aligned && ldb % 4 == 0 && ldb >= 4, lda, ldb);
+}
+
+// host-only: the two-launch plan of plan_whole_rounds_split for a product (decx_hip_sgemm_plan_split)
+int sgemm_plan_split(int M, int N, int K, int batch, long lda, long ldb, bool aligned, int* shape, int* by_columns) {
+    WholeRoundsSplit split;
+    if (aligned && lda % 4 == 0 && ldb % 4 == 0 && ldb >= 4) split = plan_whole_rounds_split(M, N, K, batch, lda, ldb);
+    if (shape) *shape = split.shape;
+    if (by_columns) *by_columns = split.by_columns ? 1 : 0;
+    return split.shape ? split.first : 0;
 }
 
 // Split-K GEMM for problems whose M x N tile count leaves most CUs idle while K is long (the short-M / long-K shapes of

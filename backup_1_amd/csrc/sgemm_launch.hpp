@@ -290,4 +290,76 @@ inline int plan_sgemm(int M, int N, int K, int batch, bool vec_a, bool vec_b, lo
     return pick_sgemm_variant(M, N, K, batch, true);
 }
 
+// What one launch of the automatic choice costs, in the tile model's unit (tile area per CU / efficiency; times
+// 2 K / 614.5e3 it is microseconds), or 0 where the model has no figure.  A summary of the pickers above for the planner
+// below -- it decides nothing by itself.
+inline double sgemm_one_launch_cost(int M, int N, int K, int batch) {
+    const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+    double cost = 0.0;
+    pick_sgemm_variant(M, N, K, batch, true, &cost);
+    if (cost == 0.0) return 0.0;
+    const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch, tiles128 = (long)cdiv(M, 128) * cdiv(N, 128) * batch;
+    const long tiles32 = (long)cdiv(M, 32) * cdiv(N, 32) * batch;
+    auto rounds = [cus](long tiles) { return (double)((tiles + cus - 1) / cus); };
+    if (100.0 * M * N * batch >= 85.0 * 16384.0 * tiles128) cost = std::min(cost, rounds(tiles128) * 16384.0 / 0.96);
+    if (4 * tiles64 > 25 * cus) {
+        if (K >= 512)
+            for (int bn : {256, 224, 192}) cost = std::min(cost, rounds((long)cdiv(M, 256) * cdiv(N, bn) * batch) * 256.0 * bn / 0.975);
+    } else {
+        // cycles per k of the small LDS-DMA tiles (pick_dma_shape) in the model's unit: 614.5e3 / 2 / 2400 per cycle
+        cost = std::min(cost, std::min(34.2 * rounds(tiles64), 9.7 * rounds(tiles32)) * 128.0);
+    }
+    return cost;
+}
+
+// A result whose 256-row tiles come in whole rounds plus a part of one (a round = one tile per CU) pays a whole round for
+// the part.  Every element's sum is the same chain of products whatever tile computes it, so the rows -- or columns --
+// that fill whole rounds can go to one launch of such tiles and the rest to a second launch, which picks its own tiles
+// (4096x4608: 288 tiles of 256x256; 4096 columns in one round, the other 512 on 128 tiles of 128x128, against two rounds
+// of 256x192).  The plan: for each of the three 256-row LDS-DMA tiles, whole rounds of it plus the one-launch cost of the
+// rest plus 4 us for the second launch; taken where the cheapest is under 96 % of the one-launch cost of the whole.
+struct WholeRoundsSplit {
+    int shape = 0;          // 26 - 28: the tile of the first launch; 0 = one launch
+    bool by_columns = false;
+    int first = 0;          // rows (columns) of the first launch
+};
+inline WholeRoundsSplit plan_whole_rounds_split(int M, int N, int K, int batch, long lda, long ldb) {
+    WholeRoundsSplit plan;
+    if (g_rt.sgemm_variant != 0 || batch != 1 || K < 512 || lda >= kDmaMaxPitch || ldb >= kDmaMaxPitch) return plan;
+    const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+    if (4 * (long)cdiv(M, 64) * cdiv(N, 64) <= 25 * cus) return plan;
+    const double whole_cost = sgemm_one_launch_cost(M, N, K, 1);
+    if (whole_cost == 0.0) return plan;
+    double best = 0.96 * whole_cost;
+    const double second_launch = 4.0 * 614.5e3 / (2.0 * K);
+    const int shapes[3] = {26, 27, 28}, widths[3] = {256, 224, 192};
+    for (int i = 0; i < 3; ++i) {
+        const long tiles_m = cdiv(M, 256), tiles_n = cdiv(N, widths[i]), whole = tiles_m * tiles_n / cus;
+        if (whole < 1 || tiles_m * tiles_n % cus == 0) continue;
+        const double first_cost = (double)whole * 256.0 * widths[i] / 0.975;
+        for (int by_columns = 0; by_columns < 2; ++by_columns) {
+            const long lines = whole * cus / (by_columns ? tiles_m : tiles_n);          // whole tile rows (columns) in the whole rounds
+            if (lines < 1 || lines >= (by_columns ? tiles_n : tiles_m)) continue;
+            const int first = (int)lines * (by_columns ? widths[i] : 256);
+            const double rest = by_columns ? sgemm_one_launch_cost(M, N - first, K, 1) : sgemm_one_launch_cost(M - first, N, K, 1);
+            if (rest == 0.0) continue;
+            const double cost = first_cost + rest + second_launch;
+            if (cost < best) {
+                best = cost;
+                plan.shape = shapes[i], plan.by_columns = by_columns != 0, plan.first = first;
+            }
+        }
+    }
+    return plan;
+}
+
+// shape 33 (convolution: the automatic choice with the small-image kernel kept out of it) and shape 34 (dense products:
+// the automatic choice in one launch, plan_whole_rounds_split switched off) are for experiments and tests: the rest of
+// the call sees shape 0
+struct ShapeForThisCall {
+    int saved;
+    explicit ShapeForThisCall(int shape) : saved(g_rt.sgemm_variant) { g_rt.sgemm_variant = shape; }
+    ~ShapeForThisCall() { g_rt.sgemm_variant = saved; }
+};
+
 }  // namespace decx_hip

@@ -425,15 +425,19 @@ SWEEP_FP32 = [(1024, 1024, 1024), (1536, 1536, 1536), (2048, 2048, 2048), (2560,
               (384, 8192, 384), (64, 65536, 1024), (128, 16384, 1024), (196, 4608, 512), (300, 200, 260), (8192, 8192, 8192),
               # tall results at most 256 wide (the shape of a lowered convolution)
               (409600, 576, 64), (147456, 1152, 128), (82944, 864, 96), (82944, 864, 224), (100000, 4096, 128), (300000, 128, 64),
-              (200000, 128, 128), (30000, 512, 48), (262144, 288, 32), (150000, 2048, 256), (200000, 1024, 32), (400000, 32, 64)]
-SWEEP_FP32_VARIANTS = [2, 3, 4, 5, 7, 8, 9, 10, 14, 15, 16, 11, 12, 13, 23, 18, 19, 20, 21, 22, 24, 25, 26, 27, 28]
+              (200000, 128, 128), (30000, 512, 48), (262144, 288, 32), (150000, 2048, 256), (200000, 1024, 32), (400000, 32, 64),
+              # results that run as two launches (whole rounds of a 256-row tile, then the rest); 34 = kept in one launch
+              (4352, 4096, 4352), (4096, 4096, 4608), (6950, 2048, 5308), (3497, 1500, 5226), (6324, 512, 5986)]
+SWEEP_FP32_VARIANTS = [2, 3, 4, 5, 7, 8, 9, 10, 14, 15, 16, 11, 12, 13, 23, 18, 19, 20, 21, 22, 24, 25, 26, 27, 28, 34]
 SWEEP_CONV = [(224, 224, 64, 128, 3), (112, 112, 128, 128, 3), (56, 56, 256, 256, 3), (28, 28, 512, 512, 3), (128, 128, 128, 128, 5),
               (512, 512, 256, 256, 3), (224, 224, 64, 64, 3), (96, 96, 128, 256, 3), (28, 28, 256, 256, 3), (14, 14, 512, 512, 3),
               (180, 180, 128, 128, 3), (208, 208, 64, 128, 3), (256, 256, 64, 128, 3), (56, 56, 64, 256, 1)]
 SWEEP_CONV_VARIANTS = [2, 3, 4, 5, 7, 9, 10, 15, 16, 17, 11, 12, 13, 23, 29, 30, 31, 33]
 SWEEP_FP16 = [(8192, 8192, 8192), (4096, 4096, 4096), (2048, 2048, 2048), (1024, 1024, 1024), (3000, 1500, 4500), (64, 65536, 1024),
-              (512, 8192, 512), (128, 16384, 2048)]
-SWEEP_FP16_VARIANTS = [1, 2, 7, 8, 9, 10, 15, 16, 17, 11]
+              (512, 8192, 512), (128, 16384, 2048),
+              # results that run as two launches (whole rounds of the 256x256 tile, then the rest); 20 = kept in one launch
+              (4352, 4096, 4352), (4013, 8192, 4775), (7336, 4096, 6806)]
+SWEEP_FP16_VARIANTS = [1, 2, 7, 8, 9, 10, 15, 16, 17, 11, 20]
 
 
 def sweep_one(capi, launch, set_variant, variants, budget_ms=25.0):

@@ -285,6 +285,17 @@ int decx_hip_set_hgemm_variant(int variant);
 int decx_hip_sgemm_plan(int M, int N, int K, int batch, long lda, long ldb, int aligned);
 int decx_hip_hgemm_plan(int M, int N, int K, int batch, long lda, long ldb, int aligned, int* splits);
 
+/* Host-only, like the two above: whether decx_hip_sgemm runs the product as two launches -- the rows (columns, when
+ * *by_columns is set to 1) that fill whole rounds of a 256-row tile, one tile per compute unit and round, on that tile
+ * (*shape = 26, 27 or 28), the rest on a kernel of its own choice (which may be split again) -- and how many rows
+ * (columns) the first launch takes; 0 = one launch (*shape = 0), -1 on bad sizes.  Either way every element is the same
+ * chain of products (GEMM.h:46 computes it in one launch).  decx_hip_set_sgemm_variant(34) keeps every product in
+ * one launch. */
+int decx_hip_sgemm_plan_split(int M, int N, int K, int batch, long lda, long ldb, int aligned, int* shape, int* by_columns);
+/* The same for decx_hip_hgemm_f32acc (GEMM.h:457-519 likewise): the first launch is on the 256x256 tile (variant 15);
+ * decx_hip_set_hgemm_variant(20) keeps every product in one launch. */
+int decx_hip_hgemm_plan_split(int M, int N, int K, int batch, long lda, long ldb, int aligned, int* by_columns);
+
 /* Host-only: 1 if the convolution kernels that work on patch-shaped tiles may run on a source tensor of these dimensions
  * (their 32-bit byte offsets, the apron's negative ones and the patches' reach past the output included, stay on the
  * right side of 2^31: see conv_patch_offsets_fit in backup_1_amd/csrc/runtime.hpp), 0 if the library takes its other

@@ -1,0 +1,94 @@
+"""Products that decx_hip_sgemm runs as two launches (whole rounds of a 256-row tile, then the rest on a kernel of its
+own choice; decx_hip_sgemm_plan_split says which): every element is the same chain of products whatever tile computes
+it, so the result has to be the one-launch result (decx_hip_set_sgemm_variant(34)) bit for bit -- on real-valued data,
+with and without "+ C", in place, with the ReLU epilogue -- and exact on small integers, at the seam above all.
+decx_hip_hgemm_f32acc does the same on its 256x256 tile (decx_hip_hgemm_plan_split; variant 20 = one launch): exact on
+small integers, and within the path's 2e-3 rule of the fp64 product on real-valued data on both sides of the seam."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from backup_1_amd import capi, workloads
+from gpu_helpers import gpu_sgemm, gpu_hgemm
+
+pytestmark = pytest.mark.gpu
+
+# (M, K, N): split by rows on the 256x256 tile, by columns on 256x224 and on 256x192, by rows on 256x192 with ragged edges
+SHAPES = [(4352, 512, 4352), (4096, 512, 4608), (2048, 512, 6212), (6324, 520, 5986)]
+
+
+def planned_split(M, K, N):
+    shape, by_columns = ctypes.c_int(0), ctypes.c_int(0)
+    first = capi.lib().decx_hip_sgemm_plan_split(M, N, K, 1, (K + 7) // 8 * 8, (N + 7) // 8 * 8, 1, ctypes.byref(shape), ctypes.byref(by_columns))
+    return first, shape.value, by_columns.value
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_two_launches_give_the_bits_of_one(gpu, shape):
+    M, K, N = shape
+    first, tile, by_columns = planned_split(M, K, N)
+    assert first > 0 and tile in (26, 27, 28), "the shape is meant to be one the library splits"
+    A, B, C = workloads.normal((M, K), 61), workloads.normal((K, N), 62), workloads.normal((M, N), 63)
+    for kwargs in ({}, {"C": C}, {"C": C, "inplace": True}, {"relu": True}):
+        two = gpu_sgemm(A, B, **kwargs)
+        one = gpu_sgemm(A, B, variant=34, **kwargs)
+        assert np.array_equal(two.view(np.uint32), one.view(np.uint32)), (shape, sorted(kwargs))
+
+
+@pytest.mark.parametrize("shape", SHAPES[:3])
+def test_two_launches_exact_on_small_integers(gpu, shape):
+    M, K, N = shape
+    assert planned_split(M, K, N)[0] > 0
+    A, B = workloads.small_ints((M, K), 64, -2, 2), workloads.small_ints((K, N), 65, -2, 2)
+    want = (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32)
+    got = gpu_sgemm(A, B)
+    assert np.array_equal(got, want), shape
+
+
+def test_rows_at_the_seam_match_the_oracle_chain(gpu, oracle):
+    M, K, N = SHAPES[0]
+    first, _, by_columns = planned_split(M, K, N)
+    assert first > 0 and not by_columns
+    A, B = workloads.normal((M, K), 66), workloads.normal((K, N), 67)
+    got = gpu_sgemm(A, B)
+    rows = [0, first - 1, first, first + 1, M - 1]
+    want = oracle.sgemm_chain(np.ascontiguousarray(A[rows]), B)
+    assert np.array_equal(got[rows].view(np.uint32), want.view(np.uint32))
+
+
+H_SHAPES = [(4352, 1024, 4352), (2048, 1024, 8448), (4013, 1032, 4775)]
+
+
+def planned_hsplit(M, K, N):
+    by_columns = ctypes.c_int(0)
+    first = capi.lib().decx_hip_hgemm_plan_split(M, N, K, 1, (K + 15) // 16 * 16, (N + 15) // 16 * 16, 1, ctypes.byref(by_columns))
+    return first, by_columns.value
+
+
+@pytest.mark.parametrize("shape", H_SHAPES)
+def test_fp16_two_launches_exact_on_small_integers(gpu, shape):
+    M, K, N = shape
+    assert planned_hsplit(M, K, N)[0] > 0, "the shape is meant to be one the library splits"
+    A, B = workloads.small_ints((M, K), 71, -1, 1), workloads.small_ints((K, N), 72, -1, 1)
+    C = workloads.small_ints((M, N), 73, -30, 30)
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    h = lambda x: x.astype(np.float16).view(np.uint16)
+    for with_c in (False, True):
+        two = gpu_hgemm(h(A), h(B), h(C) if with_c else None)
+        one = gpu_hgemm(h(A), h(B), h(C) if with_c else None, variant=20)
+        assert np.array_equal(two, one), (shape, with_c)
+        assert np.array_equal(two.view(np.float16).astype(np.float64), want + (C if with_c else 0.0)), (shape, with_c)
+
+
+def test_fp16_rows_around_the_seam_within_the_rule(gpu):
+    M, K, N = H_SHAPES[0]
+    first, by_columns = planned_hsplit(M, K, N)
+    assert first > 0 and not by_columns
+    A, B = workloads.normal((M, K), 74).astype(np.float16), workloads.normal((K, N), 75).astype(np.float16)
+    got = gpu_hgemm(A.view(np.uint16), B.view(np.uint16)).view(np.float16).astype(np.float64)
+    rows = [0, 1, first - 2, first - 1, first, first + 1, M - 2, M - 1]
+    ref = A[rows].astype(np.float64) @ B.astype(np.float64)
+    scale = np.abs(A[rows].astype(np.float64)) @ np.abs(B.astype(np.float64))
+    err = np.max((np.abs(got[rows] - ref) - np.abs(ref) / 2048.0) / np.maximum(scale, 1e-30))     # beyond the rounding of the result to binary16
+    assert err < 2e-3, err

@@ -84,6 +84,87 @@ def test_fp32_tall_results_take_the_tiles_that_pad_them_least(lib):
             assert not (K > 256 and v == 20 and N % 128 != 0 and N % 128 < 100), (M, K, N)
 
 
+def split_plan(lib, M, K, N, batch=1, lda=None, ldb=None, aligned=1):
+    shape, by_columns = ctypes.c_int(-1), ctypes.c_int(-1)
+    first = lib.decx_hip_sgemm_plan_split(M, N, K, batch, lda or pad(K, 8), ldb or pad(N, 8), aligned, ctypes.byref(shape), ctypes.byref(by_columns))
+    return first, shape.value, by_columns.value
+
+
+def test_fp32_two_launch_plans_are_whole_rounds_of_a_256_row_tile(lib):
+    """decx_hip_sgemm_plan_split over a grid: a first launch is whole tile rows (columns) of its tile that fit the whole
+    rounds of 256 compute units and leave something for the second launch; no plan for a forced variant, a batch, a short
+    K, operands the LDS-DMA tiles cannot take, or a result of whole rounds."""
+    widths = {26: 256, 27: 224, 28: 192}
+    planned = 0
+    for M in range(1500, 9000, 293):
+        for N in range(1500, 9000, 347):
+            for K in (512, 1500, 4096):
+                first, shape, by_columns = split_plan(lib, M, K, N)
+                if first == 0:
+                    assert shape == 0 and by_columns == 0
+                    continue
+                planned += 1
+                assert shape in widths, (M, K, N, shape)
+                tiles_m, tiles_n = -(-M // 256), -(-N // widths[shape])
+                whole = tiles_m * tiles_n // 256
+                assert whole >= 1 and tiles_m * tiles_n % 256 != 0
+                if by_columns:
+                    assert first % widths[shape] == 0 and 0 < first < N and first // widths[shape] * tiles_m <= whole * 256
+                    assert (first // widths[shape] + 1) * tiles_m > whole * 256        # as many columns as the rounds hold
+                else:
+                    assert first % 256 == 0 and 0 < first < M and first // 256 * tiles_n <= whole * 256
+                    assert (first // 256 + 1) * tiles_n > whole * 256
+                assert split_plan(lib, M, K, N, batch=2)[0] == 0
+                assert split_plan(lib, M, K, N, lda=DMA_MAX_PITCH)[0] == 0 and split_plan(lib, M, K, N, ldb=DMA_MAX_PITCH)[0] == 0
+                assert split_plan(lib, M, K, N, aligned=0)[0] == 0 and split_plan(lib, M, K, N, ldb=pad(N, 8) + 2)[0] == 0
+    assert planned > 100
+    # the measured ones: 4352^2 is 289 tiles of 256x256 -- 15 tile rows in one round, 512 rows left
+    assert split_plan(lib, 4352, 4096, 4352) == (3840, 26, 0)
+    assert split_plan(lib, 4096, 4096, 4608) == (3584, 27, 1) and split_plan(lib, 2048, 4096, 6212) == (6144, 28, 1)
+    for whole_rounds in ((8192, 8192, 8192), (4096, 4096, 4096), (6144, 6144, 6144), (3000, 1500, 4500), (1024, 1024, 1024)):
+        assert split_plan(lib, *whole_rounds)[0] == 0
+    assert split_plan(lib, 4352, 256, 4352)[0] == 0                                    # short K
+    for forced in (26, 7, 34):
+        lib.decx_hip_set_sgemm_variant(forced)
+        assert split_plan(lib, 4352, 4096, 4352)[0] == 0
+    lib.decx_hip_set_sgemm_variant(34)                                                 # 34 leaves the kernel choice alone
+    assert lib.decx_hip_sgemm_plan(4352, 4352, 4096, 1, 4096, 4352, 1) in FP32_TILES | FP32_DMA
+    lib.decx_hip_set_sgemm_variant(0)
+    assert split_plan(lib, 0, 8, 8)[0] == -1
+
+
+def test_fp16_two_launch_plans_are_whole_rounds_of_the_256_tile(lib):
+    def plan(M, K, N, batch=1, lda=None, ldb=None, aligned=1):
+        by_columns = ctypes.c_int(-1)
+        first = lib.decx_hip_hgemm_plan_split(M, N, K, batch, lda or pad(K, 16), ldb or pad(N, 16), aligned, ctypes.byref(by_columns))
+        return first, by_columns.value
+    planned = 0
+    for M in range(1500, 9000, 293):
+        for N in range(1500, 9000, 347):
+            for K in (512, 4096):
+                first, by_columns = plan(M, K, N)
+                if first == 0:
+                    continue
+                planned += 1
+                tiles_m, tiles_n = -(-M // 256), -(-N // 256)
+                whole = tiles_m * tiles_n // 256
+                assert whole >= 1 and tiles_m * tiles_n % 256 != 0 and first % 256 == 0
+                lines, across, extent = first // 256, (tiles_m if by_columns else tiles_n), (N if by_columns else M)
+                assert 0 < first < extent and lines * across <= whole * 256 < (lines + 1) * across
+                assert plan(M, K, N, batch=2)[0] == 0 and plan(M, K, N, aligned=0)[0] == 0 and plan(M, K, N, lda=pad(K, 16) + 4)[0] == 0
+    assert planned > 100
+    assert plan(4352, 4096, 4352) == (3840, 0)
+    for whole_rounds in ((8192, 8192, 8192), (4096, 4096, 4096), (3000, 1500, 4500), (1024, 1024, 1024), (64, 65536, 1024)):
+        assert plan(*whole_rounds)[0] == 0
+    assert plan(4352, 256, 4352)[0] == 0
+    for forced in (15, 8, 11, 20):
+        lib.decx_hip_set_hgemm_variant(forced)
+        assert plan(4352, 4096, 4352)[0] == 0
+    lib.decx_hip_set_hgemm_variant(20)                                                 # 20 leaves the kernel choice alone
+    assert lib.decx_hip_hgemm_plan(4352, 4352, 4096, 1, 4096, 4352, 1, None) in (8, 9, 15)
+    lib.decx_hip_set_hgemm_variant(0)
+
+
 def test_forced_fp32_variants_stay_where_they_can_run(lib):
     for forced in sorted(FP32_TILES | FP32_CHAINS | FP32_DMA):
         lib.decx_hip_set_sgemm_variant(forced)
