@@ -654,6 +654,27 @@ def main():
         also["fp32_ragged_3000x1500x4500"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
                                               "frac_of_fp32_matrix_peak": round(r["tflops_kernel"] / PEAK_FP32_MATRIX_TFLOPS, 4)}
         log("fp32 ragged: %.4f ms -> %.1f TFLOP/s" % (r["ms_wall"], r["tflops"]))
+        # a size that is no multiple of any tile: 289 tiles of 256x256 run as one round + 512 rows on smaller tiles
+        # (decx_hip_sgemm_plan_split); the same product kept in one launch beside it (variants 34 / 20)
+        L = capi.lib()
+        rows = 0 if args.no_verify else 8
+        r = bench_sgemm(capi, workloads, 4352, 4096, 4352, side_steps, side_warmup, 4400, verify_rows=rows)
+        prev = L.decx_hip_set_sgemm_variant(34)
+        one = bench_sgemm(capi, workloads, 4352, 4096, 4352, side_steps, side_warmup, 4400)
+        L.decx_hip_set_sgemm_variant(prev)
+        also["fp32_4352x4096x4352_two_launches"] = {"tflops": round(r["tflops"], 2), "ms_per_step": round(r["ms_wall"], 4),
+                                                    "frac_of_fp32_matrix_peak": round(r["tflops_kernel"] / PEAK_FP32_MATRIX_TFLOPS, 4),
+                                                    "verified": r.get("verified"), "verified_rows": r.get("verified_rows", 0),
+                                                    "one_launch_tflops": round(one["tflops"], 2), "one_launch_ms": round(one["ms_wall"], 4)}
+        h = bench_hgemm(capi, workloads, 0, side_steps, side_warmup, 4410, shape=(4352, 4096, 4352), verify_rows=rows)
+        prev = L.decx_hip_set_hgemm_variant(20)
+        hone = bench_hgemm(capi, workloads, 0, side_steps, side_warmup, 4410, shape=(4352, 4096, 4352))
+        L.decx_hip_set_hgemm_variant(prev)
+        also["fp16_4352x4096x4352_two_launches"] = {"tflops": round(h["tflops"], 2), "ms_per_step": round(h["ms_wall"], 4),
+                                                    "verified": h.get("verified"), "max_rel_err": h.get("max_rel_err"),
+                                                    "one_launch_tflops": round(hone["tflops"], 2), "one_launch_ms": round(hone["ms_wall"], 4)}
+        log("4352x4096x4352 in two launches: fp32 %.1f TFLOP/s (one launch %.1f), fp16 %.1f (one launch %.1f)"
+            % (r["tflops"], one["tflops"], h["tflops"], hone["tflops"]))
     if want("conv"):
         r = bench_conv(capi, workloads, side_steps, side_warmup)
         also["fp32_conv_224x224x64_128f3x3_fused_im2col"] = {
