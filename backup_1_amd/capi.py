@@ -24,7 +24,7 @@ SYMBOLS = [
     "decx_hip_sgemm_splitk", "decx_hip_sgemm_batched", "decx_hip_hgemm_f32acc_batched", "decx_hip_gemm3_host_f32", "decx_hip_gemm3_host_f16",
     "decx_hip_conv2_im2col_f32_fused", "decx_hip_conv2_im2col_f16", "decx_hip_conv2_im2col_f16_async", "decx_hip_sgemm_relu", "decx_hip_relu_f32", "decx_hip_relu_f32_async",
     "decx_hip_relu_f32_rec", "decx_hip_relu_f32_backward", "decx_hip_gemm_host_f32", "decx_hip_gemm_host_f16",
-    "decx_hip_b_read_extent", "decx_hip_sgemm_plan", "decx_hip_sgemm_plan_split", "decx_hip_hgemm_plan", "decx_hip_hgemm_plan_split", "decx_hip_conv_patch_offsets_fit", "decx_hip_set_splitk_mode", "decx_hip_hgemm_f32acc_noalloc", "decx_hip_release_tmp", "decx_hip_tmp_malloc", "decx_hip_tmp_free",
+    "decx_hip_b_read_extent", "decx_hip_sgemm_plan", "decx_hip_sgemm_plan_split", "decx_hip_hgemm_plan", "decx_hip_hgemm_plan_split", "decx_hip_conv_plan_split", "decx_hip_conv_patch_offsets_fit", "decx_hip_set_splitk_mode", "decx_hip_hgemm_f32acc_noalloc", "decx_hip_release_tmp", "decx_hip_tmp_malloc", "decx_hip_tmp_free",
 ]
 
 
@@ -81,6 +81,7 @@ def lib():
             "decx_hip_sgemm_plan": ([I, I, I, I, ctypes.c_long, ctypes.c_long, I], I),
             "decx_hip_sgemm_plan_split": ([I, I, I, I, ctypes.c_long, ctypes.c_long, I, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int)], I),
             "decx_hip_hgemm_plan_split": ([I, I, I, I, ctypes.c_long, ctypes.c_long, I, ctypes.POINTER(ctypes.c_int)], I),
+            "decx_hip_conv_plan_split": ([I, I, I, I, I, I, I, ctypes.POINTER(ctypes.c_int)], I),
             "decx_hip_hgemm_plan": ([I, I, I, I, ctypes.c_long, ctypes.c_long, I, PI], I),
             "decx_hip_conv_patch_offsets_fit": ([I, I, I, Z, I, I, I, I], I),
             "decx_hip_set_splitk_mode": ([I], I),

@@ -768,6 +768,14 @@ int decx_hip_sgemm_plan_split(int M, int N, int K, int batch, long lda, long ldb
     return sgemm_plan_split(M, N, K, batch, lda, ldb, aligned != 0, shape, by_columns);
 }
 
+int decx_hip_conv_plan_split(int H, int W, int dpitch, int N, int kh, int kw, int flag, int* shape) {
+    if (H <= 0 || W <= 0 || dpitch <= 0 || N <= 0 || kh <= 0 || kw <= 0) return -1;
+    const int Hout = flag ? H : H - 2 * (kh / 2), Wout = flag ? W : W - 2 * (kw / 2);
+    const long K = (long)kh * kw * dpitch;
+    if (Hout <= 0 || Wout <= 0 || K > 0x7fffffffL) return -1;
+    return conv_plan_split(Hout, Wout, N, (int)K, shape);
+}
+
 int decx_hip_hgemm_plan_split(int M, int N, int K, int batch, long lda, long ldb, int aligned, int* by_columns) {
     if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || lda < K || ldb < N) return -1;
     return hgemm_plan_split(M, N, K, batch, lda, ldb, aligned != 0, by_columns);

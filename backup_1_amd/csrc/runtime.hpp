@@ -90,6 +90,7 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
                   int ldd, int M, int N, int K, const Batch& batch);
 // host-only: which kernel the two entry points above take for a product of these sizes and pitches (no device call)
 int sgemm_plan(int M, int N, int K, int batch, long lda, long ldb, bool aligned);
+int conv_plan_split(int Hout, int Wout, int N, int K, int* shape);
 int sgemm_plan_split(int M, int N, int K, int batch, long lda, long ldb, bool aligned, int* shape, int* by_columns);
 int hgemm_plan(int M, int N, int K, int batch, long lda, long ldb, bool aligned, int* splits);
 int hgemm_plan_split(int M, int N, int K, int batch, long lda, long ldb, bool aligned, int* by_columns);

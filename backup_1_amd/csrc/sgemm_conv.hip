@@ -39,11 +39,39 @@ int launch_conv_chain16(const Im2colA<false>& img, const FilterB<false>& fb, con
     return 0;
 }
 
+namespace {
+// see conv_enqueue: image rows of the first of two launches, on the 256x256 tile (shape 7, one workgroup per CU), or
+// rows = 0 for one launch.  Only where one launch would take one of the big tiles, whose rounds the model counts right
+// (the 128x128 tile runs several workgroups per CU and does not come in rounds: measured, its products lose 1 - 2 %
+// when split); first launches on the 256x128 and 224x128 tiles lost 3 - 10 % on four shapes of five and are not planned.
+struct ConvRowsSplit {
+    int rows = 0, shape = 0;
+};
+ConvRowsSplit plan_conv_rows_split(int Hout, int Wout, int N, int K) {
+    ConvRowsSplit plan;
+    const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+    const long M = (long)Hout * Wout;
+    if (K < 512 || M > 0x7fffffffL) return plan;
+    double whole_cost = 0.0;
+    const int whole_shape = pick_sgemm_variant((int)M, N, K, 1, false, &whole_cost);
+    if (whole_cost == 0.0 || !(whole_shape == 7 || whole_shape == 10 || (whole_shape >= 3 && whole_shape <= 5) || whole_shape == 15)) return plan;
+    const long tiles_m = cdiv((int)M, 256), tiles_n = cdiv(N, 256), whole = tiles_m * tiles_n / cus;
+    if (whole < 1 || tiles_m * tiles_n % cus == 0) return plan;
+    const long rows = whole * cus / tiles_n * 256 / Wout;          // image rows whose tiles fit the whole rounds
+    if (rows < 1 || rows >= Hout) return plan;
+    double rest = 0.0;
+    (void)pick_sgemm_variant((int)((Hout - rows) * Wout), N, K, 1, false, &rest);
+    if (rest == 0.0) return plan;
+    if ((double)whole * 65536.0 + rest + 4.0 * 614.5e3 / (2.0 * K) < 0.96 * whole_cost) plan.rows = (int)rows, plan.shape = 7;
+    return plan;
+}
+}  // namespace
+
 int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stride, const float* filt, int N, int kh,
                  int kw, size_t filt_stride, size_t filt_row_stride, float* dst, int dst_dpitch, size_t dst_row_stride,
                  int flag, const float* bias, bool relu) {
     if (!g_rt.is_init) return need_init();
-    const bool small_kept_out = g_rt.sgemm_variant == 33;
+    const bool small_kept_out = g_rt.sgemm_variant == 33, one_launch = g_rt.sgemm_variant == 34;
     const ShapeForThisCall shape_for_this_call(small_kept_out || g_rt.sgemm_variant == 34 ? 0 : g_rt.sgemm_variant);
     if (flag != DECX_HIP_CONV_NO_COMPENSATE && flag != DECX_HIP_CONV_ZERO_COMPENSATE)
         return fail(DECX_HIP_FAIL_ERROR_FLAG, "This flag is meaningless in current context\n");   // core/error.h:67
@@ -137,19 +165,46 @@ int conv_enqueue(const float* src, int H, int W, int dpitch, size_t src_row_stri
             return launch_sconv_dma_shape(shape, a, b, bias, dst, out, M, N, K);
         }
     }
-    if (dpitch % 16 == 0) {      // a whole K step inside one tap: the tap walk runs on the scalar unit
-        Im2colAUniform a{{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes}};
-        FilterBUniform b{{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes}};
-        return conv_dispatch_uniform(variant, a, b, bias, dst, out, M, N, K, one);
+    // The register-staged tiles, on output rows row0 .. row0 + rows - 1: the loaders place output pixel m of the part at
+    // image row m / Wout - (oy - row0), so a part further down is the same launch with oy moved and dst advanced.
+    auto tiles_on_rows = [&](int shape, int row0, int rows) -> int {
+        const int part_m = rows * Wout, part_oy = oy - row0;
+        float* part_dst = dst + (size_t)row0 * dst_row_stride;
+        if (dpitch % 16 == 0) {      // a whole K step inside one tap: the tap walk runs on the scalar unit
+            Im2colAUniform a{{src, H, W, dpitch, kh, kw, part_oy, ox, Wout, part_m, K, (int)src_row_stride, (unsigned)src_bytes}};
+            FilterBUniform b{{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes}};
+            return conv_dispatch_uniform(shape, a, b, bias, part_dst, out, part_m, N, K, one);
+        }
+        if (dpitch % 8 == 0) {       // the 8 consecutive k of a staging task never straddle a tap
+            Im2colA<true> a{src, H, W, dpitch, kh, kw, part_oy, ox, Wout, part_m, K, (int)src_row_stride, (unsigned)src_bytes};
+            FilterB<true> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
+            return conv_dispatch_paired(shape, a, b, bias, part_dst, out, part_m, N, K, one);
+        }
+        Im2colA<false> a{src, H, W, dpitch, kh, kw, part_oy, ox, Wout, part_m, K, (int)src_row_stride, (unsigned)src_bytes};
+        FilterB<false> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
+        return conv_dispatch_plain(shape, a, b, bias, part_dst, out, part_m, N, K, one);
+    };
+    // Tiles that come in whole rounds plus a part of one (a round = one tile per CU) pay a whole round for the part.
+    // Every output element is the same chain of products whatever tile computes it, so the image rows that fill whole
+    // rounds of the 256x256 tile go to one launch and the rows below to a second one on the tile that is cheapest for
+    // them: taken where that costs under 96 % of the one launch, in the tile model's unit, 4 us for the second launch
+    // included (300x300x128 under 256 filters: 418 -> 383 us, 348x348x256 under 512: 2061 -> 1944).  Shape 34 keeps
+    // every convolution in one launch.
+    if (g_rt.sgemm_variant == 0 && !one_launch) {
+        const ConvRowsSplit split = plan_conv_rows_split(Hout, Wout, N, K);
+        if (split.rows > 0) {
+            if (int rc = tiles_on_rows(split.shape, 0, split.rows)) return rc;
+            return tiles_on_rows(pick_sgemm_variant((Hout - split.rows) * Wout, N, K, 1), split.rows, Hout - split.rows);
+        }
     }
-    if (dpitch % 8 == 0) {       // the 8 consecutive k of a staging task never straddle a tap
-        Im2colA<true> a{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
-        FilterB<true> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
-        return conv_dispatch_paired(variant, a, b, bias, dst, out, M, N, K, one);
-    }
-    Im2colA<false> a{src, H, W, dpitch, kh, kw, oy, ox, Wout, M, K, (int)src_row_stride, (unsigned)src_bytes};
-    FilterB<false> b{filt, N, K, dpitch, kw, (int)filt_stride, (int)filt_row_stride, (unsigned)filt_bytes};
-    return conv_dispatch_plain(variant, a, b, bias, dst, out, M, N, K, one);
+    return tiles_on_rows(variant, 0, Hout);
+}
+
+// host-only: the two-launch plan above for an output of Hout x Wout pixels under N filters (decx_hip_conv_plan_split)
+int conv_plan_split(int Hout, int Wout, int N, int K, int* shape) {
+    const ConvRowsSplit split = g_rt.sgemm_variant == 0 ? plan_conv_rows_split(Hout, Wout, N, K) : ConvRowsSplit();
+    if (shape) *shape = split.shape;
+    return split.rows;
 }
 
 }  // namespace decx_hip

@@ -431,8 +431,10 @@ SWEEP_FP32 = [(1024, 1024, 1024), (1536, 1536, 1536), (2048, 2048, 2048), (2560,
 SWEEP_FP32_VARIANTS = [2, 3, 4, 5, 7, 8, 9, 10, 14, 15, 16, 11, 12, 13, 23, 18, 19, 20, 21, 22, 24, 25, 26, 27, 28, 34]
 SWEEP_CONV = [(224, 224, 64, 128, 3), (112, 112, 128, 128, 3), (56, 56, 256, 256, 3), (28, 28, 512, 512, 3), (128, 128, 128, 128, 5),
               (512, 512, 256, 256, 3), (224, 224, 64, 64, 3), (96, 96, 128, 256, 3), (28, 28, 256, 256, 3), (14, 14, 512, 512, 3),
-              (180, 180, 128, 128, 3), (208, 208, 64, 128, 3), (256, 256, 64, 128, 3), (56, 56, 64, 256, 1)]
-SWEEP_CONV_VARIANTS = [2, 3, 4, 5, 7, 9, 10, 15, 16, 17, 11, 12, 13, 23, 29, 30, 31, 33]
+              (180, 180, 128, 128, 3), (208, 208, 64, 128, 3), (256, 256, 64, 128, 3), (56, 56, 64, 256, 1),
+              # two launches by output rows (whole rounds of the 256x256 tile, then the rest); 34 = kept in one launch
+              (300, 300, 128, 256, 3), (385, 385, 256, 256, 3)]
+SWEEP_CONV_VARIANTS = [2, 3, 4, 5, 7, 9, 10, 15, 16, 17, 11, 12, 13, 23, 29, 30, 31, 33, 34]
 SWEEP_FP16 = [(8192, 8192, 8192), (4096, 4096, 4096), (2048, 2048, 2048), (1024, 1024, 1024), (3000, 1500, 4500), (64, 65536, 1024),
               (512, 8192, 512), (128, 16384, 2048),
               # results that run as two launches (whole rounds of the 256x256 tile, then the rest); 20 = kept in one launch

@@ -295,6 +295,12 @@ int decx_hip_sgemm_plan_split(int M, int N, int K, int batch, long lda, long ldb
 /* The same for decx_hip_hgemm_f32acc (GEMM.h:457-519 likewise): the first launch is on the 256x256 tile (variant 15);
  * decx_hip_set_hgemm_variant(20) keeps every product in one launch. */
 int decx_hip_hgemm_plan_split(int M, int N, int K, int batch, long lda, long ldb, int aligned, int* by_columns);
+/* The same for decx_hip_conv2_im2col_f32 and its fused form (conv2_mk_im2col.h:167-274 runs one launch) where the
+ * convolution reaches the register-staged tiles (large images; the small-image, patch and block-chain kernels run in one
+ * launch): the output rows of the first launch, on tile *shape (7: 256x256), or 0.  The second
+ * launch computes the rows below with the same source tensor, so both sides of the seam see their real neighbours.
+ * decx_hip_set_sgemm_variant(34) keeps every convolution in one launch. */
+int decx_hip_conv_plan_split(int H, int W, int dpitch, int N, int kh, int kw, int flag, int* shape);
 
 /* Host-only: 1 if the convolution kernels that work on patch-shaped tiles may run on a source tensor of these dimensions
  * (their 32-bit byte offsets, the apron's negative ones and the patches' reach past the output included, stay on the

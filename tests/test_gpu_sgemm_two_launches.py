@@ -92,3 +92,33 @@ def test_fp16_rows_around_the_seam_within_the_rule(gpu):
     scale = np.abs(A[rows].astype(np.float64)) @ np.abs(B.astype(np.float64))
     err = np.max((np.abs(got[rows] - ref) - np.abs(ref) / 2048.0) / np.maximum(scale, 1e-30))     # beyond the rounding of the result to binary16
     assert err < 2e-3, err
+
+
+# (H, W, C, N, flag): convolutions that reach the register-staged tiles and split by output rows (decx_hip_conv_plan_split)
+CONV_SHAPES = [(274, 274, 64, 512, 1), (300, 300, 128, 256, 1), (350, 350, 96, 512, 0)]
+
+
+@pytest.mark.parametrize("shape", CONV_SHAPES)
+def test_convolution_in_two_launches(gpu, oracle, shape):
+    from gpu_helpers import gpu_conv
+    H, W, C, N, flag = shape
+    tile = ctypes.c_int(0)
+    rows = capi.lib().decx_hip_conv_plan_split(H, W, C, N, 3, 3, flag, ctypes.byref(tile))
+    assert rows > 0 and tile.value == 7, "the shape is meant to be one the library splits"
+    src, filt = workloads.normal((H, W, C), 81), 0.1 * workloads.normal((N, 3, 3, C), 82)
+    bias = workloads.normal((N,), 83)
+    two, one = gpu_conv(src, filt, flag), gpu_conv(src, filt, flag, variant=34)
+    assert np.array_equal(two.view(np.uint32), one.view(np.uint32)), shape
+    two, one = gpu_conv(src, filt, flag, bias=bias, relu=True), gpu_conv(src, filt, flag, variant=34, bias=bias, relu=True)
+    assert np.array_equal(two.view(np.uint32), one.view(np.uint32)), shape
+    # the output rows on both sides of the seam against the oracle's chain, computed on a crop of the image that gives
+    # every one of them its real neighbours
+    a, b = rows - 2, rows + 2
+    if flag:
+        crop = np.ascontiguousarray(src[a - 2:b + 2])
+        want = oracle.conv2_chain(crop, filt, 1)[2:2 + (b - a)]
+    else:
+        crop = np.ascontiguousarray(src[a:b + 2])                 # valid region: output row r reads image rows r .. r + 2
+        want = oracle.conv2_chain(crop, filt, 0)
+    got = gpu_conv(src, filt, flag)[a:b]
+    assert np.array_equal(got.view(np.uint32), np.ascontiguousarray(want).view(np.uint32)), shape

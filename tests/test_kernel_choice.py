@@ -165,6 +165,37 @@ def test_fp16_two_launch_plans_are_whole_rounds_of_the_256_tile(lib):
     lib.decx_hip_set_hgemm_variant(0)
 
 
+def test_convolution_two_launch_plans_are_whole_rounds_of_the_256_tile(lib):
+    def plan(H, W, C, N, k=3, flag=1):
+        shape = ctypes.c_int(-1)
+        rows = lib.decx_hip_conv_plan_split(H, W, C, N, k, k, flag, ctypes.byref(shape))
+        return rows, shape.value
+    planned = 0
+    for H in range(150, 1200, 37):
+        for C in (16, 48, 64, 128, 256):
+            for N in (32, 64, 128, 256, 384, 512):
+                for flag in (0, 1):
+                    rows, shape = plan(H, H + 3, C, N, flag=flag)
+                    if rows == 0:
+                        assert shape == 0
+                        continue
+                    planned += 1
+                    Hout, Wout = (H, H + 3) if flag else (H - 2, H + 1)
+                    tiles_n = -(-N // 256)
+                    whole = -(-Hout * Wout // 256) * tiles_n // 256
+                    assert shape == 7 and 0 < rows < Hout and whole >= 1 and 9 * C >= 512
+                    assert -(-rows * Wout // 256) * tiles_n <= whole * 256          # the first launch fits the whole rounds
+    assert planned > 20
+    assert plan(300, 300, 128, 256) == (218, 7)                        # measured: 418 -> 383 us
+    assert plan(224, 224, 64, 128)[0] == 0 and plan(512, 512, 256, 256)[0] == 0        # single round; four whole rounds
+    assert plan(300, 300, 16, 256)[0] == 0                             # K = 144: short
+    for forced in (7, 16, 34):
+        lib.decx_hip_set_sgemm_variant(forced)
+        assert plan(300, 300, 128, 256)[0] == 0
+    lib.decx_hip_set_sgemm_variant(0)
+    assert plan(0, 300, 128, 256)[0] == -1 and plan(2, 300, 128, 256, flag=0)[0] == -1
+
+
 def test_forced_fp32_variants_stay_where_they_can_run(lib):
     for forced in sorted(FP32_TILES | FP32_CHAINS | FP32_DMA):
         lib.decx_hip_set_sgemm_variant(forced)
