@@ -291,24 +291,29 @@ inline int plan_sgemm(int M, int N, int K, int batch, bool vec_a, bool vec_b, lo
 }
 
 // What one launch of the automatic choice costs, in the tile model's unit (tile area per CU / efficiency; times
-// 2 K / 614.5e3 it is microseconds), or 0 where the model has no figure.  A summary of the pickers above for the planner
-// below -- it decides nothing by itself.
-inline double sgemm_one_launch_cost(int M, int N, int K, int batch) {
+// 2 K / 614.5e3 it is microseconds), or 0 where the model has no figure (the block-chain kernels).  It prices the kernel
+// plan_sgemm answers, with the pickers' own figures; the planner below compares such prices, it picks no kernel.
+inline double sgemm_one_launch_cost(int M, int N, int K, int batch, long lda, long ldb) {
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
+    const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch, tiles32 = (long)cdiv(M, 32) * cdiv(N, 32) * batch;
+    auto rounds = [cus](long tiles) { return (double)((tiles + cus - 1) / cus); };
+    // cycles per k of the small LDS-DMA tiles (pick_dma_shape) in the model's unit: 614.5e3 / 2 / 2400 per cycle
+    const double per_cycle = 128.0;
+    const int plan = plan_sgemm(M, N, K, batch, true, true, lda, ldb);
+    switch (plan) {
+        case 26: return rounds((long)cdiv(M, 256) * cdiv(N, 256) * batch) * 65536.0 / 0.975;
+        case 27: return rounds((long)cdiv(M, 256) * cdiv(N, 224) * batch) * 57344.0 / 0.975;
+        case 28: return rounds((long)cdiv(M, 256) * cdiv(N, 192) * batch) * 49152.0 / 0.975;
+        case 20: return rounds((long)cdiv(M, 128) * cdiv(N, 128) * batch) * 16384.0 / 0.96;
+        case 18: case 19: return rounds(tiles64) * 34.2 * per_cycle;
+        case 24: case 25:
+            if (4 * tiles64 > 25 * cus) return (double)tiles32 / cus * 1024.0 / std::min(0.75, 0.93 * K / (K + 280.0));
+            return rounds(tiles32) * 9.7 * per_cycle;
+        case 11: case 12: case 13: case 23: return 0.0;
+        default: break;
+    }
     double cost = 0.0;
     pick_sgemm_variant(M, N, K, batch, true, &cost);
-    if (cost == 0.0) return 0.0;
-    const long tiles64 = (long)cdiv(M, 64) * cdiv(N, 64) * batch, tiles128 = (long)cdiv(M, 128) * cdiv(N, 128) * batch;
-    const long tiles32 = (long)cdiv(M, 32) * cdiv(N, 32) * batch;
-    auto rounds = [cus](long tiles) { return (double)((tiles + cus - 1) / cus); };
-    if (100.0 * M * N * batch >= 85.0 * 16384.0 * tiles128) cost = std::min(cost, rounds(tiles128) * 16384.0 / 0.96);
-    if (4 * tiles64 > 25 * cus) {
-        if (K >= 512)
-            for (int bn : {256, 224, 192}) cost = std::min(cost, rounds((long)cdiv(M, 256) * cdiv(N, bn) * batch) * 256.0 * bn / 0.975);
-    } else {
-        // cycles per k of the small LDS-DMA tiles (pick_dma_shape) in the model's unit: 614.5e3 / 2 / 2400 per cycle
-        cost = std::min(cost, std::min(34.2 * rounds(tiles64), 9.7 * rounds(tiles32)) * 128.0);
-    }
     return cost;
 }
 
@@ -328,7 +333,7 @@ inline WholeRoundsSplit plan_whole_rounds_split(int M, int N, int K, int batch, 
     if (g_rt.sgemm_variant != 0 || batch != 1 || K < 512 || lda >= kDmaMaxPitch || ldb >= kDmaMaxPitch) return plan;
     const long cus = g_rt.compute_units > 0 ? g_rt.compute_units : 256;
     if (4 * (long)cdiv(M, 64) * cdiv(N, 64) <= 25 * cus) return plan;
-    const double whole_cost = sgemm_one_launch_cost(M, N, K, 1);
+    const double whole_cost = sgemm_one_launch_cost(M, N, K, 1, lda, ldb);
     if (whole_cost == 0.0) return plan;
     double best = 0.96 * whole_cost;
     const double second_launch = 4.0 * 614.5e3 / (2.0 * K);
@@ -341,7 +346,7 @@ inline WholeRoundsSplit plan_whole_rounds_split(int M, int N, int K, int batch, 
             const long lines = whole * cus / (by_columns ? tiles_m : tiles_n);          // whole tile rows (columns) in the whole rounds
             if (lines < 1 || lines >= (by_columns ? tiles_n : tiles_m)) continue;
             const int first = (int)lines * (by_columns ? widths[i] : 256);
-            const double rest = by_columns ? sgemm_one_launch_cost(M, N - first, K, 1) : sgemm_one_launch_cost(M - first, N, K, 1);
+            const double rest = by_columns ? sgemm_one_launch_cost(M, N - first, K, 1, lda, ldb) : sgemm_one_launch_cost(M - first, N, K, 1, lda, ldb);
             if (rest == 0.0) continue;
             const double cost = first_cost + rest + second_launch;
             if (cost < best) {
