@@ -148,6 +148,72 @@ def bench_hgemm(capi, workloads, n, steps, warmup, seed, shape=None, verify_rows
     return out
 
 
+def bench_two_launch_ab(capi, seed=2024, count=40):
+    """Seeded random sizes (M, N in 1500..9000, K in 512..8192): each product as the library runs it (two launches where
+    decx_hip_*_plan_split says so) against the same product kept in one launch (variants 34 / 20), fp32 and fp16;
+    operands uniform in (-1, 1) uploaded once per size from a 64 MB host block, results compared (fp32: equal bits)."""
+    import ctypes
+    L = capi.lib()
+    rng = np.random.Generator(np.random.PCG64(seed))
+    block = (np.random.Generator(np.random.PCG64(seed + 1)).random(1 << 24, dtype=np.float32) * 2 - 1)
+    def fill(dev, count_elems, half):
+        src = block.astype(np.float16) if half else block
+        size = src.itemsize
+        for start in range(0, count_elems, src.size):
+            n = min(src.size, count_elems - start)
+            capi.check(L.decx_hip_memcpy(dev.ptr + start * size, src.ctypes.data, n * size, 1))
+    def timed(launch):
+        for _ in range(3):
+            launch()
+        capi.sync()
+        best = 1e9
+        for _ in range(3):
+            capi.timer_start()
+            for _ in range(8):
+                launch()
+            best = min(best, capi.timer_stop() / 8)
+        return best
+    rows = []
+    while len(rows) < count:
+        M, N = int(rng.integers(1500, 9000)), int(rng.integers(1500, 9000))
+        K = int(rng.choice([512, 1024, 1500, 2048, 4096, 8192]))
+        if 1.0 * M * N * K > 3.0e11:
+            continue
+        for half in (False, True):
+            unit, size = (16, 2) if half else (8, 4)
+            lda, ldb = (K + unit - 1) // unit * unit, (N + unit - 1) // unit * unit
+            tile, by_columns = ctypes.c_int(0), ctypes.c_int(0)
+            first = (L.decx_hip_hgemm_plan_split(M, N, K, 1, lda, ldb, 1, ctypes.byref(by_columns)) if half else
+                     L.decx_hip_sgemm_plan_split(M, N, K, 1, lda, ldb, 1, ctypes.byref(tile), ctypes.byref(by_columns)))
+            if first <= 0:
+                continue
+            dA, dB = capi.DeviceBuffer(M * lda * size), capi.DeviceBuffer(K * ldb * size)
+            dD, dE = capi.DeviceBuffer(M * ldb * size), capi.DeviceBuffer(M * ldb * size)
+            fill(dA, M * lda, half)
+            fill(dB, K * ldb, half)
+            gemm, knob, one_launch = ((capi.hgemm, L.decx_hip_set_hgemm_variant, 20) if half else
+                                      (capi.sgemm, L.decx_hip_set_sgemm_variant, 34))
+            t = {}
+            for v, dst in ((0, dD), (one_launch, dE), (0, dD), (one_launch, dE)):
+                knob(v)
+                t[v] = min(t.get(v, 1e9), timed(lambda: gemm(dA.ptr, lda, dB.ptr, ldb, dst.ptr, ldb, M, N, K, blocking=False)))
+            knob(0)
+            dt = np.uint16 if half else np.uint32
+            a, b = dD.download((M, ldb), dt)[:, :N], dE.download((M, ldb), dt)[:, :N]
+            if half:
+                same = bool(np.max(np.abs(a.view(np.float16).astype(np.float32) - b.view(np.float16).astype(np.float32))) <= 4e-3 * np.sqrt(K))
+            else:
+                same = bool(np.array_equal(a, b))
+            rows.append({"what": "%s %dx%dx%d (MxKxN)" % ("fp16" if half else "fp32", M, K, N),
+                         "first_launch": "%d %s" % (first, "columns" if by_columns.value else "rows") + ("" if half else " on tile %d" % tile.value),
+                         "two_launches_ms": round(t[0], 5), "one_launch_ms": round(t[one_launch], 5), "ratio": round(t[0] / t[one_launch], 4),
+                         "tflops": round(2.0 * M * N * K / t[0] / 1e9, 1), "one_launch_tflops": round(2.0 * M * N * K / t[one_launch] / 1e9, 1),
+                         "results_agree": same})
+            for d in (dA, dB, dD, dE):
+                d.free()
+    return rows
+
+
 LADDER_BUILDS = [(0, "2 LDS stages of 64 k, one tile per workgroup"), (1, "4 LDS stages of 32 k"), (2, "5 LDS stages of 32 k"),
                  (3, "2 LDS stages of 64 k, one workgroup per CU walks its tiles as one stream of K steps"),
                  (5, "2 LDS stages of 64 k, 4 waves of 128 x 128 (one per SIMD) instead of 8 of 128 x 64"),
@@ -576,7 +642,7 @@ def main():
     ap.add_argument("--sgemm-variant", type=int, default=0, help="force a fp32 tile shape (0 = automatic)")
     ap.add_argument("--hgemm-variant", type=int, default=0, help="force a fp16 tile shape (0 = automatic)")
     ap.add_argument("--no-verify", action="store_true", help="skip the post-run comparison of sampled rows with the oracle")
-    ap.add_argument("--only", default="", help="comma list of: headline,fp16,sq4096,small,ragged,conv,relu,host,cpu (default all); extra: ladder, copy, sweep")
+    ap.add_argument("--only", default="", help="comma list of: headline,fp16,sq4096,small,ragged,conv,relu,host,cpu (default all); extra: ladder, copy, sweep, twolaunch")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); --gpus %d is not supported. "
@@ -740,6 +806,12 @@ def main():
         for row in also["shape_choice_sweep"]:
             log("sweep, %-46s auto %-4s %9.5f ms | best forced %-3s %9.5f ms | auto / best %.3f"
                 % (row["what"], row["auto_variant"], row["auto_ms"], row["best_variant"], row["best_ms"], row["auto_over_best"]))
+    if "twolaunch" in only:
+        also["two_launch_ab"] = bench_two_launch_ab(capi)
+        for row in also["two_launch_ab"]:
+            log("two launches, %-34s first %-26s %9.4f ms (%6.1f TFLOP/s) | one launch %9.4f ms (%6.1f) | ratio %.3f%s"
+                % (row["what"], row["first_launch"], row["two_launches_ms"], row["tflops"], row["one_launch_ms"], row["one_launch_tflops"],
+                   row["ratio"], "" if row["results_agree"] else "  RESULTS DIFFER"))
     if "copy" in only:
         # calibration launch for the traffic counters: 1 GiB read + 1 GiB written by a plain copy kernel
         nbytes = 1 << 30
