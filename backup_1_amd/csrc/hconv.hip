@@ -135,7 +135,9 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
     }
     {
         if (take16) {
-            auto launch16 = [&](auto shape) -> int {
+            // on output rows row0 .. row0 + rows - 1: the kernel places output row y of the part at image row y - (oy - row0),
+            // so a part further down is the same launch with oy moved and dst advanced
+            auto launch16 = [&](auto shape, int row0, int rows) -> int {
                 typedef decltype(shape) S;
                 static bool attr_done = false;           // one per shape: the lambda's body is instantiated per S
                 if (!attr_done) {
@@ -143,15 +145,37 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
                                                 (int)S::LDS_BYTES));
                     attr_done = true;
                 }
+                HalfImage part_img = img;
+                part_img.oy = oy - row0, part_img.Mtot = rows * Wout;
+                HalfTensorOut part_out = out;
+                part_out.dst = out.dst + (size_t)row0 * dst_row_stride;
                 const int tn = cdiv(N, S::BN), tx = cdiv(Wout, S::PATCH_X);
-                hipLaunchKernelGGL(hconv_mfma16_kernel<S>, dim3((unsigned)(patches * tn)), dim3(S::NT), S::LDS_BYTES, g_rt.stream, img, fb, out,
-                                   Hout, N, tx, (int)patches, tn);
+                const long part_patches = (long)cdiv(rows, S::PATCH_Y) * tx;
+                hipLaunchKernelGGL(hconv_mfma16_kernel<S>, dim3((unsigned)(part_patches * tn)), dim3(S::NT), S::LDS_BYTES, g_rt.stream, part_img, fb,
+                                   part_out, rows, N, tx, (int)part_patches, tn);
                 HIP_TRY(hipGetLastError());
                 return 0;
             };
-            if (wide) return launch16(Hconv16Shape<256, 2, 4>{});      // 2x4 waves of 128 pixels x 64 filters
-            if (slim) return launch16(Hconv16Shape<64, 8, 1>{});       // 8x1 waves of 32 pixels x 64 filters
-            return launch16(Hconv16Shape<128, 4, 2>{});                // 4x2 waves of 64 pixels x 64 filters
+            auto launch_rows = [&](int row0, int rows) -> int {
+                const long part_patches = (long)cdiv(rows, 16) * cdiv(Wout, 16);
+                if (N > 128 && 2 * part_patches * cdiv(N, 256) >= cus) return launch16(Hconv16Shape<256, 2, 4>{}, row0, rows);      // 2x4 waves of 128 pixels x 64 filters
+                if (N <= 64 || 2 * part_patches * cdiv(N, 128) <= cus) return launch16(Hconv16Shape<64, 8, 1>{}, row0, rows);      // 8x1 waves of 32 pixels x 64 filters
+                return launch16(Hconv16Shape<128, 4, 2>{}, row0, rows);                // 4x2 waves of 64 pixels x 64 filters
+            };
+            // The 256-filter tiles run one per CU: tiles beyond whole rounds of them pay a round of their own (268x268x128
+            // under 256 filters, 289 tiles: 58.4 us where 256 tiles take 35.7), and a nearly empty round still costs two
+            // thirds of a full one.  While the part is at most a quarter of a round, the image rows that fill the whole
+            // rounds go to one launch and the rows below to a second one on tiles that suit their count (hgemm variant 20
+            // keeps one launch).
+            if (wide && g_rt.hgemm_variant == 0) {
+                const long row_tiles = (long)cdiv(Wout, 16) * cdiv(N, 256), whole = tiles16 / cus, part = tiles16 % cus;
+                const long first = whole * cus / row_tiles * 16;          // image rows whose tiles fit the whole rounds
+                if (whole >= 1 && part > 0 && 4 * part <= cus && first >= 16 && first < Hout) {
+                    if (int rc = launch16(Hconv16Shape<256, 2, 4>{}, 0, (int)first)) return rc;
+                    return launch_rows((int)first, Hout - (int)first);
+                }
+            }
+            return launch_rows(0, Hout);
         }
     }
     // filters 3, 5 or 7 wide: the LDS-DMA kernel that loads a tap row's pixels once for all of its taps, if a tile's patch

@@ -122,3 +122,36 @@ def test_convolution_in_two_launches(gpu, oracle, shape):
         want = oracle.conv2_chain(crop, filt, 0)
     got = gpu_conv(src, filt, flag)[a:b]
     assert np.array_equal(got.view(np.uint32), np.ascontiguousarray(want).view(np.uint32)), shape
+
+
+@pytest.mark.parametrize("shape", [(260, 264, 128, 256, 1), (358, 362, 64, 512, 0)])
+def test_fp16_convolution_in_two_launches(gpu, oracle, shape):
+    """289 (1058) tiles of 256 pixels x 256 filters on 256 compute units: whole rounds of them, then the rows below on tiles of
+    their own.  The same bits as one launch (hgemm variant 20), with bias and ReLU too, and the rows around the seam --
+    image row 240 (352) -- within the path's 2e-3 rule of the fp64 convolution of the same binary16 tensors."""
+    from gpu_helpers import gpu_hconv
+    H, W, C, N, flag = shape
+    src = workloads.normal((H, W, C), 91).astype(np.float16)
+    filt = (0.1 * workloads.normal((N, 3, 3, C), 92)).astype(np.float16)
+    bias = workloads.normal((N,), 93).astype(np.float16)
+    two, sbuf, fbuf = gpu_hconv(src, filt, flag)
+    one, _, _ = gpu_hconv(src, filt, flag, variant=20)
+    assert np.array_equal(two.view(np.uint16), one.view(np.uint16)), shape
+    two_b, _, _ = gpu_hconv(src, filt, flag, bias16=bias, relu=True)
+    one_b, _, _ = gpu_hconv(src, filt, flag, bias16=bias, relu=True, variant=20)
+    assert np.array_equal(two_b.view(np.uint16), one_b.view(np.uint16)), shape
+    Hout = H if flag else H - 2
+    tiles_per_patch_row = -(-(W if flag else W - 2) // 16) * -(-N // 256)
+    seam = (-(-Hout // 16) * tiles_per_patch_row // 256) * 256 // tiles_per_patch_row * 16
+    assert 0 < seam < Hout
+    a, b = seam - 3, seam + 3
+    if flag:
+        crop = np.ascontiguousarray(sbuf[a - 2:b + 2])
+        ref, scale = oracle.conv2_f64_f16(crop, fbuf, 1)
+        ref, scale = ref[2:2 + (b - a)], scale[2:2 + (b - a)]
+    else:
+        crop = np.ascontiguousarray(sbuf[a:b + 2])
+        ref, scale = oracle.conv2_f64_f16(crop, fbuf, 0)
+    got = two[a:b].astype(np.float64)
+    err = np.max((np.abs(got - ref) - np.abs(ref) / 2048.0) / np.maximum(scale, 1e-30))
+    assert err < 2e-3, (shape, err)
