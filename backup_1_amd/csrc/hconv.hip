@@ -162,16 +162,17 @@ int hconv_enqueue(const uint16_t* src, int H, int W, int dpitch, size_t src_row_
                 if (N <= 64 || 2 * part_patches * cdiv(N, 128) <= cus) return launch16(Hconv16Shape<64, 8, 1>{}, row0, rows);      // 8x1 waves of 32 pixels x 64 filters
                 return launch16(Hconv16Shape<128, 4, 2>{}, row0, rows);                // 4x2 waves of 64 pixels x 64 filters
             };
-            // The 256-filter tiles run one per CU: tiles beyond whole rounds of them pay a round of their own (268x268x128
-            // under 256 filters, 289 tiles: 58.4 us where 256 tiles take 35.7), and a nearly empty round still costs two
-            // thirds of a full one.  While the part is at most a quarter of a round, the image rows that fill the whole
-            // rounds go to one launch and the rows below to a second one on tiles that suit their count (hgemm variant 20
-            // keeps one launch).
+            // The tiles run one per CU: tiles beyond whole rounds of them pay a round of their own (268x268x128 under 256
+            // filters, 289 tiles: 58.4 us where 256 tiles take 35.7), and a nearly empty round still costs two thirds of
+            // a full one.  With the 256-filter tiles, while the part is at most a quarter of a round, the image rows that
+            // fill the whole rounds go to one launch and the rows below to a second one on narrower tiles, which spread
+            // them over the chip (hgemm variant 20 keeps one launch).  Not with the narrower tiles: measured, under 128
+            // filters the second launch gains 0 - 2 %, and under 64, where it has no narrower tile to go to, loses 4 - 22 %.
             if (wide && g_rt.hgemm_variant == 0) {
                 const long row_tiles = (long)cdiv(Wout, 16) * cdiv(N, 256), whole = tiles16 / cus, part = tiles16 % cus;
                 const long first = whole * cus / row_tiles * 16;          // image rows whose tiles fit the whole rounds
                 if (whole >= 1 && part > 0 && 4 * part <= cus && first >= 16 && first < Hout) {
-                    if (int rc = launch16(Hconv16Shape<256, 2, 4>{}, 0, (int)first)) return rc;
+                    if (int rc = launch_rows(0, (int)first)) return rc;
                     return launch_rows((int)first, Hout - (int)first);
                 }
             }
