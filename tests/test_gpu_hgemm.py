@@ -107,7 +107,7 @@ def test_split_k_is_the_same_on_every_run(gpu, oracle):
         capi.lib().decx_hip_set_splitk_mode(prev)
 
 
-@pytest.mark.parametrize("shape", [(4352, 128, 4352), (4352, 384, 4608), (1024, 256, 69632 + 256)])
+@pytest.mark.parametrize("shape", [(4352, 128, 4352), (4352, 384, 4608), (1024, 256, 69632 + 256), (4096, 640, 8192)])
 def test_one_workgroup_per_cu_walking_its_tiles(gpu, oracle, shape):
     # variant 17: more whole 256x256 tiles than compute units, one workgroup per CU walks several of them as one stream
     # of K steps (the next tile's first loads are issued during the last steps of the tile before).  Every accumulator
@@ -126,6 +126,9 @@ def test_one_workgroup_per_cu_walking_its_tiles(gpu, oracle, shape):
     walked = gpu_hgemm(A, B, variant=17)
     assert np.array_equal(walked, one_tile)
     assert np.array_equal(gpu_hgemm(A, B, C, variant=17), gpu_hgemm(A, B, C, variant=15))
+    if 512 <= K <= 3072:      # where the automatic choice takes the walk by itself
+        assert capi.lib().decx_hip_hgemm_plan(M, N, K, 1, (K + 15) // 16 * 16, (N + 15) // 16 * 16, 1, None) == 17
+        assert np.array_equal(gpu_hgemm(A, B), one_tile) and np.array_equal(gpu_hgemm(A, B, C), gpu_hgemm(A, B, C, variant=15))
     rows = np.random.Generator(np.random.PCG64(56)).choice(M, size=24, replace=False).astype(np.int32)
     ref, scale = oracle.gemm_f64_rows_f16(A, B, rows)
     assert rel_err_vs_abs_scale(from_bits(walked[rows]), ref, scale) < TOL

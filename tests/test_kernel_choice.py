@@ -218,8 +218,10 @@ def test_fp16_choice_over_a_grid_of_shapes(lib):
         for batch in (1, 3):
             lda, ldb = pad(K, 16), pad(N, 16)
             v = lib.decx_hip_hgemm_plan(M, N, K, batch, lda, ldb, 1, ctypes.byref(splits))
-            assert v in {8, 9, 11, 15}, (M, N, K, batch, v)                      # the automatic choices
+            assert v in {8, 9, 11, 15, 17}, (M, N, K, batch, v)                  # the automatic choices
             seen.add(v)
+            if v == 17:          # the walk over several tiles: whole tiles only, more of them than CUs, the measured range of K
+                assert batch == 1 and M % 256 == 0 and N % 256 == 0 and K % 128 == 0 and 512 <= K <= 3072 and (M // 256) * (N // 256) > 256
             if v == 11:
                 assert batch == 1 and splits.value >= 2 and K // splits.value >= 512
                 assert M * N * 4 * splits.value <= RESERVED_WORKSPACE, (M, N, K, splits.value)
@@ -227,7 +229,7 @@ def test_fp16_choice_over_a_grid_of_shapes(lib):
                 assert splits.value == 0
             assert lib.decx_hip_hgemm_plan(M, N, K, batch, lda, ldb, 0, None) == 0
             assert lib.decx_hip_hgemm_plan(M, N, K, batch, lda + 4, ldb, 1, None) == 0
-    assert seen == {8, 9, 11, 15}
+    assert seen == {8, 9, 11, 15, 17}
     # a 256-row tile of A beyond 4 GiB, 64 rows of B beyond 4 GiB: the element-wise kernel, which uses 64-bit addresses
     assert lib.decx_hip_hgemm_plan(300, 260, 200, 1, 1 << 23, 272, 1, None) == 0
     assert lib.decx_hip_hgemm_plan(300, 260, 200, 1, 208, 1 << 25, 1, None) == 0
