@@ -268,12 +268,12 @@ static int plan_hgemm(int M, int N, int K, int batch_count, bool vec, int* split
         const double cost_small = (double)((small + cus - 1) / cus) * 16384.0 / 0.75;
         // the small tile with three LDS stages holds one workgroup per CU: only worth it when there is at most one to hold
         variant = cost_big <= cost_small ? 15 : (small <= cus ? 9 : 8);
-        // several rounds of whole 256x256 tiles on a K of 512 .. 3072 (the measured range): one workgroup per CU that walks its tiles as one
+        // several rounds of whole 256x256 tiles on a K of 128 .. 3072 (the measured range; the walk needs K >= 128): one workgroup per CU that walks its tiles as one
         // stream of K steps (17) has no prologue after the first tile and stores under the next tile's loads, which a
-        // short K walk cannot hide otherwise -- 8192x512x8192 85.0 -> 75.2 us, x1024 126.8 -> 117.9, x2048 215.8 -> 210.7,
+        // short K walk cannot hide otherwise -- 8192x128x8192 49.4 -> 40.2 us, x256 58.7 -> 50.2, 16384x256x8192 105.2 -> 84.9, 8192x512x8192 85.0 -> 75.2, x1024 126.8 -> 117.9, x2048 215.8 -> 210.7,
         // x3072 307.2 -> 300.7, 6144x1024x8192 93.8 -> 87.4; level at 8192^3 (770.1 against 772.7), behind by 1 % on a
         // single round (4096x1024x4096), where hgemm_mfma16_persistent_fits says no anyway
-        if (variant == 15 && batch_count == 1 && K >= 512 && K <= 3072 && hgemm_mfma16_persistent_fits<HShape16>(M, N, K, Batch())) variant = 17;
+        if (variant == 15 && batch_count == 1 && K <= 3072 && hgemm_mfma16_persistent_fits<HShape16>(M, N, K, Batch())) variant = 17;
     }
     return variant;
 }
@@ -335,7 +335,7 @@ int hgemm_enqueue(const uint16_t* A, int lda, const uint16_t* B, int ldb, const 
     const HgemmWholeRoundsSplit split = plan_hgemm_whole_rounds_split(M, N, K, batch.count, vec);
     // the first launch of a split: whole rounds of the 256x256 tile, as the stream of K steps where plan_hgemm would take that
     auto whole_rounds = [&](int rows, int cols) -> int {
-        if (K >= 512 && K <= 3072 && hgemm_mfma16_persistent_fits<HShape16>(rows, cols, K, batch))
+        if (K <= 3072 && hgemm_mfma16_persistent_fits<HShape16>(rows, cols, K, batch))
             return launch_hgemm_mfma16_persistent<HShape16>(A, lda, B, ldb, Cin, ldc, D, ldd, rows, cols, K, batch);
         return launch_hgemm_mfma16<HShape16>(A, lda, B, ldb, Cin, ldc, D, ldd, rows, cols, K, batch);
     };

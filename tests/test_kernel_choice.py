@@ -221,7 +221,7 @@ def test_fp16_choice_over_a_grid_of_shapes(lib):
             assert v in {8, 9, 11, 15, 17}, (M, N, K, batch, v)                  # the automatic choices
             seen.add(v)
             if v == 17:          # the walk over several tiles: whole tiles only, more of them than CUs, the measured range of K
-                assert batch == 1 and M % 256 == 0 and N % 256 == 0 and K % 128 == 0 and 512 <= K <= 3072 and (M // 256) * (N // 256) > 256
+                assert batch == 1 and M % 256 == 0 and N % 256 == 0 and K % 128 == 0 and 128 <= K <= 3072 and (M // 256) * (N // 256) > 256
             if v == 11:
                 assert batch == 1 and splits.value >= 2 and K // splits.value >= 512
                 assert M * N * 4 * splits.value <= RESERVED_WORKSPACE, (M, N, K, splits.value)
